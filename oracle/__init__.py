@@ -1,0 +1,263 @@
+"""TEST INFRASTRUCTURE — CPU oracle of the sparse message-passing path.
+
+`oracle.c` restates the reference's single-threaded CPU loops in plain C;
+this module loads it with ctypes and adds numpy restatements of the Python
+code either side of those loops (graph normalisation, the GAT composition,
+the layer wrappers).  Only tests, the smoke check and the CPU-baseline leg of
+the benchmark import this package; the shipped library never does.
+
+Functions with no independent pin (see oracle.c header for the pins of the
+rest): none of the arithmetic.  The cuSPARSE-internal summation order behind
+the reference's SpmmCsr is "parity unpinned" (third-party, jittor==1.3.9.14).
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "liboracle.so")
+
+
+def build(force=False):
+    """Compile oracle.c (gcc, single thread, AVX+FMA) into liboracle.so."""
+    if force or not os.path.exists(_SO) or os.path.getmtime(_SO) < os.path.getmtime(
+            os.path.join(_HERE, "oracle.c")):
+        subprocess.check_call(["make", "-C", _HERE, "-B", "liboracle.so"],
+                              stdout=subprocess.DEVNULL)
+    return _SO
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_SO):
+            build()
+        _lib = ctypes.CDLL(_SO)
+    return _lib
+
+
+def _p(a):
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+def _i32(a):
+    a = np.ascontiguousarray(a, dtype=np.int32)
+    return a
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+# ---------------------------------------------------------------- C loops ---
+
+def cootocsr(edge_index, edge_weight, v_num):
+    """ops/cootocsr.py:28-35 -> ops/cpp/cootocsr_op.cc:24-57.
+    Returns (column_indices, row_offset, csr_edge_weight)."""
+    ei = _i32(edge_index)
+    w = _f32(edge_weight)
+    E = ei.shape[1]
+    col = np.zeros(E, np.int32)
+    off = np.zeros(v_num + 1, np.int32)
+    wo = np.zeros(E, np.float32)
+    rc = lib().orc_cootocsr(_p(ei), _p(w), ctypes.c_int64(E), ctypes.c_int32(v_num),
+                            _p(col), _p(off), _p(wo))
+    assert rc == 0
+    return col, off, wo
+
+
+def cootocsc(edge_index, edge_weight, v_num):
+    """ops/cootocsc.py:29-36 -> ops/cpp/cootocsc_op.cc:23-53.
+    Returns (row_indices, column_offset, csc_edge_weight)."""
+    ei = _i32(edge_index)
+    w = _f32(edge_weight)
+    E = ei.shape[1]
+    row = np.zeros(E, np.int32)
+    off = np.zeros(v_num + 1, np.int32)
+    wo = np.zeros(E, np.float32)
+    rc = lib().orc_cootocsc(_p(ei), _p(w), ctypes.c_int64(E), ctypes.c_int32(v_num),
+                            _p(row), _p(off), _p(wo))
+    assert rc == 0
+    return row, off, wo
+
+
+def aggregate(x, indices, offset, weight, scalar=False):
+    """ops/cpp/aggregate_op.cc:26-71: out[i,:] = sum_j w[j] * x[indices[j],:]
+    over j in [offset[i], offset[i+1]).  The number of output rows is x's
+    (aggregate_op.cc:33), as in the reference."""
+    x = _f32(x)
+    indices, offset, weight = _i32(indices), _i32(offset), _f32(weight)
+    v_num, F = x.shape
+    assert offset.shape[0] == v_num + 1
+    out = np.empty_like(x)
+    fn = lib().orc_aggregate_scalar if scalar else lib().orc_aggregate
+    fn(_p(out), _p(x), _p(indices), _p(offset), _p(weight), ctypes.c_int32(v_num),
+       ctypes.c_int32(F))
+    return out
+
+
+def edgesoftmax(x, offset):
+    """ops/cpp/edgesoftmax_op.cc:36-66.  x is [E], [E,1] (reference shapes) or
+    [E,H] (independent heads)."""
+    x = _f32(x)
+    offset = _i32(offset)
+    H = 1 if x.ndim == 1 else x.shape[1]
+    out = np.zeros_like(x)
+    if H == 1:
+        lib().orc_edgesoftmax(_p(out), _p(x), _p(offset), ctypes.c_int32(offset.shape[0] - 1))
+    else:
+        lib().orc_edgesoftmax_heads(_p(out), _p(x), _p(offset),
+                                    ctypes.c_int32(offset.shape[0] - 1), ctypes.c_int32(H))
+    return out
+
+
+def edgesoftmax_backward(grad, y, offset):
+    """ops/cpp/edgesoftmaxbackward_op.cc:27-54."""
+    grad, y = _f32(grad), _f32(y)
+    offset = _i32(offset)
+    H = 1 if y.ndim == 1 else y.shape[1]
+    out = np.zeros_like(y)
+    lib().orc_edgesoftmax_backward(_p(out), _p(grad), _p(y), _p(offset),
+                                   ctypes.c_int32(offset.shape[0] - 1), ctypes.c_int32(H))
+    return out
+
+
+def scattertoedge(x, indices, offset, flag):
+    """ops/cpp/scattertoedge_op.cc:67-88; flag 0 = by source (row_indices),
+    flag 1 = by destination (the column the edge sits in)."""
+    x = _f32(x)
+    indices, offset = _i32(indices), _i32(offset)
+    E, F = indices.shape[0], x.shape[1]
+    out = np.empty((E, F), np.float32)
+    lib().orc_scattertoedge(_p(out), _p(x), _p(indices), _p(offset),
+                            ctypes.c_int32(offset.shape[0] - 1), ctypes.c_int64(E),
+                            ctypes.c_int32(F), ctypes.c_int32(flag))
+    return out
+
+
+def edgetovertex(x, indices, offset, flag, out_rows=None):
+    """ops/cpp/edgetovertex_op.cc:36-55."""
+    x = _f32(x)
+    indices, offset = _i32(indices), _i32(offset)
+    v_num = offset.shape[0] - 1
+    out_rows = v_num if out_rows is None else out_rows
+    F = x.shape[1]
+    out = np.empty((out_rows, F), np.float32)
+    lib().orc_edgetovertex(_p(out), _p(x), _p(indices), _p(offset), ctypes.c_int32(v_num),
+                           ctypes.c_int32(out_rows), ctypes.c_int32(F), ctypes.c_int32(flag))
+    return out
+
+
+# ------------------------------------------------- numpy: graph preprocessing
+
+def add_remaining_self_loops(edge_index, edge_weight=None, fill_value=1.0, num_nodes=None):
+    """utils/loop.py:98-136: drop existing self-loops, append (i,i) for every
+    node at the END; a dropped loop's weight becomes that node's loop weight
+    (the last one wins when a node had several)."""
+    edge_index = np.asarray(edge_index)
+    N = int(edge_index.max()) + 1 if num_nodes is None else int(num_nodes)
+    row, col = edge_index[0], edge_index[1]
+    mask = row != col
+    loop_index = np.arange(N, dtype=edge_index.dtype)
+    out_index = np.concatenate([edge_index[:, mask], np.stack([loop_index, loop_index])], axis=1)
+    out_w = None
+    if edge_weight is not None:
+        edge_weight = np.asarray(edge_weight, dtype=np.float32)
+        loop_w = np.full(N, fill_value, np.float32)
+        inv = ~mask
+        if inv.any():
+            loop_w[row[inv]] = edge_weight[inv]
+        out_w = np.concatenate([edge_weight[mask], loop_w])
+    return out_index, out_w
+
+
+def _degree_by_col(col, w, N):
+    deg = np.zeros(N, np.float32)
+    np.add.at(deg, col, w)            # jt.scatter(..., reduce='add')
+    return deg
+
+
+def gcn_norm(edge_index, edge_weight=None, num_nodes=None, improved=False, add_self_loops=True):
+    """nn/conv/gcn_conv.py:18-37: w = d^-1/2[row] * w * d^-1/2[col] with the
+    degree summed by column, inf -> 0."""
+    edge_index = np.asarray(edge_index)
+    N = int(edge_index.max()) + 1 if num_nodes is None else int(num_nodes)
+    fill = 2.0 if improved else 1.0
+    if edge_weight is None:
+        edge_weight = np.ones(edge_index.shape[1], np.float32)
+    if add_self_loops:
+        edge_index, edge_weight = add_remaining_self_loops(edge_index, edge_weight, fill, N)
+    row, col = edge_index[0], edge_index[1]
+    deg = _degree_by_col(col, edge_weight, N)
+    with np.errstate(divide="ignore"):
+        dis = np.power(deg, np.float32(-0.5)).astype(np.float32)
+    dis[np.isinf(dis)] = 0
+    return edge_index, (dis[row] * edge_weight * dis[col]).astype(np.float32)
+
+
+def sage_norm(edge_index, edge_weight=None, num_nodes=None, improved=False, add_self_loops=True):
+    """nn/conv/sage_conv.py:16-40: w = w * d^-1[col]."""
+    edge_index = np.asarray(edge_index)
+    N = int(edge_index.max()) + 1 if num_nodes is None else int(num_nodes)
+    fill = 2.0 if improved else 1.0
+    if edge_weight is None:
+        edge_weight = np.ones(edge_index.shape[1], np.float32)
+    if add_self_loops:
+        edge_index, edge_weight = add_remaining_self_loops(edge_index, edge_weight, fill, N)
+    col = edge_index[1]
+    deg = _degree_by_col(col, edge_weight, N)
+    with np.errstate(divide="ignore"):
+        di = np.power(deg, np.float32(-1.0)).astype(np.float32)
+    di[np.isinf(di)] = 0
+    return edge_index, (edge_weight * di[col]).astype(np.float32)
+
+
+# ------------------------------------------------------ numpy: op wrappers ---
+
+def aggregate_with_weight(x, csc, csr=None):
+    """ops/aggregateWithWeight.py:20-30: forward feeds the CSC arrays.
+    csc = (row_indices, column_offset, edge_weight)."""
+    return aggregate(x, csc[0], csc[1], csc[2])
+
+
+def aggregate_with_weight_grad(grad_out, csr):
+    """ops/aggregateWithWeight.py:32-41: backward feeds the CSR arrays.
+    csr = (column_indices, row_offset, edge_weight)."""
+    return aggregate(grad_out, csr[0], csr[1], csr[2])
+
+
+def gat_forward(h, csc, a, slope=0.2):
+    """nn/conv/gat_conv.py:61-83 after vertex_forward: h is [V,C] (already
+    relu(x@W)), a is the [2C,1] attention vector.  Returns (out, alpha, m).
+    Single head, float32 throughout like the reference."""
+    row, off = _i32(csc[0]), _i32(csc[1])
+    h = _f32(h)
+    C = h.shape[1]
+    e_src = scattertoedge(h, row, off, 0)
+    e_dst = scattertoedge(h, row, off, 1)
+    e = np.concatenate([e_src, e_dst], axis=1)
+    out = (e @ _f32(a).reshape(2 * C, 1)).astype(np.float32)
+    m = np.where(out > 0, out, np.float32(slope) * out).astype(np.float32)
+    alpha = edgesoftmax(m, off)
+    msg = e[:, :C] * alpha
+    res = edgetovertex(msg, row, off, 1)
+    return res, alpha, m
+
+
+def gat_forward_heads(h, csc, a_src, a_dst, slope=0.2):
+    """Multi-head generalisation: h [V,H,D], a_src/a_dst [H,D]; head k is
+    gat_forward on h[:,k,:] with a = concat(a_src[k], a_dst[k]).
+    Returns (out [V,H,D], alpha [E,H])."""
+    V, H, D = h.shape
+    outs, alphas = [], []
+    for k in range(H):
+        a = np.concatenate([a_src[k], a_dst[k]]).astype(np.float32)
+        o, al, _ = gat_forward(np.ascontiguousarray(h[:, k, :]), csc, a, slope)
+        outs.append(o)
+        alphas.append(al[:, 0])
+    return np.stack(outs, axis=1), np.stack(alphas, axis=1)

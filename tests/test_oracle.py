@@ -1,0 +1,273 @@
+"""Pins the CPU oracle: reference fixtures, closed forms, library routines,
+invariants.  A mistake in oracle.c (dropped term, wrong index, transposed
+operand) must fail at least one of these.  No GPU needed."""
+import json
+import os
+
+import numpy as np
+import pytest
+import scipy.sparse as sp
+from scipy.special import softmax as sp_softmax
+
+import oracle
+
+GOLD = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_fixtures.json")))
+
+
+def closed_form_csx(edge_index, w, V, key_row):
+    """Stable counting sort written with library calls only."""
+    key = edge_index[key_row]
+    other = edge_index[1 - key_row]
+    perm = np.argsort(key, kind="stable")
+    off = np.concatenate([[0], np.cumsum(np.bincount(key, minlength=V))]).astype(np.int32)
+    return other[perm].astype(np.int32), off, w[perm].astype(np.float32), perm
+
+
+def rand_graph(rng, V, E, loops=True):
+    ei = rng.integers(0, V, size=(2, E)).astype(np.int32)
+    if not loops:
+        ei = ei[:, ei[0] != ei[1]]
+    w = rng.standard_normal(ei.shape[1]).astype(np.float32)
+    return ei, w
+
+
+# ------------------------------------------------------------- conversion ---
+
+@pytest.mark.parametrize("name", ["csr_v4", "mp_spmm_v10"])
+def test_conversion_reference_fixtures(name):
+    g = GOLD[name]
+    ei = np.array(g["edge_index"], np.int32)
+    w = np.array(g["edge_weight"], np.float32)
+    col, off, wo = oracle.cootocsr(ei, w, g["v_num"])
+    assert col.tolist() == g["csr"]["column_indices"]
+    assert off.tolist() == g["csr"]["row_offset"]
+    assert wo.tolist() == g["csr"]["edge_weight"]
+    row, coff, cw = oracle.cootocsc(ei, w, g["v_num"])
+    assert row.tolist() == g["csc"]["row_indices"]
+    assert coff.tolist() == g["csc"]["column_offset"]
+    assert cw.tolist() == g["csc"]["edge_weight"]
+
+
+def test_conversion_readme_csc_to_csr_known_answer():
+    g = GOLD["csctocsr_readme_v4"]
+    off = np.array(g["column_offset"])
+    dst = np.repeat(np.arange(len(off) - 1), np.diff(off)).astype(np.int32)
+    ei = np.stack([np.array(g["row_indices"], np.int32), dst])
+    col, roff, _ = oracle.cootocsr(ei, np.ones(ei.shape[1], np.float32), 4)
+    assert roff.tolist() == g["row_offset"]
+    assert col.tolist() == g["column_indices"]
+
+
+@pytest.mark.parametrize("V,E,seed", [(1, 0, 0), (1, 5, 1), (7, 0, 2), (50, 400, 3), (1000, 30000, 4),
+                                      (5000, 5000, 5)])
+def test_conversion_closed_form_and_invariants(V, E, seed):
+    rng = np.random.default_rng(seed)
+    ei, w = rand_graph(rng, V, E)
+    for key_row, fn in ((0, oracle.cootocsr), (1, oracle.cootocsc)):
+        idx, off, wo = fn(ei, w, V)
+        cidx, coff, cw, perm = closed_form_csx(ei, w, V, key_row)
+        assert np.array_equal(idx, cidx) and np.array_equal(off, coff)
+        assert np.array_equal(wo.view(np.int32), cw.view(np.int32))
+        assert off[0] == 0 and off[-1] == ei.shape[1] and np.all(np.diff(off) >= 0)
+        # within a row the original edge ids increase strictly (stability)
+        keys_sorted = ei[key_row][perm]
+        same = keys_sorted[1:] == keys_sorted[:-1]
+        assert np.all(perm[1:][same] > perm[:-1][same])
+
+
+def test_conversion_bruteforce_tiny():
+    rng = np.random.default_rng(11)
+    for _ in range(20):
+        V = int(rng.integers(1, 6))
+        E = int(rng.integers(0, 12))
+        ei, w = rand_graph(rng, V, E)
+        col, off, wo = oracle.cootocsr(ei, w, V)
+        slots = []
+        for r in range(V):
+            for e in range(E):
+                if ei[0, e] == r:
+                    slots.append(e)
+        assert col.tolist() == [int(ei[1, e]) for e in slots]
+        assert wo.tolist() == [float(w[e]) for e in slots]
+
+
+# ------------------------------------------------------------------- SpMM ---
+
+def test_aggregate_reference_fixture_integer_exact():
+    g = GOLD["mp_spmm_v10"]
+    x = np.array(g["x"], np.float32)
+    ei = np.array(g["edge_index"], np.int32)
+    w = np.array(g["edge_weight"], np.float32)
+    csc = oracle.cootocsc(ei, w, 10)
+    out = oracle.aggregate_with_weight(x, csc)
+    for r, vals in g["aggregate_rows"].items():
+        assert out[int(r)].tolist() == [float(v) for v in vals]
+    dense = np.zeros((10, 10))
+    dense[ei[1], ei[0]] += w                      # out[dst] += w * x[src]
+    assert np.array_equal(out, (dense @ x.astype(np.float64)).astype(np.float32))
+
+
+def test_aggregate_spmmcsr_fixture():
+    g = GOLD["spmmcsr_v3"]
+    x = np.array(g["x"], np.float32)
+    col = np.array(g["column_indices"], np.int32)
+    off = np.array(g["row_offset"], np.int32)
+    w = np.array(g["edge_weight"], np.float32)
+    assert oracle.aggregate(x, col, off, w).tolist() == g["out_no_trans"]
+    src = np.repeat(np.arange(3), np.diff(off)).astype(np.int32)
+    csc = oracle.cootocsc(np.stack([src, col]), w, 3)
+    assert oracle.aggregate(x, *csc).tolist() == g["out_trans_A"]
+
+
+@pytest.mark.parametrize("V,E,F,seed", [(64, 600, 7, 0), (64, 600, 8, 1), (300, 5000, 33, 2),
+                                        (200, 3000, 128, 3), (50, 0, 16, 4)])
+def test_aggregate_vs_scipy_fp64_and_transpose_identity(V, E, F, seed):
+    rng = np.random.default_rng(seed)
+    ei, w = rand_graph(rng, V, E)
+    x = rng.standard_normal((V, F)).astype(np.float32)
+    g = rng.standard_normal((V, F)).astype(np.float32)
+    csc = oracle.cootocsc(ei, w, V)
+    csr = oracle.cootocsr(ei, w, V)
+    A = sp.coo_matrix((w.astype(np.float64), (ei[1], ei[0])), shape=(V, V)).tocsr()
+    fwd = oracle.aggregate_with_weight(x, csc)
+    bwd = oracle.aggregate_with_weight_grad(g, csr)
+    np.testing.assert_allclose(fwd, A @ x.astype(np.float64), rtol=1e-5, atol=2e-5)
+    np.testing.assert_allclose(bwd, A.T @ g.astype(np.float64), rtol=1e-5, atol=2e-5)
+    # <A x, g> == <x, A^T g>
+    lhs = np.sum(fwd.astype(np.float64) * g)
+    rhs = np.sum(x.astype(np.float64) * bwd)
+    assert abs(lhs - rhs) <= 1e-4 * max(1.0, abs(lhs))
+    # AVX branch and scalar branch sum in the same order per feature
+    sc = oracle.aggregate(x, *csc, scalar=True)
+    np.testing.assert_allclose(fwd, sc, rtol=1e-6, atol=1e-6)
+
+
+# ----------------------------------------------------------- edge softmax ---
+
+def test_edgesoftmax_reference_fixture():
+    g = GOLD["edgesoftmax_v3"]
+    y = oracle.edgesoftmax(np.array(g["x"], np.float32), np.array(g["column_offset"], np.int32))
+    np.testing.assert_allclose(y, np.array(g["y"]), rtol=1e-6, atol=0)
+
+
+@pytest.mark.parametrize("H", [1, 2, 8])
+def test_edgesoftmax_vs_scipy_and_invariants(H):
+    rng = np.random.default_rng(5 + H)
+    V, E = 200, 3000
+    ei, w = rand_graph(rng, V, E)
+    _, off, _ = oracle.cootocsc(ei, w, V)
+    x = (3 * rng.standard_normal((E, H))).astype(np.float32)
+    y = oracle.edgesoftmax(x if H > 1 else x[:, 0], off)
+    y = y.reshape(E, H)
+    for v in range(V):
+        s, e = off[v], off[v + 1]
+        if e > s:
+            np.testing.assert_allclose(y[s:e], sp_softmax(x[s:e].astype(np.float64), axis=0),
+                                       rtol=2e-6, atol=1e-7)
+            np.testing.assert_allclose(y[s:e].sum(0), 1.0, rtol=1e-5)
+    y2 = oracle.edgesoftmax((x + np.float32(2.0)) if H > 1 else (x + np.float32(2.0))[:, 0], off)
+    np.testing.assert_allclose(y2.reshape(E, H), y, rtol=1e-5, atol=1e-7)   # shift invariance
+    # [E,1] input is the reference's GAT shape and equals the [E] answer
+    if H == 1:
+        assert np.array_equal(oracle.edgesoftmax(x, off)[:, 0], y[:, 0])
+
+
+@pytest.mark.parametrize("H", [1, 4])
+def test_edgesoftmax_backward_closed_form_and_finite_difference(H):
+    rng = np.random.default_rng(21 + H)
+    V, E = 40, 300
+    ei, w = rand_graph(rng, V, E)
+    _, off, _ = oracle.cootocsc(ei, w, V)
+    x = rng.standard_normal((E, H)).astype(np.float32)
+    g = rng.standard_normal((E, H)).astype(np.float32)
+    y = oracle.edgesoftmax(x, off).reshape(E, H)
+    dx = oracle.edgesoftmax_backward(g, y, off).reshape(E, H)
+    seg = np.repeat(np.arange(V), np.diff(off))
+    dot = np.zeros((V, H))
+    np.add.at(dot, seg, y.astype(np.float64) * g)
+    np.testing.assert_allclose(dx, y * (g - dot[seg]), rtol=1e-5, atol=1e-6)
+    segsum = np.zeros((V, H))
+    np.add.at(segsum, seg, dx)
+    np.testing.assert_allclose(segsum, 0, atol=1e-5)
+    # finite differences of the fp64 closed-form forward along a random direction
+    def f64(xx):
+        out = np.zeros_like(xx)
+        for v in range(V):
+            s, e = off[v], off[v + 1]
+            if e > s:
+                out[s:e] = sp_softmax(xx[s:e], axis=0)
+        return out
+    d = rng.standard_normal((E, H))
+    eps = 1e-6
+    fd = (np.sum(f64(x + eps * d) * g) - np.sum(f64(x - eps * d) * g)) / (2 * eps)
+    assert abs(fd - np.sum(dx * d)) < 1e-4 * max(1.0, abs(fd))
+
+
+# ------------------------------------------------------------ scatter ops ---
+
+def test_scatter_ops_vs_numpy():
+    rng = np.random.default_rng(3)
+    V, E, F = 60, 500, 5
+    ei, w = rand_graph(rng, V, E)
+    row, off, _ = oracle.cootocsc(ei, w, V)
+    dst = np.repeat(np.arange(V), np.diff(off))
+    x = rng.standard_normal((V, F)).astype(np.float32)
+    xe = rng.standard_normal((E, F)).astype(np.float32)
+    assert np.array_equal(oracle.scattertoedge(x, row, off, 0), x[row])
+    assert np.array_equal(oracle.scattertoedge(x, row, off, 1), x[dst])
+    for flag, tgt in ((0, row), (1, dst)):
+        ref = np.zeros((V, F))
+        np.add.at(ref, tgt, xe.astype(np.float64))
+        np.testing.assert_allclose(oracle.edgetovertex(xe, row, off, flag), ref, rtol=1e-5, atol=1e-5)
+
+
+# ---------------------------------------------------------- normalisation ---
+
+def test_add_remaining_self_loops_order_and_weights():
+    ei = np.array([[0, 1, 1, 2, 2], [1, 1, 2, 2, 0]], np.int32)
+    w = np.array([1, 7, 2, 9, 3], np.float32)
+    oi, ow = oracle.add_remaining_self_loops(ei, w, 1.0, 4)
+    assert oi.tolist() == [[0, 1, 2, 0, 1, 2, 3], [1, 2, 0, 0, 1, 2, 3]]
+    assert ow.tolist() == [1, 2, 3, 1, 7, 9, 1]
+
+
+def test_gcn_and_sage_norm_closed_forms():
+    rng = np.random.default_rng(8)
+    V = 30
+    ei, _ = rand_graph(rng, V, 200, loops=False)
+    oi, ow = oracle.gcn_norm(ei, None, V)
+    assert oi.shape[1] == ei.shape[1] + V and np.array_equal(oi[:, -V:], np.stack([np.arange(V)] * 2))
+    deg = np.bincount(oi[1], minlength=V).astype(np.float64)       # integer degrees, exact
+    np.testing.assert_allclose(ow, 1 / np.sqrt(deg[oi[0]] * deg[oi[1]]), rtol=1e-6)
+    si, sw = oracle.sage_norm(ei, None, V)
+    np.testing.assert_allclose(sw, 1 / deg[si[1]], rtol=1e-6)
+    # mean aggregation: every column of the normalised adjacency sums to 1
+    colsum = np.zeros(V)
+    np.add.at(colsum, si[1], sw)
+    np.testing.assert_allclose(colsum, 1, rtol=1e-5)
+
+
+# ------------------------------------------------------------ GAT pieces ----
+
+def test_gat_forward_matches_dense_fp64():
+    rng = np.random.default_rng(13)
+    V, E, C = 50, 400, 6
+    ei, w = rand_graph(rng, V, E)
+    csc = oracle.cootocsc(ei, w, V)
+    h = np.maximum(rng.standard_normal((V, C)), 0).astype(np.float32)
+    a = rng.standard_normal(2 * C).astype(np.float32)
+    out, alpha, _ = oracle.gat_forward(h, csc, a)
+    ref = np.zeros((V, C))
+    for v in range(V):
+        srcs = ei[0][ei[1] == v]
+        if len(srcs) == 0:
+            continue
+        z = h[srcs].astype(np.float64) @ a[:C] + h[v].astype(np.float64) @ a[C:]
+        z = np.where(z > 0, z, 0.2 * z)
+        al = sp_softmax(z)
+        ref[v] = al @ h[srcs]
+    np.testing.assert_allclose(out, ref, rtol=1e-4, atol=1e-5)
+    o8, a8 = oracle.gat_forward_heads(np.stack([h, 2 * h], 1), csc, np.stack([a[:C], a[:C]]),
+                                      np.stack([a[C:], a[C:]]))
+    np.testing.assert_allclose(o8[:, 0], out, rtol=1e-6, atol=1e-7)
+    assert a8.shape == (E, 2)
