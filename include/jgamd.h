@@ -1,0 +1,181 @@
+/*
+ * jgamd — C ABI of the MI355X (gfx950) sparse message-passing kernels.
+ *
+ * Drop-in boundary for the native half of jittor_geometric.ops: every entry
+ * point replaces one Jittor custom Op (or one jittor-wheel cuSPARSE op) of the
+ * reference; the citation above each declaration names it.
+ *
+ * Conventions (all entry points):
+ *   - extern "C", plain pointers and sizes; no C++ or torch types.
+ *   - All data pointers are DEVICE pointers to contiguous arrays; indices are
+ *     int32, values fp32 (the only combination the reference's hot path uses:
+ *     data/data.py:103-106 casts edge_index to int32).
+ *   - Work is enqueued on `stream` (a hipStream_t passed as void*; NULL is the
+ *     default stream).  Nothing synchronises the device; nothing allocates or
+ *     frees device memory: scratch comes in through `ws` / `ws_bytes`, sized by
+ *     the matching *_workspace() query (host-only arithmetic, needs no GPU).
+ *   - Return value: 0 = enqueued; negative = argument error found on the host
+ *     (nothing was enqueued); positive = a hipError_t from a launch.
+ *     jgamd_last_error() returns a thread-local description of the last
+ *     non-zero status.
+ *   - Outputs are overwritten (beta = 0); they need not be zeroed by the
+ *     caller, unlike the reference ops which accumulate into zero-filled Vars.
+ *   - Calls are re-entrant; two calls may overlap on one GPU when they use
+ *     different workspaces and outputs.
+ */
+#ifndef JGAMD_H
+#define JGAMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define JGAMD_OK 0
+#define JGAMD_ERR_NULL (-1)        /* a required pointer is NULL              */
+#define JGAMD_ERR_SIZE (-2)        /* negative / overflowing / inconsistent size */
+#define JGAMD_ERR_WORKSPACE (-3)   /* ws is NULL or smaller than the query says */
+#define JGAMD_ERR_UNSUPPORTED (-4) /* shape outside what the kernels handle   */
+#define JGAMD_ERR_ALIGN (-5)       /* pointer not 4-byte aligned              */
+
+/* Library version, major*10000 + minor*100 + patch. */
+int32_t jgamd_version(void);
+/* Thread-local text of the last error returned on this thread ("" if none). */
+const char *jgamd_last_error(void);
+
+/* ------------------------------------------------------------------------
+ * COO -> CSR / CSC.
+ * Replaces CootocsrOp::jit_run (ops/cpp/cootocsr_op.cc:24-57, Python wrapper
+ * ops/cootocsr.py:28-35) with key_row = 0 and CootocscOp::jit_run
+ * (ops/cpp/cootocsc_op.cc:23-53, ops/cootocsc.py:29-36) with key_row = 1.
+ *
+ *   edge_index [2,E] row-major: row 0 = source, row 1 = destination
+ *   key_row    0: group by source (CSR; out_idx = destinations)
+ *              1: group by destination (CSC; out_idx = sources)
+ *   out_off    [V+1]  out_idx [E]  out_w [E]
+ *   out_perm   optional [E]: original edge id stored at each output slot
+ *              (NULL to skip).  Not produced by the reference; used to move
+ *              per-edge tensors between the CSR and CSC orders.
+ *
+ * Result is bit-identical to the reference: a stable counting sort, i.e.
+ * inside a row the edges keep their input order; weights are copied.
+ * Edges whose key is outside [0,V) are dropped (the reference would write out
+ * of bounds); the tail of out_idx/out_w is then left untouched.
+ * Limits: 0 <= E < 2^31 - 2^20, 0 <= V < 2^31 - 1.
+ */
+int32_t jgamd_coo_to_csx_workspace(int64_t E, int32_t V, int32_t with_perm, size_t *bytes);
+int32_t jgamd_coo_to_csx(const int32_t *edge_index, const float *edge_weight, int64_t E,
+                         int32_t V, int32_t key_row, int32_t *out_idx, int32_t *out_off,
+                         float *out_w, int32_t *out_perm, void *ws, size_t ws_bytes,
+                         void *stream);
+
+/* Transpose of a compressed structure (CSR of an R x C matrix -> CSC arrays of
+ * the same matrix, or the reverse): expands the row ids and runs the stable
+ * conversion keyed on idx.  No single reference op; it is what
+ * SpmmCsr(trans_A=True) (ops/spmmcsr.py:31, cuSPARSE op(A)=T inside the
+ * jittor wheel) and the flag-0 edgetovertex backward
+ * (ops/cpp/edgetovertex_op.cc:36-45) need to run as gathers instead of
+ * scatters.  out_off has C+1 entries.  out_w / out_perm / w may be NULL.
+ */
+int32_t jgamd_csx_transpose_workspace(int64_t E, int32_t R, int32_t C, size_t *bytes);
+int32_t jgamd_csx_transpose(const int32_t *off, const int32_t *idx, const float *w, int32_t R,
+                            int32_t C, int64_t E, int32_t *out_off, int32_t *out_idx,
+                            float *out_w, int32_t *out_perm, void *ws, size_t ws_bytes,
+                            void *stream);
+
+/* ------------------------------------------------------------------------
+ * Weighted row-gather SpMM:  out[r,:] = sum_{j in [off[r],off[r+1])} w[j] * x[idx[j],:]
+ * Replaces AggregateOp::jit_run (ops/cpp/aggregate_op.cc:26-71 CPU,
+ * :74-106 CUDA; wrapper ops/aggregateWithWeight.py:20-41: forward passes the
+ * CSC arrays, backward the CSR arrays) and cusparse_ops.cusparse_spmmcsr as
+ * called by ops/spmmcsr.py:31,37.
+ *
+ *   off [R+1], idx [E], w [E], x [C,F] (leading dimension F), out [R,F]
+ *   idx == NULL means idx[j] = j (x is then per-edge, [E,F]); w == NULL means 1.
+ *   With those two the same entry point is EdgetovertexOp::jit_run
+ *   (ops/cpp/edgetovertex_op.cc:36-55): flag 1 = (idx NULL, w NULL) over the
+ *   CSC offsets; flag 0 = (idx = perm, w NULL) over the transposed offsets.
+ *
+ * Rows are summed in edge order inside one wavefront's share of the edges and
+ * pieces of a row that span several wavefronts are added in edge order by a
+ * second kernel: results are run-to-run reproducible (no float atomics) and
+ * agree with the sequential reference sum to fp32 rounding.
+ * Entries with idx outside [0,C) contribute nothing.
+ * Limits: E + R < 2^31, 1 <= F <= 65535*2048.
+ */
+int32_t jgamd_spmm_csx_workspace(int32_t R, int64_t E, int32_t F, size_t *bytes);
+int32_t jgamd_spmm_csx(const int32_t *off, const int32_t *idx, const float *w, const float *x,
+                       float *out, int32_t R, int32_t C, int64_t E, int32_t F, void *ws,
+                       size_t ws_bytes, void *stream);
+
+/* ------------------------------------------------------------------------
+ * Edge softmax over the in-edges of every destination (CSC column).
+ * Replaces EdgesoftmaxOp::jit_run (ops/cpp/edgesoftmax_op.cc:36-66, the
+ * max-subtracted CPU form; wrapper ops/edgesoftmax.py:62-69) and
+ * EdgesoftmaxbackwardOp::jit_run (ops/cpp/edgesoftmaxbackward_op.cc:27-54,
+ * wrapper ops/edgesoftmax.py:71-74).
+ *   x, y, g, dx are [E,H] row-major; H = 1 is the reference's shape ([E] or
+ *   [E,1]); H > 1 treats every head as an independent softmax.
+ *   fwd:  y = exp(x - max_col) / sum_col exp(x - max_col)
+ *   bwd:  dx = y*g - y*sum_col(y*g)
+ */
+int32_t jgamd_edge_softmax_fwd(const int32_t *off, const float *x, float *y, int32_t V,
+                               int64_t E, int32_t H, void *stream);
+int32_t jgamd_edge_softmax_bwd(const int32_t *off, const float *y, const float *g, float *dx,
+                               int32_t V, int64_t E, int32_t H, void *stream);
+
+/* ------------------------------------------------------------------------
+ * Vertex -> edge copy.  Replaces ScattertoedgeOp::jit_run
+ * (ops/cpp/scattertoedge_op.cc:67-88 CPU, :91-137 CUDA; wrapper
+ * ops/scatterToEdge.py:22-40).  flag 0: out[e,:] = x[idx[e],:] ("src");
+ * flag 1: out[e,:] = x[v,:] for every e in column v ("dst").
+ *   off [V+1], idx [E], x [V,F], out [E,F].
+ */
+int32_t jgamd_scatter_to_edge(const int32_t *off, const int32_t *idx, const float *x,
+                              float *out, int32_t V, int64_t E, int32_t F, int32_t flag,
+                              void *stream);
+
+/* ------------------------------------------------------------------------
+ * Fused GAT layer core (attention logits + edge softmax + weighted
+ * aggregation) over the CSC arrays.  Replaces the op chain of
+ * GATConv.propagate (nn/conv/gat_conv.py:61-83): ScatterToEdge x2, concat,
+ * [E,2C]x[2C,1] product, leaky_relu, EdgeSoftmax, multiply, ScatterToVertex.
+ *   h      [V,H,D]   node features after vertex_forward
+ *   a_src  [H,D], a_dst [H,D]  the two halves of GATConv.edge_weight
+ *   el,er  [V,H]  outputs: a_src.h and a_dst.h per node and head
+ *   smax, ssum [V,H] outputs: per destination and head, the max logit and
+ *          the sum of exp(logit - max) (what backward needs to rebuild alpha)
+ *   alpha  optional [E,H] output (NULL to skip): attention per CSC slot
+ *   out    [V,H,D]:  out[v,k,:] = sum_e alpha[e,k] * h[idx[e],k,:]
+ * H = 1, D = C reproduces the reference's single head.
+ */
+int32_t jgamd_gat_fwd_workspace(int32_t V, int64_t E, int32_t H, int32_t D, size_t *bytes);
+int32_t jgamd_gat_fwd(const int32_t *off, const int32_t *idx, const float *h,
+                      const float *a_src, const float *a_dst, float slope, float *el,
+                      float *er, float *smax, float *ssum, float *alpha, float *out,
+                      int32_t V, int64_t E, int32_t H, int32_t D, void *ws, size_t ws_bytes,
+                      void *stream);
+
+/* Backward of jgamd_gat_fwd.  Needs both orders of the graph: (off, idx) are
+ * the CSC arrays used forward, (t_off, t_idx) the transposed (CSR) arrays of
+ * the same edges (jgamd_csx_transpose or cootocsr).
+ *   g_out [V,H,D] upstream gradient, out [V,H,D] forward result
+ *   g_h   [V,H,D], g_a_src [H,D], g_a_dst [H,D] outputs
+ * Replaces the grad chain edgetovertex <-> scattertoedge <->
+ * edgesoftmaxbackward that Jittor autograd builds for gat_conv.py:61-83.
+ */
+int32_t jgamd_gat_bwd_workspace(int32_t V, int64_t E, int32_t H, int32_t D, size_t *bytes);
+int32_t jgamd_gat_bwd(const int32_t *off, const int32_t *idx, const int32_t *t_off,
+                      const int32_t *t_idx, const float *h, const float *a_src,
+                      const float *a_dst, float slope, const float *el, const float *er,
+                      const float *smax, const float *ssum, const float *out,
+                      const float *g_out, float *g_h, float *g_a_src, float *g_a_dst,
+                      int32_t V, int64_t E, int32_t H, int32_t D, void *ws, size_t ws_bytes,
+                      void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* JGAMD_H */

@@ -1,0 +1,57 @@
+// Shared host/device helpers for the gfx950 kernels (wave64 everywhere).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/jgamd.h"
+
+namespace jg {
+
+constexpr int kWave = 64;
+
+// Records a message for jgamd_last_error() and returns `code`.
+int32_t fail(int32_t code, const char *fmt, ...);
+// Checks the launch that was just enqueued; returns 0 or the hipError_t.
+int32_t launch_status(const char *what);
+
+inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Bump allocator over the caller's workspace (256-byte granules).
+struct Carver {
+    char *base;
+    size_t used = 0;
+    explicit Carver(void *p) : base(static_cast<char *>(p)) {}
+    template <typename T> T *take(size_t n)
+    {
+        T *r = reinterpret_cast<T *>(base + used);
+        used += align_up(n * sizeof(T), 256);
+        return r;
+    }
+};
+inline size_t carve_bytes(size_t n, size_t elem) { return align_up(n * elem, 256); }
+
+// ---- device-wide exclusive scan over int32 (scan.hip) ---------------------
+// out[i] = sum(in[0..i-1]); in == out allowed.  sums_ws needs
+// scan_ws_ints(n) int32 of scratch.
+size_t scan_ws_ints(int64_t n);
+int32_t exclusive_scan_i32(const int32_t *in, int32_t *out, int64_t n, int32_t *sums_ws,
+                           hipStream_t s);
+
+#ifdef __HIPCC__
+__device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
+// Wave index inside the block as a wave-uniform (scalar) value.
+__device__ __forceinline__ int wave_in_block()
+{
+    return __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+}
+__device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ int bcast_i(int v, int lane) { return __builtin_amdgcn_readlane(v, lane); }
+__device__ __forceinline__ float bcast_f(float v, int lane)
+{
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+#endif
+
+}  // namespace jg

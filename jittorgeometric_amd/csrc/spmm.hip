@@ -1,0 +1,328 @@
+// Weighted row-gather SpMM  out[r,:] = sum_j w[j] * x[idx[j],:]  for gfx950.
+//
+// Work split (merge-path): the R row-end markers and the E entries form one
+// sequence of M = R + E items (row r's entries, then its end marker).  Every
+// wavefront takes `chunk` consecutive items, so a 20,000-entry hub row is cut
+// into pieces and a run of empty rows costs what the same number of entries
+// would.  Inside a wavefront the feature dimension lies across the 64 lanes
+// (VEC floats per lane, NT tiles of 64*VEC features), the entries are walked
+// in order, and (idx, w) are loaded 64 at a time, one per lane, then handed
+// out with v_readlane so that every gathered row has a scalar base address.
+// The gathers of UNROLL entries are issued before the first is used.
+//
+// A row that ends inside a chunk is stored by that chunk's wavefront.  The
+// leading piece of a row that continues into the next chunk goes to
+// partial[chunk].  spmm_fixup then adds, for every row that started in an
+// earlier chunk, the pieces in chunk order.  No float atomics: the result
+// does not change from run to run.
+#include <stdlib.h>
+
+#include "common.h"
+
+namespace jg {
+
+constexpr int kSpmmThreads = 256;
+constexpr int kSpmmWaves = kSpmmThreads / kWave;
+
+template <int VEC> struct Vec;
+template <> struct Vec<1> { using type = float; };
+template <> struct Vec<2> { using type = float2; };
+template <> struct Vec<4> { using type = float4; };
+
+template <int VEC> __device__ __forceinline__ void vload(float (&d)[VEC], const float *p)
+{
+    using V = typename Vec<VEC>::type;
+    const V v = *reinterpret_cast<const V *>(p);
+    const float *f = reinterpret_cast<const float *>(&v);
+#pragma unroll
+    for (int i = 0; i < VEC; i++) d[i] = f[i];
+}
+template <int VEC> __device__ __forceinline__ void vstore(float *p, const float (&s)[VEC])
+{
+    using V = typename Vec<VEC>::type;
+    V v;
+    float *f = reinterpret_cast<float *>(&v);
+#pragma unroll
+    for (int i = 0; i < VEC; i++) f[i] = s[i];
+    *reinterpret_cast<V *>(p) = v;
+}
+
+// chunk_row[k] = the row that owns merged position k*chunk, k < nchunks;
+// chunk_row[nchunks] = R.  Row r owns positions off[r]+r .. off[r+1]+r.
+__global__ void spmm_chunk_rows(const int32_t *__restrict__ off, int R, int chunk, int nchunks,
+                                int32_t *__restrict__ chunk_row)
+{
+    const int r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (r == 0) chunk_row[nchunks] = R;
+    if (r >= R) return;
+    const int64_t lo = (int64_t)off[r] + r, hi = (int64_t)off[r + 1] + r;
+    for (int64_t k = (lo + chunk - 1) / chunk; k * chunk <= hi && k < nchunks; k++) chunk_row[k] = r;
+}
+
+template <int VEC, int NT, int UNROLL>
+__global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__restrict__ off,
+                                                           const int32_t *__restrict__ idx,
+                                                           const float *__restrict__ w,
+                                                           const float *__restrict__ x, float *__restrict__ out,
+                                                           float *__restrict__ partial,
+                                                           const int32_t *__restrict__ chunk_row, int R, int C,
+                                                           int E, int F, int chunk, int nchunks)
+{
+    const int k = blockIdx.x * kSpmmWaves + wave_in_block();
+    if (k >= nchunks) return;
+    const int lane = lane_id();
+    const int f0 = blockIdx.y * (kWave * VEC * NT) + lane * VEC;   // this lane's first feature
+    bool act[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) act[t] = f0 + t * kWave * VEC < F;
+
+    int r = uniform(chunk_row[k]);
+    const int r1 = uniform(chunk_row[k + 1]);
+    const int M = R + E;
+    const int p0 = k * chunk;
+    const int p1 = min(p0 + chunk, M);
+    int j0 = p0 - r;
+    int j1 = min(p1 - r1, E);
+    j0 = max(j0, 0);
+
+    // window of 64 row ends starting at row rb: lane l holds off[rb + 1 + l]
+    int rb = r;
+    int ends = (rb + lane < R) ? off[rb + 1 + lane] : 0x7fffffff;
+    int row_end = bcast_i(ends, 0);
+
+    float acc[NT][VEC];
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int v = 0; v < VEC; v++) acc[t][v] = 0.f;
+
+    auto flush_row = [&]() {
+        float *dst = out + (size_t)r * F + f0;
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            if (act[t]) vstore<VEC>(dst + t * kWave * VEC, acc[t]);
+#pragma unroll
+            for (int v = 0; v < VEC; v++) acc[t][v] = 0.f;
+        }
+        r++;
+        if (r - rb == kWave) {
+            rb = r;
+            ends = (rb + lane < R) ? off[rb + 1 + lane] : 0x7fffffff;
+        }
+        row_end = bcast_i(ends, r - rb);
+    };
+
+    for (int jb = j0; jb < j1; jb += kWave) {
+        const int n = min(kWave, j1 - jb);
+        int my_c;
+        float my_w;
+        {
+            const bool ok = lane < n;
+            const int jj = jb + lane;
+            my_c = idx ? (ok ? idx[jj] : 0) : jj;
+            my_w = ok ? (w ? w[jj] : 1.f) : 0.f;
+            if ((unsigned)my_c >= (unsigned)C) {
+                my_c = 0;
+                my_w = 0.f;
+            }
+        }
+        for (int i0 = 0; i0 < n; i0 += UNROLL) {
+            float xv[UNROLL][NT][VEC];
+            const bool full = i0 + UNROLL <= n;
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) {
+                if (full || i0 + u < n) {
+                    const int c = bcast_i(my_c, i0 + u);
+                    const float *src = x + (size_t)c * F + f0;
+#pragma unroll
+                    for (int t = 0; t < NT; t++)
+                        if (act[t]) vload<VEC>(xv[u][t], src + t * kWave * VEC);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) {
+                if (full || i0 + u < n) {
+                    const int jj = jb + i0 + u;
+                    while (jj == row_end && r < r1) flush_row();
+                    const float wv = bcast_f(my_w, i0 + u);
+#pragma unroll
+                    for (int t = 0; t < NT; t++)
+                        if (act[t]) {
+#pragma unroll
+                            for (int v = 0; v < VEC; v++) acc[t][v] = fmaf(wv, xv[u][t][v], acc[t][v]);
+                        }
+                }
+            }
+        }
+    }
+    while (r < r1) flush_row();   // rows whose end marker lies in this chunk after its last entry
+    if (r1 < R) {
+        float *dst = partial + (size_t)k * F + f0;
+#pragma unroll
+        for (int t = 0; t < NT; t++)
+            if (act[t]) vstore<VEC>(dst + t * kWave * VEC, acc[t]);
+    }
+}
+
+// One wavefront per chunk b: if the first row of b started in an earlier
+// chunk a and ends in b, out[row] = partial[a] + ... + partial[b-1] + out[row].
+template <int VEC, int NT>
+__global__ __launch_bounds__(kSpmmThreads) void spmm_fixup(const int32_t *__restrict__ off, float *__restrict__ out,
+                                                           const float *__restrict__ partial,
+                                                           const int32_t *__restrict__ chunk_row, int F, int chunk,
+                                                           int nchunks)
+{
+    const int k = blockIdx.x * kSpmmWaves + wave_in_block();
+    if (k >= nchunks) return;
+    const int r0 = uniform(chunk_row[k]);
+    const int r1 = uniform(chunk_row[k + 1]);
+    if (r1 <= r0) return;
+    const int lo = uniform(off[r0]) + r0;
+    if (lo >= k * chunk) return;
+    const int a = lo / chunk;
+    const int lane = lane_id();
+    const int f0 = blockIdx.y * (kWave * VEC * NT) + lane * VEC;
+    float acc[NT][VEC];
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int v = 0; v < VEC; v++) acc[t][v] = 0.f;
+    auto add = [&](const float *src) {
+#pragma unroll
+        for (int t = 0; t < NT; t++)
+            if (f0 + t * kWave * VEC < F) {
+                float v[VEC];
+                vload<VEC>(v, src + f0 + t * kWave * VEC);
+#pragma unroll
+                for (int i = 0; i < VEC; i++) acc[t][i] += v[i];
+            }
+    };
+#pragma unroll 4
+    for (int kk = a; kk < k; kk++) add(partial + (size_t)kk * F);
+    float *dst = out + (size_t)r0 * F;
+    add(dst);
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+        if (f0 + t * kWave * VEC < F) vstore<VEC>(dst + f0 + t * kWave * VEC, acc[t]);
+}
+
+// ------------------------------------------------------------------ host ---
+static int env_int(const char *name, int dflt)
+{
+    const char *s = getenv(name);
+    if (!s || !*s) return dflt;
+    int v = atoi(s);
+    return v > 0 ? v : dflt;
+}
+
+// Items per wavefront: enough chunks to fill the 256 CUs many times over,
+// few enough that the per-chunk partial row stays a small share of the work.
+static int pick_chunk(int64_t M)
+{
+    static const int forced = env_int("JGAMD_SPMM_CHUNK", 0);
+    if (forced) return forced;
+    int c = 256;
+    while (c > 32 && M / c < 32768) c >>= 1;
+    return c;
+}
+
+struct SpmmShape {
+    int vec, nt, slabs, chunk, nchunks;
+};
+
+static SpmmShape spmm_shape(int32_t R, int64_t E, int32_t F, bool aligned16, bool aligned8)
+{
+    SpmmShape s{};
+    s.vec = (F % 4 == 0 && aligned16) ? 4 : (F % 2 == 0 && aligned8) ? 2 : 1;
+    // prefer the narrowest vector that still covers F with one tile per lane:
+    // more lanes per row keeps every load instruction a full 64-lane access
+    while (s.vec > 1 && F <= kWave * (s.vec / 2)) s.vec >>= 1;
+    int per_tile = kWave * s.vec;
+    int tiles = (int)ceil_div(F, per_tile);
+    s.nt = tiles <= 8 ? tiles : 8;
+    if (s.nt == 7) s.nt = 8;
+    s.slabs = (int)ceil_div(F, per_tile * s.nt);
+    const int64_t M = (int64_t)R + E;
+    s.chunk = pick_chunk(M);
+    s.nchunks = (int)ceil_div(M > 0 ? M : 1, s.chunk);
+    return s;
+}
+
+static size_t spmm_ws_bytes(int32_t R, int64_t E, int32_t F)
+{
+    SpmmShape s = spmm_shape(R, E, F, true, true);
+    return carve_bytes((size_t)s.nchunks + 1, 4) + carve_bytes((size_t)s.nchunks * (size_t)F, 4);
+}
+
+template <int VEC, int NT>
+static void launch_spmm(const SpmmShape &s, const int32_t *off, const int32_t *idx, const float *w, const float *x,
+                        float *out, float *partial, const int32_t *chunk_row, int R, int C, int E, int F,
+                        hipStream_t st)
+{
+    dim3 grid((unsigned)ceil_div(s.nchunks, kSpmmWaves), (unsigned)s.slabs), block(kSpmmThreads);
+    // gathers in flight per wavefront: bounded by the registers they land in
+    constexpr int U = (VEC * NT >= 16) ? 4 : (VEC * NT >= 8 ? 8 : 16);
+    hipLaunchKernelGGL((spmm_merge<VEC, NT, U>), grid, block, 0, st, off, idx, w, x, out, partial, chunk_row, R, C,
+                       E, F, s.chunk, s.nchunks);
+    hipLaunchKernelGGL((spmm_fixup<VEC, NT>), grid, block, 0, st, off, out, partial, chunk_row, F, s.chunk,
+                       s.nchunks);
+}
+
+}  // namespace jg
+
+using namespace jg;
+
+static int32_t check_spmm_sizes(int32_t R, int64_t E, int32_t F)
+{
+    if (R < 0 || E < 0 || F < 0) return fail(JGAMD_ERR_SIZE, "spmm_csx: negative size");
+    if ((int64_t)R + E >= ((int64_t)1 << 31) - 4096)
+        return fail(JGAMD_ERR_SIZE, "spmm_csx: R + E = %lld does not fit int32", (long long)((int64_t)R + E));
+    return 0;
+}
+
+extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_workspace(int32_t R, int64_t E, int32_t F, size_t *bytes)
+{
+    if (!bytes) return fail(JGAMD_ERR_NULL, "spmm_csx_workspace: bytes is NULL");
+    if (int32_t rc = check_spmm_sizes(R, E, F)) return rc;
+    *bytes = (R == 0 || F == 0) ? 0 : spmm_ws_bytes(R, E, F);
+    return 0;
+}
+
+extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx(const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out,
+                                  int32_t R, int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes,
+                                  void *stream)
+{
+    if (int32_t rc = check_spmm_sizes(R, E, F)) return rc;
+    if (C < 0) return fail(JGAMD_ERR_SIZE, "spmm_csx: negative C");
+    if (R == 0 || F == 0) return 0;
+    if (!off || !out) return fail(JGAMD_ERR_NULL, "spmm_csx: off/out is NULL");
+    if (E > 0 && !x) return fail(JGAMD_ERR_NULL, "spmm_csx: x is NULL with E > 0");
+    if (E > 0 && C == 0) return fail(JGAMD_ERR_SIZE, "spmm_csx: E > 0 entries but x has no rows");
+    if ((((uintptr_t)x | (uintptr_t)out) & 3) != 0) return fail(JGAMD_ERR_ALIGN, "spmm_csx: x/out not 4-byte aligned");
+    const size_t need = spmm_ws_bytes(R, E, F);
+    if (!ws || ws_bytes < need)
+        return fail(JGAMD_ERR_WORKSPACE, "spmm_csx: workspace %zu < %zu bytes", ws ? ws_bytes : (size_t)0, need);
+    if (((uintptr_t)ws & 255) != 0) return fail(JGAMD_ERR_ALIGN, "spmm_csx: workspace not 256-byte aligned");
+
+    const uintptr_t bits = (uintptr_t)x | (uintptr_t)out;
+    const SpmmShape s = spmm_shape(R, E, F, (bits & 15) == 0, (bits & 7) == 0);
+    Carver carve(ws);
+    int32_t *chunk_row = carve.take<int32_t>((size_t)s.nchunks + 1);
+    float *partial = carve.take<float>((size_t)s.nchunks * (size_t)F);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+
+    hipLaunchKernelGGL(spmm_chunk_rows, dim3((unsigned)ceil_div(R, 256)), dim3(256), 0, st, off, R, s.chunk,
+                       s.nchunks, chunk_row);
+#define JG_CASE(V, N)                                                                                \
+    if (s.vec == V && s.nt == N) {                                                                   \
+        launch_spmm<V, N>(s, off, idx, w, x, out, partial, chunk_row, R, C, (int)E, F, st);          \
+        return launch_status("spmm_csx");                                                            \
+    }
+#define JG_CASES(V) JG_CASE(V, 1) JG_CASE(V, 2) JG_CASE(V, 3) JG_CASE(V, 4) JG_CASE(V, 5) JG_CASE(V, 6) JG_CASE(V, 8)
+    JG_CASES(1)
+    JG_CASES(2)
+    JG_CASES(4)
+#undef JG_CASES
+#undef JG_CASE
+    return fail(JGAMD_ERR_UNSUPPORTED, "spmm_csx: no kernel for F=%d (vec %d, tiles %d)", F, s.vec, s.nt);
+}

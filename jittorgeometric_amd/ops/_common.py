@@ -1,0 +1,55 @@
+"""Helpers shared by the operator wrappers."""
+import torch
+
+from .. import _lib
+
+
+def as_i32(t, name):
+    if t.dtype != torch.int32:
+        # the reference's Data casts edge_index to int32 (data/data.py:103-106);
+        # int64 inputs (tests/test_spmmcsr.py:14-15) are narrowed the same way
+        t = t.to(torch.int32)
+    return t.contiguous()
+
+
+def as_f32(t, name):
+    if t.dtype != torch.float32:
+        t = t.to(torch.float32)
+    return t.contiguous()
+
+
+def transposed(holder, off, idx, w, R, C):
+    """(off_t, idx_t, w_t, perm) of a compressed structure, built on first use
+    and kept on the CSR/CSC object it belongs to."""
+    cached = getattr(holder, "_jgamd_transposed", None)
+    if cached is not None and cached[4] is off and cached[5] is idx and cached[6] is w:
+        return cached[:4]
+    lib = _lib.load()
+    dev = _lib.require_gpu(off, idx, w)
+    E = idx.shape[0]
+    off_t = torch.empty(C + 1, dtype=torch.int32, device=dev)
+    idx_t = torch.empty(E, dtype=torch.int32, device=dev)
+    w_t = torch.empty(E, dtype=torch.float32, device=dev) if w is not None else None
+    perm = torch.empty(E, dtype=torch.int32, device=dev)
+    nbytes = _lib.query(lib.jgamd_csx_transpose_workspace, E, R, C)
+    ws = _lib.workspace(nbytes, dev)
+    _lib.check(lib.jgamd_csx_transpose(_lib.ptr(off), _lib.ptr(idx), _lib.ptr(w), R, C, E, _lib.ptr(off_t),
+                                       _lib.ptr(idx_t), _lib.ptr(w_t), _lib.ptr(perm), _lib.ptr(ws), nbytes,
+                                       _lib.stream_ptr(dev)))
+    holder._jgamd_transposed = (off_t, idx_t, w_t, perm, off, idx, w)
+    return off_t, idx_t, w_t, perm
+
+
+def spmm(off, idx, w, x, R):
+    """out[r,:] = sum_j w[j] * x[idx[j],:]; idx/w may be None (identity / ones)."""
+    lib = _lib.load()
+    dev = _lib.require_gpu(off, x, idx, w)
+    x = as_f32(x, "x")
+    C, F = x.shape
+    E = int(idx.shape[0]) if idx is not None else C
+    out = torch.empty((R, F), dtype=torch.float32, device=dev)
+    nbytes = _lib.query(lib.jgamd_spmm_csx_workspace, R, E, F)
+    ws = _lib.workspace(nbytes, dev)
+    _lib.check(lib.jgamd_spmm_csx(_lib.ptr(off), _lib.ptr(idx), _lib.ptr(w), _lib.ptr(x), _lib.ptr(out), R, C, E, F,
+                                  _lib.ptr(ws), nbytes, _lib.stream_ptr(dev)))
+    return out

@@ -1,0 +1,48 @@
+"""SpMM on a CSR matrix.  Same call as jittor_geometric.ops.SpmmCsr
+(ops/spmmcsr.py:21-44), whose arithmetic is cuSPARSE inside the jittor wheel.
+trans_A=True (the default) multiplies by the transpose of the CSR matrix:
+out[c] = sum over entries (r, c) of w * x[r]."""
+import torch
+
+from .. import _lib
+from ._common import as_f32, as_i32, spmm, transposed
+
+# False: backward is the exact transpose of forward (the true gradient).
+# True: backward re-applies the forward product, as the reference does
+# (ops/spmmcsr.py:35-39); the two agree whenever the matrix is symmetric,
+# e.g. for gcn_norm weights on an undirected graph.
+REFERENCE_GRAD = False
+
+
+def _product(x, csr, trans_A):
+    col = as_i32(csr.column_indices, "column_indices")
+    off = as_i32(csr.row_offset, "row_offset")
+    w = as_f32(csr.edge_weight, "edge_weight")
+    v_num = off.shape[0] - 1
+    if trans_A:
+        # the transposed product is run as a gather over the transposed arrays,
+        # built once per CSR object (stable, so the result is reproducible)
+        if col is not csr.column_indices or off is not csr.row_offset or w is not csr.edge_weight:
+            csr.column_indices, csr.row_offset, csr.edge_weight = col, off, w
+        off_t, idx_t, w_t, _ = transposed(csr, off, col, w, v_num, v_num)
+        return spmm(off_t, idx_t, w_t, x, v_num)
+    return spmm(off, col, w, x, v_num)
+
+
+class SpmmCsrFunc(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, csr, trans_A, trans_B):
+        if trans_B:
+            raise _lib.JgamdError("SpmmCsr: trans_B=True is not supported")
+        ctx.csr = csr
+        ctx.trans_A = trans_A
+        return _product(x, csr, trans_A)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        trans = ctx.trans_A if REFERENCE_GRAD else not ctx.trans_A
+        return _product(grad_output.contiguous(), ctx.csr, trans), None, None, None
+
+
+def SpmmCsr(x, csr, trans_A=True, trans_B=False):
+    return SpmmCsrFunc.apply(x, csr, trans_A, trans_B)

@@ -1,0 +1,140 @@
+"""COO -> CSR/CSC on the GPU against the CPU oracle: bit-exact, through the
+C ABI (jittorgeometric_amd.ops -> ctypes -> libjgamd.so)."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from util import dev, rand_graph, to_gpu
+
+pytestmark = pytest.mark.gpu
+
+GOLD = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_fixtures.json")))
+
+
+def run_both(ei, w, V):
+    from jittorgeometric_amd.ops import cootocsc, cootocsr
+    csr = cootocsr(to_gpu(ei), to_gpu(w), V)
+    csc = cootocsc(to_gpu(ei), to_gpu(w), V)
+    torch.cuda.synchronize()
+    return csr, csc
+
+
+def check_exact(ei, w, V):
+    csr, csc = run_both(ei, w, V)
+    col, roff, rw = oracle.cootocsr(ei, w, V)
+    row, coff, cw = oracle.cootocsc(ei, w, V)
+    assert np.array_equal(csr.row_offset.cpu().numpy(), roff)
+    assert np.array_equal(csr.column_indices.cpu().numpy(), col)
+    assert np.array_equal(csr.edge_weight.cpu().numpy().view(np.int32), rw.view(np.int32))
+    assert np.array_equal(csc.column_offset.cpu().numpy(), coff)
+    assert np.array_equal(csc.row_indices.cpu().numpy(), row)
+    assert np.array_equal(csc.edge_weight.cpu().numpy().view(np.int32), cw.view(np.int32))
+    assert csr.column_indices.dtype == torch.int32 and csr.edge_weight.dtype == torch.float32
+
+
+@pytest.mark.parametrize("name", ["csr_v4", "mp_spmm_v10"])
+def test_reference_fixtures(name):
+    g = GOLD[name]
+    ei = np.array(g["edge_index"], np.int32)
+    w = np.array(g["edge_weight"], np.float32)
+    csr, csc = run_both(ei, w, g["v_num"])
+    assert csr.column_indices.tolist() == g["csr"]["column_indices"]
+    assert csr.row_offset.tolist() == g["csr"]["row_offset"]
+    assert csr.edge_weight.tolist() == g["csr"]["edge_weight"]
+    assert csc.row_indices.tolist() == g["csc"]["row_indices"]
+    assert csc.column_offset.tolist() == g["csc"]["column_offset"]
+    assert csc.edge_weight.tolist() == g["csc"]["edge_weight"]
+
+
+@pytest.mark.parametrize("V,E,hubs,seed", [
+    (1, 0, 0, 0), (1, 9, 0, 1), (5, 0, 0, 2), (4, 100, 0, 3), (1000, 1, 0, 4),
+    (1024, 20000, 3, 5), (1025, 20000, 3, 6), (2708, 13264, 0, 7), (5000, 8191, 2, 8),
+    (5000, 8192, 2, 9), (5000, 8193, 2, 10), (70001, 300000, 5, 11), (300000, 1000000, 4, 12),
+    (4194304, 600000, 3, 13), (2100000, 2500000, 2, 14),
+])
+def test_random_graphs_bit_exact(V, E, hubs, seed):
+    rng = np.random.default_rng(seed)
+    ei, w = rand_graph(rng, V, E, hubs)
+    check_exact(ei, w, V)
+
+
+def test_all_edges_one_row_and_sorted_and_reversed_inputs():
+    rng = np.random.default_rng(20)
+    V, E = 3000, 50000
+    ei, w = rand_graph(rng, V, E)
+    one = ei.copy()
+    one[0, :] = 17                              # a single 50,000-edge row
+    check_exact(one, w, V)
+    order = np.argsort(ei[0], kind="stable")
+    check_exact(ei[:, order], w[order], V)      # already sorted by source
+    check_exact(ei[:, order[::-1]].copy(), w[order[::-1]].copy(), V)
+
+
+def test_weights_are_copied_bitwise_including_nan_inf_and_negative_zero():
+    rng = np.random.default_rng(21)
+    V, E = 500, 4000
+    ei, w = rand_graph(rng, V, E)
+    w[:8] = [np.nan, np.inf, -np.inf, -0.0, 0.0, 1e-45, -1e38, 3.0]
+    check_exact(ei, w, V)
+
+
+def test_deterministic_across_runs():
+    rng = np.random.default_rng(22)
+    V, E = 20000, 400000
+    ei, w = rand_graph(rng, V, E, hubs=3)
+    a, _ = run_both(ei, w, V)
+    b, _ = run_both(ei, w, V)
+    assert torch.equal(a.column_indices, b.column_indices) and torch.equal(a.edge_weight, b.edge_weight)
+
+
+def test_permutation_output_and_transpose():
+    from jittorgeometric_amd.ops.cootocsr import _convert
+    from jittorgeometric_amd.ops._common import transposed
+    from jittorgeometric_amd import CSR
+    rng = np.random.default_rng(23)
+    V, E = 9000, 120000
+    ei, w = rand_graph(rng, V, E, hubs=2)
+    idx, off, wo, perm = _convert(to_gpu(ei), to_gpu(w), V, 0, with_perm=True)
+    perm = perm.cpu().numpy()
+    want = np.argsort(ei[0], kind="stable")
+    assert np.array_equal(perm, want)
+    assert np.array_equal(idx.cpu().numpy(), ei[1][want])
+    # transpose of the CSR equals the CSC of the CSR-ordered edge list
+    holder = CSR(idx, off, wo)
+    off_t, idx_t, w_t, perm_t = transposed(holder, off, idx, wo, V, V)
+    src_sorted = ei[0][want]
+    dst_sorted = ei[1][want]
+    row, coff, cw = oracle.cootocsc(np.stack([src_sorted, dst_sorted]), w[want], V)
+    assert np.array_equal(off_t.cpu().numpy(), coff)
+    assert np.array_equal(idx_t.cpu().numpy(), row)
+    assert np.array_equal(w_t.cpu().numpy(), cw)
+    assert np.array_equal(perm_t.cpu().numpy(), np.argsort(dst_sorted, kind="stable"))
+
+
+def test_int64_edge_index_is_narrowed_like_the_reference_data_class():
+    from jittorgeometric_amd.ops import cootocsr
+    g = GOLD["csr_v4"]
+    ei = torch.tensor(g["edge_index"], dtype=torch.int64, device=dev())
+    w = torch.tensor(g["edge_weight"], dtype=torch.float32, device=dev())
+    csr = cootocsr(ei, w, 4)
+    assert csr.column_indices.tolist() == g["csr"]["column_indices"]
+
+
+def test_cpu_tensors_are_refused():
+    from jittorgeometric_amd import _lib
+    from jittorgeometric_amd.ops import cootocsr
+    with pytest.raises(_lib.JgamdError):
+        cootocsr(torch.zeros((2, 3), dtype=torch.int32), torch.zeros(3), 4)
+
+
+def test_powerlaw_1m_full_size_bit_exact():
+    """Benchmark configuration: 1M nodes, 16M power-law edges + self-loops,
+    gcn_norm weights, edge order as generated (random)."""
+    from jittorgeometric_amd import synthetic
+    ei, V = synthetic.make("powerlaw_1m")
+    ei, w = oracle.gcn_norm(ei, None, V)
+    check_exact(ei.astype(np.int32), w, V)
