@@ -110,6 +110,17 @@ int32_t jgamd_spmm_csx(const int32_t *off, const int32_t *idx, const float *w, c
                        float *out, int32_t R, int32_t C, int64_t E, int32_t F, void *ws,
                        size_t ws_bytes, void *stream);
 
+/* Benchmark support; no counterpart in the reference.  Runs jgamd_spmm_csx
+ * `iters` times on `stream`, with one hipEvent pair around each launch of the
+ * gather kernel (spmm_merge) and one around each whole call (three launches),
+ * WAITS for the stream after every call, and returns the two mean durations
+ * in milliseconds.  Unlike every other entry point it synchronises and
+ * creates/destroys events. */
+int32_t jgamd_spmm_csx_timed(const int32_t *off, const int32_t *idx, const float *w, const float *x,
+                             float *out, int32_t R, int32_t C, int64_t E, int32_t F, void *ws,
+                             size_t ws_bytes, void *stream, int32_t iters, float *kernel_ms,
+                             float *call_ms);
+
 /* ------------------------------------------------------------------------
  * Edge softmax over the in-edges of every destination (CSC column).
  * Replaces EdgesoftmaxOp::jit_run (ops/cpp/edgesoftmax_op.cc:36-66, the

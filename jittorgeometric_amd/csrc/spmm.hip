@@ -76,8 +76,9 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__rest
 #pragma unroll
     for (int t = 0; t < NT; t++) act[t] = f0 + t * kWave * VEC < F;
 
-    int r = uniform(chunk_row[k]);
-    const int r1 = uniform(chunk_row[k + 1]);
+    // rows are clamped so that a malformed off/E pair cannot index outside the arrays
+    const int r1 = min(max(uniform(chunk_row[k + 1]), 0), R);
+    int r = min(max(uniform(chunk_row[k]), 0), r1);
     const int M = R + E;
     const int p0 = k * chunk;
     const int p1 = min(p0 + chunk, M);
@@ -179,7 +180,7 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_fixup(const int32_t *__rest
     if (r1 <= r0) return;
     const int lo = uniform(off[r0]) + r0;
     if (lo >= k * chunk) return;
-    const int a = lo / chunk;
+    const int a = max(lo, 0) / chunk;
     const int lane = lane_id();
     const int f0 = blockIdx.y * (kWave * VEC * NT) + lane * VEC;
     float acc[NT][VEC];
@@ -257,13 +258,15 @@ static size_t spmm_ws_bytes(int32_t R, int64_t E, int32_t F)
 template <int VEC, int NT>
 static void launch_spmm(const SpmmShape &s, const int32_t *off, const int32_t *idx, const float *w, const float *x,
                         float *out, float *partial, const int32_t *chunk_row, int R, int C, int E, int F,
-                        hipStream_t st)
+                        hipStream_t st, hipEvent_t k0 = nullptr, hipEvent_t k1 = nullptr)
 {
     dim3 grid((unsigned)ceil_div(s.nchunks, kSpmmWaves), (unsigned)s.slabs), block(kSpmmThreads);
     // gathers in flight per wavefront: bounded by the registers they land in
     constexpr int U = (VEC * NT >= 16) ? 4 : (VEC * NT >= 8 ? 8 : 16);
+    if (k0) (void)hipEventRecord(k0, st);
     hipLaunchKernelGGL((spmm_merge<VEC, NT, U>), grid, block, 0, st, off, idx, w, x, out, partial, chunk_row, R, C,
                        E, F, s.chunk, s.nchunks);
+    if (k1) (void)hipEventRecord(k1, st);
     hipLaunchKernelGGL((spmm_fixup<VEC, NT>), grid, block, 0, st, off, out, partial, chunk_row, F, s.chunk,
                        s.nchunks);
 }
@@ -288,9 +291,9 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_workspa
     return 0;
 }
 
-extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx(const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out,
-                                  int32_t R, int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes,
-                                  void *stream)
+static int32_t spmm_call(const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out,
+                         int32_t R, int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, void *stream,
+                         hipEvent_t k0, hipEvent_t k1)
 {
     if (int32_t rc = check_spmm_sizes(R, E, F)) return rc;
     if (C < 0) return fail(JGAMD_ERR_SIZE, "spmm_csx: negative C");
@@ -315,7 +318,7 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx(const i
                        s.nchunks, chunk_row);
 #define JG_CASE(V, N)                                                                                \
     if (s.vec == V && s.nt == N) {                                                                   \
-        launch_spmm<V, N>(s, off, idx, w, x, out, partial, chunk_row, R, C, (int)E, F, st);          \
+        launch_spmm<V, N>(s, off, idx, w, x, out, partial, chunk_row, R, C, (int)E, F, st, k0, k1);  \
         return launch_status("spmm_csx");                                                            \
     }
 #define JG_CASES(V) JG_CASE(V, 1) JG_CASE(V, 2) JG_CASE(V, 3) JG_CASE(V, 4) JG_CASE(V, 5) JG_CASE(V, 6) JG_CASE(V, 8)
@@ -325,4 +328,44 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx(const i
 #undef JG_CASES
 #undef JG_CASE
     return fail(JGAMD_ERR_UNSUPPORTED, "spmm_csx: no kernel for F=%d (vec %d, tiles %d)", F, s.vec, s.nt);
+}
+
+extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx(const int32_t *off, const int32_t *idx,
+                                                                         const float *w, const float *x, float *out,
+                                                                         int32_t R, int32_t C, int64_t E, int32_t F,
+                                                                         void *ws, size_t ws_bytes, void *stream)
+{
+    return spmm_call(off, idx, w, x, out, R, C, E, F, ws, ws_bytes, stream, nullptr, nullptr);
+}
+
+extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_timed(
+    const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out, int32_t R, int32_t C,
+    int64_t E, int32_t F, void *ws, size_t ws_bytes, void *stream, int32_t iters, float *kernel_ms, float *call_ms)
+{
+    if (iters < 1 || iters > 4096) return fail(JGAMD_ERR_SIZE, "spmm_csx_timed: iters must be in [1, 4096]");
+    if (!kernel_ms || !call_ms) return fail(JGAMD_ERR_NULL, "spmm_csx_timed: NULL result pointer");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipEvent_t ev[4];
+    for (auto &e : ev)
+        if (hipEventCreate(&e) != hipSuccess) return fail(JGAMD_ERR_UNSUPPORTED, "spmm_csx_timed: hipEventCreate failed");
+    double ksum = 0, csum = 0;
+    int32_t rc = 0;
+    for (int i = 0; i < iters && rc == 0; i++) {
+        (void)hipEventRecord(ev[0], st);
+        rc = spmm_call(off, idx, w, x, out, R, C, E, F, ws, ws_bytes, stream, ev[1], ev[2]);
+        (void)hipEventRecord(ev[3], st);
+        if (hipEventSynchronize(ev[3]) != hipSuccess && rc == 0)
+            rc = fail(JGAMD_ERR_UNSUPPORTED, "spmm_csx_timed: hipEventSynchronize failed");
+        float k = 0, c = 0;
+        if (rc == 0 && R > 0 && F > 0) {
+            (void)hipEventElapsedTime(&k, ev[1], ev[2]);
+            (void)hipEventElapsedTime(&c, ev[0], ev[3]);
+        }
+        ksum += k;
+        csum += c;
+    }
+    for (auto &e : ev) (void)hipEventDestroy(e);
+    *kernel_ms = (float)(ksum / iters);
+    *call_ms = (float)(csum / iters);
+    return rc;
 }

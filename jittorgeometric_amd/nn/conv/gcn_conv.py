@@ -1,0 +1,72 @@
+"""GCN layer with the constructor and call signature of the reference's
+GCNConv (nn/conv/gcn_conv.py:40-116) on torch tensors."""
+import torch
+from torch import nn
+
+from ...ops import SpmmCsr, aggregateWithWeight
+from ...utils import add_remaining_self_loops
+from ...utils.num_nodes import maybe_num_nodes
+from ..inits import glorot, zeros
+
+
+def _degree_norm(edge_index, edge_weight, num_nodes, improved, add_self_loops, power):
+    fill_value = 2.0 if improved else 1.0
+    num_nodes = maybe_num_nodes(edge_index, num_nodes)
+    if edge_weight is None:
+        edge_weight = torch.ones((edge_index.size(1),), dtype=torch.float32, device=edge_index.device)
+    if add_self_loops:
+        edge_index, edge_weight = add_remaining_self_loops(edge_index, edge_weight, fill_value, num_nodes)
+    row, col = edge_index[0].long(), edge_index[1].long()
+    deg = torch.zeros((num_nodes,), dtype=edge_weight.dtype, device=edge_weight.device)
+    deg.scatter_add_(0, col, edge_weight)
+    dinv = deg.pow(power)
+    dinv.masked_fill_(dinv == float("inf"), 0)
+    return edge_index, edge_weight, dinv, row, col
+
+
+def gcn_norm(edge_index, edge_weight=None, num_nodes=None, improved=False, add_self_loops=True, dtype=None):
+    """Symmetric normalisation w = d^-1/2[row] * w * d^-1/2[col] with the
+    degree summed by column (nn/conv/gcn_conv.py:18-37)."""
+    edge_index, edge_weight, dis, row, col = _degree_norm(edge_index, edge_weight, num_nodes, improved,
+                                                          add_self_loops, -0.5)
+    return edge_index, dis[row] * edge_weight * dis[col]
+
+
+class GCNConv(nn.Module):
+    """out = A_hat (x W) + b.  `spmm=True` routes through SpmmCsr(x, csr), as
+    the reference does on a GPU (gcn_conv.py:96-97); `spmm=False` through
+    aggregateWithWeight(x, csc, csr) (gcn_conv.py:98-99)."""
+
+    def __init__(self, in_channels, out_channels, bias=True, spmm=True, **kwargs):
+        super().__init__()
+        self.in_channels = in_channels
+        self.out_channels = out_channels
+        self.weight = nn.Parameter(torch.empty(in_channels, out_channels))
+        self.bias = nn.Parameter(torch.empty(out_channels)) if bias else None
+        self.spmm = spmm
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        glorot(self.weight)
+        zeros(self.bias)
+
+    def forward(self, x, csc, csr):
+        x = x @ self.weight
+        if self.spmm:
+            out = self.propagate_spmm(x=x, csr=csr)
+        else:
+            out = self.propagate_msg(x=x, csc=csc, csr=csr)
+        if self.bias is not None:
+            out = out + self.bias
+        return out
+
+    execute = forward
+
+    def propagate_msg(self, x, csc, csr):
+        return aggregateWithWeight(x, csc, csr)
+
+    def propagate_spmm(self, x, csr):
+        return SpmmCsr(x, csr)
+
+    def __repr__(self):
+        return "{}({}, {})".format(self.__class__.__name__, self.in_channels, self.out_channels)

@@ -1,0 +1,91 @@
+"""GraphSAGE (mean) layer with the constructor and call signature of the
+reference's SAGEConv (nn/conv/sage_conv.py:43-240) on torch tensors."""
+import torch
+from torch import nn
+
+from ...ops import SpmmCsr, aggregateWithWeight, cootocsc, cootocsr
+from ..inits import glorot, zeros
+from .gcn_conv import _degree_norm
+
+
+def sage_norm(edge_index, edge_weight=None, num_nodes=None, improved=False, add_self_loops=True, dtype=None):
+    """Mean weights w * d^-1[col] (nn/conv/sage_conv.py:16-40)."""
+    edge_index, edge_weight, dinv, row, col = _degree_norm(edge_index, edge_weight, num_nodes, improved,
+                                                           add_self_loops, -1.0)
+    return edge_index, edge_weight * dinv[col]
+
+
+class SAGEConv(nn.Module):
+    """out = mean_aggregate(x) W1 (+ x W_root) (+ b); aggregation happens at
+    the input width, before the dense product (sage_conv.py:172-190)."""
+
+    def __init__(self, in_channels, out_channels, improved=False, cached=False, add_self_loops=True,
+                 normalize=True, project=False, root_weight=True, bias=True, spmm=True, **kwargs):
+        super().__init__()
+        self.in_channels = in_channels
+        self.out_channels = out_channels
+        self.improved = improved
+        self.cached = cached
+        self.add_self_loops = add_self_loops
+        self.normalize = normalize
+        self.project = project
+        self._cached_edge_index = None
+        if project:
+            self.weight_proj = nn.Parameter(torch.empty(in_channels, in_channels))
+            self.bias_proj = nn.Parameter(torch.empty(in_channels))
+        else:
+            self.weight_proj = None
+            self.bias_proj = None
+        self.weight1 = nn.Parameter(torch.empty(in_channels, out_channels))
+        self.root_weight = nn.Parameter(torch.empty(in_channels, out_channels)) if root_weight else None
+        self.bias = nn.Parameter(torch.empty(out_channels)) if bias else None
+        self.spmm = spmm
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        if self.project:
+            glorot(self.weight_proj)
+            zeros(self.bias_proj)
+        glorot(self.weight1)
+        glorot(self.root_weight)
+        zeros(self.bias)
+        self._cached_edge_index = None
+
+    def forward(self, x, edge_index=None, edge_weight=None, csc=None, csr=None):
+        if csc is None or csr is None:
+            cache = self._cached_edge_index
+            if cache is None:
+                if self.normalize:
+                    edge_index, edge_weight = sage_norm(edge_index, edge_weight, x.size(0), self.improved,
+                                                        self.add_self_loops)
+                with torch.no_grad():
+                    csc = cootocsc(edge_index, edge_weight, x.size(0))
+                    csr = cootocsr(edge_index, edge_weight, x.size(0))
+                if self.cached:
+                    self._cached_edge_index = (edge_index, edge_weight, csr, csc)
+            else:
+                edge_index, edge_weight, csr, csc = cache
+        xs = (x, x)
+        if self.weight_proj is not None:
+            xs = (torch.relu(xs[0] @ self.weight_proj + self.bias_proj), xs[1])
+        if self.spmm:
+            out = self.propagate_spmm(x=xs[0], csr=csr)
+        else:
+            out = self.propagate_msg(x=xs[0], csc=csc, csr=csr)
+        out = out @ self.weight1
+        if self.root_weight is not None:
+            out = out + xs[1] @ self.root_weight
+        if self.bias is not None:
+            out = out + self.bias
+        return out
+
+    execute = forward
+
+    def propagate_msg(self, x, csc, csr):
+        return aggregateWithWeight(x, csc, csr)
+
+    def propagate_spmm(self, x, csr):
+        return SpmmCsr(x, csr)
+
+    def __repr__(self):
+        return "{}({}, {})".format(self.__class__.__name__, self.in_channels, self.out_channels)
