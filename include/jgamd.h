@@ -170,8 +170,11 @@ int32_t jgamd_gat_fwd(const int32_t *off, const int32_t *idx, const float *h,
                       void *stream);
 
 /* Backward of jgamd_gat_fwd.  Needs both orders of the graph: (off, idx) are
- * the CSC arrays used forward, (t_off, t_idx) the transposed (CSR) arrays of
- * the same edges (jgamd_csx_transpose or cootocsr).
+ * the CSC arrays used forward, (t_off, t_idx, t_perm) their transpose as
+ * produced by jgamd_csx_transpose (t_perm[j] = CSC slot of transposed slot j).
+ * With H > 1 the head width D must span a power-of-two number of lanes
+ * (D in {1,2,4,...,256}); other shapes return JGAMD_ERR_UNSUPPORTED and are
+ * served by the unfused operator chain.
  *   g_out [V,H,D] upstream gradient, out [V,H,D] forward result
  *   g_h   [V,H,D], g_a_src [H,D], g_a_dst [H,D] outputs
  * Replaces the grad chain edgetovertex <-> scattertoedge <->
@@ -179,7 +182,7 @@ int32_t jgamd_gat_fwd(const int32_t *off, const int32_t *idx, const float *h,
  */
 int32_t jgamd_gat_bwd_workspace(int32_t V, int64_t E, int32_t H, int32_t D, size_t *bytes);
 int32_t jgamd_gat_bwd(const int32_t *off, const int32_t *idx, const int32_t *t_off,
-                      const int32_t *t_idx, const float *h, const float *a_src,
+                      const int32_t *t_idx, const int32_t *t_perm, const float *h, const float *a_src,
                       const float *a_dst, float slope, const float *el, const float *er,
                       const float *smax, const float *ssum, const float *out,
                       const float *g_out, float *g_h, float *g_a_src, float *g_a_dst,

@@ -27,7 +27,7 @@ SIGNATURES = {
     "jgamd_gat_fwd": [_P, _P, _P, _P, _P, _F32, _P, _P, _P, _P, _P, _P, _I32, _I64, _I32, _I32, _P,
                       _c.c_size_t, _P],
     "jgamd_gat_bwd_workspace": [_I32, _I64, _I32, _I32, _SZP],
-    "jgamd_gat_bwd": [_P, _P, _P, _P, _P, _P, _P, _F32, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I32, _I64,
+    "jgamd_gat_bwd": [_P, _P, _P, _P, _P, _P, _P, _P, _F32, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I32, _I64,
                       _I32, _I32, _P, _c.c_size_t, _P],
 }
 

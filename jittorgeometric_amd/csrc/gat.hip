@@ -1,29 +1,777 @@
-// Fused GAT layer core (placeholder until the kernels land).
+// Fused GAT layer core for gfx950: attention logits, edge softmax and the
+// weighted aggregation in one pass over the CSC arrays; backward in one pass
+// over the transposed (CSR) arrays.
+//
+// Reference chain being replaced (nn/conv/gat_conv.py:61-83):
+//   e = [h[src] | h[dst]]  (two [E,C] copies + concat)      scattertoedge_op.cc
+//   z = leaky_relu(e @ a, 0.2)                               [E,1]
+//   alpha = edge softmax of z per destination                edgesoftmax_op.cc
+//   out[dst] = sum alpha * h[src]                            edgetovertex_op.cc
+// With a = [a_src | a_dst]:  e @ a = a_src.h[src] + a_dst.h[dst] = el[src] + er[dst],
+// two per-node scalars per head, so no [E,C] tensor is ever materialised.
+//
+// Work split and lane layout are those of the SpMM kernel: merge-path chunks
+// of (row ends + entries) per wavefront, features across lanes.  The softmax
+// is carried as a running (max, sum) per lane and head, rescaling the
+// accumulator when the max grows; a row cut by a chunk boundary leaves its
+// unnormalised (acc, max, sum) piece in scratch and a second kernel merges
+// the pieces in order.  No float atomics anywhere.
+#include <math.h>
+
 #include "common.h"
+
+namespace jg {
+
+constexpr int kGatThreads = 256;
+constexpr int kGatWaves = kGatThreads / kWave;
+// gathers in flight per wavefront, bounded by the registers they land in
+constexpr int gat_unroll(int regs) { return regs >= 16 ? 2 : regs >= 8 ? 4 : 8; }
+
+template <int VEC> struct GVec;
+template <> struct GVec<1> { using type = float; };
+template <> struct GVec<2> { using type = float2; };
+template <> struct GVec<4> { using type = float4; };
+
+template <int VEC> __device__ __forceinline__ void gload(float (&d)[VEC], const float *p)
+{
+    using V = typename GVec<VEC>::type;
+    const V v = *reinterpret_cast<const V *>(p);
+    const float *f = reinterpret_cast<const float *>(&v);
+#pragma unroll
+    for (int i = 0; i < VEC; i++) d[i] = f[i];
+}
+template <int VEC> __device__ __forceinline__ void gstore(float *p, const float (&s)[VEC])
+{
+    using V = typename GVec<VEC>::type;
+    V v;
+    float *f = reinterpret_cast<float *>(&v);
+#pragma unroll
+    for (int i = 0; i < VEC; i++) f[i] = s[i];
+    *reinterpret_cast<V *>(p) = v;
+}
+
+__device__ __forceinline__ float lrelu(float z, float slope) { return z > 0.f ? z : slope * z; }
+
+// chunk_row as in spmm.hip: the row owning merged position k*chunk.
+__global__ void gat_chunk_rows(const int32_t *__restrict__ off, int R, int chunk, int nchunks,
+                               int32_t *__restrict__ chunk_row)
+{
+    const int r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (r == 0) chunk_row[nchunks] = R;
+    if (r >= R) return;
+    const int64_t lo = (int64_t)off[r] + r, hi = (int64_t)off[r + 1] + r;
+    for (int64_t k = (lo + chunk - 1) / chunk; k * chunk <= hi && k < nchunks; k++) chunk_row[k] = r;
+}
+
+// el[v,k] = a_src[k,:].h[v,k,:], er[v,k] = a_dst[k,:].h[v,k,:]
+__global__ void gat_node_scores(const float *__restrict__ h, const float *__restrict__ a_src,
+                                const float *__restrict__ a_dst, float *__restrict__ el, float *__restrict__ er,
+                                int64_t VH, int H, int D)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= VH) return;
+    const int k = (int)(i % H);
+    const float *row = h + i * D;
+    const float *as = a_src + (int64_t)k * D, *ad = a_dst + (int64_t)k * D;
+    float s = 0.f, d = 0.f;
+    for (int j = 0; j < D; j++) {
+        const float v = row[j];
+        s = fmaf(v, as[j], s);
+        d = fmaf(v, ad[j], d);
+    }
+    el[i] = s;
+    er[i] = d;
+}
+
+// ----------------------------------------------------------------- forward ---
+template <int VEC, int NT>
+__global__ __launch_bounds__(kGatThreads) void gat_fwd_merge(
+    const int32_t *__restrict__ off, const int32_t *__restrict__ idx, const float *__restrict__ h,
+    const float *__restrict__ el, const float *__restrict__ er, float slope, float *__restrict__ out,
+    float *__restrict__ smax, float *__restrict__ ssum, float *__restrict__ partial, float *__restrict__ pmax,
+    float *__restrict__ psum, const int32_t *__restrict__ chunk_row, int R, int E, int H, int D, int chunk,
+    int nchunks)
+{
+    constexpr int kGatUnroll = gat_unroll(VEC * NT);
+    const int k = blockIdx.x * kGatWaves + wave_in_block();
+    if (k >= nchunks) return;
+    const int lane = lane_id();
+    const int F = H * D;
+    const int f0 = lane * VEC;
+    bool act[NT], lead[NT];
+    int head[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        const int f = f0 + t * kWave * VEC;
+        act[t] = f < F;
+        head[t] = act[t] ? f / D : 0;
+        lead[t] = act[t] && (f % D == 0);
+    }
+    const int r1 = min(max(uniform(chunk_row[k + 1]), 0), R);
+    int r = min(max(uniform(chunk_row[k]), 0), r1);
+    const int p0 = k * chunk;
+    const int p1 = min(p0 + chunk, R + E);
+    const int j0 = max(p0 - r, 0);
+    const int j1 = min(p1 - r1, E);
+    // the first row of the chunk began in an earlier chunk: its piece stays unnormalised
+    bool continued = (r < R) && (uniform(off[r]) + r < p0);
+
+    int rb = r;
+    int ends = (rb + lane < R) ? off[rb + 1 + lane] : 0x7fffffff;
+    int row_end = bcast_i(ends, 0);
+
+    float m[NT], l[NT], acc[NT][VEC], er_r[NT];
+    auto reset = [&]() {
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            m[t] = -INFINITY;
+            l[t] = 0.f;
+#pragma unroll
+            for (int v = 0; v < VEC; v++) acc[t][v] = 0.f;
+            er_r[t] = (act[t] && r < R) ? er[(size_t)r * H + head[t]] : 0.f;
+        }
+    };
+    reset();
+
+    auto flush_row = [&]() {
+        float *dst = out + (size_t)r * F + f0;
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            if (act[t]) {
+                float o[VEC];
+                const float inv = continued ? 1.f : (l[t] > 0.f ? 1.f / l[t] : 0.f);
+#pragma unroll
+                for (int v = 0; v < VEC; v++) o[v] = acc[t][v] * inv;
+                gstore<VEC>(dst + t * kWave * VEC, o);
+                if (lead[t]) {
+                    smax[(size_t)r * H + head[t]] = m[t];
+                    ssum[(size_t)r * H + head[t]] = l[t];
+                }
+            }
+        }
+        continued = false;
+        r++;
+        if (r - rb == kWave) {
+            rb = r;
+            ends = (rb + lane < R) ? off[rb + 1 + lane] : 0x7fffffff;
+        }
+        row_end = bcast_i(ends, r - rb);
+        reset();
+    };
+
+    for (int jb = j0; jb < j1; jb += kWave) {
+        const int n = min(kWave, j1 - jb);
+        int my_c = -1;
+        if (lane < n) {
+            my_c = idx[jb + lane];
+            if ((unsigned)my_c >= (unsigned)R) my_c = -1;
+        }
+        for (int i0 = 0; i0 < n; i0 += kGatUnroll) {
+            float xv[kGatUnroll][NT][VEC], sv[kGatUnroll][NT];
+#pragma unroll
+            for (int u = 0; u < kGatUnroll; u++) {
+                if (i0 + u < n) {
+                    const int c = bcast_i(my_c, i0 + u);
+                    if (c >= 0) {
+                        const float *src = h + (size_t)c * F + f0;
+                        const float *sl = el + (size_t)c * H;
+#pragma unroll
+                        for (int t = 0; t < NT; t++)
+                            if (act[t]) {
+                                gload<VEC>(xv[u][t], src + t * kWave * VEC);
+                                sv[u][t] = sl[head[t]];
+                            }
+                    }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kGatUnroll; u++) {
+                if (i0 + u < n) {
+                    const int jj = jb + i0 + u;
+                    while (jj == row_end && r < r1) flush_row();
+                    const int c = bcast_i(my_c, i0 + u);
+                    if (c >= 0) {
+#pragma unroll
+                        for (int t = 0; t < NT; t++)
+                            if (act[t]) {
+                                const float s = lrelu(sv[u][t] + er_r[t], slope);
+                                const float mn = fmaxf(m[t], s);
+                                const float sc = expf(m[t] - mn);     // 0 on the first entry (m = -inf)
+                                const float p = expf(s - mn);
+                                l[t] = fmaf(l[t], sc, p);
+#pragma unroll
+                                for (int v = 0; v < VEC; v++) acc[t][v] = fmaf(acc[t][v], sc, p * xv[u][t][v]);
+                                m[t] = mn;
+                            }
+                    }
+                }
+            }
+        }
+    }
+    while (r < r1) flush_row();
+    if (r1 < R) {
+        float *dst = partial + (size_t)k * F + f0;
+#pragma unroll
+        for (int t = 0; t < NT; t++)
+            if (act[t]) {
+                gstore<VEC>(dst + t * kWave * VEC, acc[t]);
+                if (lead[t]) {
+                    pmax[(size_t)k * H + head[t]] = m[t];
+                    psum[(size_t)k * H + head[t]] = l[t];
+                }
+            }
+    }
+}
+
+// Merges, in chunk order, the pieces of a row that started in an earlier
+// chunk and ends in chunk k (its last piece sits unnormalised in out/smax/ssum).
+template <int VEC, int NT>
+__global__ __launch_bounds__(kGatThreads) void gat_fwd_fixup(const int32_t *__restrict__ off, float *__restrict__ out,
+                                                             float *__restrict__ smax, float *__restrict__ ssum,
+                                                             const float *__restrict__ partial,
+                                                             const float *__restrict__ pmax,
+                                                             const float *__restrict__ psum,
+                                                             const int32_t *__restrict__ chunk_row, int H, int D,
+                                                             int chunk, int nchunks)
+{
+    const int k = blockIdx.x * kGatWaves + wave_in_block();
+    if (k >= nchunks) return;
+    const int r0 = uniform(chunk_row[k]);
+    const int r1 = uniform(chunk_row[k + 1]);
+    if (r1 <= r0) return;
+    const int lo = uniform(off[r0]) + r0;
+    if (lo >= k * chunk) return;
+    const int a = max(lo, 0) / chunk;
+    const int F = H * D;
+    const int f0 = lane_id() * VEC;
+    float M[NT], L[NT], acc[NT][VEC];
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        M[t] = -INFINITY;
+        L[t] = 0.f;
+#pragma unroll
+        for (int v = 0; v < VEC; v++) acc[t][v] = 0.f;
+    }
+    auto merge = [&](const float *vec, const float *pm, const float *pl) {
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const int f = f0 + t * kWave * VEC;
+            if (f < F) {
+                const float mi = pm[f / D], li = pl[f / D];
+                if (li > 0.f) {
+                    float x[VEC];
+                    gload<VEC>(x, vec + f);
+                    const float mn = fmaxf(M[t], mi);
+                    const float so = expf(M[t] - mn), si = expf(mi - mn);
+                    L[t] = L[t] * so + li * si;
+#pragma unroll
+                    for (int v = 0; v < VEC; v++) acc[t][v] = acc[t][v] * so + x[v] * si;
+                    M[t] = mn;
+                }
+            }
+        }
+    };
+    for (int kk = a; kk < k; kk++) merge(partial + (size_t)kk * F, pmax + (size_t)kk * H, psum + (size_t)kk * H);
+    merge(out + (size_t)r0 * F, smax + (size_t)r0 * H, ssum + (size_t)r0 * H);
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        const int f = f0 + t * kWave * VEC;
+        if (f < F) {
+            float o[VEC];
+            const float inv = L[t] > 0.f ? 1.f / L[t] : 0.f;
+#pragma unroll
+            for (int v = 0; v < VEC; v++) o[v] = acc[t][v] * inv;
+            gstore<VEC>(out + (size_t)r0 * F + f, o);
+        }
+    }
+    // every lane of a head holds the same (M, L); the head's first lane stores them
+    // after all lanes have read the old values above (same wavefront, program order)
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        const int f = f0 + t * kWave * VEC;
+        if (f < F && f % D == 0) {
+            smax[(size_t)r0 * H + f / D] = M[t];
+            ssum[(size_t)r0 * H + f / D] = L[t];
+        }
+    }
+}
+
+// Column (destination) of every CSC slot by binary search; one thread per (slot, head).
+__global__ void gat_alpha(const int32_t *__restrict__ off, const int32_t *__restrict__ idx,
+                          const float *__restrict__ el, const float *__restrict__ er,
+                          const float *__restrict__ smax, const float *__restrict__ ssum, float slope,
+                          float *__restrict__ alpha, int V, int64_t E, int H)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= E * H) return;
+    const int64_t j = i / H;
+    const int k = (int)(i % H);
+    int lo = 0, hi = V;
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if ((int64_t)off[mid] <= j) lo = mid; else hi = mid;
+    }
+    const int c = idx[j];
+    float a = 0.f;
+    if ((unsigned)c < (unsigned)V) {
+        const float s = lrelu(el[(size_t)c * H + k] + er[(size_t)lo * H + k], slope);
+        a = expf(s - smax[(size_t)lo * H + k]) / ssum[(size_t)lo * H + k];
+    }
+    alpha[i] = a;
+}
+
+// ---------------------------------------------------------------- backward ---
+// stat[v,k] = (er, smax, 1/ssum, g_out[v,k,:].out[v,k,:])
+__global__ void gat_bwd_node_stats(const float *__restrict__ er, const float *__restrict__ smax,
+                                   const float *__restrict__ ssum, const float *__restrict__ g_out,
+                                   const float *__restrict__ out, float4 *__restrict__ stat, int64_t VH, int D)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= VH) return;
+    const float *g = g_out + i * D, *o = out + i * D;
+    float dot = 0.f;
+    for (int j = 0; j < D; j++) dot = fmaf(g[j], o[j], dot);
+    const float l = ssum[i];
+    stat[i] = make_float4(er[i], smax[i], l > 0.f ? 1.f / l : 0.f, dot);
+}
+
+// Pass over the transposed arrays: row r = source, entries = destinations c.
+//   alpha  = exp(lrelu(el[r]+er[c]) - smax[c]) / ssum[c]
+//   galpha = g_out[c,k,:].h[r,k,:]                     (reduced over the head's lanes)
+//   gz     = alpha (galpha - g_out[c,k,:].out[c,k,:]) * lrelu'(z)
+//   g_h[r,:] += alpha g_out[c,:];  g_el[r,k] += gz;  gz_csc[perm[j],k] = gz
+// lph = lanes per head (power of two) when H > 1; for H == 1 the whole
+// wavefront (all tiles) reduces into the single head.
+template <int VEC, int NT>
+__global__ __launch_bounds__(kGatThreads) void gat_bwd_merge(
+    const int32_t *__restrict__ t_off, const int32_t *__restrict__ t_idx, const int32_t *__restrict__ t_perm,
+    const float *__restrict__ h, const float *__restrict__ el, const float4 *__restrict__ stat,
+    const float *__restrict__ g_out, float slope, float *__restrict__ g_h, float *__restrict__ g_el,
+    float *__restrict__ gz_csc, float *__restrict__ partial, float *__restrict__ pel,
+    const int32_t *__restrict__ chunk_row, int R, int E, int H, int D, int lph, int chunk, int nchunks)
+{
+    constexpr int kGatUnroll = gat_unroll(VEC * NT);
+    const int k = blockIdx.x * kGatWaves + wave_in_block();
+    if (k >= nchunks) return;
+    const int lane = lane_id();
+    const int F = H * D;
+    const int f0 = lane * VEC;
+    bool act[NT], lead[NT];
+    int head[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        const int f = f0 + t * kWave * VEC;
+        act[t] = f < F;
+        head[t] = act[t] ? f / D : 0;
+        lead[t] = act[t] && (f % D == 0);
+    }
+    const int r1 = min(max(uniform(chunk_row[k + 1]), 0), R);
+    int r = min(max(uniform(chunk_row[k]), 0), r1);
+    const int p0 = k * chunk;
+    const int p1 = min(p0 + chunk, R + E);
+    const int j0 = max(p0 - r, 0);
+    const int j1 = min(p1 - r1, E);
+
+    int rb = r;
+    int ends = (rb + lane < R) ? t_off[rb + 1 + lane] : 0x7fffffff;
+    int row_end = bcast_i(ends, 0);
+
+    float acc[NT][VEC], gel[NT], hr[NT][VEC], el_r[NT];
+    auto reset = [&]() {
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            gel[t] = 0.f;
+#pragma unroll
+            for (int v = 0; v < VEC; v++) {
+                acc[t][v] = 0.f;
+                hr[t][v] = 0.f;
+            }
+            el_r[t] = 0.f;
+            if (act[t] && r < R) {
+                gload<VEC>(hr[t], h + (size_t)r * F + f0 + t * kWave * VEC);
+                el_r[t] = el[(size_t)r * H + head[t]];
+            }
+        }
+    };
+    reset();
+    auto store_piece = [&](float *vec, float *elp) {
+#pragma unroll
+        for (int t = 0; t < NT; t++)
+            if (act[t]) {
+                gstore<VEC>(vec + f0 + t * kWave * VEC, acc[t]);
+                if (lead[t]) elp[head[t]] = gel[t];
+            }
+    };
+    auto flush_row = [&]() {
+        store_piece(g_h + (size_t)r * F, g_el + (size_t)r * H);
+        r++;
+        if (r - rb == kWave) {
+            rb = r;
+            ends = (rb + lane < R) ? t_off[rb + 1 + lane] : 0x7fffffff;
+        }
+        row_end = bcast_i(ends, r - rb);
+        reset();
+    };
+
+    for (int jb = j0; jb < j1; jb += kWave) {
+        const int n = min(kWave, j1 - jb);
+        int my_c = -1, my_p = 0;
+        if (lane < n) {
+            my_c = t_idx[jb + lane];
+            my_p = t_perm[jb + lane];
+            if ((unsigned)my_c >= (unsigned)R || (unsigned)my_p >= (unsigned)E) my_c = -1;
+        }
+        for (int i0 = 0; i0 < n; i0 += kGatUnroll) {
+            float gv[kGatUnroll][NT][VEC];
+            float4 st[kGatUnroll][NT];
+#pragma unroll
+            for (int u = 0; u < kGatUnroll; u++) {
+                if (i0 + u < n) {
+                    const int c = bcast_i(my_c, i0 + u);
+                    if (c >= 0) {
+                        const float *src = g_out + (size_t)c * F + f0;
+                        const float4 *ss = stat + (size_t)c * H;
+#pragma unroll
+                        for (int t = 0; t < NT; t++)
+                            if (act[t]) {
+                                gload<VEC>(gv[u][t], src + t * kWave * VEC);
+                                st[u][t] = ss[head[t]];
+                            }
+                    }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kGatUnroll; u++) {
+                if (i0 + u < n) {
+                    const int jj = jb + i0 + u;
+                    while (jj == row_end && r < r1) flush_row();
+                    const int c = bcast_i(my_c, i0 + u);
+                    if (c >= 0) {
+                        const int slot = bcast_i(my_p, i0 + u);
+                        float dot[NT];
+#pragma unroll
+                        for (int t = 0; t < NT; t++) {
+                            dot[t] = 0.f;
+                            if (act[t]) {
+#pragma unroll
+                                for (int v = 0; v < VEC; v++) dot[t] = fmaf(gv[u][t][v], hr[t][v], dot[t]);
+                            }
+                        }
+                        if (H == 1) {
+                            float s = 0.f;
+#pragma unroll
+                            for (int t = 0; t < NT; t++) s += dot[t];
+                            for (int o = 1; o < kWave; o <<= 1) s += __shfl_xor(s, o, kWave);
+#pragma unroll
+                            for (int t = 0; t < NT; t++) dot[t] = s;
+                        } else {
+#pragma unroll
+                            for (int t = 0; t < NT; t++)
+                                for (int o = 1; o < lph; o <<= 1) dot[t] += __shfl_xor(dot[t], o, kWave);
+                        }
+#pragma unroll
+                        for (int t = 0; t < NT; t++)
+                            if (act[t]) {
+                                const float z = el_r[t] + st[u][t].x;
+                                const float alpha = expf(lrelu(z, slope) - st[u][t].y) * st[u][t].z;
+                                const float gz = alpha * (dot[t] - st[u][t].w) * (z > 0.f ? 1.f : slope);
+                                gel[t] += gz;
+#pragma unroll
+                                for (int v = 0; v < VEC; v++) acc[t][v] = fmaf(alpha, gv[u][t][v], acc[t][v]);
+                                if (lead[t]) gz_csc[(size_t)slot * H + head[t]] = gz;
+                            }
+                    }
+                }
+            }
+        }
+    }
+    while (r < r1) flush_row();
+    if (r1 < R) store_piece(partial + (size_t)k * F, pel + (size_t)k * H);
+}
+
+template <int VEC, int NT>
+__global__ __launch_bounds__(kGatThreads) void gat_bwd_fixup(const int32_t *__restrict__ t_off,
+                                                             float *__restrict__ g_h, float *__restrict__ g_el,
+                                                             const float *__restrict__ partial,
+                                                             const float *__restrict__ pel,
+                                                             const int32_t *__restrict__ chunk_row, int H, int D,
+                                                             int chunk, int nchunks)
+{
+    const int k = blockIdx.x * kGatWaves + wave_in_block();
+    if (k >= nchunks) return;
+    const int r0 = uniform(chunk_row[k]);
+    const int r1 = uniform(chunk_row[k + 1]);
+    if (r1 <= r0) return;
+    const int lo = uniform(t_off[r0]) + r0;
+    if (lo >= k * chunk) return;
+    const int a = max(lo, 0) / chunk;
+    const int F = H * D;
+    const int f0 = lane_id() * VEC;
+    float acc[NT][VEC], gel[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        gel[t] = 0.f;
+#pragma unroll
+        for (int v = 0; v < VEC; v++) acc[t][v] = 0.f;
+    }
+    auto add = [&](const float *vec, const float *elp) {
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const int f = f0 + t * kWave * VEC;
+            if (f < F) {
+                float x[VEC];
+                gload<VEC>(x, vec + f);
+#pragma unroll
+                for (int v = 0; v < VEC; v++) acc[t][v] += x[v];
+                gel[t] += elp[f / D];
+            }
+        }
+    };
+    for (int kk = a; kk < k; kk++) add(partial + (size_t)kk * F, pel + (size_t)kk * H);
+    add(g_h + (size_t)r0 * F, g_el + (size_t)r0 * H);
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        const int f = f0 + t * kWave * VEC;
+        if (f < F) gstore<VEC>(g_h + (size_t)r0 * F + f, acc[t]);
+    }
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        const int f = f0 + t * kWave * VEC;
+        if (f < F && f % D == 0) g_el[(size_t)r0 * H + f / D] = gel[t];
+    }
+}
+
+// g_er[c,k] = sum of gz over the CSC slots of column c (contiguous), one wave per column group.
+__global__ __launch_bounds__(256) void gat_segment_sum(const int32_t *__restrict__ off, const float *__restrict__ gz,
+                                                       float *__restrict__ g_er, int V, int H)
+{
+    // thread per (column, head); columns are short on average, hubs are a few thousand slots
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (int64_t)V * H) return;
+    const int c = (int)(i / H), k = (int)(i % H);
+    float s = 0.f;
+    for (int j = off[c]; j < off[c + 1]; j++) s += gz[(size_t)j * H + k];
+    g_er[i] = s;
+}
+
+// g_h[v,f] += g_el[v,k] a_src[f] + g_er[v,k] a_dst[f]; per-block partial sums of
+// g_el*h and g_er*h over the block's rows go to red[block][2][F].
+constexpr int kRedRows = 128;
+__global__ __launch_bounds__(256) void gat_bwd_finish(const float *__restrict__ h, const float *__restrict__ a_src,
+                                                      const float *__restrict__ a_dst,
+                                                      const float *__restrict__ g_el, const float *__restrict__ g_er,
+                                                      float *__restrict__ g_h, float *__restrict__ red, int V, int H,
+                                                      int D)
+{
+    const int F = H * D;
+    const int v0 = blockIdx.x * kRedRows;
+    const int v1 = min(V, v0 + kRedRows);
+    for (int f = threadIdx.x; f < F; f += blockDim.x) {
+        const int k = f / D;
+        const float as = a_src[f], ad = a_dst[f];
+        float ss = 0.f, sd = 0.f;
+        for (int v = v0; v < v1; v++) {
+            const float gl = g_el[(size_t)v * H + k], gr = g_er[(size_t)v * H + k];
+            const float hv = h[(size_t)v * F + f];
+            g_h[(size_t)v * F + f] += gl * as + gr * ad;
+            ss = fmaf(gl, hv, ss);
+            sd = fmaf(gr, hv, sd);
+        }
+        red[((size_t)blockIdx.x * 2 + 0) * F + f] = ss;
+        red[((size_t)blockIdx.x * 2 + 1) * F + f] = sd;
+    }
+}
+
+__global__ void gat_bwd_reduce(const float *__restrict__ red, int nblocks, int F, float *__restrict__ g_a_src,
+                               float *__restrict__ g_a_dst)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= 2 * F) return;
+    const int which = i / F, f = i % F;
+    float s = 0.f;
+    for (int b = 0; b < nblocks; b++) s += red[((size_t)b * 2 + which) * F + f];
+    (which ? g_a_dst : g_a_src)[f] = s;
+}
+
+// ------------------------------------------------------------------ host ---
+struct GatShape {
+    int vec, nt, chunk, nchunks, lph;
+    bool bwd_ok;
+};
+
+static GatShape gat_shape(int32_t V, int64_t E, int32_t H, int32_t D)
+{
+    GatShape s{};
+    const int F = H * D;
+    s.vec = D % 4 == 0 ? 4 : D % 2 == 0 ? 2 : 1;
+    while (s.vec > 1 && F <= kWave * (s.vec / 2)) s.vec >>= 1;
+    s.nt = (int)ceil_div(F, kWave * s.vec);
+    const int64_t M = (int64_t)V + E;
+    s.chunk = 128;
+    while (s.chunk > 32 && M / s.chunk < 32768) s.chunk >>= 1;
+    s.nchunks = (int)ceil_div(M > 0 ? M : 1, s.chunk);
+    s.lph = D / s.vec;
+    s.bwd_ok = H == 1 || (s.lph >= 1 && s.lph <= kWave && (s.lph & (s.lph - 1)) == 0);
+    return s;
+}
+
+static int32_t check_gat(const char *who, int32_t V, int64_t E, int32_t H, int32_t D)
+{
+    if (V < 0 || E < 0 || H < 1 || D < 1) return fail(JGAMD_ERR_SIZE, "%s: bad size (V=%d E=%lld H=%d D=%d)", who, V, (long long)E, H, D);
+    if ((int64_t)V + E >= ((int64_t)1 << 31) - 4096) return fail(JGAMD_ERR_SIZE, "%s: V + E does not fit int32", who);
+    if ((int64_t)H * D > 2048) return fail(JGAMD_ERR_UNSUPPORTED, "%s: H*D = %lld above 2048", who, (long long)H * D);
+    GatShape s = gat_shape(V, E, H, D);
+    if (s.nt > 8) return fail(JGAMD_ERR_UNSUPPORTED, "%s: H*D = %d needs %d feature tiles (max 8) at vector width %d", who, H * D, s.nt, s.vec);
+    return 0;
+}
+
+static size_t gat_fwd_ws(int32_t V, int64_t E, int32_t H, int32_t D)
+{
+    GatShape s = gat_shape(V, E, H, D);
+    return carve_bytes((size_t)s.nchunks + 1, 4) + carve_bytes((size_t)s.nchunks * H * D, 4) +
+           2 * carve_bytes((size_t)s.nchunks * H, 4);
+}
+
+static size_t gat_bwd_ws(int32_t V, int64_t E, int32_t H, int32_t D)
+{
+    GatShape s = gat_shape(V, E, H, D);
+    const size_t nred = (size_t)ceil_div(V > 0 ? V : 1, kRedRows);
+    return carve_bytes((size_t)s.nchunks + 1, 4) + carve_bytes((size_t)s.nchunks * H * D, 4) +
+           carve_bytes((size_t)s.nchunks * H, 4) + carve_bytes((size_t)V * H, 16) + carve_bytes((size_t)E * H, 4) +
+           2 * carve_bytes((size_t)V * H, 4) + carve_bytes(nred * 2 * H * D, 4);
+}
+
+#define JG_GAT_DISPATCH(CALL)                         \
+    switch (s.vec * 16 + s.nt) {                      \
+        CALL(1, 1) CALL(1, 2) CALL(1, 3) CALL(1, 4) CALL(1, 5) CALL(1, 6) CALL(1, 7) CALL(1, 8) \
+        CALL(2, 1) CALL(2, 2) CALL(2, 3) CALL(2, 4) CALL(2, 5) CALL(2, 6) CALL(2, 7) CALL(2, 8) \
+        CALL(4, 1) CALL(4, 2) CALL(4, 3) CALL(4, 4) CALL(4, 5) CALL(4, 6) CALL(4, 7) CALL(4, 8) \
+    default: break;                                   \
+    }
+
+}  // namespace jg
 
 using namespace jg;
 #define JG_EXPORT extern "C" __attribute__((visibility("default")))
 
-JG_EXPORT int32_t jgamd_gat_fwd_workspace(int32_t, int64_t, int32_t, int32_t, size_t *bytes)
+JG_EXPORT int32_t jgamd_gat_fwd_workspace(int32_t V, int64_t E, int32_t H, int32_t D, size_t *bytes)
 {
-    if (bytes) *bytes = 0;
-    return fail(JGAMD_ERR_UNSUPPORTED, "gat_fwd: not implemented");
+    if (!bytes) return fail(JGAMD_ERR_NULL, "gat_fwd_workspace: bytes is NULL");
+    if (int32_t rc = check_gat("gat_fwd", V, E, H, D)) return rc;
+    *bytes = V == 0 ? 0 : gat_fwd_ws(V, E, H, D);
+    return 0;
 }
-JG_EXPORT int32_t jgamd_gat_fwd(const int32_t *, const int32_t *, const float *, const float *, const float *, float,
-                                float *, float *, float *, float *, float *, float *, int32_t, int64_t, int32_t,
-                                int32_t, void *, size_t, void *)
+
+JG_EXPORT int32_t jgamd_gat_fwd(const int32_t *off, const int32_t *idx, const float *h, const float *a_src,
+                                const float *a_dst, float slope, float *el, float *er, float *smax, float *ssum,
+                                float *alpha, float *out, int32_t V, int64_t E, int32_t H, int32_t D, void *ws,
+                                size_t ws_bytes, void *stream)
 {
-    return fail(JGAMD_ERR_UNSUPPORTED, "gat_fwd: not implemented");
+    if (int32_t rc = check_gat("gat_fwd", V, E, H, D)) return rc;
+    if (V == 0) return 0;
+    if (!off || !h || !a_src || !a_dst || !el || !er || !smax || !ssum || !out)
+        return fail(JGAMD_ERR_NULL, "gat_fwd: NULL array");
+    if (E > 0 && !idx) return fail(JGAMD_ERR_NULL, "gat_fwd: idx is NULL with E > 0");
+    if ((((uintptr_t)h | (uintptr_t)out) & 15) != 0) return fail(JGAMD_ERR_ALIGN, "gat_fwd: h/out not 16-byte aligned");
+    const size_t need = gat_fwd_ws(V, E, H, D);
+    if (!ws || ws_bytes < need) return fail(JGAMD_ERR_WORKSPACE, "gat_fwd: workspace %zu < %zu bytes", ws ? ws_bytes : (size_t)0, need);
+    if (((uintptr_t)ws & 255) != 0) return fail(JGAMD_ERR_ALIGN, "gat_fwd: workspace not 256-byte aligned");
+    const GatShape s = gat_shape(V, E, H, D);
+    Carver carve(ws);
+    int32_t *chunk_row = carve.take<int32_t>((size_t)s.nchunks + 1);
+    float *partial = carve.take<float>((size_t)s.nchunks * H * D);
+    float *pmax = carve.take<float>((size_t)s.nchunks * H);
+    float *psum = carve.take<float>((size_t)s.nchunks * H);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int64_t VH = (int64_t)V * H;
+    hipLaunchKernelGGL(gat_node_scores, dim3((unsigned)ceil_div(VH, 256)), dim3(256), 0, st, h, a_src, a_dst, el, er,
+                       VH, H, D);
+    hipLaunchKernelGGL(gat_chunk_rows, dim3((unsigned)ceil_div(V, 256)), dim3(256), 0, st, off, V, s.chunk, s.nchunks,
+                       chunk_row);
+    dim3 grid((unsigned)ceil_div(s.nchunks, kGatWaves)), block(kGatThreads);
+#define JG_FWD(VV, NN)                                                                                           \
+    case VV * 16 + NN:                                                                                           \
+        hipLaunchKernelGGL((gat_fwd_merge<VV, NN>), grid, block, 0, st, off, idx, h, el, er, slope, out, smax,   \
+                           ssum, partial, pmax, psum, chunk_row, V, (int)E, H, D, s.chunk, s.nchunks);           \
+        hipLaunchKernelGGL((gat_fwd_fixup<VV, NN>), grid, block, 0, st, off, out, smax, ssum, partial, pmax,     \
+                           psum, chunk_row, H, D, s.chunk, s.nchunks);                                           \
+        break;
+    JG_GAT_DISPATCH(JG_FWD)
+#undef JG_FWD
+    if (alpha && E > 0)
+        hipLaunchKernelGGL(gat_alpha, dim3((unsigned)ceil_div(E * H, 256)), dim3(256), 0, st, off, idx, el, er, smax,
+                           ssum, slope, alpha, V, E, H);
+    return launch_status("gat_fwd");
 }
-JG_EXPORT int32_t jgamd_gat_bwd_workspace(int32_t, int64_t, int32_t, int32_t, size_t *bytes)
+
+JG_EXPORT int32_t jgamd_gat_bwd_workspace(int32_t V, int64_t E, int32_t H, int32_t D, size_t *bytes)
 {
-    if (bytes) *bytes = 0;
-    return fail(JGAMD_ERR_UNSUPPORTED, "gat_bwd: not implemented");
+    if (!bytes) return fail(JGAMD_ERR_NULL, "gat_bwd_workspace: bytes is NULL");
+    if (int32_t rc = check_gat("gat_bwd", V, E, H, D)) return rc;
+    if (!gat_shape(V, E, H, D).bwd_ok)
+        return fail(JGAMD_ERR_UNSUPPORTED, "gat_bwd: with H > 1 the head width D=%d must give a power-of-two lane count", D);
+    *bytes = V == 0 ? 0 : gat_bwd_ws(V, E, H, D);
+    return 0;
 }
-JG_EXPORT int32_t jgamd_gat_bwd(const int32_t *, const int32_t *, const int32_t *, const int32_t *, const float *,
-                                const float *, const float *, float, const float *, const float *, const float *,
-                                const float *, const float *, const float *, float *, float *, float *, int32_t,
-                                int64_t, int32_t, int32_t, void *, size_t, void *)
+
+JG_EXPORT int32_t jgamd_gat_bwd(const int32_t *off, const int32_t *idx, const int32_t *t_off, const int32_t *t_idx,
+                                const int32_t *t_perm, const float *h, const float *a_src, const float *a_dst,
+                                float slope, const float *el, const float *er, const float *smax, const float *ssum,
+                                const float *out, const float *g_out, float *g_h, float *g_a_src, float *g_a_dst,
+                                int32_t V, int64_t E, int32_t H, int32_t D, void *ws, size_t ws_bytes, void *stream)
 {
-    return fail(JGAMD_ERR_UNSUPPORTED, "gat_bwd: not implemented");
+    (void)idx;
+    if (int32_t rc = check_gat("gat_bwd", V, E, H, D)) return rc;
+    const GatShape s = gat_shape(V, E, H, D);
+    if (!s.bwd_ok)
+        return fail(JGAMD_ERR_UNSUPPORTED, "gat_bwd: with H > 1 the head width D=%d must give a power-of-two lane count", D);
+    if (!g_a_src || !g_a_dst) return fail(JGAMD_ERR_NULL, "gat_bwd: NULL gradient output");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int F = H * D;
+    if (V == 0) {
+        hipLaunchKernelGGL(gat_bwd_reduce, dim3((unsigned)ceil_div(2 * F, 256)), dim3(256), 0, st, nullptr, 0, F,
+                           g_a_src, g_a_dst);
+        return launch_status("gat_bwd");
+    }
+    if (!off || !t_off || !h || !a_src || !a_dst || !el || !er || !smax || !ssum || !out || !g_out || !g_h)
+        return fail(JGAMD_ERR_NULL, "gat_bwd: NULL array");
+    if (E > 0 && (!t_idx || !t_perm)) return fail(JGAMD_ERR_NULL, "gat_bwd: transposed arrays are NULL with E > 0");
+    if ((((uintptr_t)h | (uintptr_t)g_out | (uintptr_t)g_h) & 15) != 0)
+        return fail(JGAMD_ERR_ALIGN, "gat_bwd: h/g_out/g_h not 16-byte aligned");
+    const size_t need = gat_bwd_ws(V, E, H, D);
+    if (!ws || ws_bytes < need) return fail(JGAMD_ERR_WORKSPACE, "gat_bwd: workspace %zu < %zu bytes", ws ? ws_bytes : (size_t)0, need);
+    if (((uintptr_t)ws & 255) != 0) return fail(JGAMD_ERR_ALIGN, "gat_bwd: workspace not 256-byte aligned");
+    Carver carve(ws);
+    int32_t *chunk_row = carve.take<int32_t>((size_t)s.nchunks + 1);
+    float *partial = carve.take<float>((size_t)s.nchunks * F);
+    float *pel = carve.take<float>((size_t)s.nchunks * H);
+    float4 *stat = carve.take<float4>((size_t)V * H);
+    float *gz = carve.take<float>((size_t)E * H);
+    float *g_el = carve.take<float>((size_t)V * H);
+    float *g_er = carve.take<float>((size_t)V * H);
+    const int nred = (int)ceil_div(V, kRedRows);
+    float *red = carve.take<float>((size_t)nred * 2 * F);
+    const int64_t VH = (int64_t)V * H;
+
+    hipLaunchKernelGGL(gat_bwd_node_stats, dim3((unsigned)ceil_div(VH, 256)), dim3(256), 0, st, er, smax, ssum, g_out,
+                       out, stat, VH, D);
+    hipLaunchKernelGGL(gat_chunk_rows, dim3((unsigned)ceil_div(V, 256)), dim3(256), 0, st, t_off, V, s.chunk,
+                       s.nchunks, chunk_row);
+    dim3 grid((unsigned)ceil_div(s.nchunks, kGatWaves)), block(kGatThreads);
+#define JG_BWD(VV, NN)                                                                                             \
+    case VV * 16 + NN:                                                                                             \
+        hipLaunchKernelGGL((gat_bwd_merge<VV, NN>), grid, block, 0, st, t_off, t_idx, t_perm, h, el, stat, g_out,  \
+                           slope, g_h, g_el, gz, partial, pel, chunk_row, V, (int)E, H, D, s.lph, s.chunk,         \
+                           s.nchunks);                                                                             \
+        hipLaunchKernelGGL((gat_bwd_fixup<VV, NN>), grid, block, 0, st, t_off, g_h, g_el, partial, pel, chunk_row, \
+                           H, D, s.chunk, s.nchunks);                                                              \
+        break;
+    JG_GAT_DISPATCH(JG_BWD)
+#undef JG_BWD
+    hipLaunchKernelGGL(gat_segment_sum, dim3((unsigned)ceil_div(VH, 256)), dim3(256), 0, st, off, gz, g_er, V, H);
+    hipLaunchKernelGGL(gat_bwd_finish, dim3((unsigned)nred), dim3(256), 0, st, h, a_src, a_dst, g_el, g_er, g_h, red,
+                       V, H, D);
+    hipLaunchKernelGGL(gat_bwd_reduce, dim3((unsigned)ceil_div(2 * F, 256)), dim3(256), 0, st, red, nred, F, g_a_src,
+                       g_a_dst);
+    return launch_status("gat_bwd");
 }

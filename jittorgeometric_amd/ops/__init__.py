@@ -1,6 +1,10 @@
 """Operators with the names and argument order of jittor_geometric.ops
-(ops/__init__.py:5-13)."""
+(ops/__init__.py:5-13), plus the fused GAT core."""
 from .aggregateWithWeight import aggregateWithWeight  # noqa: F401
 from .cootocsc import cootocsc  # noqa: F401
 from .cootocsr import cootocsr  # noqa: F401
+from .edgesoftmax import EdgeSoftmax  # noqa: F401
+from .gat import gat_aggregate  # noqa: F401
+from .scatterToEdge import ScatterToEdge  # noqa: F401
+from .scatterToVertex import ScatterToVertex  # noqa: F401
 from .spmmcsr import SpmmCsr  # noqa: F401

@@ -1,0 +1,46 @@
+"""Softmax over the in-edges of every destination.  Same call as
+jittor_geometric.ops.EdgeSoftmax (ops/edgesoftmax.py:62-80); the loops of
+ops/cpp/edgesoftmax_op.cc:36-66 and edgesoftmaxbackward_op.cc:27-54 run as
+csrc/edge_ops.hip.  x is [E] or [E,1] as in the reference, or [E,H] for H
+independent heads."""
+import torch
+
+from .. import _lib
+from ._common import as_f32
+
+
+def _heads(x):
+    return 1 if x.dim() == 1 else int(x.shape[1])
+
+
+class EdgeSoftmaxFunc(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, csc):
+        lib = _lib.load()
+        dev = _lib.require_gpu(x, csc.column_offset)
+        x = as_f32(x, "x")
+        off = csc.column_offset
+        V, E, H = off.shape[0] - 1, x.shape[0], _heads(x)
+        y = torch.empty_like(x)
+        _lib.check(lib.jgamd_edge_softmax_fwd(_lib.ptr(off), _lib.ptr(x), _lib.ptr(y), V, E, H,
+                                              _lib.stream_ptr(dev)))
+        ctx.save_for_backward(y)
+        ctx.csc = csc
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        lib = _lib.load()
+        (y,) = ctx.saved_tensors
+        off = ctx.csc.column_offset
+        g = as_f32(grad_output, "grad")
+        dev = _lib.require_gpu(g, y)
+        V, E, H = off.shape[0] - 1, y.shape[0], _heads(y)
+        dx = torch.empty_like(y)
+        _lib.check(lib.jgamd_edge_softmax_bwd(_lib.ptr(off), _lib.ptr(y), _lib.ptr(g), _lib.ptr(dx), V, E, H,
+                                              _lib.stream_ptr(dev)))
+        return dx, None
+
+
+def EdgeSoftmax(x, csc):
+    return EdgeSoftmaxFunc.apply(x, csc)

@@ -1,0 +1,79 @@
+"""Fused GAT core: logits, edge softmax and weighted aggregation in one
+kernel pass (csrc/gat.hip).  No single counterpart in the reference: it
+replaces the chain ScatterToEdge x2 -> concat -> matmul -> leaky_relu ->
+EdgeSoftmax -> multiply -> ScatterToVertex of GATConv.propagate
+(nn/conv/gat_conv.py:61-83) and the gradient chain Jittor derives from it."""
+import torch
+
+from .. import _lib
+from ._common import as_f32, transposed
+
+
+def fused_supported(H, D, backward=True):
+    """Shapes the fused kernels take; others go through the operator chain."""
+    F = H * D
+    vec = 4 if D % 4 == 0 else 2 if D % 2 == 0 else 1
+    while vec > 1 and F <= 64 * (vec // 2):
+        vec //= 2
+    if F > 2048 or -(-F // (64 * vec)) > 8:
+        return False
+    if backward and H > 1:
+        lph = D // vec
+        return 1 <= lph <= 64 and (lph & (lph - 1)) == 0
+    return True
+
+
+def gat_forward_raw(h, csc, a_src, a_dst, slope=0.2, want_alpha=False):
+    """h [V,H,D], a_src/a_dst [H,D] -> dict(out, el, er, smax, ssum, alpha)."""
+    lib = _lib.load()
+    dev = _lib.require_gpu(h, csc.row_indices, csc.column_offset, a_src, a_dst)
+    h, a_src, a_dst = as_f32(h, "h"), as_f32(a_src, "a_src"), as_f32(a_dst, "a_dst")
+    V, H, D = h.shape
+    E = csc.row_indices.shape[0]
+    mk = lambda *s: torch.empty(s, dtype=torch.float32, device=dev)
+    out, el, er, smax, ssum = mk(V, H, D), mk(V, H), mk(V, H), mk(V, H), mk(V, H)
+    alpha = mk(E, H) if want_alpha else None
+    nbytes = _lib.query(lib.jgamd_gat_fwd_workspace, V, E, H, D)
+    ws = _lib.workspace(nbytes, dev)
+    _lib.check(lib.jgamd_gat_fwd(_lib.ptr(csc.column_offset), _lib.ptr(csc.row_indices), _lib.ptr(h),
+                                 _lib.ptr(a_src), _lib.ptr(a_dst), float(slope), _lib.ptr(el), _lib.ptr(er),
+                                 _lib.ptr(smax), _lib.ptr(ssum), _lib.ptr(alpha), _lib.ptr(out), V, E, H, D,
+                                 _lib.ptr(ws), nbytes, _lib.stream_ptr(dev)))
+    return dict(out=out, el=el, er=er, smax=smax, ssum=ssum, alpha=alpha)
+
+
+class GatFusedFunc(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, h, a_src, a_dst, csc, slope):
+        r = gat_forward_raw(h, csc, a_src, a_dst, slope)
+        ctx.save_for_backward(h, a_src, a_dst, r["el"], r["er"], r["smax"], r["ssum"], r["out"])
+        ctx.csc = csc
+        ctx.slope = slope
+        return r["out"]
+
+    @staticmethod
+    def backward(ctx, g_out):
+        lib = _lib.load()
+        h, a_src, a_dst, el, er, smax, ssum, out = ctx.saved_tensors
+        csc = ctx.csc
+        g_out = as_f32(g_out, "g_out")
+        dev = _lib.require_gpu(g_out, h)
+        V, H, D = h.shape
+        E = csc.row_indices.shape[0]
+        off_t, idx_t, _, perm = transposed(csc, csc.column_offset, csc.row_indices, csc.edge_weight, V, V)
+        g_h = torch.empty_like(h)
+        g_as, g_ad = torch.empty_like(a_src), torch.empty_like(a_dst)
+        nbytes = _lib.query(lib.jgamd_gat_bwd_workspace, V, E, H, D)
+        ws = _lib.workspace(nbytes, dev)
+        _lib.check(lib.jgamd_gat_bwd(_lib.ptr(csc.column_offset), _lib.ptr(csc.row_indices), _lib.ptr(off_t),
+                                     _lib.ptr(idx_t), _lib.ptr(perm), _lib.ptr(h), _lib.ptr(a_src), _lib.ptr(a_dst),
+                                     float(ctx.slope), _lib.ptr(el), _lib.ptr(er), _lib.ptr(smax), _lib.ptr(ssum),
+                                     _lib.ptr(out), _lib.ptr(g_out), _lib.ptr(g_h), _lib.ptr(g_as), _lib.ptr(g_ad),
+                                     V, E, H, D, _lib.ptr(ws), nbytes, _lib.stream_ptr(dev)))
+        return g_h, g_as, g_ad, None, None
+
+
+def gat_aggregate(h, csc, a_src, a_dst, slope=0.2):
+    """out[v,k,:] = sum over in-edges e of v of softmax_e(leaky_relu(a_src[k].h[src(e),k] +
+    a_dst[k].h[v,k])) * h[src(e),k,:]; differentiable in h, a_src, a_dst."""
+    return GatFusedFunc.apply(h, a_src, a_dst, csc, slope)

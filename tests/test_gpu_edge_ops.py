@@ -1,0 +1,115 @@
+"""Edge softmax (forward/backward) and the scatter operators on the GPU
+against the CPU oracle, through the operator wrappers and the C ABI."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from util import assert_close, dev, rand_graph, to_gpu
+
+pytestmark = pytest.mark.gpu
+
+GOLD = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_fixtures.json")))
+
+
+def make_csc(ei, w, V):
+    from jittorgeometric_amd.ops import cootocsc
+    return cootocsc(to_gpu(ei), to_gpu(w), V), oracle.cootocsc(ei, w, V)
+
+
+def test_edgesoftmax_reference_fixture_and_gradient():
+    from jittorgeometric_amd import CSC
+    from jittorgeometric_amd.ops import EdgeSoftmax
+    g = GOLD["edgesoftmax_v3"]
+    csc = CSC(torch.tensor(g["row_indices"], dtype=torch.int32, device=dev()),
+              torch.tensor(g["column_offset"], dtype=torch.int32, device=dev()),
+              torch.ones(4, device=dev()))
+    x = torch.tensor(g["x"], device=dev(), requires_grad=True)
+    y = EdgeSoftmax(x, csc)
+    np.testing.assert_allclose(y.detach().cpu().numpy(), np.array(g["y"]), rtol=1e-6)
+    # the reference test feeds the output to BCELoss against ones (tests/test_edgesoftmax.py:31-33)
+    loss = torch.nn.functional.binary_cross_entropy(y, torch.ones_like(y))
+    loss.backward()
+    yh = y.detach().cpu().numpy()
+    gy = (-1.0 / yh / 4.0).astype(np.float32)
+    want = oracle.edgesoftmax_backward(gy, yh, np.array(g["column_offset"], np.int32))
+    assert_close(x.grad.cpu().numpy(), want, rtol=1e-5, atol=1e-6, what="BCE gradient")
+
+
+@pytest.mark.parametrize("V,E,H,hubs,seed", [
+    (1, 0, 1, 0, 0), (1, 300, 1, 0, 1), (300, 2000, 1, 2, 2), (300, 2000, 2, 2, 3), (5000, 40000, 8, 3, 4),
+    (2000, 300000, 1, 2, 5), (2000, 100000, 4, 1, 6), (700, 9000, 3, 2, 7), (700, 9000, 16, 2, 8),
+    (20000, 30000, 64, 0, 9), (100, 5000, 128, 1, 10),
+])
+def test_edgesoftmax_forward_backward(V, E, H, hubs, seed):
+    from jittorgeometric_amd.ops import EdgeSoftmax
+    rng = np.random.default_rng(seed)
+    ei, w = rand_graph(rng, V, E, hubs, hub_share=0.5)
+    csc, (row, off, _) = make_csc(ei, w, V)
+    x = (3 * rng.standard_normal((E, H))).astype(np.float32)
+    g = rng.standard_normal((E, H)).astype(np.float32)
+    xt = to_gpu(x).requires_grad_(True)
+    y = EdgeSoftmax(xt, csc)
+    y.backward(to_gpu(g))
+    want = oracle.edgesoftmax(x, off).reshape(E, H)
+    assert_close(y.detach().cpu().numpy(), want, rtol=1e-5, atol=1e-7, what="softmax")
+    # backward: compare on the oracle's own y so that only the backward kernel is judged
+    wantg = oracle.edgesoftmax_backward(g, y.detach().cpu().numpy(), off).reshape(E, H)
+    seg = np.repeat(np.arange(V), np.diff(off))
+    scale = np.zeros((V, H))
+    np.add.at(scale, seg, np.abs(want.astype(np.float64) * g))
+    assert_close(xt.grad.cpu().numpy(), wantg, scale=np.abs(wantg) + want * scale[seg], what="softmax backward")
+
+
+def test_edgesoftmax_reference_shapes_E_and_E1():
+    from jittorgeometric_amd.ops import EdgeSoftmax
+    rng = np.random.default_rng(30)
+    V, E = 400, 5000
+    ei, w = rand_graph(rng, V, E, 2)
+    csc, (row, off, _) = make_csc(ei, w, V)
+    x = rng.standard_normal(E).astype(np.float32)
+    y1 = EdgeSoftmax(to_gpu(x), csc)
+    y2 = EdgeSoftmax(to_gpu(x.reshape(E, 1)), csc)
+    assert y1.shape == (E,) and y2.shape == (E, 1)
+    assert torch.equal(y1, y2[:, 0])
+    assert_close(y1.cpu().numpy(), oracle.edgesoftmax(x, off), rtol=1e-5, atol=1e-7)
+
+
+def test_edgesoftmax_large_logits_stay_finite():
+    from jittorgeometric_amd.ops import EdgeSoftmax
+    rng = np.random.default_rng(31)
+    V, E = 100, 3000
+    ei, w = rand_graph(rng, V, E)
+    csc, (row, off, _) = make_csc(ei, w, V)
+    x = (200 * rng.standard_normal(E)).astype(np.float32)      # exp(x) alone would overflow
+    y = EdgeSoftmax(to_gpu(x), csc).cpu().numpy()
+    assert np.isfinite(y).all()
+    assert_close(y, oracle.edgesoftmax(x, off), rtol=1e-5, atol=1e-7)
+
+
+@pytest.mark.parametrize("V,E,F,seed", [(1, 0, 4, 0), (60, 500, 5, 1), (3000, 50000, 16, 2), (500, 20000, 128, 3),
+                                        (5000, 3000, 33, 4)])
+def test_scatter_ops_and_their_gradients(V, E, F, seed):
+    from jittorgeometric_amd.ops import ScatterToEdge, ScatterToVertex
+    rng = np.random.default_rng(seed)
+    ei, w = rand_graph(rng, V, E, hubs=2 if V > 10 else 0, hub_share=0.4)
+    csc, (row, off, _) = make_csc(ei, w, V)
+    x = rng.standard_normal((V, F)).astype(np.float32)
+    xe = rng.standard_normal((E, F)).astype(np.float32)
+    for flow, flag in (("src", 0), ("dst", 1)):
+        xt = to_gpu(x).requires_grad_(True)
+        out = ScatterToEdge(xt, csc, flow)
+        assert np.array_equal(out.detach().cpu().numpy(), oracle.scattertoedge(x, row, off, flag))
+        out.backward(to_gpu(xe))
+        want = oracle.edgetovertex(xe, row, off, flag)
+        scale = oracle.edgetovertex(np.abs(xe), row, off, flag)
+        assert_close(xt.grad.cpu().numpy(), want, scale, what="ScatterToEdge grad %s" % flow)
+    et = to_gpu(xe).requires_grad_(True)
+    out = ScatterToVertex(et, csc, "src")
+    want = oracle.edgetovertex(xe, row, off, 1)
+    assert_close(out.detach().cpu().numpy(), want, oracle.edgetovertex(np.abs(xe), row, off, 1), what="ScatterToVertex")
+    out.backward(to_gpu(x))
+    assert np.array_equal(et.grad.cpu().numpy(), oracle.scattertoedge(x, row, off, 1))
