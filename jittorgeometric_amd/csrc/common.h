@@ -39,6 +39,11 @@ size_t scan_ws_ints(int64_t n);
 int32_t exclusive_scan_i32(const int32_t *in, int32_t *out, int64_t n, int32_t *sums_ws,
                            hipStream_t s);
 
+// ---- row-gather SpMM for use by other kernels' host code (spmm.hip) ---------
+size_t spmm_ws_bytes(int32_t R, int64_t E, int32_t F);
+int32_t spmm_enqueue(const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out, int32_t R,
+                     int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, hipStream_t s);
+
 #ifdef __HIPCC__
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
 // Wave index inside the block as a wave-uniform (scalar) value.

@@ -64,6 +64,7 @@ __global__ void gat_chunk_rows(const int32_t *__restrict__ off, int R, int chunk
 }
 
 // el[v,k] = a_src[k,:].h[v,k,:], er[v,k] = a_dst[k,:].h[v,k,:]
+// Generic form: one thread per (node, head) walks the head's D values.
 __global__ void gat_node_scores(const float *__restrict__ h, const float *__restrict__ a_src,
                                 const float *__restrict__ a_dst, float *__restrict__ el, float *__restrict__ er,
                                 int64_t VH, int H, int D)
@@ -81,6 +82,34 @@ __global__ void gat_node_scores(const float *__restrict__ h, const float *__rest
     }
     el[i] = s;
     er[i] = d;
+}
+
+// Coalesced form for D = 4*lph with lph a power of two <= 64: the array is
+// read as one stream of float4, lph consecutive lanes hold one (node, head)
+// and fold their partial dot products with xor-shuffles.
+__global__ __launch_bounds__(256) void gat_node_scores_vec(const float4 *__restrict__ h,
+                                                           const float4 *__restrict__ a_src,
+                                                           const float4 *__restrict__ a_dst, float *__restrict__ el,
+                                                           float *__restrict__ er, int64_t n4, int H, int lph)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // float4 index into h
+    float s = 0.f, d = 0.f;
+    if (i < n4) {
+        const float4 v = h[i];
+        const int64_t vh = i / lph;                 // (node, head) pair
+        const int q = (int)(vh % H) * lph + (int)(i % lph);
+        const float4 as = a_src[q], ad = a_dst[q];
+        s = v.x * as.x + v.y * as.y + v.z * as.z + v.w * as.w;
+        d = v.x * ad.x + v.y * ad.y + v.z * ad.z + v.w * ad.w;
+    }
+    for (int o = 1; o < lph; o <<= 1) {
+        s += __shfl_xor(s, o, kWave);
+        d += __shfl_xor(d, o, kWave);
+    }
+    if (i < n4 && i % lph == 0) {
+        el[i / lph] = s;
+        er[i / lph] = d;
+    }
 }
 
 // ----------------------------------------------------------------- forward ---
@@ -271,7 +300,40 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_fixup(const int32_t *__re
             }
         }
     };
-    for (int kk = a; kk < k; kk++) merge(partial + (size_t)kk * F, pmax + (size_t)kk * H, psum + (size_t)kk * H);
+    // pieces are fetched kBatch at a time (independent loads in flight), then merged in order
+    constexpr int kBatch = VEC * NT >= 16 ? 2 : (VEC * NT >= 8 ? 4 : 8);
+    for (int kb = a; kb < k; kb += kBatch) {
+        float x[kBatch][NT][VEC], pm[kBatch][NT], pl[kBatch][NT];
+#pragma unroll
+        for (int b = 0; b < kBatch; b++)
+            if (kb + b < k) {
+#pragma unroll
+                for (int t = 0; t < NT; t++) {
+                    const int f = f0 + t * kWave * VEC;
+                    if (f < F) {
+                        gload<VEC>(x[b][t], partial + (size_t)(kb + b) * F + f);
+                        pm[b][t] = pmax[(size_t)(kb + b) * H + f / D];
+                        pl[b][t] = psum[(size_t)(kb + b) * H + f / D];
+                    }
+                }
+            }
+#pragma unroll
+        for (int b = 0; b < kBatch; b++)
+            if (kb + b < k) {
+#pragma unroll
+                for (int t = 0; t < NT; t++) {
+                    const int f = f0 + t * kWave * VEC;
+                    if (f < F && pl[b][t] > 0.f) {
+                        const float mn = fmaxf(M[t], pm[b][t]);
+                        const float so = expf(M[t] - mn), si = expf(pm[b][t] - mn);
+                        L[t] = L[t] * so + pl[b][t] * si;
+#pragma unroll
+                        for (int v = 0; v < VEC; v++) acc[t][v] = acc[t][v] * so + x[b][t][v] * si;
+                        M[t] = mn;
+                    }
+                }
+            }
+    }
     merge(out + (size_t)r0 * F, smax + (size_t)r0 * H, ssum + (size_t)r0 * H);
 #pragma unroll
     for (int t = 0; t < NT; t++) {
@@ -333,6 +395,28 @@ __global__ void gat_bwd_node_stats(const float *__restrict__ er, const float *__
     for (int j = 0; j < D; j++) dot = fmaf(g[j], o[j], dot);
     const float l = ssum[i];
     stat[i] = make_float4(er[i], smax[i], l > 0.f ? 1.f / l : 0.f, dot);
+}
+
+// Coalesced form (D = 4*lph, lph a power of two <= 64), as gat_node_scores_vec.
+__global__ __launch_bounds__(256) void gat_bwd_node_stats_vec(const float *__restrict__ er,
+                                                              const float *__restrict__ smax,
+                                                              const float *__restrict__ ssum,
+                                                              const float4 *__restrict__ g_out,
+                                                              const float4 *__restrict__ out,
+                                                              float4 *__restrict__ stat, int64_t n4, int lph)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    float dot = 0.f;
+    if (i < n4) {
+        const float4 g = g_out[i], o = out[i];
+        dot = g.x * o.x + g.y * o.y + g.z * o.z + g.w * o.w;
+    }
+    for (int o = 1; o < lph; o <<= 1) dot += __shfl_xor(dot, o, kWave);
+    if (i < n4 && i % lph == 0) {
+        const int64_t vh = i / lph;
+        const float l = ssum[vh];
+        stat[vh] = make_float4(er[vh], smax[vh], l > 0.f ? 1.f / l : 0.f, dot);
+    }
 }
 
 // Pass over the transposed arrays: row r = source, entries = destinations c.
@@ -527,7 +611,35 @@ __global__ __launch_bounds__(kGatThreads) void gat_bwd_fixup(const int32_t *__re
             }
         }
     };
-    for (int kk = a; kk < k; kk++) add(partial + (size_t)kk * F, pel + (size_t)kk * H);
+    constexpr int kBatch = VEC * NT >= 16 ? 2 : (VEC * NT >= 8 ? 4 : 8);
+    for (int kb = a; kb < k; kb += kBatch) {
+        float x[kBatch][NT][VEC], pe[kBatch][NT];
+#pragma unroll
+        for (int b = 0; b < kBatch; b++)
+            if (kb + b < k) {
+#pragma unroll
+                for (int t = 0; t < NT; t++) {
+                    const int f = f0 + t * kWave * VEC;
+                    if (f < F) {
+                        gload<VEC>(x[b][t], partial + (size_t)(kb + b) * F + f);
+                        pe[b][t] = pel[(size_t)(kb + b) * H + f / D];
+                    }
+                }
+            }
+#pragma unroll
+        for (int b = 0; b < kBatch; b++)
+            if (kb + b < k) {
+#pragma unroll
+                for (int t = 0; t < NT; t++) {
+                    const int f = f0 + t * kWave * VEC;
+                    if (f < F) {
+#pragma unroll
+                        for (int v = 0; v < VEC; v++) acc[t][v] += x[b][t][v];
+                        gel[t] += pe[b][t];
+                    }
+                }
+            }
+    }
     add(g_h + (size_t)r0 * F, g_el + (size_t)r0 * H);
 #pragma unroll
     for (int t = 0; t < NT; t++) {
@@ -541,22 +653,9 @@ __global__ __launch_bounds__(kGatThreads) void gat_bwd_fixup(const int32_t *__re
     }
 }
 
-// g_er[c,k] = sum of gz over the CSC slots of column c (contiguous), one wave per column group.
-__global__ __launch_bounds__(256) void gat_segment_sum(const int32_t *__restrict__ off, const float *__restrict__ gz,
-                                                       float *__restrict__ g_er, int V, int H)
-{
-    // thread per (column, head); columns are short on average, hubs are a few thousand slots
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= (int64_t)V * H) return;
-    const int c = (int)(i / H), k = (int)(i % H);
-    float s = 0.f;
-    for (int j = off[c]; j < off[c + 1]; j++) s += gz[(size_t)j * H + k];
-    g_er[i] = s;
-}
-
 // g_h[v,f] += g_el[v,k] a_src[f] + g_er[v,k] a_dst[f]; per-block partial sums of
 // g_el*h and g_er*h over the block's rows go to red[block][2][F].
-constexpr int kRedRows = 128;
+constexpr int kRedRows = 256;
 __global__ __launch_bounds__(256) void gat_bwd_finish(const float *__restrict__ h, const float *__restrict__ a_src,
                                                       const float *__restrict__ a_dst,
                                                       const float *__restrict__ g_el, const float *__restrict__ g_er,
@@ -582,15 +681,27 @@ __global__ __launch_bounds__(256) void gat_bwd_finish(const float *__restrict__ 
     }
 }
 
-__global__ void gat_bwd_reduce(const float *__restrict__ red, int nblocks, int F, float *__restrict__ g_a_src,
-                               float *__restrict__ g_a_dst)
+// Sums red[0..nblocks) per (which, f): 64 features per block, 16 strided
+// groups of partials added in a fixed order, then the 16 group sums in order.
+__global__ __launch_bounds__(1024) void gat_bwd_reduce(const float *__restrict__ red, int nblocks, int F,
+                                                       float *__restrict__ g_a_src, float *__restrict__ g_a_dst)
 {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= 2 * F) return;
-    const int which = i / F, f = i % F;
+    __shared__ float part[16][64];
+    const int col = blockIdx.x * 64 + (threadIdx.x & 63);   // index into [2][F]
+    const int grp = threadIdx.x >> 6;
     float s = 0.f;
-    for (int b = 0; b < nblocks; b++) s += red[((size_t)b * 2 + which) * F + f];
-    (which ? g_a_dst : g_a_src)[f] = s;
+    if (col < 2 * F) {
+        const int which = col / F, f = col % F;
+        for (int b = grp; b < nblocks; b += 16) s += red[((size_t)b * 2 + which) * F + f];
+    }
+    part[grp][threadIdx.x & 63] = s;
+    __syncthreads();
+    if (grp == 0 && col < 2 * F) {
+        float t = 0.f;
+#pragma unroll
+        for (int g = 0; g < 16; g++) t += part[g][threadIdx.x];
+        (col / F ? g_a_dst : g_a_src)[col % F] = t;
+    }
 }
 
 // ------------------------------------------------------------------ host ---
@@ -613,6 +724,13 @@ static GatShape gat_shape(int32_t V, int64_t E, int32_t H, int32_t D)
     s.lph = D / s.vec;
     s.bwd_ok = H == 1 || (s.lph >= 1 && s.lph <= kWave && (s.lph & (s.lph - 1)) == 0);
     return s;
+}
+
+// float4 streaming form of the node kernels: D = 4*lph, lph a power of two <= 64
+static bool vec_nodes_ok(int D)
+{
+    const int lph = D / 4;
+    return D % 4 == 0 && lph >= 1 && lph <= kWave && (lph & (lph - 1)) == 0;
 }
 
 static int32_t check_gat(const char *who, int32_t V, int64_t E, int32_t H, int32_t D)
@@ -638,7 +756,8 @@ static size_t gat_bwd_ws(int32_t V, int64_t E, int32_t H, int32_t D)
     const size_t nred = (size_t)ceil_div(V > 0 ? V : 1, kRedRows);
     return carve_bytes((size_t)s.nchunks + 1, 4) + carve_bytes((size_t)s.nchunks * H * D, 4) +
            carve_bytes((size_t)s.nchunks * H, 4) + carve_bytes((size_t)V * H, 16) + carve_bytes((size_t)E * H, 4) +
-           2 * carve_bytes((size_t)V * H, 4) + carve_bytes(nred * 2 * H * D, 4);
+           2 * carve_bytes((size_t)V * H, 4) + carve_bytes(nred * 2 * H * D, 4) +
+           align_up(spmm_ws_bytes(V, E, H), 256);
 }
 
 #define JG_GAT_DISPATCH(CALL)                         \
@@ -684,8 +803,13 @@ JG_EXPORT int32_t jgamd_gat_fwd(const int32_t *off, const int32_t *idx, const fl
     float *psum = carve.take<float>((size_t)s.nchunks * H);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int64_t VH = (int64_t)V * H;
-    hipLaunchKernelGGL(gat_node_scores, dim3((unsigned)ceil_div(VH, 256)), dim3(256), 0, st, h, a_src, a_dst, el, er,
-                       VH, H, D);
+    if (vec_nodes_ok(D) && (((uintptr_t)a_src | (uintptr_t)a_dst) & 15) == 0)
+        hipLaunchKernelGGL(gat_node_scores_vec, dim3((unsigned)ceil_div(VH * (D / 4), 256)), dim3(256), 0, st,
+                           reinterpret_cast<const float4 *>(h), reinterpret_cast<const float4 *>(a_src),
+                           reinterpret_cast<const float4 *>(a_dst), el, er, VH * (D / 4), H, D / 4);
+    else
+        hipLaunchKernelGGL(gat_node_scores, dim3((unsigned)ceil_div(VH, 256)), dim3(256), 0, st, h, a_src, a_dst, el,
+                           er, VH, H, D);
     hipLaunchKernelGGL(gat_chunk_rows, dim3((unsigned)ceil_div(V, 256)), dim3(256), 0, st, off, V, s.chunk, s.nchunks,
                        chunk_row);
     dim3 grid((unsigned)ceil_div(s.nchunks, kGatWaves)), block(kGatThreads);
@@ -729,7 +853,7 @@ JG_EXPORT int32_t jgamd_gat_bwd(const int32_t *off, const int32_t *idx, const in
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int F = H * D;
     if (V == 0) {
-        hipLaunchKernelGGL(gat_bwd_reduce, dim3((unsigned)ceil_div(2 * F, 256)), dim3(256), 0, st, nullptr, 0, F,
+        hipLaunchKernelGGL(gat_bwd_reduce, dim3((unsigned)ceil_div(2 * F, 64)), dim3(1024), 0, st, nullptr, 0, F,
                            g_a_src, g_a_dst);
         return launch_status("gat_bwd");
     }
@@ -753,8 +877,14 @@ JG_EXPORT int32_t jgamd_gat_bwd(const int32_t *off, const int32_t *idx, const in
     float *red = carve.take<float>((size_t)nred * 2 * F);
     const int64_t VH = (int64_t)V * H;
 
-    hipLaunchKernelGGL(gat_bwd_node_stats, dim3((unsigned)ceil_div(VH, 256)), dim3(256), 0, st, er, smax, ssum, g_out,
-                       out, stat, VH, D);
+    void *spmm_ws = carve.base + carve.used;
+    if (vec_nodes_ok(D) && (((uintptr_t)out) & 15) == 0)
+        hipLaunchKernelGGL(gat_bwd_node_stats_vec, dim3((unsigned)ceil_div(VH * (D / 4), 256)), dim3(256), 0, st, er,
+                           smax, ssum, reinterpret_cast<const float4 *>(g_out), reinterpret_cast<const float4 *>(out),
+                           stat, VH * (D / 4), D / 4);
+    else
+        hipLaunchKernelGGL(gat_bwd_node_stats, dim3((unsigned)ceil_div(VH, 256)), dim3(256), 0, st, er, smax, ssum,
+                           g_out, out, stat, VH, D);
     hipLaunchKernelGGL(gat_chunk_rows, dim3((unsigned)ceil_div(V, 256)), dim3(256), 0, st, t_off, V, s.chunk,
                        s.nchunks, chunk_row);
     dim3 grid((unsigned)ceil_div(s.nchunks, kGatWaves)), block(kGatThreads);
@@ -768,10 +898,14 @@ JG_EXPORT int32_t jgamd_gat_bwd(const int32_t *off, const int32_t *idx, const in
         break;
     JG_GAT_DISPATCH(JG_BWD)
 #undef JG_BWD
-    hipLaunchKernelGGL(gat_segment_sum, dim3((unsigned)ceil_div(VH, 256)), dim3(256), 0, st, off, gz, g_er, V, H);
+    // g_er[c,k] = sum of gz over the (contiguous) CSC slots of column c: the row-gather SpMM
+    // with identity indices and unit weights on the [E,H] array
+    if (int32_t rc = spmm_enqueue(off, nullptr, nullptr, gz, g_er, V, (int32_t)E, E, H, spmm_ws,
+                                  spmm_ws_bytes(V, E, H), st))
+        return rc;
     hipLaunchKernelGGL(gat_bwd_finish, dim3((unsigned)nred), dim3(256), 0, st, h, a_src, a_dst, g_el, g_er, g_h, red,
                        V, H, D);
-    hipLaunchKernelGGL(gat_bwd_reduce, dim3((unsigned)ceil_div(2 * F, 256)), dim3(256), 0, st, red, nred, F, g_a_src,
+    hipLaunchKernelGGL(gat_bwd_reduce, dim3((unsigned)ceil_div(2 * F, 64)), dim3(1024), 0, st, red, nred, F, g_a_src,
                        g_a_dst);
     return launch_status("gat_bwd");
 }

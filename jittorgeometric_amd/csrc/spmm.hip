@@ -188,6 +188,29 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_fixup(const int32_t *__rest
     for (int t = 0; t < NT; t++)
 #pragma unroll
         for (int v = 0; v < VEC; v++) acc[t][v] = 0.f;
+    // pieces are fetched kBatch at a time (independent loads in flight), then added in order
+    constexpr int kBatch = VEC * NT >= 16 ? 2 : (VEC * NT >= 8 ? 4 : 8);
+    for (int kb = a; kb < k; kb += kBatch) {
+        float v[kBatch][NT][VEC];
+#pragma unroll
+        for (int b = 0; b < kBatch; b++)
+            if (kb + b < k) {
+                const float *src = partial + (size_t)(kb + b) * F + f0;
+#pragma unroll
+                for (int t = 0; t < NT; t++)
+                    if (f0 + t * kWave * VEC < F) vload<VEC>(v[b][t], src + t * kWave * VEC);
+            }
+#pragma unroll
+        for (int b = 0; b < kBatch; b++)
+            if (kb + b < k) {
+#pragma unroll
+                for (int t = 0; t < NT; t++)
+                    if (f0 + t * kWave * VEC < F) {
+#pragma unroll
+                        for (int i = 0; i < VEC; i++) acc[t][i] += v[b][t][i];
+                    }
+            }
+    }
     auto add = [&](const float *src) {
 #pragma unroll
         for (int t = 0; t < NT; t++)
@@ -198,8 +221,6 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_fixup(const int32_t *__rest
                 for (int i = 0; i < VEC; i++) acc[t][i] += v[i];
             }
     };
-#pragma unroll 4
-    for (int kk = a; kk < k; kk++) add(partial + (size_t)kk * F);
     float *dst = out + (size_t)r0 * F;
     add(dst);
 #pragma unroll
@@ -249,7 +270,7 @@ static SpmmShape spmm_shape(int32_t R, int64_t E, int32_t F, bool aligned16, boo
     return s;
 }
 
-static size_t spmm_ws_bytes(int32_t R, int64_t E, int32_t F)
+size_t spmm_ws_bytes(int32_t R, int64_t E, int32_t F)
 {
     SpmmShape s = spmm_shape(R, E, F, true, true);
     return carve_bytes((size_t)s.nchunks + 1, 4) + carve_bytes((size_t)s.nchunks * (size_t)F, 4);
@@ -337,6 +358,14 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx(const i
 {
     return spmm_call(off, idx, w, x, out, R, C, E, F, ws, ws_bytes, stream, nullptr, nullptr);
 }
+
+namespace jg {
+int32_t spmm_enqueue(const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out, int32_t R,
+                     int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, hipStream_t s)
+{
+    return spmm_call(off, idx, w, x, out, R, C, E, F, ws, ws_bytes, s, nullptr, nullptr);
+}
+}  // namespace jg
 
 extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_timed(
     const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out, int32_t R, int32_t C,
