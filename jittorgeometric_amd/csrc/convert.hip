@@ -3,21 +3,26 @@
 // The reference (ops/cpp/cootocsr_op.cc:35-53, cootocsc_op.cc:33-51) is a
 // sequential counting sort: histogram of the key, prefix sum, then a scatter
 // in input order, so edges of one row keep their input order.  Atomics on a
-// GPU cannot give that order, so the scatter is done as two stable
-// partitions, each ranking its items with wave-level match + popcount:
+// GPU cannot give that order (and 10^7 global atomics write through to
+// memory), so the sort is two stable partitions that rank their items with
+// wave-level match + popcount and count only in LDS:
 //
-//   1. histogram   : off[key] += 1 (global atomics) and, per block, a count of
-//                    the block's items per BUCKET (bucket = key >> shift,
-//                    at most 2048 buckets).
-//   2. scans       : off -> exclusive prefix (the final offsets); the
-//                    (bucket, block) count table -> exclusive prefix, which
-//                    is each block's write cursor in each bucket.
-//   3. partition   : every block re-reads its items and writes them, as
-//                    12/16-byte records, to their bucket in input order.
-//   4. bucket sort : one block per bucket walks the bucket's records in
-//                    order and places each at off[key] + (rank among equal
-//                    keys so far); the bucket's output window is a few
-//                    hundred KB, so these scattered writes combine in L2.
+//   1. bucket histogram : per block of 8192 edges, LDS counts per BUCKET
+//                         (bucket = key >> shift, <= 2048 buckets).
+//   2. scan             : the (bucket, block) table -> each block's write
+//                         cursor in each bucket (and every bucket's extent).
+//   3. partition        : every block re-reads its edges and writes them, as
+//                         12/16-byte records, to their bucket in input order.
+//   4. sub-block plan   : buckets are cut into sub-blocks of <= 32768
+//                         records, so a hub's bucket is many blocks' work.
+//   5. sub-block count  : LDS counts per key of the bucket (<= 2048 keys).
+//   6. bucket offsets   : per bucket, prefix over its sub-blocks and keys ->
+//                         the final offsets array and every sub-block's
+//                         first output slot per key.
+//   7. sub-block scatter: records are walked in order and placed at
+//                         cursor[key] + (rank among equal keys so far); a
+//                         bucket's output window is a few hundred KB, so the
+//                         scattered 4-byte stores combine in L2.
 //
 // Two levels of at most 2048 bins each cover V <= 2^22 vertices.
 #include "common.h"
@@ -52,30 +57,26 @@ __device__ __forceinline__ int32_t get_id(const Rec4 &r) { return r.id; }
 
 // ---------------------------------------------------------------- step 1 ---
 // keys: the key row of edge_index.  Items with key outside [0,V) are ignored
-// here and in every later step.
-__global__ __launch_bounds__(kPartThreads) void csx_histogram(const int32_t *__restrict__ keys, int64_t E,
-                                                              int32_t V, int shift, int nbins,
-                                                              int32_t *__restrict__ off_counts,
-                                                              int32_t *__restrict__ table, int nblocks)
+// here and in every later step.  table is [nbins][nblocks] (+1 trailing zero).
+__global__ __launch_bounds__(kPartThreads) void csx_bucket_histogram(const int32_t *__restrict__ keys, int64_t E,
+                                                                     int32_t V, int shift, int nbins,
+                                                                     int32_t *__restrict__ table, int nblocks)
 {
     __shared__ int bins[kMaxBins];
     for (int b = threadIdx.x; b < nbins; b += kPartThreads) bins[b] = 0;
     __syncthreads();
-    int64_t base = (int64_t)blockIdx.x * kTile;
+    const int64_t base = (int64_t)blockIdx.x * kTile;
 #pragma unroll 4
     for (int i = 0; i < kItems; i++) {
-        int64_t e = base + (int64_t)i * kPartThreads + threadIdx.x;
+        const int64_t e = base + (int64_t)i * kPartThreads + threadIdx.x;
         if (e < E) {
-            int32_t k = keys[e];
-            if ((uint32_t)k < (uint32_t)V) {
-                atomicAdd(&off_counts[k], 1);
-                atomicAdd(&bins[k >> shift], 1);
-            }
+            const int32_t k = keys[e];
+            if ((uint32_t)k < (uint32_t)V) atomicAdd(&bins[k >> shift], 1);
         }
     }
     __syncthreads();
-    for (int b = threadIdx.x; b < nbins; b += kPartThreads)
-        table[(int64_t)b * nblocks + blockIdx.x] = bins[b];
+    for (int b = threadIdx.x; b < nbins; b += kPartThreads) table[(int64_t)b * nblocks + blockIdx.x] = bins[b];
+    if (blockIdx.x == 0 && threadIdx.x == 0) table[(int64_t)nbins * nblocks] = 0;
 }
 
 // ------------------------------------------------------- stable tile rank ---
@@ -175,43 +176,165 @@ __global__ __launch_bounds__(kPartThreads) void csx_partition(Loader in, int shi
 }
 
 // ---------------------------------------------------------------- step 4 ---
-// One block per bucket: keys [b << shift, (b+1) << shift) and the records
-// recs[off[first key] .. off[last key + 1]).  Chunks of kTile records are
-// ranked in order; cursor[] (LDS) carries each key's next free slot from one
-// chunk to the next.
+// After the scan, bucket b holds records [table[b*nblocks], table[(b+1)*nblocks]).
+// Cuts every bucket into sub-blocks of at most kSubRecords records (at least
+// one per bucket): sub_first[b] = first sub-block of b, sub_bucket[s] = bucket
+// of sub-block s (-1 for the unused tail of the max_sub launch slots).
+constexpr int kSubRecords = 4 * kTile;
+
+__global__ __launch_bounds__(1024) void csx_plan_subblocks(const int32_t *__restrict__ table, int nblocks,
+                                                           int nbuckets, int max_sub,
+                                                           int32_t *__restrict__ sub_bucket,
+                                                           int32_t *__restrict__ sub_first)
+{
+    __shared__ int first[kMaxBins + 1];
+    for (int b = threadIdx.x; b < nbuckets; b += 1024) {
+        const int size = table[(int64_t)(b + 1) * nblocks] - table[(int64_t)b * nblocks];
+        first[b] = size <= kSubRecords ? 1 : (size + kSubRecords - 1) / kSubRecords;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int run = 0;
+        for (int b = 0; b < nbuckets; b++) {
+            const int n = first[b];
+            first[b] = run;
+            run += n;
+        }
+        first[nbuckets] = run;
+    }
+    __syncthreads();
+    for (int b = threadIdx.x; b <= nbuckets; b += 1024) sub_first[b] = first[b];
+    for (int b = threadIdx.x; b < nbuckets; b += 1024)
+        for (int s = first[b]; s < first[b + 1] && s < max_sub; s++) sub_bucket[s] = b;
+    for (int s = first[nbuckets] + threadIdx.x; s < max_sub; s += 1024) sub_bucket[s] = -1;
+}
+
+struct SubRange {
+    int bucket, begin, end;
+};
+__device__ __forceinline__ SubRange sub_range(const int32_t *table, int nblocks, const int32_t *sub_bucket,
+                                              const int32_t *sub_first, int s)
+{
+    SubRange r;
+    r.bucket = sub_bucket[s];
+    if (r.bucket < 0) {
+        r.begin = r.end = 0;
+        return r;
+    }
+    const int b0 = table[(int64_t)r.bucket * nblocks], b1 = table[(int64_t)(r.bucket + 1) * nblocks];
+    r.begin = b0 + (s - sub_first[r.bucket]) * kSubRecords;
+    r.end = min(b1, r.begin + kSubRecords);
+    return r;
+}
+
+// ---------------------------------------------------------------- step 5 ---
+// cnt2[s][key] = records of sub-block s whose low key bits are `key`.
+template <typename Rec>
+__global__ __launch_bounds__(kPartThreads) void csx_sub_count(const Rec *__restrict__ recs,
+                                                              const int32_t *__restrict__ table, int nblocks,
+                                                              const int32_t *__restrict__ sub_bucket,
+                                                              const int32_t *__restrict__ sub_first, int shift,
+                                                              int32_t *__restrict__ cnt2)
+{
+    __shared__ int bins[kMaxBins];
+    const SubRange r = sub_range(table, nblocks, sub_bucket, sub_first, blockIdx.x);
+    if (r.bucket < 0) return;
+    const int nkeys = 1 << shift, mask = nkeys - 1;
+    for (int k = threadIdx.x; k < nkeys; k += kPartThreads) bins[k] = 0;
+    __syncthreads();
+    for (int e = r.begin + threadIdx.x; e < r.end; e += kPartThreads) atomicAdd(&bins[recs[e].key & mask], 1);
+    __syncthreads();
+    for (int k = threadIdx.x; k < nkeys; k += kPartThreads) cnt2[(int64_t)blockIdx.x * nkeys + k] = bins[k];
+}
+
+// ---------------------------------------------------------------- step 6 ---
+// One block per bucket.  For every key of the bucket: exclusive prefix of its
+// counts over the bucket's sub-blocks, then an exclusive prefix over the keys
+// (+ the bucket's first slot) = off[key]; cnt2[s][key] becomes the first
+// output slot of sub-block s for that key.
+__global__ __launch_bounds__(kPartThreads) void csx_bucket_offsets(const int32_t *__restrict__ table, int nblocks,
+                                                                   int nbuckets,
+                                                                   const int32_t *__restrict__ sub_first, int shift,
+                                                                   int32_t V, int32_t *__restrict__ cnt2,
+                                                                   int32_t *__restrict__ off)
+{
+    __shared__ int wave_tot[kPartWaves];
+    __shared__ int carry;
+    const int b = blockIdx.x;
+    const int nkeys = 1 << shift;
+    const int s0 = sub_first[b], s1 = sub_first[b + 1];
+    const int64_t k0 = (int64_t)b << shift;
+    if (threadIdx.x == 0) carry = table[(int64_t)b * nblocks];
+    __syncthreads();
+    for (int kb = 0; kb < nkeys; kb += kPartThreads) {
+        const int k = kb + threadIdx.x;
+        int total = 0;
+        if (k < nkeys)
+            for (int s = s0; s < s1; s++) {
+                const int c = cnt2[(int64_t)s * nkeys + k];
+                cnt2[(int64_t)s * nkeys + k] = total;
+                total += c;
+            }
+        // block-exclusive scan of `total` in key order
+        int inc = total;
+#pragma unroll
+        for (int d = 1; d < kWave; d <<= 1) {
+            const int t = __shfl_up(inc, d, kWave);
+            if (lane_id() >= d) inc += t;
+        }
+        const int w = threadIdx.x >> 6;
+        if (lane_id() == kWave - 1) wave_tot[w] = inc;
+        __syncthreads();
+        int before = carry;
+        for (int v = 0; v < w; v++) before += wave_tot[v];
+        const int key_base = before + inc - total;
+        if (k < nkeys) {
+            if (k0 + k < V) off[k0 + k] = key_base;
+            for (int s = s0; s < s1; s++) cnt2[(int64_t)s * nkeys + k] += key_base;
+        }
+        __syncthreads();
+        if (threadIdx.x == kPartThreads - 1) carry = key_base + total;
+        __syncthreads();
+    }
+    if (b == nbuckets - 1 && threadIdx.x == 0) off[V] = table[(int64_t)nbuckets * nblocks];
+}
+
+// ---------------------------------------------------------------- step 7 ---
+// One block per sub-block: chunks of kTile records are ranked in order;
+// cursor[] (LDS) carries each key's next free slot from one chunk to the next.
 template <typename Rec, bool PERM>
-__global__ __launch_bounds__(kPartThreads) void csx_bucket_sort(const Rec *__restrict__ recs,
-                                                                const int32_t *__restrict__ off, int32_t V,
-                                                                int shift, int nbits,
+__global__ __launch_bounds__(kPartThreads) void csx_sub_scatter(const Rec *__restrict__ recs,
+                                                                const int32_t *__restrict__ table, int nblocks,
+                                                                const int32_t *__restrict__ sub_bucket,
+                                                                const int32_t *__restrict__ sub_first,
+                                                                const int32_t *__restrict__ cnt2, int shift,
                                                                 int32_t *__restrict__ out_idx,
                                                                 uint32_t *__restrict__ out_w,
                                                                 int32_t *__restrict__ out_perm)
 {
     extern __shared__ int lds[];
+    const SubRange sr = sub_range(table, nblocks, sub_bucket, sub_first, blockIdx.x);
+    if (sr.bucket < 0) return;
     const int nkeys = 1 << shift;
     int *cursor = lds;               // [nkeys]
     int *cnt = lds + nkeys;          // [kPartWaves][nkeys]
-    const int64_t k0 = (int64_t)blockIdx.x << shift;
-    const int64_t k1 = min((int64_t)V, k0 + nkeys);
-    const int begin = off[k0], end = off[k1];
-    for (int k = threadIdx.x; k < nkeys; k += kPartThreads)
-        cursor[k] = k0 + k < V ? off[k0 + k] : end;
+    for (int k = threadIdx.x; k < nkeys; k += kPartThreads) cursor[k] = cnt2[(int64_t)blockIdx.x * nkeys + k];
     __syncthreads();
     const int w = threadIdx.x >> 6;
     const int mask = nkeys - 1;
-    for (int chunk = begin; chunk < end; chunk += kTile) {
+    for (int chunk = sr.begin; chunk < sr.end; chunk += kTile) {
         const int base = chunk + w * kWaveSpan + lane_id();
         Rec rec[kItems];
         int bin[kItems], pos[kItems];
 #pragma unroll
         for (int r = 0; r < kItems; r++) {
-            int e = base + r * kWave;
-            bool ok = e < end;
+            const int e = base + r * kWave;
+            const bool ok = e < sr.end;
             if (ok) rec[r] = recs[e];
             bin[r] = ok ? (rec[r].key & mask) : -1;
         }
         tile_rank(
-            cnt, nkeys, nbits, bin, pos, [&](int b) { return cursor[b]; },
+            cnt, nkeys, shift, bin, pos, [&](int b) { return cursor[b]; },
             [&](int b, int next) { cursor[b] = next; });
 #pragma unroll
         for (int r = 0; r < kItems; r++)
@@ -244,9 +367,10 @@ __global__ void fill_i32(int32_t *p, int64_t n, int32_t v)
 
 // ------------------------------------------------------------------ host ---
 struct ConvPlan {
-    int shift;        // low key bits handled by the bucket sort
+    int shift;        // low key bits handled inside a bucket
     int nbuckets;     // bins of the partition
-    int64_t nblocks;  // tiles of kTile items
+    int64_t nblocks;  // tiles of kTile edges
+    int max_sub;      // upper bound on the number of sub-blocks
 };
 
 static ConvPlan make_plan(int64_t E, int32_t V)
@@ -258,22 +382,21 @@ static ConvPlan make_plan(int64_t E, int32_t V)
     p.shift = bits > 10 ? bits - 10 : 0;
     if (p.shift > kMaxBinBits) p.shift = kMaxBinBits;
     p.nbuckets = (int)ceil_div(V > 0 ? V : 1, (int64_t)1 << p.shift);
+    p.max_sub = (int)(E / kSubRecords) + p.nbuckets;
     return p;
-}
-
-static int64_t scan_len(const ConvPlan &p, int32_t V)
-{
-    int64_t table = (int64_t)p.nbuckets * p.nblocks;
-    return table > (int64_t)V + 1 ? table : (int64_t)V + 1;
 }
 
 static size_t conv_ws_bytes(int64_t E, int32_t V, bool perm)
 {
     ConvPlan p = make_plan(E, V);
+    const size_t table_n = (size_t)p.nbuckets * (size_t)p.nblocks + 1;
     size_t b = 0;
-    b += carve_bytes((size_t)p.nbuckets * (size_t)p.nblocks, 4);
-    b += carve_bytes(scan_ws_ints(scan_len(p, V)), 4);
+    b += carve_bytes(table_n, 4);
+    b += carve_bytes(scan_ws_ints((int64_t)table_n), 4);
     b += carve_bytes((size_t)E, perm ? sizeof(Rec4) : sizeof(Rec3));
+    b += carve_bytes((size_t)p.max_sub, 4);
+    b += carve_bytes((size_t)p.nbuckets + 1, 4);
+    b += carve_bytes((size_t)p.max_sub << p.shift, 4);
     return b;
 }
 
@@ -292,22 +415,27 @@ static int32_t convert(const int32_t *keys, const int32_t *others, const float *
     using Rec = typename RecOf<PERM>::type;
     const ConvPlan p = make_plan(E, V);
     Carver carve(ws);
-    const size_t table_n = (size_t)p.nbuckets * (size_t)p.nblocks;
+    const size_t table_n = (size_t)p.nbuckets * (size_t)p.nblocks + 1;
     int32_t *table = carve.take<int32_t>(table_n);
-    int32_t *sums = carve.take<int32_t>(scan_ws_ints(scan_len(p, V)));
+    int32_t *sums = carve.take<int32_t>(scan_ws_ints((int64_t)table_n));
     Rec *recs = carve.take<Rec>((size_t)E);
+    int32_t *sub_bucket = carve.take<int32_t>((size_t)p.max_sub);
+    int32_t *sub_first = carve.take<int32_t>((size_t)p.nbuckets + 1);
+    int32_t *cnt2 = carve.take<int32_t>((size_t)p.max_sub << p.shift);
     const unsigned nb = (unsigned)p.nblocks;
+    const int nblk = (int)nb;
     int32_t rc;
 
-    hipLaunchKernelGGL(fill_i32, dim3((unsigned)ceil_div((int64_t)V + 1, 256)), dim3(256), 0, s, out_off,
-                       (int64_t)V + 1, 0);
-    if (E == 0) return launch_status("coo_to_csx(fill)");
+    if (E == 0) {
+        hipLaunchKernelGGL(fill_i32, dim3((unsigned)ceil_div((int64_t)V + 1, 256)), dim3(256), 0, s, out_off,
+                           (int64_t)V + 1, 0);
+        return launch_status("coo_to_csx(fill)");
+    }
 
     int bbits = 0;
     while ((1 << bbits) < p.nbuckets) bbits++;
-    hipLaunchKernelGGL(csx_histogram, dim3(nb), dim3(kPartThreads), 0, s, keys, E, V, p.shift, p.nbuckets, out_off,
-                       table, (int)nb);
-    if ((rc = exclusive_scan_i32(out_off, out_off, (int64_t)V + 1, sums, s))) return rc;
+    hipLaunchKernelGGL(csx_bucket_histogram, dim3(nb), dim3(kPartThreads), 0, s, keys, E, V, p.shift, p.nbuckets,
+                       table, nblk);
     if ((rc = exclusive_scan_i32(table, table, (int64_t)table_n, sums, s))) return rc;
 
     CooLoader<Rec> in{keys, others, reinterpret_cast<const uint32_t *>(w), E, V};
@@ -315,14 +443,20 @@ static int32_t convert(const int32_t *keys, const int32_t *others, const float *
     const size_t part_lds = (size_t)kPartWaves * p.nbuckets * sizeof(int);
     allow_lds(part, part_lds);
     hipLaunchKernelGGL(part, dim3(nb), dim3(kPartThreads), part_lds, s, in, p.shift, 0x7fffffff, p.nbuckets, bbits,
-                       table, (int)nb, recs);
+                       table, nblk, recs);
 
+    hipLaunchKernelGGL(csx_plan_subblocks, dim3(1), dim3(1024), 0, s, table, nblk, p.nbuckets, p.max_sub, sub_bucket,
+                       sub_first);
+    hipLaunchKernelGGL(csx_sub_count<Rec>, dim3((unsigned)p.max_sub), dim3(kPartThreads), 0, s, recs, table, nblk,
+                       sub_bucket, sub_first, p.shift, cnt2);
+    hipLaunchKernelGGL(csx_bucket_offsets, dim3((unsigned)p.nbuckets), dim3(kPartThreads), 0, s, table, nblk,
+                       p.nbuckets, sub_first, p.shift, V, cnt2, out_off);
     const int nkeys = 1 << p.shift;
-    auto sort = csx_bucket_sort<Rec, PERM>;
-    const size_t sort_lds = (size_t)(kPartWaves + 1) * nkeys * sizeof(int);
-    allow_lds(sort, sort_lds);
-    hipLaunchKernelGGL(sort, dim3((unsigned)p.nbuckets), dim3(kPartThreads), sort_lds, s, recs, out_off, V, p.shift,
-                       p.shift, out_idx, reinterpret_cast<uint32_t *>(out_w), out_perm);
+    auto scat = csx_sub_scatter<Rec, PERM>;
+    const size_t scat_lds = (size_t)(kPartWaves + 1) * nkeys * sizeof(int);
+    allow_lds(scat, scat_lds);
+    hipLaunchKernelGGL(scat, dim3((unsigned)p.max_sub), dim3(kPartThreads), scat_lds, s, recs, table, nblk,
+                       sub_bucket, sub_first, cnt2, p.shift, out_idx, reinterpret_cast<uint32_t *>(out_w), out_perm);
     return launch_status("coo_to_csx");
 }
 
