@@ -27,6 +27,9 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 F = 128
+# FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 per spmm_merge launch on this exact (seeded) workload;
+# factors from a plain 1 GiB copy in the same counter runs.
+PROFILED_TRAFFIC_BYTES = 7.161e9
 
 
 def spmm_bytes(R, E, feat):
@@ -41,8 +44,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the single-thread CPU timing")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (known traffic, for scaling rocprof counters)")
-    ap.add_argument("--traffic-bytes", type=float, default=None,
-                    help="HBM bytes per spmm_merge launch from a separate rocprofv3 --pmc run")
+    ap.add_argument("--traffic-bytes", type=float, default=PROFILED_TRAFFIC_BYTES,
+                    help="bytes moved between L2 and the fabric per spmm_merge launch, from the separate "
+                         "rocprofv3 --pmc runs summarised under profiles/ (counters cannot be read in-process)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only; --gpus %d is not supported "
@@ -118,9 +122,12 @@ def main():
     layer = GCNConv(F, F, spmm=False).to(dev)
     xg = x.clone().requires_grad_(True)
 
+    g_up = torch.randn(V, F, device=dev)
+
     def layer_step():
-        out_l = layer(xg, csc, csr)
-        out_l.sum().backward()
+        layer.zero_grad(set_to_none=True)
+        xg.grad = None
+        layer(xg, csc, csr).backward(g_up)
     gcn_ms = timed(layer_step, 10, 2)
 
     # ---- CPU baseline: the reference's single-threaded loop (oracle port) ----
@@ -170,9 +177,11 @@ def main():
         "coo_to_csc_edges_per_s": round(E / (conv_csc_ms * 1e-3)),
         "coo_to_csr_ms": round(conv_csr_ms, 4),
         "gcn_layer_fwd_bwd_ms": round(gcn_ms, 4),
-        "gcn_layer_shape": "GCNConv(128->128) on the same graph, aggregateWithWeight path, x.grad and W.grad",
+        "gcn_layer_shape": "GCNConv(128->128) on the same graph, aggregateWithWeight path: x@W, SpMM, bias; "
+                           "backward SpMM, W.grad, x.grad",
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": args.traffic_bytes,
+                     "traffic_source": "profiles/spmm_merge_f128_powerlaw_1m.txt",
                      "kernel": "spmm_merge<2,1,16>", "kernel_ms": round(k_ms.value, 4),
                      "call_ms": round(c_ms.value, 4), "algorithmic_bytes": bytes_step},
         "cpu_baseline": cpu,

@@ -252,16 +252,110 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_merge(
     }
 }
 
-// Merges, in chunk order, the pieces of a row that started in an earlier
-// chunk and ends in chunk k (its last piece sits unnormalised in out/smax/ssum).
+// Running softmax state of one row piece per lane: acc (unnormalised), max, sum.
+template <int VEC, int NT> struct SoftState {
+    float M[NT], L[NT], acc[NT][VEC];
+    __device__ __forceinline__ void clear()
+    {
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            M[t] = -INFINITY;
+            L[t] = 0.f;
+#pragma unroll
+            for (int v = 0; v < VEC; v++) acc[t][v] = 0.f;
+        }
+    }
+    // Merges pieces first..last-1 of (vec [.,F], pmax [.,H], psum [.,H]) in order;
+    // a few pieces are fetched at a time so that their loads overlap.
+    __device__ __forceinline__ void merge(const float *__restrict__ vec, const float *__restrict__ pmax,
+                                          const float *__restrict__ psum, int first, int last, int F, int H, int D,
+                                          int f0)
+    {
+        constexpr int kBatch = VEC * NT >= 16 ? 2 : (VEC * NT >= 8 ? 4 : 8);
+        for (int kb = first; kb < last; kb += kBatch) {
+            float x[kBatch][NT][VEC], pm[kBatch][NT], pl[kBatch][NT];
+#pragma unroll
+            for (int b = 0; b < kBatch; b++)
+                if (kb + b < last) {
+#pragma unroll
+                    for (int t = 0; t < NT; t++) {
+                        const int f = f0 + t * kWave * VEC;
+                        if (f < F) {
+                            gload<VEC>(x[b][t], vec + (size_t)(kb + b) * F + f);
+                            pm[b][t] = pmax[(size_t)(kb + b) * H + f / D];
+                            pl[b][t] = psum[(size_t)(kb + b) * H + f / D];
+                        }
+                    }
+                }
+#pragma unroll
+            for (int b = 0; b < kBatch; b++)
+                if (kb + b < last) {
+#pragma unroll
+                    for (int t = 0; t < NT; t++) {
+                        const int f = f0 + t * kWave * VEC;
+                        if (f < F && pl[b][t] > 0.f) {
+                            const float mn = fmaxf(M[t], pm[b][t]);
+                            const float so = expf(M[t] - mn), si = expf(pm[b][t] - mn);
+                            L[t] = L[t] * so + pl[b][t] * si;
+#pragma unroll
+                            for (int v = 0; v < VEC; v++) acc[t][v] = acc[t][v] * so + x[b][t][v] * si;
+                            M[t] = mn;
+                        }
+                    }
+                }
+        }
+    }
+};
+
+// Pieces of a long row are pre-merged in groups of kGatGroup consecutive
+// chunks (see spmm_group_sums): group g's wavefront merges the pieces of the
+// row that continues past the end of the group.
+constexpr int kGatGroup = 32;
+
 template <int VEC, int NT>
-__global__ __launch_bounds__(kGatThreads) void gat_fwd_fixup(const int32_t *__restrict__ off, float *__restrict__ out,
-                                                             float *__restrict__ smax, float *__restrict__ ssum,
+__global__ __launch_bounds__(kGatThreads) void gat_fwd_group(const int32_t *__restrict__ off,
                                                              const float *__restrict__ partial,
                                                              const float *__restrict__ pmax,
                                                              const float *__restrict__ psum,
-                                                             const int32_t *__restrict__ chunk_row, int H, int D,
-                                                             int chunk, int nchunks)
+                                                             float *__restrict__ gvec, float *__restrict__ gmax,
+                                                             float *__restrict__ gsum,
+                                                             const int32_t *__restrict__ chunk_row, int R, int H,
+                                                             int D, int chunk, int nchunks)
+{
+    const int g = blockIdx.x * kGatWaves + wave_in_block();
+    const int kend = (g + 1) * kGatGroup;
+    if (kend >= nchunks) return;
+    const int r = uniform(chunk_row[kend]);
+    if (r >= R) return;
+    const int lo = uniform(off[r]) + r;
+    if (lo >= kend * chunk) return;
+    const int a = max(max(lo, 0) / chunk, g * kGatGroup);
+    const int F = H * D;
+    const int f0 = lane_id() * VEC;
+    SoftState<VEC, NT> st;
+    st.clear();
+    st.merge(partial, pmax, psum, a, kend, F, H, D, f0);
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        const int f = f0 + t * kWave * VEC;
+        if (f < F) {
+            gstore<VEC>(gvec + (size_t)g * F + f, st.acc[t]);
+            if (f % D == 0) {
+                gmax[(size_t)g * H + f / D] = st.M[t];
+                gsum[(size_t)g * H + f / D] = st.L[t];
+            }
+        }
+    }
+}
+
+// Merges, in chunk order, the pieces of a row that started in an earlier
+// chunk and ends in chunk k (its last piece sits unnormalised in out/smax/ssum).
+template <int VEC, int NT>
+__global__ __launch_bounds__(kGatThreads) void gat_fwd_fixup(
+    const int32_t *__restrict__ off, float *__restrict__ out, float *__restrict__ smax, float *__restrict__ ssum,
+    const float *__restrict__ partial, const float *__restrict__ pmax, const float *__restrict__ psum,
+    const float *__restrict__ gvec, const float *__restrict__ gmax, const float *__restrict__ gsum,
+    const int32_t *__restrict__ chunk_row, int H, int D, int chunk, int nchunks)
 {
     const int k = blockIdx.x * kGatWaves + wave_in_block();
     if (k >= nchunks) return;
@@ -273,87 +367,36 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_fixup(const int32_t *__re
     const int a = max(lo, 0) / chunk;
     const int F = H * D;
     const int f0 = lane_id() * VEC;
-    float M[NT], L[NT], acc[NT][VEC];
-#pragma unroll
-    for (int t = 0; t < NT; t++) {
-        M[t] = -INFINITY;
-        L[t] = 0.f;
-#pragma unroll
-        for (int v = 0; v < VEC; v++) acc[t][v] = 0.f;
+    SoftState<VEC, NT> st;
+    st.clear();
+    const int ga = a / kGatGroup, gb = k / kGatGroup;
+    if (ga == gb) {
+        st.merge(partial, pmax, psum, a, k, F, H, D, f0);
+    } else {
+        st.merge(gvec, gmax, gsum, ga, gb, F, H, D, f0);
+        st.merge(partial, pmax, psum, gb * kGatGroup, k, F, H, D, f0);
     }
-    auto merge = [&](const float *vec, const float *pm, const float *pl) {
-#pragma unroll
-        for (int t = 0; t < NT; t++) {
-            const int f = f0 + t * kWave * VEC;
-            if (f < F) {
-                const float mi = pm[f / D], li = pl[f / D];
-                if (li > 0.f) {
-                    float x[VEC];
-                    gload<VEC>(x, vec + f);
-                    const float mn = fmaxf(M[t], mi);
-                    const float so = expf(M[t] - mn), si = expf(mi - mn);
-                    L[t] = L[t] * so + li * si;
-#pragma unroll
-                    for (int v = 0; v < VEC; v++) acc[t][v] = acc[t][v] * so + x[v] * si;
-                    M[t] = mn;
-                }
-            }
-        }
-    };
-    // pieces are fetched kBatch at a time (independent loads in flight), then merged in order
-    constexpr int kBatch = VEC * NT >= 16 ? 2 : (VEC * NT >= 8 ? 4 : 8);
-    for (int kb = a; kb < k; kb += kBatch) {
-        float x[kBatch][NT][VEC], pm[kBatch][NT], pl[kBatch][NT];
-#pragma unroll
-        for (int b = 0; b < kBatch; b++)
-            if (kb + b < k) {
-#pragma unroll
-                for (int t = 0; t < NT; t++) {
-                    const int f = f0 + t * kWave * VEC;
-                    if (f < F) {
-                        gload<VEC>(x[b][t], partial + (size_t)(kb + b) * F + f);
-                        pm[b][t] = pmax[(size_t)(kb + b) * H + f / D];
-                        pl[b][t] = psum[(size_t)(kb + b) * H + f / D];
-                    }
-                }
-            }
-#pragma unroll
-        for (int b = 0; b < kBatch; b++)
-            if (kb + b < k) {
-#pragma unroll
-                for (int t = 0; t < NT; t++) {
-                    const int f = f0 + t * kWave * VEC;
-                    if (f < F && pl[b][t] > 0.f) {
-                        const float mn = fmaxf(M[t], pm[b][t]);
-                        const float so = expf(M[t] - mn), si = expf(pm[b][t] - mn);
-                        L[t] = L[t] * so + pl[b][t] * si;
-#pragma unroll
-                        for (int v = 0; v < VEC; v++) acc[t][v] = acc[t][v] * so + x[b][t][v] * si;
-                        M[t] = mn;
-                    }
-                }
-            }
-    }
-    merge(out + (size_t)r0 * F, smax + (size_t)r0 * H, ssum + (size_t)r0 * H);
+    st.merge(out, smax, ssum, r0, r0 + 1, F, H, D, f0);
 #pragma unroll
     for (int t = 0; t < NT; t++) {
         const int f = f0 + t * kWave * VEC;
         if (f < F) {
             float o[VEC];
-            const float inv = L[t] > 0.f ? 1.f / L[t] : 0.f;
+            const float inv = st.L[t] > 0.f ? 1.f / st.L[t] : 0.f;
 #pragma unroll
-            for (int v = 0; v < VEC; v++) o[v] = acc[t][v] * inv;
+            for (int v = 0; v < VEC; v++) o[v] = st.acc[t][v] * inv;
             gstore<VEC>(out + (size_t)r0 * F + f, o);
         }
     }
-    // every lane of a head holds the same (M, L); the head's first lane stores them
-    // after all lanes have read the old values above (same wavefront, program order)
+    // every lane of a head holds the same (M, L); the head's first lane stores them.  The
+    // loads of the old values above are complete before these stores issue (their
+    // results feed the stored values, same wavefront).
 #pragma unroll
     for (int t = 0; t < NT; t++) {
         const int f = f0 + t * kWave * VEC;
         if (f < F && f % D == 0) {
-            smax[(size_t)r0 * H + f / D] = M[t];
-            ssum[(size_t)r0 * H + f / D] = L[t];
+            smax[(size_t)r0 * H + f / D] = st.M[t];
+            ssum[(size_t)r0 * H + f / D] = st.L[t];
         }
     }
 }
@@ -573,11 +616,97 @@ __global__ __launch_bounds__(kGatThreads) void gat_bwd_merge(
     if (r1 < R) store_piece(partial + (size_t)k * F, pel + (size_t)k * H);
 }
 
+// Plain sums of backward pieces: vec [.,F] and per-head scalars elp [.,H].
+template <int VEC, int NT> struct SumState {
+    float acc[NT][VEC], gel[NT];
+    __device__ __forceinline__ void clear()
+    {
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            gel[t] = 0.f;
+#pragma unroll
+            for (int v = 0; v < VEC; v++) acc[t][v] = 0.f;
+        }
+    }
+    __device__ __forceinline__ void add(const float *__restrict__ vec, const float *__restrict__ elp, int first,
+                                        int last, int F, int H, int D, int f0)
+    {
+        constexpr int kBatch = VEC * NT >= 16 ? 2 : (VEC * NT >= 8 ? 4 : 8);
+        for (int kb = first; kb < last; kb += kBatch) {
+            float x[kBatch][NT][VEC], pe[kBatch][NT];
+#pragma unroll
+            for (int b = 0; b < kBatch; b++)
+                if (kb + b < last) {
+#pragma unroll
+                    for (int t = 0; t < NT; t++) {
+                        const int f = f0 + t * kWave * VEC;
+                        if (f < F) {
+                            gload<VEC>(x[b][t], vec + (size_t)(kb + b) * F + f);
+                            pe[b][t] = elp[(size_t)(kb + b) * H + f / D];
+                        }
+                    }
+                }
+#pragma unroll
+            for (int b = 0; b < kBatch; b++)
+                if (kb + b < last) {
+#pragma unroll
+                    for (int t = 0; t < NT; t++) {
+                        const int f = f0 + t * kWave * VEC;
+                        if (f < F) {
+#pragma unroll
+                            for (int v = 0; v < VEC; v++) acc[t][v] += x[b][t][v];
+                            gel[t] += pe[b][t];
+                        }
+                    }
+                }
+        }
+    }
+    __device__ __forceinline__ void store(float *vec, float *elp, int F, int D, int f0) const
+    {
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const int f = f0 + t * kWave * VEC;
+            if (f < F) gstore<VEC>(vec + f, acc[t]);
+        }
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const int f = f0 + t * kWave * VEC;
+            if (f < F && f % D == 0) elp[f / D] = gel[t];
+        }
+    }
+};
+
+template <int VEC, int NT>
+__global__ __launch_bounds__(kGatThreads) void gat_bwd_group(const int32_t *__restrict__ t_off,
+                                                             const float *__restrict__ partial,
+                                                             const float *__restrict__ pel, float *__restrict__ gvec,
+                                                             float *__restrict__ gel,
+                                                             const int32_t *__restrict__ chunk_row, int R, int H,
+                                                             int D, int chunk, int nchunks)
+{
+    const int g = blockIdx.x * kGatWaves + wave_in_block();
+    const int kend = (g + 1) * kGatGroup;
+    if (kend >= nchunks) return;
+    const int r = uniform(chunk_row[kend]);
+    if (r >= R) return;
+    const int lo = uniform(t_off[r]) + r;
+    if (lo >= kend * chunk) return;
+    const int a = max(max(lo, 0) / chunk, g * kGatGroup);
+    const int F = H * D;
+    const int f0 = lane_id() * VEC;
+    SumState<VEC, NT> st;
+    st.clear();
+    st.add(partial, pel, a, kend, F, H, D, f0);
+    st.store(gvec + (size_t)g * F, gel + (size_t)g * H, F, D, f0);
+}
+
 template <int VEC, int NT>
 __global__ __launch_bounds__(kGatThreads) void gat_bwd_fixup(const int32_t *__restrict__ t_off,
                                                              float *__restrict__ g_h, float *__restrict__ g_el,
                                                              const float *__restrict__ partial,
                                                              const float *__restrict__ pel,
+                                                             const float *__restrict__ gvec,
+                                                             const float *__restrict__ gel,
                                                              const int32_t *__restrict__ chunk_row, int H, int D,
                                                              int chunk, int nchunks)
 {
@@ -591,66 +720,17 @@ __global__ __launch_bounds__(kGatThreads) void gat_bwd_fixup(const int32_t *__re
     const int a = max(lo, 0) / chunk;
     const int F = H * D;
     const int f0 = lane_id() * VEC;
-    float acc[NT][VEC], gel[NT];
-#pragma unroll
-    for (int t = 0; t < NT; t++) {
-        gel[t] = 0.f;
-#pragma unroll
-        for (int v = 0; v < VEC; v++) acc[t][v] = 0.f;
+    SumState<VEC, NT> st;
+    st.clear();
+    const int ga = a / kGatGroup, gb = k / kGatGroup;
+    if (ga == gb) {
+        st.add(partial, pel, a, k, F, H, D, f0);
+    } else {
+        st.add(gvec, gel, ga, gb, F, H, D, f0);
+        st.add(partial, pel, gb * kGatGroup, k, F, H, D, f0);
     }
-    auto add = [&](const float *vec, const float *elp) {
-#pragma unroll
-        for (int t = 0; t < NT; t++) {
-            const int f = f0 + t * kWave * VEC;
-            if (f < F) {
-                float x[VEC];
-                gload<VEC>(x, vec + f);
-#pragma unroll
-                for (int v = 0; v < VEC; v++) acc[t][v] += x[v];
-                gel[t] += elp[f / D];
-            }
-        }
-    };
-    constexpr int kBatch = VEC * NT >= 16 ? 2 : (VEC * NT >= 8 ? 4 : 8);
-    for (int kb = a; kb < k; kb += kBatch) {
-        float x[kBatch][NT][VEC], pe[kBatch][NT];
-#pragma unroll
-        for (int b = 0; b < kBatch; b++)
-            if (kb + b < k) {
-#pragma unroll
-                for (int t = 0; t < NT; t++) {
-                    const int f = f0 + t * kWave * VEC;
-                    if (f < F) {
-                        gload<VEC>(x[b][t], partial + (size_t)(kb + b) * F + f);
-                        pe[b][t] = pel[(size_t)(kb + b) * H + f / D];
-                    }
-                }
-            }
-#pragma unroll
-        for (int b = 0; b < kBatch; b++)
-            if (kb + b < k) {
-#pragma unroll
-                for (int t = 0; t < NT; t++) {
-                    const int f = f0 + t * kWave * VEC;
-                    if (f < F) {
-#pragma unroll
-                        for (int v = 0; v < VEC; v++) acc[t][v] += x[b][t][v];
-                        gel[t] += pe[b][t];
-                    }
-                }
-            }
-    }
-    add(g_h + (size_t)r0 * F, g_el + (size_t)r0 * H);
-#pragma unroll
-    for (int t = 0; t < NT; t++) {
-        const int f = f0 + t * kWave * VEC;
-        if (f < F) gstore<VEC>(g_h + (size_t)r0 * F + f, acc[t]);
-    }
-#pragma unroll
-    for (int t = 0; t < NT; t++) {
-        const int f = f0 + t * kWave * VEC;
-        if (f < F && f % D == 0) g_el[(size_t)r0 * H + f / D] = gel[t];
-    }
+    st.add(g_h, g_el, r0, r0 + 1, F, H, D, f0);
+    st.store(g_h + (size_t)r0 * F, g_el + (size_t)r0 * H, F, D, f0);
 }
 
 // g_h[v,f] += g_el[v,k] a_src[f] + g_er[v,k] a_dst[f]; per-block partial sums of
@@ -746,15 +826,17 @@ static int32_t check_gat(const char *who, int32_t V, int64_t E, int32_t H, int32
 static size_t gat_fwd_ws(int32_t V, int64_t E, int32_t H, int32_t D)
 {
     GatShape s = gat_shape(V, E, H, D);
+    const size_t ng = (size_t)ceil_div(s.nchunks, kGatGroup);
     return carve_bytes((size_t)s.nchunks + 1, 4) + carve_bytes((size_t)s.nchunks * H * D, 4) +
-           2 * carve_bytes((size_t)s.nchunks * H, 4);
+           2 * carve_bytes((size_t)s.nchunks * H, 4) + carve_bytes(ng * H * D, 4) + 2 * carve_bytes(ng * H, 4);
 }
 
 static size_t gat_bwd_ws(int32_t V, int64_t E, int32_t H, int32_t D)
 {
     GatShape s = gat_shape(V, E, H, D);
     const size_t nred = (size_t)ceil_div(V > 0 ? V : 1, kRedRows);
-    return carve_bytes((size_t)s.nchunks + 1, 4) + carve_bytes((size_t)s.nchunks * H * D, 4) +
+    const size_t ng = (size_t)ceil_div(s.nchunks, kGatGroup);
+    return carve_bytes(ng * H * D, 4) + carve_bytes(ng * H, 4) + carve_bytes((size_t)s.nchunks + 1, 4) + carve_bytes((size_t)s.nchunks * H * D, 4) +
            carve_bytes((size_t)s.nchunks * H, 4) + carve_bytes((size_t)V * H, 16) + carve_bytes((size_t)E * H, 4) +
            2 * carve_bytes((size_t)V * H, 4) + carve_bytes(nred * 2 * H * D, 4) +
            align_up(spmm_ws_bytes(V, E, H), 256);
@@ -801,6 +883,10 @@ JG_EXPORT int32_t jgamd_gat_fwd(const int32_t *off, const int32_t *idx, const fl
     float *partial = carve.take<float>((size_t)s.nchunks * H * D);
     float *pmax = carve.take<float>((size_t)s.nchunks * H);
     float *psum = carve.take<float>((size_t)s.nchunks * H);
+    const int ngroups = (int)ceil_div(s.nchunks, kGatGroup);
+    float *gvec = carve.take<float>((size_t)ngroups * H * D);
+    float *gmax = carve.take<float>((size_t)ngroups * H);
+    float *gsum = carve.take<float>((size_t)ngroups * H);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int64_t VH = (int64_t)V * H;
     if (vec_nodes_ok(D) && (((uintptr_t)a_src | (uintptr_t)a_dst) & 15) == 0)
@@ -817,8 +903,12 @@ JG_EXPORT int32_t jgamd_gat_fwd(const int32_t *off, const int32_t *idx, const fl
     case VV * 16 + NN:                                                                                           \
         hipLaunchKernelGGL((gat_fwd_merge<VV, NN>), grid, block, 0, st, off, idx, h, el, er, slope, out, smax,   \
                            ssum, partial, pmax, psum, chunk_row, V, (int)E, H, D, s.chunk, s.nchunks);           \
+        if (ngroups > 1)                                                                                         \
+            hipLaunchKernelGGL((gat_fwd_group<VV, NN>), dim3((unsigned)ceil_div(ngroups, kGatWaves)), block, 0,  \
+                               st, off, partial, pmax, psum, gvec, gmax, gsum, chunk_row, V, H, D, s.chunk,      \
+                               s.nchunks);                                                                       \
         hipLaunchKernelGGL((gat_fwd_fixup<VV, NN>), grid, block, 0, st, off, out, smax, ssum, partial, pmax,     \
-                           psum, chunk_row, H, D, s.chunk, s.nchunks);                                           \
+                           psum, gvec, gmax, gsum, chunk_row, H, D, s.chunk, s.nchunks);                         \
         break;
     JG_GAT_DISPATCH(JG_FWD)
 #undef JG_FWD
@@ -866,6 +956,9 @@ JG_EXPORT int32_t jgamd_gat_bwd(const int32_t *off, const int32_t *idx, const in
     if (!ws || ws_bytes < need) return fail(JGAMD_ERR_WORKSPACE, "gat_bwd: workspace %zu < %zu bytes", ws ? ws_bytes : (size_t)0, need);
     if (((uintptr_t)ws & 255) != 0) return fail(JGAMD_ERR_ALIGN, "gat_bwd: workspace not 256-byte aligned");
     Carver carve(ws);
+    const int ngroups = (int)ceil_div(s.nchunks, kGatGroup);
+    float *gvec = carve.take<float>((size_t)ngroups * F);
+    float *ggel = carve.take<float>((size_t)ngroups * H);
     int32_t *chunk_row = carve.take<int32_t>((size_t)s.nchunks + 1);
     float *partial = carve.take<float>((size_t)s.nchunks * F);
     float *pel = carve.take<float>((size_t)s.nchunks * H);
@@ -893,8 +986,11 @@ JG_EXPORT int32_t jgamd_gat_bwd(const int32_t *off, const int32_t *idx, const in
         hipLaunchKernelGGL((gat_bwd_merge<VV, NN>), grid, block, 0, st, t_off, t_idx, t_perm, h, el, stat, g_out,  \
                            slope, g_h, g_el, gz, partial, pel, chunk_row, V, (int)E, H, D, s.lph, s.chunk,         \
                            s.nchunks);                                                                             \
-        hipLaunchKernelGGL((gat_bwd_fixup<VV, NN>), grid, block, 0, st, t_off, g_h, g_el, partial, pel, chunk_row, \
-                           H, D, s.chunk, s.nchunks);                                                              \
+        if (ngroups > 1)                                                                                           \
+            hipLaunchKernelGGL((gat_bwd_group<VV, NN>), dim3((unsigned)ceil_div(ngroups, kGatWaves)), block, 0,    \
+                               st, t_off, partial, pel, gvec, ggel, chunk_row, V, H, D, s.chunk, s.nchunks);       \
+        hipLaunchKernelGGL((gat_bwd_fixup<VV, NN>), grid, block, 0, st, t_off, g_h, g_el, partial, pel, gvec,      \
+                           ggel, chunk_row, H, D, s.chunk, s.nchunks);                                             \
         break;
     JG_GAT_DISPATCH(JG_BWD)
 #undef JG_BWD

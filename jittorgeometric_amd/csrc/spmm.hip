@@ -21,13 +21,16 @@
 
 namespace jg {
 
+#ifndef JG_NT
+#define JG_NT 1
+#endif
 constexpr int kSpmmThreads = 256;
 constexpr int kSpmmWaves = kSpmmThreads / kWave;
 
 template <int VEC> struct Vec;
 template <> struct Vec<1> { using type = float; };
-template <> struct Vec<2> { using type = float2; };
-template <> struct Vec<4> { using type = float4; };
+template <> struct Vec<2> { typedef float type __attribute__((ext_vector_type(2))); };
+template <> struct Vec<4> { typedef float type __attribute__((ext_vector_type(4))); };
 
 template <int VEC> __device__ __forceinline__ void vload(float (&d)[VEC], const float *p)
 {
@@ -46,6 +49,18 @@ template <int VEC> __device__ __forceinline__ void vstore(float *p, const float 
     for (int i = 0; i < VEC; i++) f[i] = s[i];
     *reinterpret_cast<V *>(p) = v;
 }
+// Streaming variants: data touched once (indices, weights, the output) is
+// marked non-temporal so that it does not displace gathered x rows from L2.
+template <int VEC> __device__ __forceinline__ void vstore_stream(float *p, const float (&s)[VEC])
+{
+    using V = typename Vec<VEC>::type;
+    V v;
+    float *f = reinterpret_cast<float *>(&v);
+#pragma unroll
+    for (int i = 0; i < VEC; i++) f[i] = s[i];
+    __builtin_nontemporal_store(v, reinterpret_cast<V *>(p));
+}
+template <typename T> __device__ __forceinline__ T load_stream(const T *p) { return __builtin_nontemporal_load(p); }
 
 // chunk_row[k] = the row that owns merged position k*chunk, k < nchunks;
 // chunk_row[nchunks] = R.  Row r owns positions off[r]+r .. off[r+1]+r.
@@ -101,7 +116,7 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__rest
         float *dst = out + (size_t)r * F + f0;
 #pragma unroll
         for (int t = 0; t < NT; t++) {
-            if (act[t]) vstore<VEC>(dst + t * kWave * VEC, acc[t]);
+            if (act[t]) { if (JG_NT) vstore_stream<VEC>(dst + t * kWave * VEC, acc[t]); else vstore<VEC>(dst + t * kWave * VEC, acc[t]); }
 #pragma unroll
             for (int v = 0; v < VEC; v++) acc[t][v] = 0.f;
         }
@@ -120,8 +135,8 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__rest
         {
             const bool ok = lane < n;
             const int jj = jb + lane;
-            my_c = idx ? (ok ? idx[jj] : 0) : jj;
-            my_w = ok ? (w ? w[jj] : 1.f) : 0.f;
+            my_c = idx ? (ok ? (JG_NT ? load_stream(idx + jj) : idx[jj]) : 0) : jj;
+            my_w = ok ? (w ? (JG_NT ? load_stream(w + jj) : w[jj]) : 1.f) : 0.f;
             if ((unsigned)my_c >= (unsigned)C) {
                 my_c = 0;
                 my_w = 0.f;
@@ -165,11 +180,78 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__rest
     }
 }
 
+// Adds pieces src[first..last) (rows of F floats) to acc in order, fetching a
+// few at a time so that the loads are in flight together.
+template <int VEC, int NT>
+__device__ __forceinline__ void add_pieces(float (&acc)[NT][VEC], const float *__restrict__ src, int first, int last,
+                                           int F, int f0)
+{
+    constexpr int kBatch = VEC * NT >= 16 ? 2 : (VEC * NT >= 8 ? 4 : 8);
+    for (int kb = first; kb < last; kb += kBatch) {
+        float v[kBatch][NT][VEC];
+#pragma unroll
+        for (int b = 0; b < kBatch; b++)
+            if (kb + b < last) {
+                const float *p = src + (size_t)(kb + b) * F + f0;
+#pragma unroll
+                for (int t = 0; t < NT; t++)
+                    if (f0 + t * kWave * VEC < F) vload<VEC>(v[b][t], p + t * kWave * VEC);
+            }
+#pragma unroll
+        for (int b = 0; b < kBatch; b++)
+            if (kb + b < last) {
+#pragma unroll
+                for (int t = 0; t < NT; t++)
+                    if (f0 + t * kWave * VEC < F) {
+#pragma unroll
+                        for (int i = 0; i < VEC; i++) acc[t][i] += v[b][t][i];
+                    }
+            }
+    }
+}
+
+// A row cut into thousands of pieces (a hub with millions of entries) would
+// make its last wavefront add them all one after the other.  Pieces are
+// therefore pre-summed in groups of kGroup consecutive chunks: group g's
+// wavefront adds, in order, the pieces of the row that continues past the end
+// of the group (a suffix of the group's chunks) into group_sum[g].
+constexpr int kGroup = 32;
+
+template <int VEC, int NT>
+__global__ __launch_bounds__(kSpmmThreads) void spmm_group_sums(const int32_t *__restrict__ off,
+                                                                const float *__restrict__ partial,
+                                                                float *__restrict__ group_sum,
+                                                                const int32_t *__restrict__ chunk_row, int R, int F,
+                                                                int chunk, int nchunks)
+{
+    const int g = blockIdx.x * kSpmmWaves + wave_in_block();
+    const int kend = (g + 1) * kGroup;            // first chunk after the group
+    if (kend >= nchunks) return;                  // the last group has no row continuing past it
+    const int r = uniform(chunk_row[kend]);       // row that owns the first item after the group
+    if (r >= R) return;
+    const int lo = uniform(off[r]) + r;           // merged position of the row's first item
+    if (lo >= kend * chunk) return;               // it starts after the group: nothing continues
+    const int a = max(max(lo, 0) / chunk, g * kGroup);
+    const int f0 = blockIdx.y * (kWave * VEC * NT) + lane_id() * VEC;
+    float acc[NT][VEC];
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int v = 0; v < VEC; v++) acc[t][v] = 0.f;
+    add_pieces<VEC, NT>(acc, partial, a, kend, F, f0);
+    float *dst = group_sum + (size_t)g * F + f0;
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+        if (f0 + t * kWave * VEC < F) vstore<VEC>(dst + t * kWave * VEC, acc[t]);
+}
+
 // One wavefront per chunk b: if the first row of b started in an earlier
-// chunk a and ends in b, out[row] = partial[a] + ... + partial[b-1] + out[row].
+// chunk a and ends in b, out[row] = (pieces a .. b-1, in order) + out[row];
+// whole groups between a and b come from group_sum.
 template <int VEC, int NT>
 __global__ __launch_bounds__(kSpmmThreads) void spmm_fixup(const int32_t *__restrict__ off, float *__restrict__ out,
                                                            const float *__restrict__ partial,
+                                                           const float *__restrict__ group_sum,
                                                            const int32_t *__restrict__ chunk_row, int F, int chunk,
                                                            int nchunks)
 {
@@ -188,41 +270,17 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_fixup(const int32_t *__rest
     for (int t = 0; t < NT; t++)
 #pragma unroll
         for (int v = 0; v < VEC; v++) acc[t][v] = 0.f;
-    // pieces are fetched kBatch at a time (independent loads in flight), then added in order
-    constexpr int kBatch = VEC * NT >= 16 ? 2 : (VEC * NT >= 8 ? 4 : 8);
-    for (int kb = a; kb < k; kb += kBatch) {
-        float v[kBatch][NT][VEC];
-#pragma unroll
-        for (int b = 0; b < kBatch; b++)
-            if (kb + b < k) {
-                const float *src = partial + (size_t)(kb + b) * F + f0;
-#pragma unroll
-                for (int t = 0; t < NT; t++)
-                    if (f0 + t * kWave * VEC < F) vload<VEC>(v[b][t], src + t * kWave * VEC);
-            }
-#pragma unroll
-        for (int b = 0; b < kBatch; b++)
-            if (kb + b < k) {
-#pragma unroll
-                for (int t = 0; t < NT; t++)
-                    if (f0 + t * kWave * VEC < F) {
-#pragma unroll
-                        for (int i = 0; i < VEC; i++) acc[t][i] += v[b][t][i];
-                    }
-            }
+    const int ga = a / kGroup, gb = k / kGroup;
+    if (ga == gb) {
+        add_pieces<VEC, NT>(acc, partial, a, k, F, f0);
+    } else {
+        // group ga's sum starts at piece a (the row continues past that group),
+        // groups ga+1 .. gb-1 belong to the row entirely, the rest of gb is added piecewise
+        add_pieces<VEC, NT>(acc, group_sum, ga, gb, F, f0);
+        add_pieces<VEC, NT>(acc, partial, gb * kGroup, k, F, f0);
     }
-    auto add = [&](const float *src) {
-#pragma unroll
-        for (int t = 0; t < NT; t++)
-            if (f0 + t * kWave * VEC < F) {
-                float v[VEC];
-                vload<VEC>(v, src + f0 + t * kWave * VEC);
-#pragma unroll
-                for (int i = 0; i < VEC; i++) acc[t][i] += v[i];
-            }
-    };
     float *dst = out + (size_t)r0 * F;
-    add(dst);
+    add_pieces<VEC, NT>(acc, dst, 0, 1, F, f0);
 #pragma unroll
     for (int t = 0; t < NT; t++)
         if (f0 + t * kWave * VEC < F) vstore<VEC>(dst + f0 + t * kWave * VEC, acc[t]);
@@ -243,7 +301,7 @@ static int pick_chunk(int64_t M)
 {
     static const int forced = env_int("JGAMD_SPMM_CHUNK", 0);
     if (forced) return forced;
-    int c = 256;
+    int c = 512;
     while (c > 32 && M / c < 32768) c >>= 1;
     return c;
 }
@@ -273,13 +331,14 @@ static SpmmShape spmm_shape(int32_t R, int64_t E, int32_t F, bool aligned16, boo
 size_t spmm_ws_bytes(int32_t R, int64_t E, int32_t F)
 {
     SpmmShape s = spmm_shape(R, E, F, true, true);
-    return carve_bytes((size_t)s.nchunks + 1, 4) + carve_bytes((size_t)s.nchunks * (size_t)F, 4);
+    return carve_bytes((size_t)s.nchunks + 1, 4) + carve_bytes((size_t)s.nchunks * (size_t)F, 4) +
+           carve_bytes((size_t)ceil_div(s.nchunks, kGroup) * (size_t)F, 4);
 }
 
 template <int VEC, int NT>
 static void launch_spmm(const SpmmShape &s, const int32_t *off, const int32_t *idx, const float *w, const float *x,
-                        float *out, float *partial, const int32_t *chunk_row, int R, int C, int E, int F,
-                        hipStream_t st, hipEvent_t k0 = nullptr, hipEvent_t k1 = nullptr)
+                        float *out, float *partial, float *group_sum, const int32_t *chunk_row, int R, int C, int E,
+                        int F, hipStream_t st, hipEvent_t k0 = nullptr, hipEvent_t k1 = nullptr)
 {
     dim3 grid((unsigned)ceil_div(s.nchunks, kSpmmWaves), (unsigned)s.slabs), block(kSpmmThreads);
     // gathers in flight per wavefront: bounded by the registers they land in
@@ -288,7 +347,11 @@ static void launch_spmm(const SpmmShape &s, const int32_t *off, const int32_t *i
     hipLaunchKernelGGL((spmm_merge<VEC, NT, U>), grid, block, 0, st, off, idx, w, x, out, partial, chunk_row, R, C,
                        E, F, s.chunk, s.nchunks);
     if (k1) (void)hipEventRecord(k1, st);
-    hipLaunchKernelGGL((spmm_fixup<VEC, NT>), grid, block, 0, st, off, out, partial, chunk_row, F, s.chunk,
+    const int ngroups = (int)ceil_div(s.nchunks, kGroup);
+    if (ngroups > 1)
+        hipLaunchKernelGGL((spmm_group_sums<VEC, NT>), dim3((unsigned)ceil_div(ngroups, kSpmmWaves), (unsigned)s.slabs),
+                           block, 0, st, off, partial, group_sum, chunk_row, R, F, s.chunk, s.nchunks);
+    hipLaunchKernelGGL((spmm_fixup<VEC, NT>), grid, block, 0, st, off, out, partial, group_sum, chunk_row, F, s.chunk,
                        s.nchunks);
 }
 
@@ -333,13 +396,14 @@ static int32_t spmm_call(const int32_t *off, const int32_t *idx, const float *w,
     Carver carve(ws);
     int32_t *chunk_row = carve.take<int32_t>((size_t)s.nchunks + 1);
     float *partial = carve.take<float>((size_t)s.nchunks * (size_t)F);
+    float *group_sum = carve.take<float>((size_t)ceil_div(s.nchunks, kGroup) * (size_t)F);
     hipStream_t st = static_cast<hipStream_t>(stream);
 
     hipLaunchKernelGGL(spmm_chunk_rows, dim3((unsigned)ceil_div(R, 256)), dim3(256), 0, st, off, R, s.chunk,
                        s.nchunks, chunk_row);
 #define JG_CASE(V, N)                                                                                \
     if (s.vec == V && s.nt == N) {                                                                   \
-        launch_spmm<V, N>(s, off, idx, w, x, out, partial, chunk_row, R, C, (int)E, F, st, k0, k1);  \
+        launch_spmm<V, N>(s, off, idx, w, x, out, partial, group_sum, chunk_row, R, C, (int)E, F, st, k0, k1); \
         return launch_status("spmm_csx");                                                            \
     }
 #define JG_CASES(V) JG_CASE(V, 1) JG_CASE(V, 2) JG_CASE(V, 3) JG_CASE(V, 4) JG_CASE(V, 5) JG_CASE(V, 6) JG_CASE(V, 8)
