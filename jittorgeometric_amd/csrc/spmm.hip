@@ -88,8 +88,12 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__rest
     const int lane = lane_id();
     const int f0 = blockIdx.y * (kWave * VEC * NT) + lane * VEC;   // this lane's first feature
     bool act[NT];
+    int fo[NT];   // feature offset this lane loads from in tile t (0 when the lane is past F)
 #pragma unroll
-    for (int t = 0; t < NT; t++) act[t] = f0 + t * kWave * VEC < F;
+    for (int t = 0; t < NT; t++) {
+        act[t] = f0 + t * kWave * VEC < F;
+        fo[t] = act[t] ? f0 + t * kWave * VEC : 0;
+    }
 
     // rows are clamped so that a malformed off/E pair cannot index outside the arrays
     const int r1 = min(max(uniform(chunk_row[k + 1]), 0), R);
@@ -143,30 +147,30 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__rest
             }
         }
         for (int i0 = 0; i0 < n; i0 += UNROLL) {
+            // Issue phase: straight-line code, no branches and no lane predicates, so that the
+            // UNROLL gathers leave back to back.  Slots past n re-read row my_c = 0 of a lane
+            // that holds no entry (harmless, weight 0, never accumulated); lanes past F read
+            // the start of the row instead of being masked off.
             float xv[UNROLL][NT][VEC];
-            const bool full = i0 + UNROLL <= n;
 #pragma unroll
             for (int u = 0; u < UNROLL; u++) {
-                if (full || i0 + u < n) {
-                    const int c = bcast_i(my_c, i0 + u);
-                    const float *src = x + (size_t)c * F + f0;
+                const int c = bcast_i(my_c, (i0 + u) & (kWave - 1));
+                const float *src = x + (size_t)c * F;
 #pragma unroll
-                    for (int t = 0; t < NT; t++)
-                        if (act[t]) vload<VEC>(xv[u][t], src + t * kWave * VEC);
-                }
+                for (int t = 0; t < NT; t++) vload<VEC>(xv[u][t], src + fo[t]);
             }
+            // Consume phase, in entry order.
 #pragma unroll
             for (int u = 0; u < UNROLL; u++) {
-                if (full || i0 + u < n) {
+                if (i0 + u < n) {
                     const int jj = jb + i0 + u;
                     while (jj == row_end && r < r1) flush_row();
                     const float wv = bcast_f(my_w, i0 + u);
 #pragma unroll
-                    for (int t = 0; t < NT; t++)
-                        if (act[t]) {
+                    for (int t = 0; t < NT; t++) {
 #pragma unroll
-                            for (int v = 0; v < VEC; v++) acc[t][v] = fmaf(wv, xv[u][t][v], acc[t][v]);
-                        }
+                        for (int v = 0; v < VEC; v++) acc[t][v] = fmaf(wv, xv[u][t][v], acc[t][v]);
+                    }
                 }
             }
         }

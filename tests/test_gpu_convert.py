@@ -138,3 +138,24 @@ def test_powerlaw_1m_full_size_bit_exact():
     ei, V = synthetic.make("powerlaw_1m")
     ei, w = oracle.gcn_norm(ei, None, V)
     check_exact(ei.astype(np.int32), w, V)
+
+
+def test_dense_233k_full_size_bit_exact():
+    """Benchmark configuration 4: 232,965 nodes, ~115M lognormal-degree edges +
+    self-loops (source-sorted input, so the CSR side is a pure copy and the CSC
+    side a full sort)."""
+    from jittorgeometric_amd import synthetic
+    ei, V = synthetic.make("dense_233k")
+    ei, w = oracle.gcn_norm(ei, None, V)
+    check_exact(ei.astype(np.int32), w, V)
+
+
+def test_one_hub_with_millions_of_edges_bit_exact():
+    """A single key owning 3M of 8M edges: its bucket is cut into many
+    sub-blocks (the uncapped power-law configuration has such a hub)."""
+    rng = np.random.default_rng(77)
+    V, E = 600000, 8000000
+    ei, w = rand_graph(rng, V, E)
+    ei[0, rng.random(E) < 0.38] = 31337
+    ei[1, rng.random(E) < 0.38] = 4242
+    check_exact(ei, w, V)

@@ -134,3 +134,14 @@ def test_transpose_identity_at_full_size_and_oracle_on_a_row_sample():
     ocsc = oracle.cootocsc(ei, w, V)
     want = oracle.aggregate_with_weight(x, ocsc)
     assert_close(out.detach().cpu().numpy(), want, abs_scale(x, *ocsc), what="config 2 forward")
+
+
+def test_hub_row_with_millions_of_entries_uses_grouped_piece_sums():
+    """One destination with 2.5M in-edges: its row is cut into ~10^4 pieces
+    whose sums are grouped before the final add."""
+    rng = np.random.default_rng(78)
+    V, E, F = 50000, 3000000, 32
+    ei, w = rand_graph(rng, V, E)
+    ei[1, :2500000] = 777
+    ei[0, 2500000:2900000] = 5            # and a 400k-entry row for the backward direction
+    check_fwd_bwd(ei, w, V, F)
