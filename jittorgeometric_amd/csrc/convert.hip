@@ -66,13 +66,17 @@ __global__ __launch_bounds__(kPartThreads) void csx_bucket_histogram(const int32
     for (int b = threadIdx.x; b < nbins; b += kPartThreads) bins[b] = 0;
     __syncthreads();
     const int64_t base = (int64_t)blockIdx.x * kTile;
-#pragma unroll 4
+    // all loads first (index clamped instead of predicated), then the counting
+    int32_t k[kItems];
+#pragma unroll
     for (int i = 0; i < kItems; i++) {
         const int64_t e = base + (int64_t)i * kPartThreads + threadIdx.x;
-        if (e < E) {
-            const int32_t k = keys[e];
-            if ((uint32_t)k < (uint32_t)V) atomicAdd(&bins[k >> shift], 1);
-        }
+        k[i] = keys[e < E ? e : E - 1];
+    }
+#pragma unroll
+    for (int i = 0; i < kItems; i++) {
+        const int64_t e = base + (int64_t)i * kPartThreads + threadIdx.x;
+        if (e < E && (uint32_t)k[i] < (uint32_t)V) atomicAdd(&bins[k[i] >> shift], 1);
     }
     __syncthreads();
     for (int b = threadIdx.x; b < nbins; b += kPartThreads) table[(int64_t)b * nblocks + blockIdx.x] = bins[b];
@@ -141,14 +145,18 @@ template <typename Rec> struct CooLoader {
     const uint32_t *w;
     int64_t n;
     int32_t V;
-    __device__ __forceinline__ bool load(int64_t e, Rec &r) const
+    // Branch-free: the index is clamped, validity is judged afterwards.
+    __device__ __forceinline__ void load(int64_t e, Rec &r) const
     {
-        if (e >= n) return false;
-        r.key = keys[e];
-        r.other = others[e];
-        r.w = w ? w[e] : 0u;
-        set_id(r, (int32_t)e);
-        return (uint32_t)r.key < (uint32_t)V;
+        const int64_t c = e < n ? e : n - 1;
+        r.key = keys[c];
+        r.other = others[c];
+        r.w = w ? w[c] : 0u;
+        set_id(r, (int32_t)c);
+    }
+    __device__ __forceinline__ bool valid(int64_t e, const Rec &r) const
+    {
+        return e < n && (uint32_t)r.key < (uint32_t)V;
     }
 };
 template <typename Rec, typename Loader>
@@ -162,10 +170,10 @@ __global__ __launch_bounds__(kPartThreads) void csx_partition(Loader in, int shi
     Rec rec[kItems];
     int bin[kItems], pos[kItems];
 #pragma unroll
-    for (int r = 0; r < kItems; r++) {
-        bool ok = in.load(base + (int64_t)r * kWave, rec[r]);
-        bin[r] = ok ? ((rec[r].key >> shift) & mask) : -1;
-    }
+    for (int r = 0; r < kItems; r++) in.load(base + (int64_t)r * kWave, rec[r]);
+#pragma unroll
+    for (int r = 0; r < kItems; r++)
+        bin[r] = in.valid(base + (int64_t)r * kWave, rec[r]) ? ((rec[r].key >> shift) & mask) : -1;
     const int blk = blockIdx.x;
     tile_rank(
         cnt, nbins, nbits, bin, pos, [&](int b) { return table[(int64_t)b * nblocks + blk]; },
@@ -242,7 +250,15 @@ __global__ __launch_bounds__(kPartThreads) void csx_sub_count(const Rec *__restr
     const int nkeys = 1 << shift, mask = nkeys - 1;
     for (int k = threadIdx.x; k < nkeys; k += kPartThreads) bins[k] = 0;
     __syncthreads();
-    for (int e = r.begin + threadIdx.x; e < r.end; e += kPartThreads) atomicAdd(&bins[recs[e].key & mask], 1);
+    constexpr int kBatch = 8;
+    for (int e0 = r.begin + threadIdx.x; e0 < r.end; e0 += kBatch * kPartThreads) {
+        int32_t k[kBatch];
+#pragma unroll
+        for (int i = 0; i < kBatch; i++) k[i] = recs[min(e0 + i * kPartThreads, r.end - 1)].key;
+#pragma unroll
+        for (int i = 0; i < kBatch; i++)
+            if (e0 + i * kPartThreads < r.end) atomicAdd(&bins[k[i] & mask], 1);
+    }
     __syncthreads();
     for (int k = threadIdx.x; k < nkeys; k += kPartThreads) cnt2[(int64_t)blockIdx.x * nkeys + k] = bins[k];
 }
@@ -327,12 +343,9 @@ __global__ __launch_bounds__(kPartThreads) void csx_sub_scatter(const Rec *__res
         Rec rec[kItems];
         int bin[kItems], pos[kItems];
 #pragma unroll
-        for (int r = 0; r < kItems; r++) {
-            const int e = base + r * kWave;
-            const bool ok = e < sr.end;
-            if (ok) rec[r] = recs[e];
-            bin[r] = ok ? (rec[r].key & mask) : -1;
-        }
+        for (int r = 0; r < kItems; r++) rec[r] = recs[min(base + r * kWave, sr.end - 1)];
+#pragma unroll
+        for (int r = 0; r < kItems; r++) bin[r] = base + r * kWave < sr.end ? (rec[r].key & mask) : -1;
         tile_rank(
             cnt, nkeys, shift, bin, pos, [&](int b) { return cursor[b]; },
             [&](int b, int next) { cursor[b] = next; });

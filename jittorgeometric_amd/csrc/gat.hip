@@ -128,13 +128,14 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_merge(
     const int F = H * D;
     const int f0 = lane * VEC;
     bool act[NT], lead[NT];
-    int head[NT];
+    int head[NT], fo[NT];
 #pragma unroll
     for (int t = 0; t < NT; t++) {
         const int f = f0 + t * kWave * VEC;
         act[t] = f < F;
         head[t] = act[t] ? f / D : 0;
         lead[t] = act[t] && (f % D == 0);
+        fo[t] = act[t] ? f : 0;
     }
     const int r1 = min(max(uniform(chunk_row[k + 1]), 0), R);
     int r = min(max(uniform(chunk_row[k]), 0), r1);
@@ -196,21 +197,18 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_merge(
             if ((unsigned)my_c >= (unsigned)R) my_c = -1;
         }
         for (int i0 = 0; i0 < n; i0 += kGatUnroll) {
+            // issue phase: straight-line, no branches or lane predicates (slots past n and
+            // dropped entries read row 0; lanes past F read the start of the row)
             float xv[kGatUnroll][NT][VEC], sv[kGatUnroll][NT];
 #pragma unroll
             for (int u = 0; u < kGatUnroll; u++) {
-                if (i0 + u < n) {
-                    const int c = bcast_i(my_c, i0 + u);
-                    if (c >= 0) {
-                        const float *src = h + (size_t)c * F + f0;
-                        const float *sl = el + (size_t)c * H;
+                const int c = max(bcast_i(my_c, (i0 + u) & (kWave - 1)), 0);
+                const float *src = h + (size_t)c * F;
+                const float *sl = el + (size_t)c * H;
 #pragma unroll
-                        for (int t = 0; t < NT; t++)
-                            if (act[t]) {
-                                gload<VEC>(xv[u][t], src + t * kWave * VEC);
-                                sv[u][t] = sl[head[t]];
-                            }
-                    }
+                for (int t = 0; t < NT; t++) {
+                    gload<VEC>(xv[u][t], src + fo[t]);
+                    sv[u][t] = sl[head[t]];
                 }
             }
 #pragma unroll
@@ -274,19 +272,20 @@ template <int VEC, int NT> struct SoftState {
         constexpr int kBatch = VEC * NT >= 16 ? 2 : (VEC * NT >= 8 ? 4 : 8);
         for (int kb = first; kb < last; kb += kBatch) {
             float x[kBatch][NT][VEC], pm[kBatch][NT], pl[kBatch][NT];
+            // issue phase without branches: slots past `last` re-read the last piece and
+            // lanes past F read offset 0; both are ignored below
 #pragma unroll
-            for (int b = 0; b < kBatch; b++)
-                if (kb + b < last) {
+            for (int b = 0; b < kBatch; b++) {
+                const size_t pc = (size_t)min(kb + b, last - 1);
 #pragma unroll
-                    for (int t = 0; t < NT; t++) {
-                        const int f = f0 + t * kWave * VEC;
-                        if (f < F) {
-                            gload<VEC>(x[b][t], vec + (size_t)(kb + b) * F + f);
-                            pm[b][t] = pmax[(size_t)(kb + b) * H + f / D];
-                            pl[b][t] = psum[(size_t)(kb + b) * H + f / D];
-                        }
-                    }
+                for (int t = 0; t < NT; t++) {
+                    const int f = f0 + t * kWave * VEC;
+                    const int fc = f < F ? f : 0;
+                    gload<VEC>(x[b][t], vec + pc * F + fc);
+                    pm[b][t] = pmax[pc * H + fc / D];
+                    pl[b][t] = psum[pc * H + fc / D];
                 }
+            }
 #pragma unroll
             for (int b = 0; b < kBatch; b++)
                 if (kb + b < last) {
@@ -484,13 +483,14 @@ __global__ __launch_bounds__(kGatThreads) void gat_bwd_merge(
     const int F = H * D;
     const int f0 = lane * VEC;
     bool act[NT], lead[NT];
-    int head[NT];
+    int head[NT], fo[NT];
 #pragma unroll
     for (int t = 0; t < NT; t++) {
         const int f = f0 + t * kWave * VEC;
         act[t] = f < F;
         head[t] = act[t] ? f / D : 0;
         lead[t] = act[t] && (f % D == 0);
+        fo[t] = act[t] ? f : 0;
     }
     const int r1 = min(max(uniform(chunk_row[k + 1]), 0), R);
     int r = min(max(uniform(chunk_row[k]), 0), r1);
@@ -553,18 +553,13 @@ __global__ __launch_bounds__(kGatThreads) void gat_bwd_merge(
             float4 st[kGatUnroll][NT];
 #pragma unroll
             for (int u = 0; u < kGatUnroll; u++) {
-                if (i0 + u < n) {
-                    const int c = bcast_i(my_c, i0 + u);
-                    if (c >= 0) {
-                        const float *src = g_out + (size_t)c * F + f0;
-                        const float4 *ss = stat + (size_t)c * H;
+                const int c = max(bcast_i(my_c, (i0 + u) & (kWave - 1)), 0);
+                const float *src = g_out + (size_t)c * F;
+                const float4 *ss = stat + (size_t)c * H;
 #pragma unroll
-                        for (int t = 0; t < NT; t++)
-                            if (act[t]) {
-                                gload<VEC>(gv[u][t], src + t * kWave * VEC);
-                                st[u][t] = ss[head[t]];
-                            }
-                    }
+                for (int t = 0; t < NT; t++) {
+                    gload<VEC>(gv[u][t], src + fo[t]);
+                    st[u][t] = ss[head[t]];
                 }
             }
 #pragma unroll
@@ -635,17 +630,16 @@ template <int VEC, int NT> struct SumState {
         for (int kb = first; kb < last; kb += kBatch) {
             float x[kBatch][NT][VEC], pe[kBatch][NT];
 #pragma unroll
-            for (int b = 0; b < kBatch; b++)
-                if (kb + b < last) {
+            for (int b = 0; b < kBatch; b++) {
+                const size_t pc = (size_t)min(kb + b, last - 1);
 #pragma unroll
-                    for (int t = 0; t < NT; t++) {
-                        const int f = f0 + t * kWave * VEC;
-                        if (f < F) {
-                            gload<VEC>(x[b][t], vec + (size_t)(kb + b) * F + f);
-                            pe[b][t] = elp[(size_t)(kb + b) * H + f / D];
-                        }
-                    }
+                for (int t = 0; t < NT; t++) {
+                    const int f = f0 + t * kWave * VEC;
+                    const int fc = f < F ? f : 0;
+                    gload<VEC>(x[b][t], vec + pc * F + fc);
+                    pe[b][t] = elp[pc * H + fc / D];
                 }
+            }
 #pragma unroll
             for (int b = 0; b < kBatch; b++)
                 if (kb + b < last) {

@@ -192,15 +192,18 @@ __device__ __forceinline__ void add_pieces(float (&acc)[NT][VEC], const float *_
 {
     constexpr int kBatch = VEC * NT >= 16 ? 2 : (VEC * NT >= 8 ? 4 : 8);
     for (int kb = first; kb < last; kb += kBatch) {
+        // issue phase without branches: slots past `last` re-read the last piece, lanes past F
+        // read offset 0; both are ignored below
         float v[kBatch][NT][VEC];
 #pragma unroll
-        for (int b = 0; b < kBatch; b++)
-            if (kb + b < last) {
-                const float *p = src + (size_t)(kb + b) * F + f0;
+        for (int b = 0; b < kBatch; b++) {
+            const float *p = src + (size_t)min(kb + b, last - 1) * F;
 #pragma unroll
-                for (int t = 0; t < NT; t++)
-                    if (f0 + t * kWave * VEC < F) vload<VEC>(v[b][t], p + t * kWave * VEC);
+            for (int t = 0; t < NT; t++) {
+                const int f = f0 + t * kWave * VEC;
+                vload<VEC>(v[b][t], p + (f < F ? f : 0));
             }
+        }
 #pragma unroll
         for (int b = 0; b < kBatch; b++)
             if (kb + b < last) {
