@@ -29,7 +29,7 @@ HBM_PEAK_GBPS = 8000.0
 F = 128
 # FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 per spmm_merge launch on this exact (seeded) workload;
 # factors from a plain 1 GiB copy in the same counter runs.
-PROFILED_TRAFFIC_BYTES = 7.161e9
+PROFILED_TRAFFIC_BYTES = 7.077e9
 
 
 def spmm_bytes(R, E, feat):
@@ -130,6 +130,28 @@ def main():
         layer(xg, csc, csr).backward(g_up)
     gcn_ms = timed(layer_step, 10, 2)
 
+    # ---- fused GAT layer core on the 169k-node configuration ----------------------
+    from jittorgeometric_amd.ops import gat_aggregate
+    from jittorgeometric_amd.ops.gat import gat_forward_raw
+    from jittorgeometric_amd.utils import add_remaining_self_loops
+    gei_np, gV = synthetic.make("gat_169k")
+    gei, _ = add_remaining_self_loops(torch.from_numpy(gei_np).to(dev), None, 1.0, gV)
+    gei = gei.contiguous()
+    gE = gei.shape[1]
+    gcsc = cootocsc(gei, torch.ones(gE, device=dev), gV)
+    H, D = 8, 16
+    gh = torch.randn(gV, H, D, device=dev, requires_grad=True)
+    ga_s = (torch.randn(H, D, device=dev) / 4).requires_grad_(True)
+    ga_d = (torch.randn(H, D, device=dev) / 4).requires_grad_(True)
+    gg = torch.randn(gV, H, D, device=dev)
+    gat_fwd_ms = timed(lambda: gat_forward_raw(gh.detach(), gcsc, ga_s.detach(), ga_d.detach(), 0.2), 20, 3)
+
+    def gat_step():
+        gh.grad = ga_s.grad = ga_d.grad = None
+        gat_aggregate(gh, gcsc, ga_s, ga_d, 0.2).backward(gg)
+    gat_fb_ms = timed(gat_step, 20, 3)
+    gat_bytes = gE * (4 + 4 * H * D) + gV * (4 + 8 * H + 4 * H * D) + gV * H * D * 4 + 2 * gV * H * 4
+
     # ---- CPU baseline: the reference's single-threaded loop (oracle port) ----
     cpu = None
     if not args.no_cpu_baseline:
@@ -179,9 +201,14 @@ def main():
         "gcn_layer_fwd_bwd_ms": round(gcn_ms, 4),
         "gcn_layer_shape": "GCNConv(128->128) on the same graph, aggregateWithWeight path: x@W, SpMM, bias; "
                            "backward SpMM, W.grad, x.grad",
+        "gat_fused_fwd_ms": round(gat_fwd_ms, 4),
+        "gat_fused_fwd_bwd_ms": round(gat_fb_ms, 4),
+        "gat_fused_fwd_algorithmic_gbps": round(gat_bytes / (gat_fwd_ms * 1e-3) / 1e9, 1),
+        "gat_shape": "V=%d, E=%d (power-law exp 2.3 + self-loops), 8 heads x 16" % (gV, gE),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": args.traffic_bytes,
-                     "traffic_source": "profiles/spmm_merge_f128_powerlaw_1m.txt",
+                     "traffic_source": "profiles/bench_workload_mi355x.txt",
+                     "traffic_rate_gbps": round(args.traffic_bytes / (k_ms.value * 1e-3) / 1e9, 1) if args.traffic_bytes else None,
                      "kernel": "spmm_merge<2,1,16>", "kernel_ms": round(k_ms.value, 4),
                      "call_ms": round(c_ms.value, 4), "algorithmic_bytes": bytes_step},
         "cpu_baseline": cpu,

@@ -52,15 +52,24 @@ template <int VEC> __device__ __forceinline__ void gstore(float *p, const float 
 
 __device__ __forceinline__ float lrelu(float z, float slope) { return z > 0.f ? z : slope * z; }
 
-// chunk_row as in spmm.hip: the row owning merged position k*chunk.
+// chunk_row[k] = the row owning merged position k*chunk (row r owns positions
+// off[r]+r .. off[r+1]+r, an increasing function of r): binary search per chunk.
 __global__ void gat_chunk_rows(const int32_t *__restrict__ off, int R, int chunk, int nchunks,
                                int32_t *__restrict__ chunk_row)
 {
-    const int r = blockIdx.x * blockDim.x + threadIdx.x;
-    if (r == 0) chunk_row[nchunks] = R;
-    if (r >= R) return;
-    const int64_t lo = (int64_t)off[r] + r, hi = (int64_t)off[r + 1] + r;
-    for (int64_t k = (lo + chunk - 1) / chunk; k * chunk <= hi && k < nchunks; k++) chunk_row[k] = r;
+    const int k = blockIdx.x * blockDim.x + threadIdx.x;
+    if (k > nchunks) return;
+    if (k == nchunks) {
+        chunk_row[k] = R;
+        return;
+    }
+    const int64_t p = (int64_t)k * chunk;
+    int lo = 0, hi = R;                      // largest r in [0,R) with off[r] + r <= p
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if ((int64_t)off[mid] + mid <= p) lo = mid; else hi = mid;
+    }
+    chunk_row[k] = lo;
 }
 
 // el[v,k] = a_src[k,:].h[v,k,:], er[v,k] = a_dst[k,:].h[v,k,:]
@@ -729,7 +738,7 @@ __global__ __launch_bounds__(kGatThreads) void gat_bwd_fixup(const int32_t *__re
 
 // g_h[v,f] += g_el[v,k] a_src[f] + g_er[v,k] a_dst[f]; per-block partial sums of
 // g_el*h and g_er*h over the block's rows go to red[block][2][F].
-constexpr int kRedRows = 256;
+constexpr int kRedRows = 128;
 __global__ __launch_bounds__(256) void gat_bwd_finish(const float *__restrict__ h, const float *__restrict__ a_src,
                                                       const float *__restrict__ a_dst,
                                                       const float *__restrict__ g_el, const float *__restrict__ g_er,
@@ -739,16 +748,28 @@ __global__ __launch_bounds__(256) void gat_bwd_finish(const float *__restrict__ 
     const int F = H * D;
     const int v0 = blockIdx.x * kRedRows;
     const int v1 = min(V, v0 + kRedRows);
+    constexpr int kB = 8;                     // rows fetched together
     for (int f = threadIdx.x; f < F; f += blockDim.x) {
         const int k = f / D;
         const float as = a_src[f], ad = a_dst[f];
         float ss = 0.f, sd = 0.f;
-        for (int v = v0; v < v1; v++) {
-            const float gl = g_el[(size_t)v * H + k], gr = g_er[(size_t)v * H + k];
-            const float hv = h[(size_t)v * F + f];
-            g_h[(size_t)v * F + f] += gl * as + gr * ad;
-            ss = fmaf(gl, hv, ss);
-            sd = fmaf(gr, hv, sd);
+        for (int vb = v0; vb < v1; vb += kB) {
+            float gl[kB], gr[kB], hv[kB], gh[kB];
+#pragma unroll
+            for (int i = 0; i < kB; i++) {
+                const size_t v = (size_t)min(vb + i, v1 - 1);
+                gl[i] = g_el[v * H + k];
+                gr[i] = g_er[v * H + k];
+                hv[i] = h[v * F + f];
+                gh[i] = g_h[v * F + f];
+            }
+#pragma unroll
+            for (int i = 0; i < kB; i++)
+                if (vb + i < v1) {
+                    g_h[(size_t)(vb + i) * F + f] = gh[i] + gl[i] * as + gr[i] * ad;
+                    ss = fmaf(gl[i], hv[i], ss);
+                    sd = fmaf(gr[i], hv[i], sd);
+                }
         }
         red[((size_t)blockIdx.x * 2 + 0) * F + f] = ss;
         red[((size_t)blockIdx.x * 2 + 1) * F + f] = sd;
@@ -792,8 +813,10 @@ static GatShape gat_shape(int32_t V, int64_t E, int32_t H, int32_t D)
     while (s.vec > 1 && F <= kWave * (s.vec / 2)) s.vec >>= 1;
     s.nt = (int)ceil_div(F, kWave * s.vec);
     const int64_t M = (int64_t)V + E;
+    // items per wavefront: the start-up chain of a chunk (row lookup, offsets, indices, first
+    // gathers) is a few microseconds, so chunks stay at 64 items or more
     s.chunk = 128;
-    while (s.chunk > 32 && M / s.chunk < 32768) s.chunk >>= 1;
+    while (s.chunk > 64 && M / s.chunk < 16384) s.chunk >>= 1;
     s.nchunks = (int)ceil_div(M > 0 ? M : 1, s.chunk);
     s.lph = D / s.vec;
     s.bwd_ok = H == 1 || (s.lph >= 1 && s.lph <= kWave && (s.lph & (s.lph - 1)) == 0);
@@ -890,8 +913,8 @@ JG_EXPORT int32_t jgamd_gat_fwd(const int32_t *off, const int32_t *idx, const fl
     else
         hipLaunchKernelGGL(gat_node_scores, dim3((unsigned)ceil_div(VH, 256)), dim3(256), 0, st, h, a_src, a_dst, el,
                            er, VH, H, D);
-    hipLaunchKernelGGL(gat_chunk_rows, dim3((unsigned)ceil_div(V, 256)), dim3(256), 0, st, off, V, s.chunk, s.nchunks,
-                       chunk_row);
+    hipLaunchKernelGGL(gat_chunk_rows, dim3((unsigned)ceil_div(s.nchunks + 1, 256)), dim3(256), 0, st, off, V, s.chunk,
+                       s.nchunks, chunk_row);
     dim3 grid((unsigned)ceil_div(s.nchunks, kGatWaves)), block(kGatThreads);
 #define JG_FWD(VV, NN)                                                                                           \
     case VV * 16 + NN:                                                                                           \
@@ -972,7 +995,7 @@ JG_EXPORT int32_t jgamd_gat_bwd(const int32_t *off, const int32_t *idx, const in
     else
         hipLaunchKernelGGL(gat_bwd_node_stats, dim3((unsigned)ceil_div(VH, 256)), dim3(256), 0, st, er, smax, ssum,
                            g_out, out, stat, VH, D);
-    hipLaunchKernelGGL(gat_chunk_rows, dim3((unsigned)ceil_div(V, 256)), dim3(256), 0, st, t_off, V, s.chunk,
+    hipLaunchKernelGGL(gat_chunk_rows, dim3((unsigned)ceil_div(s.nchunks + 1, 256)), dim3(256), 0, st, t_off, V, s.chunk,
                        s.nchunks, chunk_row);
     dim3 grid((unsigned)ceil_div(s.nchunks, kGatWaves)), block(kGatThreads);
 #define JG_BWD(VV, NN)                                                                                             \

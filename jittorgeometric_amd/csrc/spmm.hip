@@ -63,15 +63,25 @@ template <int VEC> __device__ __forceinline__ void vstore_stream(float *p, const
 template <typename T> __device__ __forceinline__ T load_stream(const T *p) { return __builtin_nontemporal_load(p); }
 
 // chunk_row[k] = the row that owns merged position k*chunk, k < nchunks;
-// chunk_row[nchunks] = R.  Row r owns positions off[r]+r .. off[r+1]+r.
+// chunk_row[nchunks] = R.  Row r owns positions off[r]+r .. off[r+1]+r, an
+// increasing function of r, so each chunk finds its row by binary search
+// (a hub row spans thousands of chunks; per-chunk search keeps the work even).
 __global__ void spmm_chunk_rows(const int32_t *__restrict__ off, int R, int chunk, int nchunks,
                                 int32_t *__restrict__ chunk_row)
 {
-    const int r = blockIdx.x * blockDim.x + threadIdx.x;
-    if (r == 0) chunk_row[nchunks] = R;
-    if (r >= R) return;
-    const int64_t lo = (int64_t)off[r] + r, hi = (int64_t)off[r + 1] + r;
-    for (int64_t k = (lo + chunk - 1) / chunk; k * chunk <= hi && k < nchunks; k++) chunk_row[k] = r;
+    const int k = blockIdx.x * blockDim.x + threadIdx.x;
+    if (k > nchunks) return;
+    if (k == nchunks) {
+        chunk_row[k] = R;
+        return;
+    }
+    const int64_t p = (int64_t)k * chunk;
+    int lo = 0, hi = R;                      // largest r in [0,R) with off[r] + r <= p
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if ((int64_t)off[mid] + mid <= p) lo = mid; else hi = mid;
+    }
+    chunk_row[k] = lo;
 }
 
 template <int VEC, int NT, int UNROLL>
@@ -406,8 +416,8 @@ static int32_t spmm_call(const int32_t *off, const int32_t *idx, const float *w,
     float *group_sum = carve.take<float>((size_t)ceil_div(s.nchunks, kGroup) * (size_t)F);
     hipStream_t st = static_cast<hipStream_t>(stream);
 
-    hipLaunchKernelGGL(spmm_chunk_rows, dim3((unsigned)ceil_div(R, 256)), dim3(256), 0, st, off, R, s.chunk,
-                       s.nchunks, chunk_row);
+    hipLaunchKernelGGL(spmm_chunk_rows, dim3((unsigned)ceil_div(s.nchunks + 1, 256)), dim3(256), 0, st, off, R,
+                       s.chunk, s.nchunks, chunk_row);
 #define JG_CASE(V, N)                                                                                \
     if (s.vec == V && s.nt == N) {                                                                   \
         launch_spmm<V, N>(s, off, idx, w, x, out, partial, group_sum, chunk_row, R, C, (int)E, F, st, k0, k1); \
