@@ -21,9 +21,6 @@
 
 namespace jg {
 
-#ifndef JG_NT
-#define JG_NT 1
-#endif
 constexpr int kSpmmThreads = 256;
 constexpr int kSpmmWaves = kSpmmThreads / kWave;
 
@@ -84,7 +81,10 @@ __global__ void spmm_chunk_rows(const int32_t *__restrict__ off, int R, int chun
     chunk_row[k] = lo;
 }
 
-template <int VEC, int NT, int UNROLL>
+// WIDE = false: every row of x starts less than 4 GiB from x, so a gathered
+// row is addressed as (scalar base) + (32-bit byte offset): one readlane and
+// one vector add per entry.  WIDE = true keeps 64-bit row arithmetic.
+template <int VEC, int NT, int UNROLL, bool WIDE>
 __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__restrict__ off,
                                                            const int32_t *__restrict__ idx,
                                                            const float *__restrict__ w,
@@ -93,17 +93,22 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__rest
                                                            const int32_t *__restrict__ chunk_row, int R, int C,
                                                            int E, int F, int chunk, int nchunks)
 {
+    static_assert(kWave % UNROLL == 0, "groups tile a 64-entry batch");
     const int k = blockIdx.x * kSpmmWaves + wave_in_block();
     if (k >= nchunks) return;
     const int lane = lane_id();
     const int f0 = blockIdx.y * (kWave * VEC * NT) + lane * VEC;   // this lane's first feature
     bool act[NT];
-    int fo[NT];   // feature offset this lane loads from in tile t (0 when the lane is past F)
+    int fo[NT];           // feature offset this lane loads from in tile t (0 when the lane is past F)
+    uint32_t fo_bytes[NT];
 #pragma unroll
     for (int t = 0; t < NT; t++) {
         act[t] = f0 + t * kWave * VEC < F;
         fo[t] = act[t] ? f0 + t * kWave * VEC : 0;
+        fo_bytes[t] = (uint32_t)fo[t] * 4u;
     }
+    const char *xb = reinterpret_cast<const char *>(x);
+    const uint32_t row_bytes = (uint32_t)F * 4u;
 
     // rows are clamped so that a malformed off/E pair cannot index outside the arrays
     const int r1 = min(max(uniform(chunk_row[k + 1]), 0), R);
@@ -115,10 +120,13 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__rest
     int j1 = min(p1 - r1, E);
     j0 = max(j0, 0);
 
-    // window of 64 row ends starting at row rb: lane l holds off[rb + 1 + l]
+    // window of 64 row ends starting at row rb: lane l holds off[rb + 1 + l].
+    // row_end = entry index at which row r ends; "never" once r has reached r1
+    // (the chunk's last, unfinished row), so the per-entry test is one compare.
+    constexpr int kNever = 0x7fffffff;
     int rb = r;
-    int ends = (rb + lane < R) ? off[rb + 1 + lane] : 0x7fffffff;
-    int row_end = bcast_i(ends, 0);
+    int ends = (rb + lane < R) ? off[rb + 1 + lane] : kNever;
+    int row_end = r < r1 ? bcast_i(ends, 0) : kNever;
 
     float acc[NT][VEC];
 #pragma unroll
@@ -130,16 +138,16 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__rest
         float *dst = out + (size_t)r * F + f0;
 #pragma unroll
         for (int t = 0; t < NT; t++) {
-            if (act[t]) { if (JG_NT) vstore_stream<VEC>(dst + t * kWave * VEC, acc[t]); else vstore<VEC>(dst + t * kWave * VEC, acc[t]); }
+            if (act[t]) vstore_stream<VEC>(dst + t * kWave * VEC, acc[t]);
 #pragma unroll
             for (int v = 0; v < VEC; v++) acc[t][v] = 0.f;
         }
         r++;
         if (r - rb == kWave) {
             rb = r;
-            ends = (rb + lane < R) ? off[rb + 1 + lane] : 0x7fffffff;
+            ends = (rb + lane < R) ? off[rb + 1 + lane] : kNever;
         }
-        row_end = bcast_i(ends, r - rb);
+        row_end = r < r1 ? bcast_i(ends, r - rb) : kNever;
     };
 
     for (int jb = j0; jb < j1; jb += kWave) {
@@ -149,39 +157,60 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__rest
         {
             const bool ok = lane < n;
             const int jj = jb + lane;
-            my_c = idx ? (ok ? (JG_NT ? load_stream(idx + jj) : idx[jj]) : 0) : jj;
-            my_w = ok ? (w ? (JG_NT ? load_stream(w + jj) : w[jj]) : 1.f) : 0.f;
+            my_c = idx ? (ok ? load_stream(idx + jj) : 0) : jj;
+            my_w = ok ? (w ? load_stream(w + jj) : 1.f) : 0.f;
             if ((unsigned)my_c >= (unsigned)C) {
                 my_c = 0;
                 my_w = 0.f;
             }
         }
+        // what each lane contributes to addressing: its row's byte offset, or its row index
+        const int my_a = WIDE ? my_c : (int)((uint32_t)my_c * row_bytes);
         for (int i0 = 0; i0 < n; i0 += UNROLL) {
+            // rotate the group's UNROLL entries into lanes 0..UNROLL-1 so that the
+            // broadcasts below take immediate lane numbers
+            const int from = (lane + i0) & (kWave - 1);
+            const int g_a = __shfl(my_a, from, kWave);
+            const float g_w = __shfl(my_w, from, kWave);
             // Issue phase: straight-line code, no branches and no lane predicates, so that the
-            // UNROLL gathers leave back to back.  Slots past n re-read row my_c = 0 of a lane
-            // that holds no entry (harmless, weight 0, never accumulated); lanes past F read
-            // the start of the row instead of being masked off.
+            // UNROLL gathers leave back to back.  Slots past n re-read the row of a lane that
+            // holds no entry (offset 0, weight 0, never accumulated); lanes past F read the
+            // start of the row instead of being masked off.
             float xv[UNROLL][NT][VEC];
 #pragma unroll
             for (int u = 0; u < UNROLL; u++) {
-                const int c = bcast_i(my_c, (i0 + u) & (kWave - 1));
-                const float *src = x + (size_t)c * F;
+                const int a = bcast_i(g_a, u);
 #pragma unroll
-                for (int t = 0; t < NT; t++) vload<VEC>(xv[u][t], src + fo[t]);
-            }
-            // Consume phase, in entry order.
-#pragma unroll
-            for (int u = 0; u < UNROLL; u++) {
-                if (i0 + u < n) {
-                    const int jj = jb + i0 + u;
-                    while (jj == row_end && r < r1) flush_row();
-                    const float wv = bcast_f(my_w, i0 + u);
-#pragma unroll
-                    for (int t = 0; t < NT; t++) {
-#pragma unroll
-                        for (int v = 0; v < VEC; v++) acc[t][v] = fmaf(wv, xv[u][t][v], acc[t][v]);
-                    }
+                for (int t = 0; t < NT; t++) {
+                    if (WIDE)
+                        vload<VEC>(xv[u][t], x + (size_t)a * F + fo[t]);
+                    else
+                        vload<VEC>(xv[u][t], reinterpret_cast<const float *>(
+                                                 xb + (size_t)((uint32_t)a + fo_bytes[t])));
                 }
+            }
+            // Consume phase, in entry order.  `left` = entries of this group before row r ends.
+            int left = row_end - (jb + i0);
+            const int m = min(UNROLL, n - i0);
+            auto consume = [&](int u) {
+                if (u == left) {
+                    do flush_row(); while (row_end == jb + i0 + u);
+                    left = row_end - (jb + i0);
+                }
+                const float wv = bcast_f(g_w, u);
+#pragma unroll
+                for (int t = 0; t < NT; t++) {
+#pragma unroll
+                    for (int v = 0; v < VEC; v++) acc[t][v] = fmaf(wv, xv[u][t][v], acc[t][v]);
+                }
+            };
+            if (m == UNROLL) {
+#pragma unroll
+                for (int u = 0; u < UNROLL; u++) consume(u);
+            } else {
+#pragma unroll
+                for (int u = 0; u < UNROLL; u++)
+                    if (u < m) consume(u);
             }
         }
     }
@@ -359,10 +388,15 @@ static void launch_spmm(const SpmmShape &s, const int32_t *off, const int32_t *i
 {
     dim3 grid((unsigned)ceil_div(s.nchunks, kSpmmWaves), (unsigned)s.slabs), block(kSpmmThreads);
     // gathers in flight per wavefront: bounded by the registers they land in
-    constexpr int U = (VEC * NT >= 16) ? 4 : (VEC * NT >= 8 ? 8 : 16);
+    constexpr int U = (VEC * NT >= 16) ? 4 : (VEC * NT >= 8 ? 8 : (VEC * NT >= 2 ? 16 : 32));
     if (k0) (void)hipEventRecord(k0, st);
-    hipLaunchKernelGGL((spmm_merge<VEC, NT, U>), grid, block, 0, st, off, idx, w, x, out, partial, chunk_row, R, C,
-                       E, F, s.chunk, s.nchunks);
+    // 32-bit byte offsets reach every row of x when C*F*4 < 2^32
+    if ((uint64_t)C * (uint64_t)F * 4u < ((uint64_t)1 << 32))
+        hipLaunchKernelGGL((spmm_merge<VEC, NT, U, false>), grid, block, 0, st, off, idx, w, x, out, partial,
+                           chunk_row, R, C, E, F, s.chunk, s.nchunks);
+    else
+        hipLaunchKernelGGL((spmm_merge<VEC, NT, U, true>), grid, block, 0, st, off, idx, w, x, out, partial,
+                           chunk_row, R, C, E, F, s.chunk, s.nchunks);
     if (k1) (void)hipEventRecord(k1, st);
     const int ngroups = (int)ceil_div(s.nchunks, kGroup);
     if (ngroups > 1)
