@@ -131,11 +131,15 @@ int32_t jgamd_spmm_csx_timed(const int32_t *off, const int32_t *idx, const float
  *   [E,1]); H > 1 treats every head as an independent softmax.
  *   fwd:  y = exp(x - max_col) / sum_col exp(x - max_col)
  *   bwd:  dx = y*g - y*sum_col(y*g)
+ * The workspace holds the list of hub columns (more than 512 entries), which
+ * get a whole thread block each.
  */
+int32_t jgamd_edge_softmax_workspace(int32_t V, int64_t E, size_t *bytes);
 int32_t jgamd_edge_softmax_fwd(const int32_t *off, const float *x, float *y, int32_t V,
-                               int64_t E, int32_t H, void *stream);
+                               int64_t E, int32_t H, void *ws, size_t ws_bytes, void *stream);
 int32_t jgamd_edge_softmax_bwd(const int32_t *off, const float *y, const float *g, float *dx,
-                               int32_t V, int64_t E, int32_t H, void *stream);
+                               int32_t V, int64_t E, int32_t H, void *ws, size_t ws_bytes,
+                               void *stream);
 
 /* ------------------------------------------------------------------------
  * Vertex -> edge copy.  Replaces ScattertoedgeOp::jit_run

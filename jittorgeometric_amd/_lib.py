@@ -20,8 +20,9 @@ SIGNATURES = {
     "jgamd_spmm_csx": [_P, _P, _P, _P, _P, _I32, _I32, _I64, _I32, _P, _c.c_size_t, _P],
     "jgamd_spmm_csx_timed": [_P, _P, _P, _P, _P, _I32, _I32, _I64, _I32, _P, _c.c_size_t, _P, _I32,
                              _c.POINTER(_c.c_float), _c.POINTER(_c.c_float)],
-    "jgamd_edge_softmax_fwd": [_P, _P, _P, _I32, _I64, _I32, _P],
-    "jgamd_edge_softmax_bwd": [_P, _P, _P, _P, _I32, _I64, _I32, _P],
+    "jgamd_edge_softmax_workspace": [_I32, _I64, _SZP],
+    "jgamd_edge_softmax_fwd": [_P, _P, _P, _I32, _I64, _I32, _P, _c.c_size_t, _P],
+    "jgamd_edge_softmax_bwd": [_P, _P, _P, _P, _I32, _I64, _I32, _P, _c.c_size_t, _P],
     "jgamd_scatter_to_edge": [_P, _P, _P, _P, _I32, _I64, _I32, _I32, _P],
     "jgamd_gat_fwd_workspace": [_I32, _I64, _I32, _I32, _SZP],
     "jgamd_gat_fwd": [_P, _P, _P, _P, _P, _F32, _P, _P, _P, _P, _P, _P, _I32, _I64, _I32, _I32, _P,

@@ -6,17 +6,42 @@
 // of two, H | G) owns one column; lane l of the group always sees head l % H,
 // so the three passes (max, sum of exp, normalise) need only xor-shuffles
 // between lanes H, 2H, ... apart.  G is picked from the mean column length so
-// that short columns do not idle a whole wavefront.
+// that short columns do not idle a whole wavefront.  Columns longer than
+// kLongColumn entries (hubs) are skipped by the group kernel, collected into a
+// list, and each handled by a whole 1024-thread block with LDS reductions.
 #include "common.h"
 
 namespace jg {
 
 constexpr int kEdgeThreads = 256;
+constexpr int kLongColumn = 512;   // entries; longer columns get a block each
+constexpr int kRegItems = 8;       // values per lane held in registers on the short-column path
 
 template <int G, typename Op> __device__ __forceinline__ float group_reduce(float v, int H, Op op)
 {
     for (int o = H; o < G; o <<= 1) v = op(v, __shfl_xor(v, o, kWave));
     return v;
+}
+
+// Walks positions first, first+G, ... below e, kRegItems at a time: the loads of a batch are
+// issued together (index clamped, not predicated), then f(position, a[p], b[p]) runs on the
+// positions inside the range.
+template <int G, typename F>
+__device__ __forceinline__ void group_walk(const float *__restrict__ a, const float *__restrict__ b, int64_t first,
+                                           int64_t e, F f)
+{
+    for (int64_t p0 = first; p0 < e; p0 += (int64_t)kRegItems * G) {
+        float va[kRegItems], vb[kRegItems];
+#pragma unroll
+        for (int i = 0; i < kRegItems; i++) {
+            const int64_t p = min(p0 + (int64_t)i * G, e - 1);
+            va[i] = a[p];
+            vb[i] = b[p];
+        }
+#pragma unroll
+        for (int i = 0; i < kRegItems; i++)
+            if (p0 + (int64_t)i * G < e) f(p0 + (int64_t)i * G, va[i], vb[i]);
+    }
 }
 
 // x -> y = exp(x - max) / sum exp(x - max) per (column, head);
@@ -29,14 +54,40 @@ __global__ __launch_bounds__(kEdgeThreads) void edge_softmax_fwd_k(const int32_t
     const int gl = threadIdx.x % G;
     const int64_t ngroups = (int64_t)gridDim.x * (kEdgeThreads / G);
     for (int64_t c = (int64_t)blockIdx.x * (kEdgeThreads / G) + threadIdx.x / G; c < V; c += ngroups) {
+        if (off[c + 1] - off[c] > kLongColumn) continue;   // left to the block-per-column kernel
         const int64_t s = (int64_t)off[c] * H, e = (int64_t)off[c + 1] * H;
+        if (e <= s) continue;
+        if (e - s <= (int64_t)kRegItems * G) {
+            // the whole column fits in kRegItems values per lane: one trip to memory, all loads
+            // issued together (index clamped, not predicated), the three passes run on registers
+            float v[kRegItems];
+#pragma unroll
+            for (int i = 0; i < kRegItems; i++) v[i] = x[min(s + gl + (int64_t)i * G, e - 1)];
+            float m = -INFINITY;
+#pragma unroll
+            for (int i = 0; i < kRegItems; i++)
+                if (s + gl + (int64_t)i * G < e) m = fmaxf(m, v[i]);
+            m = group_reduce<G>(m, H, [](float a, float b) { return fmaxf(a, b); });
+            float t = 0.f;
+#pragma unroll
+            for (int i = 0; i < kRegItems; i++) {
+                v[i] = expf(v[i] - m);
+                if (s + gl + (int64_t)i * G < e) t += v[i];
+            }
+            t = group_reduce<G>(t, H, [](float a, float b) { return a + b; });
+#pragma unroll
+            for (int i = 0; i < kRegItems; i++)
+                if (s + gl + (int64_t)i * G < e) y[s + gl + (int64_t)i * G] = v[i] / t;
+            continue;
+        }
+        // longer columns: the same three passes, kRegItems loads in flight per lane
         float m = -INFINITY;
-        for (int64_t p = s + gl; p < e; p += G) m = fmaxf(m, x[p]);
+        group_walk<G>(x, x, s + gl, e, [&](int64_t, float v, float) { m = fmaxf(m, v); });
         m = group_reduce<G>(m, H, [](float a, float b) { return fmaxf(a, b); });
         float t = 0.f;
-        for (int64_t p = s + gl; p < e; p += G) t += expf(x[p] - m);
+        group_walk<G>(x, x, s + gl, e, [&](int64_t, float v, float) { t += expf(v - m); });
         t = group_reduce<G>(t, H, [](float a, float b) { return a + b; });
-        for (int64_t p = s + gl; p < e; p += G) y[p] = expf(x[p] - m) / t;
+        group_walk<G>(x, x, s + gl, e, [&](int64_t p, float v, float) { y[p] = expf(v - m) / t; });
     }
 }
 
@@ -50,12 +101,133 @@ __global__ __launch_bounds__(kEdgeThreads) void edge_softmax_bwd_k(const int32_t
     const int gl = threadIdx.x % G;
     const int64_t ngroups = (int64_t)gridDim.x * (kEdgeThreads / G);
     for (int64_t c = (int64_t)blockIdx.x * (kEdgeThreads / G) + threadIdx.x / G; c < V; c += ngroups) {
+        if (off[c + 1] - off[c] > kLongColumn) continue;
         const int64_t s = (int64_t)off[c] * H, e = (int64_t)off[c + 1] * H;
+        if (e <= s) continue;
+        if (e - s <= (int64_t)kRegItems * G) {
+            float yv[kRegItems], gv[kRegItems];
+#pragma unroll
+            for (int i = 0; i < kRegItems; i++) {
+                const int64_t p = min(s + gl + (int64_t)i * G, e - 1);
+                yv[i] = y[p];
+                gv[i] = g[p];
+            }
+            float dot = 0.f;
+#pragma unroll
+            for (int i = 0; i < kRegItems; i++)
+                if (s + gl + (int64_t)i * G < e) dot += yv[i] * gv[i];
+            dot = group_reduce<G>(dot, H, [](float a, float b) { return a + b; });
+#pragma unroll
+            for (int i = 0; i < kRegItems; i++)
+                if (s + gl + (int64_t)i * G < e) dx[s + gl + (int64_t)i * G] = yv[i] * gv[i] - yv[i] * dot;
+            continue;
+        }
         float dot = 0.f;
-        for (int64_t p = s + gl; p < e; p += G) dot += y[p] * g[p];
+        group_walk<G>(y, g, s + gl, e, [&](int64_t, float yv, float gv) { dot += yv * gv; });
         dot = group_reduce<G>(dot, H, [](float a, float b) { return a + b; });
-        for (int64_t p = s + gl; p < e; p += G) dx[p] = y[p] * g[p] - y[p] * dot;
+        group_walk<G>(y, g, s + gl, e, [&](int64_t p, float yv, float gv) { dx[p] = yv * gv - yv * dot; });
     }
+}
+
+// ---- hub columns ------------------------------------------------------------
+__global__ void edge_zero_counter(int32_t *counter) { *counter = 0; }
+
+// list[0..*counter) = columns with more than kLongColumn entries (any order:
+// each is processed independently).
+__global__ void edge_list_long(const int32_t *__restrict__ off, int V, int32_t *__restrict__ counter,
+                               int32_t *__restrict__ list, int capacity)
+{
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= V) return;
+    if (off[c + 1] - off[c] > kLongColumn) {
+        const int slot = atomicAdd(counter, 1);
+        if (slot < capacity) list[slot] = c;
+    }
+}
+
+// Per-head reduction over the block: thread t holds head t % H (kLongThreads % H == 0),
+// so folding halves of at least H keeps heads apart.  Result for head h in red[h].
+constexpr int kLongThreads = 1024;
+constexpr int kLongBatch = 8;      // values per thread fetched together
+
+template <typename Op> __device__ __forceinline__ float block_head_reduce(float v, int H, float *red, Op op)
+{
+    __syncthreads();
+    red[threadIdx.x] = v;
+    __syncthreads();
+    for (int o = kLongThreads / 2; o >= H; o >>= 1) {
+        if ((int)threadIdx.x < o) red[threadIdx.x] = op(red[threadIdx.x], red[threadIdx.x + o]);
+        __syncthreads();
+    }
+    return red[threadIdx.x % H];
+}
+
+// Walks this thread's values of [s,e) (stride kLongThreads) kLongBatch at a time: the loads of a
+// batch are issued together (index clamped, not predicated), then `f(position, value...)` runs on
+// the ones inside the range.
+template <typename F> __device__ __forceinline__ void long_walk1(const float *__restrict__ a, int64_t s, int64_t e, F f)
+{
+    for (int64_t p0 = s + threadIdx.x; p0 < e; p0 += (int64_t)kLongBatch * kLongThreads) {
+        float v[kLongBatch];
+#pragma unroll
+        for (int i = 0; i < kLongBatch; i++) v[i] = a[min(p0 + (int64_t)i * kLongThreads, e - 1)];
+#pragma unroll
+        for (int i = 0; i < kLongBatch; i++)
+            if (p0 + (int64_t)i * kLongThreads < e) f(p0 + (int64_t)i * kLongThreads, v[i]);
+    }
+}
+template <typename F>
+__device__ __forceinline__ void long_walk2(const float *__restrict__ a, const float *__restrict__ b, int64_t s,
+                                           int64_t e, F f)
+{
+    for (int64_t p0 = s + threadIdx.x; p0 < e; p0 += (int64_t)kLongBatch * kLongThreads) {
+        float va[kLongBatch], vb[kLongBatch];
+#pragma unroll
+        for (int i = 0; i < kLongBatch; i++) {
+            const int64_t p = min(p0 + (int64_t)i * kLongThreads, e - 1);
+            va[i] = a[p];
+            vb[i] = b[p];
+        }
+#pragma unroll
+        for (int i = 0; i < kLongBatch; i++)
+            if (p0 + (int64_t)i * kLongThreads < e) f(p0 + (int64_t)i * kLongThreads, va[i], vb[i]);
+    }
+}
+
+__global__ __launch_bounds__(kLongThreads) void edge_softmax_fwd_long(const int32_t *__restrict__ off,
+                                                                      const float *__restrict__ x,
+                                                                      float *__restrict__ y, int H,
+                                                                      const int32_t *__restrict__ counter,
+                                                                      const int32_t *__restrict__ list)
+{
+    __shared__ float red[kLongThreads];
+    if ((int)blockIdx.x >= *counter) return;
+    const int c = list[blockIdx.x];
+    const int64_t s = (int64_t)off[c] * H, e = (int64_t)off[c + 1] * H;
+    float m = -INFINITY;
+    long_walk1(x, s, e, [&](int64_t, float v) { m = fmaxf(m, v); });
+    m = block_head_reduce(m, H, red, [](float a, float b) { return fmaxf(a, b); });
+    float t = 0.f;
+    long_walk1(x, s, e, [&](int64_t, float v) { t += expf(v - m); });
+    t = block_head_reduce(t, H, red, [](float a, float b) { return a + b; });
+    long_walk1(x, s, e, [&](int64_t p, float v) { y[p] = expf(v - m) / t; });
+}
+
+__global__ __launch_bounds__(kLongThreads) void edge_softmax_bwd_long(const int32_t *__restrict__ off,
+                                                                      const float *__restrict__ y,
+                                                                      const float *__restrict__ g,
+                                                                      float *__restrict__ dx, int H,
+                                                                      const int32_t *__restrict__ counter,
+                                                                      const int32_t *__restrict__ list)
+{
+    __shared__ float red[kLongThreads];
+    if ((int)blockIdx.x >= *counter) return;
+    const int c = list[blockIdx.x];
+    const int64_t s = (int64_t)off[c] * H, e = (int64_t)off[c + 1] * H;
+    float dot = 0.f;
+    long_walk2(y, g, s, e, [&](int64_t, float yv, float gv) { dot += yv * gv; });
+    dot = block_head_reduce(dot, H, red, [](float a, float b) { return a + b; });
+    long_walk2(y, g, s, e, [&](int64_t p, float yv, float gv) { dx[p] = yv * gv - yv * dot; });
 }
 
 // Any H (not a power of two, or above 64): one thread per (column, head).
@@ -162,8 +334,46 @@ template <typename K, typename... A> static void launch_groups(K k, int G, int V
     hipLaunchKernelGGL(k, dim3((unsigned)blocks), dim3(kEdgeThreads), 0, s, a...);
 }
 
+// Scratch of the hub-column path: a counter and the list of long columns
+// (at most E / kLongColumn of them).
+static int long_capacity(int32_t V, int64_t E)
+{
+    const int64_t c = E / kLongColumn + 1;
+    return (int)(c < (int64_t)V ? c : (int64_t)V);
+}
+static size_t softmax_ws_bytes(int32_t V, int64_t E) { return 256 + carve_bytes((size_t)long_capacity(V, E), 4); }
+
+static int32_t check_softmax_ws(const char *who, const void *ws, size_t have, int32_t V, int64_t E)
+{
+    const size_t need = softmax_ws_bytes(V, E);
+    if (!ws || have < need) return fail(JGAMD_ERR_WORKSPACE, "%s: workspace %zu < %zu bytes", who, ws ? have : (size_t)0, need);
+    if (((uintptr_t)ws & 255) != 0) return fail(JGAMD_ERR_ALIGN, "%s: workspace not 256-byte aligned", who);
+    return 0;
+}
+
+JG_EXPORT int32_t jgamd_edge_softmax_workspace(int32_t V, int64_t E, size_t *bytes)
+{
+    if (!bytes) return fail(JGAMD_ERR_NULL, "edge_softmax_workspace: bytes is NULL");
+    if (V < 0 || E < 0) return fail(JGAMD_ERR_SIZE, "edge_softmax_workspace: negative size");
+    *bytes = (V == 0 || E == 0) ? 0 : softmax_ws_bytes(V, E);
+    return 0;
+}
+
+// Fills list/counter with the hub columns; returns the launch bound for the block-per-column kernel.
+static int list_long_columns(const int32_t *off, int32_t V, int64_t E, void *ws, int32_t **counter, int32_t **list,
+                             hipStream_t s)
+{
+    Carver carve(ws);
+    *counter = carve.take<int32_t>(1);
+    const int cap = long_capacity(V, E);
+    *list = carve.take<int32_t>((size_t)cap);
+    hipLaunchKernelGGL(edge_zero_counter, dim3(1), dim3(1), 0, s, *counter);
+    hipLaunchKernelGGL(edge_list_long, dim3((unsigned)ceil_div(V, 256)), dim3(256), 0, s, off, V, *counter, *list, cap);
+    return cap;
+}
+
 JG_EXPORT int32_t jgamd_edge_softmax_fwd(const int32_t *off, const float *x, float *y, int32_t V, int64_t E,
-                                         int32_t H, void *stream)
+                                         int32_t H, void *ws, size_t ws_bytes, void *stream)
 {
     if (int32_t rc = check_softmax("edge_softmax_fwd", off, x, y, V, E, H)) return rc;
     if (V == 0 || E == 0) return 0;
@@ -173,6 +383,7 @@ JG_EXPORT int32_t jgamd_edge_softmax_fwd(const int32_t *off, const float *x, flo
                            y, V, H);
         return launch_status("edge_softmax_fwd");
     }
+    if (int32_t rc = check_softmax_ws("edge_softmax_fwd", ws, ws_bytes, V, E)) return rc;
     switch (pick_group(E, V, H)) {
     case 1: case 2: case 4: launch_groups(edge_softmax_fwd_k<4>, 4, V, s, off, x, y, V, H); break;
     case 8: launch_groups(edge_softmax_fwd_k<8>, 8, V, s, off, x, y, V, H); break;
@@ -180,11 +391,14 @@ JG_EXPORT int32_t jgamd_edge_softmax_fwd(const int32_t *off, const float *x, flo
     case 32: launch_groups(edge_softmax_fwd_k<32>, 32, V, s, off, x, y, V, H); break;
     default: launch_groups(edge_softmax_fwd_k<64>, 64, V, s, off, x, y, V, H); break;
     }
+    int32_t *counter, *list;
+    const int cap = list_long_columns(off, V, E, ws, &counter, &list, s);
+    hipLaunchKernelGGL(edge_softmax_fwd_long, dim3((unsigned)cap), dim3(kLongThreads), 0, s, off, x, y, H, counter, list);
     return launch_status("edge_softmax_fwd");
 }
 
 JG_EXPORT int32_t jgamd_edge_softmax_bwd(const int32_t *off, const float *y, const float *g, float *dx, int32_t V,
-                                         int64_t E, int32_t H, void *stream)
+                                         int64_t E, int32_t H, void *ws, size_t ws_bytes, void *stream)
 {
     if (int32_t rc = check_softmax("edge_softmax_bwd", off, y, dx, V, E, H)) return rc;
     if (E > 0 && !g) return fail(JGAMD_ERR_NULL, "edge_softmax_bwd: g is NULL");
@@ -195,6 +409,7 @@ JG_EXPORT int32_t jgamd_edge_softmax_bwd(const int32_t *off, const float *y, con
                            g, dx, V, H);
         return launch_status("edge_softmax_bwd");
     }
+    if (int32_t rc = check_softmax_ws("edge_softmax_bwd", ws, ws_bytes, V, E)) return rc;
     switch (pick_group(E, V, H)) {
     case 1: case 2: case 4: launch_groups(edge_softmax_bwd_k<4>, 4, V, s, off, y, g, dx, V, H); break;
     case 8: launch_groups(edge_softmax_bwd_k<8>, 8, V, s, off, y, g, dx, V, H); break;
@@ -202,6 +417,10 @@ JG_EXPORT int32_t jgamd_edge_softmax_bwd(const int32_t *off, const float *y, con
     case 32: launch_groups(edge_softmax_bwd_k<32>, 32, V, s, off, y, g, dx, V, H); break;
     default: launch_groups(edge_softmax_bwd_k<64>, 64, V, s, off, y, g, dx, V, H); break;
     }
+    int32_t *counter, *list;
+    const int cap = list_long_columns(off, V, E, ws, &counter, &list, s);
+    hipLaunchKernelGGL(edge_softmax_bwd_long, dim3((unsigned)cap), dim3(kLongThreads), 0, s, off, y, g, dx, H, counter,
+                       list);
     return launch_status("edge_softmax_bwd");
 }
 

@@ -22,7 +22,9 @@ class EdgeSoftmaxFunc(torch.autograd.Function):
         off = csc.column_offset
         V, E, H = off.shape[0] - 1, x.shape[0], _heads(x)
         y = torch.empty_like(x)
-        _lib.check(lib.jgamd_edge_softmax_fwd(_lib.ptr(off), _lib.ptr(x), _lib.ptr(y), V, E, H,
+        nbytes = _lib.query(lib.jgamd_edge_softmax_workspace, V, E)
+        ws = _lib.workspace(nbytes, dev)
+        _lib.check(lib.jgamd_edge_softmax_fwd(_lib.ptr(off), _lib.ptr(x), _lib.ptr(y), V, E, H, _lib.ptr(ws), nbytes,
                                               _lib.stream_ptr(dev)))
         ctx.save_for_backward(y)
         ctx.csc = csc
@@ -37,8 +39,10 @@ class EdgeSoftmaxFunc(torch.autograd.Function):
         dev = _lib.require_gpu(g, y)
         V, E, H = off.shape[0] - 1, y.shape[0], _heads(y)
         dx = torch.empty_like(y)
+        nbytes = _lib.query(lib.jgamd_edge_softmax_workspace, V, E)
+        ws = _lib.workspace(nbytes, dev)
         _lib.check(lib.jgamd_edge_softmax_bwd(_lib.ptr(off), _lib.ptr(y), _lib.ptr(g), _lib.ptr(dx), V, E, H,
-                                              _lib.stream_ptr(dev)))
+                                              _lib.ptr(ws), nbytes, _lib.stream_ptr(dev)))
         return dx, None
 
 

@@ -68,9 +68,11 @@ def test_argument_errors_are_reported_not_launched(lib):
     assert lib.jgamd_spmm_csx(bad, bad, bad, ctypes.c_void_p(258), bad, 4, 4, 5, 8, bad, 1 << 30, None) == -5
     assert lib.jgamd_spmm_csx(bad, bad, bad, bad, bad, 4, 4, 5, 8, bad, 8, None) == -3
     assert lib.jgamd_spmm_csx(bad, bad, bad, bad, bad, 0, 4, 0, 8, None, 0, None) == 0                # nothing to do
-    assert lib.jgamd_edge_softmax_fwd(bad, bad, bad, 4, 5, 0, None) == -2
-    assert lib.jgamd_edge_softmax_fwd(None, bad, bad, 4, 5, 1, None) == -1
-    assert lib.jgamd_edge_softmax_bwd(bad, bad, None, bad, 4, 5, 1, None) == -1
+    assert lib.jgamd_edge_softmax_fwd(bad, bad, bad, 4, 5, 0, bad, 1 << 20, None) == -2
+    assert lib.jgamd_edge_softmax_fwd(None, bad, bad, 4, 5, 1, bad, 1 << 20, None) == -1
+    assert lib.jgamd_edge_softmax_fwd(bad, bad, bad, 4, 5, 1, None, 0, None) == -3
+    assert lib.jgamd_edge_softmax_bwd(bad, bad, None, bad, 4, 5, 1, bad, 1 << 20, None) == -1
+    assert lib.jgamd_edge_softmax_workspace(4, 5, ctypes.byref(n)) == 0 and n.value >= 260
     assert lib.jgamd_scatter_to_edge(bad, bad, bad, bad, 4, 5, 8, 3, None) == -2
     assert lib.jgamd_gat_fwd_workspace(10, 10, 4, 1024, ctypes.byref(n)) == -4
     assert lib.jgamd_gat_bwd_workspace(10, 10, 3, 7, ctypes.byref(n)) == -4
