@@ -63,7 +63,8 @@ const char *jgamd_last_error(void);
  * inside a row the edges keep their input order; weights are copied.
  * Edges whose key is outside [0,V) are dropped (the reference would write out
  * of bounds); the tail of out_idx/out_w is then left untouched.
- * Limits: 0 <= E < 2^31 - 2^20, 0 <= V < 2^31 - 1.
+ * Limits: 0 <= E < 2^31 - 2^20, 0 <= V < 2^31 - 1 (V <= 2^22 takes the
+ * two-level path, larger V plain radix passes over the same records).
  */
 int32_t jgamd_coo_to_csx_workspace(int64_t E, int32_t V, int32_t with_perm, size_t *bytes);
 int32_t jgamd_coo_to_csx(const int32_t *edge_index, const float *edge_weight, int64_t E,

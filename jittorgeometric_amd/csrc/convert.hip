@@ -24,7 +24,10 @@
 //                         bucket's output window is a few hundred KB, so the
 //                         scattered 4-byte stores combine in L2.
 //
-// Two levels of at most 2048 bins each cover V <= 2^22 vertices.
+// Two levels of at most 2048 bins each cover V <= 2^22 vertices.  Above that
+// the records are sorted by plain LSD passes of the same stable partition
+// (11-bit digits, least significant first), the offsets are read off the
+// sorted keys, and the records are unpacked.
 #include "common.h"
 
 namespace jg {
@@ -159,6 +162,63 @@ template <typename Rec> struct CooLoader {
         return e < n && (uint32_t)r.key < (uint32_t)V;
     }
 };
+// Loader for the later LSD passes: items are records; only the first *count
+// slots hold records (edges with out-of-range keys were dropped by pass 0).
+template <typename Rec> struct RecLoader {
+    const Rec *recs;
+    const int32_t *count;
+    int64_t cap;      // upper bound of *count (> 0)
+    __device__ __forceinline__ void load(int64_t e, Rec &r) const { r = recs[e < cap ? e : cap - 1]; }
+    __device__ __forceinline__ bool valid(int64_t e, const Rec &) const { return e < (int64_t)*count; }
+};
+
+// Per-block counts of one digit ((key >> shift) & mask) for any loader.
+template <typename Rec, typename Loader>
+__global__ __launch_bounds__(kPartThreads) void csx_digit_histogram(Loader in, int shift, int mask, int nbins,
+                                                                    int32_t *__restrict__ table, int nblocks)
+{
+    __shared__ int bins[kMaxBins];
+    for (int b = threadIdx.x; b < nbins; b += kPartThreads) bins[b] = 0;
+    __syncthreads();
+    const int64_t base = (int64_t)blockIdx.x * kTile;
+    Rec rec[kItems];
+#pragma unroll
+    for (int i = 0; i < kItems; i++) in.load(base + (int64_t)i * kPartThreads + threadIdx.x, rec[i]);
+#pragma unroll
+    for (int i = 0; i < kItems; i++)
+        if (in.valid(base + (int64_t)i * kPartThreads + threadIdx.x, rec[i]))
+            atomicAdd(&bins[(rec[i].key >> shift) & mask], 1);
+    __syncthreads();
+    for (int b = threadIdx.x; b < nbins; b += kPartThreads) table[(int64_t)b * nblocks + blockIdx.x] = bins[b];
+    if (blockIdx.x == 0 && threadIdx.x == 0) table[(int64_t)nbins * nblocks] = 0;
+}
+
+__global__ void csx_save_count(const int32_t *__restrict__ table_end, int32_t *__restrict__ count)
+{
+    *count = *table_end;
+}
+
+// Records sorted by key -> offsets (off[k] = first position whose key is >= k)
+// and the unpacked output arrays.  One thread per position 0..cap (inclusive).
+template <typename Rec, bool PERM>
+__global__ void csx_unpack_sorted(const Rec *__restrict__ recs, const int32_t *__restrict__ count, int64_t cap,
+                                  int32_t V, int32_t *__restrict__ off, int32_t *__restrict__ out_idx,
+                                  uint32_t *__restrict__ out_w, int32_t *__restrict__ out_perm)
+{
+    const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t n = *count;
+    if (p > n || p > cap) return;
+    const int64_t prev = p > 0 ? recs[p - 1].key : -1;
+    const int64_t cur = p < n ? recs[p].key : (int64_t)V;
+    for (int64_t k = prev + 1; k <= cur; k++) off[k] = (int32_t)p;
+    if (p < n) {
+        const Rec r = recs[p];
+        out_idx[p] = r.other;
+        if (out_w) out_w[p] = r.w;
+        if (PERM) out_perm[p] = get_id(r);
+    }
+}
+
 template <typename Rec, typename Loader>
 __global__ __launch_bounds__(kPartThreads) void csx_partition(Loader in, int shift, int mask, int nbins,
                                                               int nbits, const int32_t *__restrict__ table,
@@ -384,6 +444,7 @@ struct ConvPlan {
     int nbuckets;     // bins of the partition
     int64_t nblocks;  // tiles of kTile edges
     int max_sub;      // upper bound on the number of sub-blocks
+    int digits;       // > 0: V above 2^22, plain LSD passes of 11 bits each
 };
 
 static ConvPlan make_plan(int64_t E, int32_t V)
@@ -392,6 +453,13 @@ static ConvPlan make_plan(int64_t E, int32_t V)
     int bits = 0;
     while (bits < 31 && ((int64_t)1 << bits) < (int64_t)V) bits++;   // keys < 2^bits
     p.nblocks = ceil_div(E > 0 ? E : 1, kTile);
+    if (bits > 2 * kMaxBinBits) {
+        p.digits = (bits + kMaxBinBits - 1) / kMaxBinBits;
+        p.shift = 0;
+        p.nbuckets = kMaxBins;
+        p.max_sub = 1;
+        return p;
+    }
     p.shift = bits > 10 ? bits - 10 : 0;
     if (p.shift > kMaxBinBits) p.shift = kMaxBinBits;
     p.nbuckets = (int)ceil_div(V > 0 ? V : 1, (int64_t)1 << p.shift);
@@ -406,7 +474,7 @@ static size_t conv_ws_bytes(int64_t E, int32_t V, bool perm)
     size_t b = 0;
     b += carve_bytes(table_n, 4);
     b += carve_bytes(scan_ws_ints((int64_t)table_n), 4);
-    b += carve_bytes((size_t)E, perm ? sizeof(Rec4) : sizeof(Rec3));
+    b += carve_bytes((size_t)E, perm ? sizeof(Rec4) : sizeof(Rec3)) * (p.digits > 0 ? 2 : 1);
     b += carve_bytes((size_t)p.max_sub, 4);
     b += carve_bytes((size_t)p.nbuckets + 1, 4);
     b += carve_bytes((size_t)p.max_sub << p.shift, 4);
@@ -443,6 +511,41 @@ static int32_t convert(const int32_t *keys, const int32_t *others, const float *
         hipLaunchKernelGGL(fill_i32, dim3((unsigned)ceil_div((int64_t)V + 1, 256)), dim3(256), 0, s, out_off,
                            (int64_t)V + 1, 0);
         return launch_status("coo_to_csx(fill)");
+    }
+
+    if (p.digits > 0) {
+        // V > 2^22: LSD passes over 11-bit digits; sub_first doubles as the record count
+        Rec *bufs[2] = {recs, carve.take<Rec>((size_t)E)};
+        int32_t *count = sub_first;
+        const size_t lds = (size_t)kPartWaves * kMaxBins * sizeof(int);
+        for (int d = 0; d < p.digits; d++) {
+            const int shift = d * kMaxBinBits;
+            Rec *dst = bufs[d & 1];
+            if (d == 0) {
+                CooLoader<Rec> in{keys, others, reinterpret_cast<const uint32_t *>(w), E, V};
+                hipLaunchKernelGGL((csx_digit_histogram<Rec, CooLoader<Rec>>), dim3(nb), dim3(kPartThreads), 0, s, in,
+                                   shift, kMaxBins - 1, kMaxBins, table, nblk);
+                if ((rc = exclusive_scan_i32(table, table, (int64_t)table_n, sums, s))) return rc;
+                hipLaunchKernelGGL(csx_save_count, dim3(1), dim3(1), 0, s, table + (table_n - 1), count);
+                auto part = csx_partition<Rec, CooLoader<Rec>>;
+                allow_lds(part, lds);
+                hipLaunchKernelGGL(part, dim3(nb), dim3(kPartThreads), lds, s, in, shift, kMaxBins - 1, kMaxBins,
+                                   kMaxBinBits, table, nblk, dst);
+            } else {
+                RecLoader<Rec> in{bufs[(d - 1) & 1], count, E};
+                hipLaunchKernelGGL((csx_digit_histogram<Rec, RecLoader<Rec>>), dim3(nb), dim3(kPartThreads), 0, s, in,
+                                   shift, kMaxBins - 1, kMaxBins, table, nblk);
+                if ((rc = exclusive_scan_i32(table, table, (int64_t)table_n, sums, s))) return rc;
+                auto part = csx_partition<Rec, RecLoader<Rec>>;
+                allow_lds(part, lds);
+                hipLaunchKernelGGL(part, dim3(nb), dim3(kPartThreads), lds, s, in, shift, kMaxBins - 1, kMaxBins,
+                                   kMaxBinBits, table, nblk, dst);
+            }
+        }
+        hipLaunchKernelGGL((csx_unpack_sorted<Rec, PERM>), dim3((unsigned)ceil_div(E + 1, 256)), dim3(256), 0, s,
+                           bufs[(p.digits - 1) & 1], count, E, V, out_off, out_idx,
+                           reinterpret_cast<uint32_t *>(out_w), out_perm);
+        return launch_status("coo_to_csx(lsd)");
     }
 
     int bbits = 0;
@@ -482,8 +585,7 @@ static int32_t check_conv_sizes(const char *who, int64_t E, int32_t V)
     if (E < 0 || V < 0) return fail(JGAMD_ERR_SIZE, "%s: negative size (E=%lld, V=%d)", who, (long long)E, V);
     if (E >= ((int64_t)1 << 31) - ((int64_t)1 << 20))
         return fail(JGAMD_ERR_SIZE, "%s: E=%lld does not fit int32 offsets", who, (long long)E);
-    if ((int64_t)V > ((int64_t)1 << (2 * kMaxBinBits)))
-        return fail(JGAMD_ERR_UNSUPPORTED, "%s: V=%d above 2^22 is not supported", who, V);
+    if (V == INT32_MAX) return fail(JGAMD_ERR_SIZE, "%s: V too large", who);
     return 0;
 }
 

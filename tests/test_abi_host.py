@@ -55,7 +55,8 @@ def test_argument_errors_are_reported_not_launched(lib):
     bad = ctypes.c_void_p(256)          # never dereferenced: every call below fails validation first
     assert lib.jgamd_coo_to_csx_workspace(-1, 4, 0, ctypes.byref(n)) == -2
     assert lib.jgamd_coo_to_csx_workspace(1 << 31, 4, 0, ctypes.byref(n)) == -2
-    assert lib.jgamd_coo_to_csx_workspace(10, (1 << 22) + 1, 0, ctypes.byref(n)) == -4
+    assert lib.jgamd_coo_to_csx_workspace(10, (1 << 22) + 1, 0, ctypes.byref(n)) == 0      # LSD path
+    assert lib.jgamd_coo_to_csx_workspace(10, 2**31 - 1, 0, ctypes.byref(n)) == -2
     assert lib.jgamd_coo_to_csx_workspace(10, 4, 0, None) == -1
     assert lib.jgamd_coo_to_csx(bad, bad, 5, 4, 2, bad, bad, bad, None, bad, 1 << 30, None) == -2      # key_row
     assert lib.jgamd_coo_to_csx(bad, bad, 5, 4, 0, bad, bad, bad, None, None, 0, None) == -3          # no workspace

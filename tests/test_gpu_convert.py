@@ -55,6 +55,7 @@ def test_reference_fixtures(name):
     (1024, 20000, 3, 5), (1025, 20000, 3, 6), (2708, 13264, 0, 7), (5000, 8191, 2, 8),
     (5000, 8192, 2, 9), (5000, 8193, 2, 10), (70001, 300000, 5, 11), (300000, 1000000, 4, 12),
     (4194304, 600000, 3, 13), (2100000, 2500000, 2, 14),
+    (4194305, 700000, 3, 15), (9000000, 3000000, 2, 16), (70000000, 100000, 1, 17),
 ])
 def test_random_graphs_bit_exact(V, E, hubs, seed):
     rng = np.random.default_rng(seed)
