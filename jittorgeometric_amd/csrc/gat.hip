@@ -52,6 +52,12 @@ template <int VEC> __device__ __forceinline__ void gstore(float *p, const float 
 
 __device__ __forceinline__ float lrelu(float z, float slope) { return z > 0.f ? z : slope * z; }
 
+// exp for arguments <= 0 in the per-edge loops: the hardware exp2 on x*log2(e), relative error
+// about |x| * 2^-23.  A term with large |x| is a correspondingly tiny share of its softmax sum
+// (|x| = 16 -> 1e-7 of the largest term), so the weights stay well inside 1e-6 relative; the
+// library expf costs ~20 VALU instructions per call and made these kernels VALU-bound.
+__device__ __forceinline__ float fast_exp(float x) { return __expf(x); }
+
 // chunk_row[k] = the row owning merged position k*chunk (row r owns positions
 // off[r]+r .. off[r+1]+r, an increasing function of r): binary search per chunk.
 __global__ void gat_chunk_rows(const int32_t *__restrict__ off, int R, int chunk, int nchunks,
@@ -121,6 +127,25 @@ __global__ __launch_bounds__(256) void gat_node_scores_vec(const float4 *__restr
     }
 }
 
+// Sum of v over aligned groups of `lanes` consecutive lanes (a power of two), left in every
+// lane of the group.  Up to 16 lanes the exchanges are DPP modifiers on the adds (quad
+// permutes, then the half-row and row mirrors); only 32 and 64 go through the LDS crossbar.
+template <int CTRL> __device__ __forceinline__ float dpp_add(float v)
+{
+    const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false);
+    return v + __int_as_float(moved);
+}
+__device__ __forceinline__ float lane_group_sum(float v, int lanes)
+{
+    if (lanes >= 2) v = dpp_add<0xB1>(v);    // quad_perm [1,0,3,2]
+    if (lanes >= 4) v = dpp_add<0x4E>(v);    // quad_perm [2,3,0,1]
+    if (lanes >= 8) v = dpp_add<0x141>(v);   // row_half_mirror
+    if (lanes >= 16) v = dpp_add<0x140>(v);  // row_mirror
+    if (lanes >= 32) v += __shfl_xor(v, 16, kWave);
+    if (lanes >= 64) v += __shfl_xor(v, 32, kWave);
+    return v;
+}
+
 // ----------------------------------------------------------------- forward ---
 template <int VEC, int NT>
 __global__ __launch_bounds__(kGatThreads) void gat_fwd_merge(
@@ -159,7 +184,14 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_merge(
     int ends = (rb + lane < R) ? off[rb + 1 + lane] : 0x7fffffff;
     int row_end = bcast_i(ends, 0);
 
-    float m[NT], l[NT], acc[NT][VEC], er_r[NT];
+    // er of the current row and, already on its way, of the next one: a row end must not
+    // wait for a fresh load (rows are a handful of entries long)
+    float m[NT], l[NT], acc[NT][VEC], er_r[NT], er_next[NT];
+    auto fetch_next = [&]() {
+        const size_t rn = (size_t)min(r + 1, R - 1);
+#pragma unroll
+        for (int t = 0; t < NT; t++) er_next[t] = er[rn * H + head[t]];
+    };
     auto reset = [&]() {
 #pragma unroll
         for (int t = 0; t < NT; t++) {
@@ -167,9 +199,15 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_merge(
             l[t] = 0.f;
 #pragma unroll
             for (int v = 0; v < VEC; v++) acc[t][v] = 0.f;
-            er_r[t] = (act[t] && r < R) ? er[(size_t)r * H + head[t]] : 0.f;
+            er_r[t] = er_next[t];
         }
+        fetch_next();
     };
+    {
+        const size_t rc = (size_t)min(r, R - 1);
+#pragma unroll
+        for (int t = 0; t < NT; t++) er_next[t] = er[rc * H + head[t]];
+    }
     reset();
 
     auto flush_row = [&]() {
@@ -232,8 +270,8 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_merge(
                             if (act[t]) {
                                 const float s = lrelu(sv[u][t] + er_r[t], slope);
                                 const float mn = fmaxf(m[t], s);
-                                const float sc = expf(m[t] - mn);     // 0 on the first entry (m = -inf)
-                                const float p = expf(s - mn);
+                                const float sc = fast_exp(m[t] - mn);   // 0 on the first entry (m = -inf)
+                                const float p = fast_exp(s - mn);
                                 l[t] = fmaf(l[t], sc, p);
 #pragma unroll
                                 for (int v = 0; v < VEC; v++) acc[t][v] = fmaf(acc[t][v], sc, p * xv[u][t][v]);
@@ -512,23 +550,31 @@ __global__ __launch_bounds__(kGatThreads) void gat_bwd_merge(
     int ends = (rb + lane < R) ? t_off[rb + 1 + lane] : 0x7fffffff;
     int row_end = bcast_i(ends, 0);
 
-    float acc[NT][VEC], gel[NT], hr[NT][VEC], el_r[NT];
+    // h row and el of the current source row and, already on their way, of the next one: a
+    // row end must not wait for fresh loads (lanes past F read offset 0 and are ignored)
+    float acc[NT][VEC], gel[NT], hr[NT][VEC], el_r[NT], hr_next[NT][VEC], el_next[NT];
+    auto fetch_row = [&](int row) {
+        const size_t rc = (size_t)min(row, R - 1);
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            gload<VEC>(hr_next[t], h + rc * F + fo[t]);
+            el_next[t] = el[rc * H + head[t]];
+        }
+    };
     auto reset = [&]() {
 #pragma unroll
         for (int t = 0; t < NT; t++) {
             gel[t] = 0.f;
+            el_r[t] = el_next[t];
 #pragma unroll
             for (int v = 0; v < VEC; v++) {
                 acc[t][v] = 0.f;
-                hr[t][v] = 0.f;
-            }
-            el_r[t] = 0.f;
-            if (act[t] && r < R) {
-                gload<VEC>(hr[t], h + (size_t)r * F + f0 + t * kWave * VEC);
-                el_r[t] = el[(size_t)r * H + head[t]];
+                hr[t][v] = hr_next[t][v];
             }
         }
+        fetch_row(r + 1);
     };
+    fetch_row(r);
     reset();
     auto store_piece = [&](float *vec, float *elp) {
 #pragma unroll
@@ -592,24 +638,23 @@ __global__ __launch_bounds__(kGatThreads) void gat_bwd_merge(
                             float s = 0.f;
 #pragma unroll
                             for (int t = 0; t < NT; t++) s += dot[t];
-                            for (int o = 1; o < kWave; o <<= 1) s += __shfl_xor(s, o, kWave);
+                            s = lane_group_sum(s, kWave);
 #pragma unroll
                             for (int t = 0; t < NT; t++) dot[t] = s;
                         } else {
 #pragma unroll
-                            for (int t = 0; t < NT; t++)
-                                for (int o = 1; o < lph; o <<= 1) dot[t] += __shfl_xor(dot[t], o, kWave);
+                            for (int t = 0; t < NT; t++) dot[t] = lane_group_sum(dot[t], lph);
                         }
 #pragma unroll
                         for (int t = 0; t < NT; t++)
                             if (act[t]) {
                                 const float z = el_r[t] + st[u][t].x;
-                                const float alpha = expf(lrelu(z, slope) - st[u][t].y) * st[u][t].z;
+                                const float alpha = fast_exp(lrelu(z, slope) - st[u][t].y) * st[u][t].z;
                                 const float gz = alpha * (dot[t] - st[u][t].w) * (z > 0.f ? 1.f : slope);
                                 gel[t] += gz;
 #pragma unroll
                                 for (int v = 0; v < VEC; v++) acc[t][v] = fmaf(alpha, gv[u][t][v], acc[t][v]);
-                                if (lead[t]) gz_csc[(size_t)slot * H + head[t]] = gz;
+                                if (lead[t]) gz_csc[(uint32_t)slot * (uint32_t)H + (uint32_t)head[t]] = gz;
                             }
                     }
                 }
@@ -941,6 +986,7 @@ JG_EXPORT int32_t jgamd_gat_bwd_workspace(int32_t V, int64_t E, int32_t H, int32
     if (int32_t rc = check_gat("gat_bwd", V, E, H, D)) return rc;
     if (!gat_shape(V, E, H, D).bwd_ok)
         return fail(JGAMD_ERR_UNSUPPORTED, "gat_bwd: with H > 1 the head width D=%d must give a power-of-two lane count", D);
+    if ((int64_t)E * H >= ((int64_t)1 << 32)) return fail(JGAMD_ERR_UNSUPPORTED, "gat_bwd: E*H does not fit 32 bits");
     *bytes = V == 0 ? 0 : gat_bwd_ws(V, E, H, D);
     return 0;
 }
@@ -956,6 +1002,7 @@ JG_EXPORT int32_t jgamd_gat_bwd(const int32_t *off, const int32_t *idx, const in
     const GatShape s = gat_shape(V, E, H, D);
     if (!s.bwd_ok)
         return fail(JGAMD_ERR_UNSUPPORTED, "gat_bwd: with H > 1 the head width D=%d must give a power-of-two lane count", D);
+    if ((int64_t)E * H >= ((int64_t)1 << 32)) return fail(JGAMD_ERR_UNSUPPORTED, "gat_bwd: E*H does not fit 32 bits");
     if (!g_a_src || !g_a_dst) return fail(JGAMD_ERR_NULL, "gat_bwd: NULL gradient output");
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int F = H * D;
