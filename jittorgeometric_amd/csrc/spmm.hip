@@ -345,8 +345,9 @@ static int env_int(const char *name, int dflt)
 // few enough that the per-chunk partial row stays a small share of the work.
 static int pick_chunk(int64_t M)
 {
+    // benchmark override, read once per process (the workspace query and the launch agree)
     static const int forced = env_int("JGAMD_SPMM_CHUNK", 0);
-    if (forced) return forced;
+    if (forced) return forced < 16 ? 16 : (forced > 4096 ? 4096 : forced);
     int c = 512;
     while (c > 32 && M / c < 32768) c >>= 1;
     return c;
