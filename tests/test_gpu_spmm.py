@@ -145,3 +145,49 @@ def test_hub_row_with_millions_of_entries_uses_grouped_piece_sums():
     ei[1, :2500000] = 777
     ei[0, 2500000:2900000] = 5            # and a 400k-entry row for the backward direction
     check_fwd_bwd(ei, w, V, F)
+
+
+def test_dense_233k_full_size_odd_width():
+    """Benchmark configuration 4 at F=41 (rows of x are not line-aligned): forward over
+    the CSC arrays against the oracle's sequential sums, backward through the
+    transpose identity."""
+    from jittorgeometric_amd import synthetic
+    from jittorgeometric_amd.ops import aggregateWithWeight
+    ei, V = synthetic.make("dense_233k")
+    ei, w = oracle.gcn_norm(ei, None, V)
+    ei = ei.astype(np.int32)
+    F = 41
+    rng = np.random.default_rng(44)
+    x = rng.standard_normal((V, F)).astype(np.float32)
+    g = rng.standard_normal((V, F)).astype(np.float32)
+    csc, csr = gpu_csx(ei, w, V)
+    xt = to_gpu(x).requires_grad_(True)
+    out = aggregateWithWeight(xt, csc, csr)
+    out.backward(to_gpu(g))
+    ocsc = oracle.cootocsc(ei, w, V)
+    want = oracle.aggregate_with_weight(x, ocsc)
+    assert_close(out.detach().cpu().numpy(), want, abs_scale(x, *ocsc), what="config 4 forward F=41")
+    lhs = (out.detach().double() * to_gpu(g).double()).sum().item()
+    rhs = (xt.grad.double() * to_gpu(x).double()).sum().item()
+    assert abs(lhs - rhs) <= 1e-6 * (out.detach().abs().double() * to_gpu(g).abs().double()).sum().item()
+
+
+def test_wide_rows_take_the_64_bit_address_path():
+    """x larger than 4 GiB: gathered rows are addressed with 64-bit arithmetic."""
+    from jittorgeometric_amd.ops._common import spmm
+    rng = np.random.default_rng(45)
+    C, F, R, E = 4_300_000, 256, 3000, 40000          # C*F*4 = 4.4e9 bytes
+    x = torch.empty((C, F), dtype=torch.float32, device=dev())
+    x.normal_()
+    src = np.concatenate([rng.integers(0, C, E - 8), np.arange(C - 8, C)]).astype(np.int32)   # reach the last rows
+    dst = rng.integers(0, R, E).astype(np.int32)
+    w = rng.standard_normal(E).astype(np.float32)
+    row, off, cw = oracle.cootocsc(np.stack([src, dst]), w, R)
+    out = spmm(to_gpu(off), to_gpu(row), to_gpu(cw), x, R).cpu().numpy()
+    xs = x[torch.from_numpy(row.astype(np.int64)).to(dev())].cpu().numpy().astype(np.float64)   # [E,F] gathered rows
+    want = np.zeros((R, F))
+    seg = np.repeat(np.arange(R), np.diff(off))
+    np.add.at(want, seg, xs * cw[:, None].astype(np.float64))
+    scale = np.zeros((R, F))
+    np.add.at(scale, seg, np.abs(xs) * np.abs(cw[:, None]))
+    assert_close(out, want, scale, what="wide x")
