@@ -10,6 +10,7 @@ from torch import nn
 
 from ...ops import EdgeSoftmax, ScatterToEdge, ScatterToVertex, gat_aggregate
 from ...ops.gat import fused_supported
+from ..dense import xw
 from ..inits import glorot
 from .message_passiong_nts import MessagePassingNts
 
@@ -69,7 +70,7 @@ class GATConv(MessagePassingNts):
         return ScatterToVertex(edge, csc, "src")
 
     def vertex_forward(self, x):
-        return torch.relu(x @ self.weight)
+        return torch.relu(xw(x, self.weight))
 
     def __repr__(self):
         return "{}({}, {})".format(self.__class__.__name__, self.in_channels, self.out_channels)

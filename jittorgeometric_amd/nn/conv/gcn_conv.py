@@ -6,6 +6,7 @@ from torch import nn
 from ...ops import SpmmCsr, aggregateWithWeight
 from ...utils import add_remaining_self_loops
 from ...utils.num_nodes import maybe_num_nodes
+from ..dense import xw
 from ..inits import glorot, zeros
 
 
@@ -51,7 +52,7 @@ class GCNConv(nn.Module):
         zeros(self.bias)
 
     def forward(self, x, csc, csr):
-        x = x @ self.weight
+        x = xw(x, self.weight)
         if self.spmm:
             out = self.propagate_spmm(x=x, csr=csr)
         else:

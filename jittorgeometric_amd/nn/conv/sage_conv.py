@@ -4,6 +4,7 @@ import torch
 from torch import nn
 
 from ...ops import SpmmCsr, aggregateWithWeight, cootocsc, cootocsr
+from ..dense import xw
 from ..inits import glorot, zeros
 from .gcn_conv import _degree_norm
 
@@ -72,9 +73,9 @@ class SAGEConv(nn.Module):
             out = self.propagate_spmm(x=xs[0], csr=csr)
         else:
             out = self.propagate_msg(x=xs[0], csc=csc, csr=csr)
-        out = out @ self.weight1
+        out = xw(out, self.weight1)
         if self.root_weight is not None:
-            out = out + xs[1] @ self.root_weight
+            out = out + xw(xs[1], self.root_weight)
         if self.bias is not None:
             out = out + self.bias
         return out
