@@ -196,6 +196,16 @@ int32_t jgamd_gat_bwd(const int32_t *off, const int32_t *idx, const int32_t *t_o
                       int32_t V, int64_t E, int32_t H, int32_t D, void *ws, size_t ws_bytes,
                       void *stream);
 
+/* ------------------------------------------------------------------------
+ * Column sums of a row-major [R,F] matrix: out[f] = sum_r x[r,f].  The bias
+ * gradient of the conv layers (`out += self.bias`, nn/conv/gcn_conv.py:100-101,
+ * nn/conv/sage_conv.py:189-190; Jittor derives the reduction).  Two stages,
+ * fixed order, no atomics.
+ */
+int32_t jgamd_column_sum_workspace(int64_t R, int32_t F, size_t *bytes);
+int32_t jgamd_column_sum(const float *x, float *out, int64_t R, int32_t F, void *ws,
+                         size_t ws_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

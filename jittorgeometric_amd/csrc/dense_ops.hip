@@ -1,0 +1,103 @@
+// Column sums of a row-major [R,F] matrix: the bias gradient of the conv
+// layers (out += bias in gcn_conv.py:100-101 of the reference; its backward
+// is a sum over all nodes).  Two deterministic stages: every block sums a
+// stripe of rows into partial[block][F], one more kernel adds the partials in
+// block order.  Narrow odd widths (47 classes) are where a generic reduction
+// falls off a cliff; here a block's threads are laid out as
+// (row group, column) so that each pass reads a contiguous run of whole rows.
+#include "common.h"
+
+namespace jg {
+
+constexpr int kColThreads = 256;
+constexpr int kColStripe = 2048;   // rows per block
+
+__global__ __launch_bounds__(kColThreads) void column_partial_sums(const float *__restrict__ x, int64_t R, int F,
+                                                                   float *__restrict__ partial)
+{
+    __shared__ float red[kColThreads];
+    const int cols = F < kColThreads ? F : kColThreads;     // columns handled per slab
+    const int groups = kColThreads / cols;                  // rows read together
+    const int c = threadIdx.x % cols, g = threadIdx.x / cols;
+    const int64_t r0 = (int64_t)blockIdx.x * kColStripe;
+    const int64_t r1 = r0 + kColStripe < R ? r0 + kColStripe : R;
+    for (int slab = 0; slab < F; slab += cols) {
+        const int col = slab + c;
+        float s = 0.f;
+        if (g < groups && col < F) {
+            constexpr int kB = 8;                            // loads in flight per thread
+            for (int64_t rb = r0 + g; rb < r1; rb += (int64_t)kB * groups) {
+                float v[kB];
+#pragma unroll
+                for (int i = 0; i < kB; i++) {
+                    const int64_t r = rb + (int64_t)i * groups;
+                    v[i] = x[(r < r1 ? r : r1 - 1) * F + col];
+                }
+#pragma unroll
+                for (int i = 0; i < kB; i++)
+                    if (rb + (int64_t)i * groups < r1) s += v[i];
+            }
+        }
+        __syncthreads();
+        red[threadIdx.x] = s;
+        __syncthreads();
+        if (g == 0 && col < F) {
+            float t = 0.f;
+            for (int k = 0; k < groups; k++) t += red[k * cols + c];
+            partial[(size_t)blockIdx.x * F + col] = t;
+        }
+    }
+}
+
+__global__ void column_final_sums(const float *__restrict__ partial, int nblocks, int F, float *__restrict__ out)
+{
+    __shared__ float part[16][64];
+    const int col = blockIdx.x * 64 + (threadIdx.x & 63);
+    const int grp = threadIdx.x >> 6;
+    float s = 0.f;
+    if (col < F)
+        for (int b = grp; b < nblocks; b += 16) s += partial[(size_t)b * F + col];
+    part[grp][threadIdx.x & 63] = s;
+    __syncthreads();
+    if (grp == 0 && col < F) {
+        float t = 0.f;
+#pragma unroll
+        for (int k = 0; k < 16; k++) t += part[k][threadIdx.x];
+        out[col] = t;
+    }
+}
+
+}  // namespace jg
+
+using namespace jg;
+#define JG_EXPORT extern "C" __attribute__((visibility("default")))
+
+static size_t colsum_ws(int64_t R, int32_t F) { return carve_bytes((size_t)ceil_div(R > 0 ? R : 1, kColStripe) * F, 4); }
+
+JG_EXPORT int32_t jgamd_column_sum_workspace(int64_t R, int32_t F, size_t *bytes)
+{
+    if (!bytes) return fail(JGAMD_ERR_NULL, "column_sum_workspace: bytes is NULL");
+    if (R < 0 || F < 0) return fail(JGAMD_ERR_SIZE, "column_sum: negative size");
+    *bytes = F == 0 ? 0 : colsum_ws(R, F);
+    return 0;
+}
+
+JG_EXPORT int32_t jgamd_column_sum(const float *x, float *out, int64_t R, int32_t F, void *ws, size_t ws_bytes,
+                                   void *stream)
+{
+    if (R < 0 || F < 0) return fail(JGAMD_ERR_SIZE, "column_sum: negative size");
+    if (F == 0) return 0;
+    if (!out) return fail(JGAMD_ERR_NULL, "column_sum: out is NULL");
+    if (R > 0 && !x) return fail(JGAMD_ERR_NULL, "column_sum: x is NULL");
+    const size_t need = colsum_ws(R, F);
+    if (!ws || ws_bytes < need) return fail(JGAMD_ERR_WORKSPACE, "column_sum: workspace %zu < %zu bytes", ws ? ws_bytes : (size_t)0, need);
+    if (((uintptr_t)ws & 255) != 0) return fail(JGAMD_ERR_ALIGN, "column_sum: workspace not 256-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    float *partial = static_cast<float *>(ws);
+    const int nblocks = (int)ceil_div(R > 0 ? R : 1, kColStripe);
+    if (R > 0)
+        hipLaunchKernelGGL(column_partial_sums, dim3((unsigned)nblocks), dim3(kColThreads), 0, st, x, R, F, partial);
+    hipLaunchKernelGGL(column_final_sums, dim3((unsigned)ceil_div(F, 64)), dim3(1024), 0, st, partial, R > 0 ? nblocks : 0,
+                       F, out);
+    return launch_status("column_sum");
+}

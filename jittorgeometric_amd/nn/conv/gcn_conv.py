@@ -3,11 +3,25 @@ GCNConv (nn/conv/gcn_conv.py:40-116) on torch tensors."""
 import torch
 from torch import nn
 
-from ...ops import SpmmCsr, aggregateWithWeight
+from ...ops import SpmmCsr, aggregateWithWeight, cootocsc
 from ...utils import add_remaining_self_loops
 from ...utils.num_nodes import maybe_num_nodes
-from ..dense import xw
+from ..dense import add_bias, xw
 from ..inits import glorot, zeros
+
+
+def _degree_by_col(edge_index, edge_weight, num_nodes):
+    """deg[v] = sum of the weights of the edges whose destination is v
+    (jt.scatter(..., reduce='add') by col in gcn_conv.py:33-34).  On the GPU it
+    is the column sum of the CSC arrays: conversion + gather-sum, in a fixed
+    order and without the same-address atomics a hub destination causes."""
+    if edge_weight.is_cuda and edge_weight.dtype == torch.float32 and edge_index.shape[1] > 0:
+        from ...ops._common import spmm
+        csc = cootocsc(edge_index.contiguous(), edge_weight, num_nodes)
+        return spmm(csc.column_offset, None, None, csc.edge_weight.view(-1, 1), num_nodes).view(-1)
+    deg = torch.zeros((num_nodes,), dtype=edge_weight.dtype, device=edge_weight.device)
+    deg.scatter_add_(0, edge_index[1].long(), edge_weight)
+    return deg
 
 
 def _degree_norm(edge_index, edge_weight, num_nodes, improved, add_self_loops, power):
@@ -18,8 +32,7 @@ def _degree_norm(edge_index, edge_weight, num_nodes, improved, add_self_loops, p
     if add_self_loops:
         edge_index, edge_weight = add_remaining_self_loops(edge_index, edge_weight, fill_value, num_nodes)
     row, col = edge_index[0].long(), edge_index[1].long()
-    deg = torch.zeros((num_nodes,), dtype=edge_weight.dtype, device=edge_weight.device)
-    deg.scatter_add_(0, col, edge_weight)
+    deg = _degree_by_col(edge_index, edge_weight, num_nodes)
     dinv = deg.pow(power)
     dinv.masked_fill_(dinv == float("inf"), 0)
     return edge_index, edge_weight, dinv, row, col
@@ -58,7 +71,7 @@ class GCNConv(nn.Module):
         else:
             out = self.propagate_msg(x=x, csc=csc, csr=csr)
         if self.bias is not None:
-            out = out + self.bias
+            out = add_bias(out, self.bias)
         return out
 
     execute = forward

@@ -4,7 +4,7 @@ import torch
 from torch import nn
 
 from ...ops import SpmmCsr, aggregateWithWeight, cootocsc, cootocsr
-from ..dense import xw
+from ..dense import add_bias, xw
 from ..inits import glorot, zeros
 from .gcn_conv import _degree_norm
 
@@ -77,7 +77,7 @@ class SAGEConv(nn.Module):
         if self.root_weight is not None:
             out = out + xw(xs[1], self.root_weight)
         if self.bias is not None:
-            out = out + self.bias
+            out = add_bias(out, self.bias)
         return out
 
     execute = forward

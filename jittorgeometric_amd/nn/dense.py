@@ -42,3 +42,37 @@ def xw(x, weight):
     if x.dim() != 2 or not x.is_contiguous():
         return x @ weight
     return _XW.apply(x, weight)
+
+
+def column_sum(x):
+    """sum over rows of a contiguous [R,F] float32 GPU tensor (csrc/dense_ops.hip)."""
+    from .. import _lib
+    lib = _lib.load()
+    dev = _lib.require_gpu(x)
+    R, F = x.shape
+    out = torch.empty(F, dtype=torch.float32, device=dev)
+    nbytes = _lib.query(lib.jgamd_column_sum_workspace, R, F)
+    ws = _lib.workspace(nbytes, dev)
+    _lib.check(lib.jgamd_column_sum(_lib.ptr(x), _lib.ptr(out), R, F, _lib.ptr(ws), nbytes, _lib.stream_ptr(dev)))
+    return out
+
+
+class _AddBias(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, bias):
+        return x + bias
+
+    @staticmethod
+    def backward(ctx, g):
+        gb = None
+        if ctx.needs_input_grad[1]:
+            if g.is_cuda and g.dim() == 2 and g.dtype == torch.float32:
+                gb = column_sum(g.contiguous())
+            else:
+                gb = g.sum(0)
+        return g, gb
+
+
+def add_bias(x, bias):
+    """x + bias (broadcast over rows) whose bias gradient is the library's column sum."""
+    return _AddBias.apply(x, bias)

@@ -122,3 +122,37 @@ def test_spmmcsr_reference_grad_switch():
             assert_close(xt.grad.cpu().numpy(), want, np.abs(want) + 1.0, what="REFERENCE_GRAD=%s" % flag)
     finally:
         spmmcsr.REFERENCE_GRAD = False
+
+
+@pytest.mark.parametrize("R,F", [(1, 1), (5000, 47), (100000, 7), (70000, 128), (3000, 602), (0, 16), (2049, 256)])
+def test_bias_gradient_column_sum(R, F):
+    from jittorgeometric_amd.nn.dense import add_bias, column_sum
+    rng = np.random.default_rng(R + F)
+    g = rng.standard_normal((R, F)).astype(np.float32)
+    got = column_sum(to_gpu(g)).cpu().numpy() if R > 0 else column_sum(torch.empty((0, F), device=dev())).cpu().numpy()
+    want = g.astype(np.float64).sum(0)
+    assert_close(got, want, np.abs(g).astype(np.float64).sum(0), what="column sum")
+    if R > 0:
+        b = torch.zeros(F, device=dev(), requires_grad=True)
+        x = to_gpu(g).requires_grad_(True)
+        add_bias(x, b).backward(to_gpu(g))
+        assert_close(b.grad.cpu().numpy(), (g.astype(np.float64) ** 1).sum(0), np.abs(g).astype(np.float64).sum(0))
+        assert torch.equal(x.grad, to_gpu(g))
+
+
+def test_gcn_norm_with_hub_destination_matches_oracle():
+    from jittorgeometric_amd.nn import gcn_norm, sage_norm
+    from util import rand_graph
+    rng = np.random.default_rng(91)
+    V, E = 20000, 400000
+    ei, _ = rand_graph(rng, V, E, hubs=1, hub_share=0.6)
+    # several self-loops on one node make "which weight becomes the loop weight" order-dependent
+    # in the reference too (utils/loop.py:130-132); keep at most none
+    ei = ei[:, ei[0] != ei[1]]
+    w = rng.random(ei.shape[1]).astype(np.float32) + 0.5
+    for fn, ofn in ((gcn_norm, oracle.gcn_norm), (sage_norm, oracle.sage_norm)):
+        gi, gw = fn(to_gpu(ei), to_gpu(w), V)
+        oi, ow = ofn(ei, w, V)
+        assert np.array_equal(gi.cpu().numpy(), oi)
+        # degrees of 10^5-edge hubs are float sums in different orders
+        assert_close(gw.cpu().numpy(), ow, rtol=2e-4, atol=0, what=fn.__name__)
