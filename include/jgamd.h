@@ -106,7 +106,8 @@ int32_t jgamd_csx_transpose(const int32_t *off, const int32_t *idx, const float 
  * Entries with idx outside [0,C) contribute nothing.
  * Limits: E + R < 2^31, 1 <= F <= 65535*2048.
  * Environment: JGAMD_SPMM_CHUNK=<16..4096> overrides the number of merged items
- * per wavefront (tuning aid; read once per process).
+ * per wavefront; JGAMD_SPMM_STAGE=lds|reg forces how (idx, w) are staged
+ * (tuning aids; read once per process).
  */
 int32_t jgamd_spmm_csx_workspace(int32_t R, int64_t E, int32_t F, size_t *bytes);
 int32_t jgamd_spmm_csx(const int32_t *off, const int32_t *idx, const float *w, const float *x,

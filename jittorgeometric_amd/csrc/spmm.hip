@@ -6,9 +6,12 @@
 // into pieces and a run of empty rows costs what the same number of entries
 // would.  Inside a wavefront the feature dimension lies across the 64 lanes
 // (VEC floats per lane, NT tiles of 64*VEC features), the entries are walked
-// in order, and (idx, w) are loaded 64 at a time, one per lane, then handed
-// out with v_readlane so that every gathered row has a scalar base address.
-// The gathers of UNROLL entries are issued before the first is used.
+// in order, and (idx, w) are loaded 64 at a time, one per lane, then staged:
+// through the wavefront's LDS slice (every lane reads entry i at the same
+// address, a broadcast) for F >= 64, or rotated with a shuffle and handed out
+// with v_readlane for narrower rows, where the two extra LDS waits per group
+// show.  Either way a gathered row is (scalar base) + (32-bit byte offset),
+// and the gathers of UNROLL entries are issued before the first is used.
 //
 // A row that ends inside a chunk is stored by that chunk's wavefront.  The
 // leading piece of a row that continues into the next chunk goes to
@@ -22,6 +25,8 @@
 namespace jg {
 
 constexpr int kSpmmThreads = 256;
+// (idx, w) staging: through LDS from this width up, through registers (shuffle + readlane) below
+constexpr int kLdsStageMinWidth = 64;
 constexpr int kSpmmWaves = kSpmmThreads / kWave;
 
 template <int VEC> struct Vec;
@@ -84,7 +89,7 @@ __global__ void spmm_chunk_rows(const int32_t *__restrict__ off, int R, int chun
 // WIDE = false: every row of x starts less than 4 GiB from x, so a gathered
 // row is addressed as (scalar base) + (32-bit byte offset): one readlane and
 // one vector add per entry.  WIDE = true keeps 64-bit row arithmetic.
-template <int VEC, int NT, int UNROLL, bool WIDE>
+template <int VEC, int NT, int UNROLL, bool WIDE, bool LDS>
 __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__restrict__ off,
                                                            const int32_t *__restrict__ idx,
                                                            const float *__restrict__ w,
@@ -94,6 +99,8 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__rest
                                                            int E, int F, int chunk, int nchunks)
 {
     static_assert(kWave % UNROLL == 0, "groups tile a 64-entry batch");
+    __shared__ int2 staged_all[LDS ? kSpmmThreads : 1];
+    int2 *staged = staged_all + (LDS ? (threadIdx.x & ~(kWave - 1)) : 0);   // this wavefront's 64 slots
     const int k = blockIdx.x * kSpmmWaves + wave_in_block();
     if (k >= nchunks) return;
     const int lane = lane_id();
@@ -166,12 +173,20 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__rest
         }
         // what each lane contributes to addressing: its row's byte offset, or its row index
         const int my_a = WIDE ? my_c : (int)((uint32_t)my_c * row_bytes);
+        if (LDS) {
+            // stage the batch's (address term, weight) pairs in this wavefront's LDS slice; every
+            // lane then reads entry i at the same address (a broadcast read, no VALU involved)
+            __builtin_amdgcn_wave_barrier();
+            staged[lane] = make_int2(my_a, __float_as_int(my_w));
+            __builtin_amdgcn_wave_barrier();
+        }
         for (int i0 = 0; i0 < n; i0 += UNROLL) {
-            // rotate the group's UNROLL entries into lanes 0..UNROLL-1 so that the
+            // registers: rotate the group's UNROLL entries into lanes 0..UNROLL-1 so that the
             // broadcasts below take immediate lane numbers
             const int from = (lane + i0) & (kWave - 1);
-            const int g_a = __shfl(my_a, from, kWave);
-            const float g_w = __shfl(my_w, from, kWave);
+            const int g_a = LDS ? 0 : __shfl(my_a, from, kWave);
+            const float g_w = LDS ? 0.f : __shfl(my_w, from, kWave);
+            float wl[UNROLL];
             // Issue phase: straight-line code, no branches and no lane predicates, so that the
             // UNROLL gathers leave back to back.  Slots past n re-read the row of a lane that
             // holds no entry (offset 0, weight 0, never accumulated); lanes past F read the
@@ -179,7 +194,14 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__rest
             float xv[UNROLL][NT][VEC];
 #pragma unroll
             for (int u = 0; u < UNROLL; u++) {
-                const int a = bcast_i(g_a, u);
+                int a;
+                if (LDS) {
+                    const int2 e = staged[i0 + u];
+                    a = e.x;
+                    wl[u] = __int_as_float(e.y);
+                } else {
+                    a = bcast_i(g_a, u);
+                }
 #pragma unroll
                 for (int t = 0; t < NT; t++) {
                     if (WIDE)
@@ -197,7 +219,7 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__rest
                     do flush_row(); while (row_end == jb + i0 + u);
                     left = row_end - (jb + i0);
                 }
-                const float wv = bcast_f(g_w, u);
+                const float wv = LDS ? wl[u] : bcast_f(g_w, u);
 #pragma unroll
                 for (int t = 0; t < NT; t++) {
 #pragma unroll
@@ -391,13 +413,22 @@ static void launch_spmm(const SpmmShape &s, const int32_t *off, const int32_t *i
     // gathers in flight per wavefront: bounded by the registers they land in
     constexpr int U = (VEC * NT >= 16) ? 4 : (VEC * NT >= 8 ? 8 : (VEC * NT >= 2 ? 16 : 32));
     if (k0) (void)hipEventRecord(k0, st);
-    // 32-bit byte offsets reach every row of x when C*F*4 < 2^32
-    if ((uint64_t)C * (uint64_t)F * 4u < ((uint64_t)1 << 32))
-        hipLaunchKernelGGL((spmm_merge<VEC, NT, U, false>), grid, block, 0, st, off, idx, w, x, out, partial,
-                           chunk_row, R, C, E, F, s.chunk, s.nchunks);
-    else
-        hipLaunchKernelGGL((spmm_merge<VEC, NT, U, true>), grid, block, 0, st, off, idx, w, x, out, partial,
-                           chunk_row, R, C, E, F, s.chunk, s.nchunks);
+    // 32-bit byte offsets reach every row of x when C*F*4 < 2^32.  (idx, w) staging: LDS or
+    // registers (JGAMD_SPMM_STAGE=lds|reg overrides the default).
+    static const int stage_env = [] {
+        const char *e = getenv("JGAMD_SPMM_STAGE");
+        return !e ? 0 : (e[0] == 'l' ? 1 : (e[0] == 'r' ? 2 : 0));
+    }();
+    const bool lds = stage_env ? stage_env == 1 : F >= kLdsStageMinWidth;
+    const bool narrow = (uint64_t)C * (uint64_t)F * 4u < ((uint64_t)1 << 32);
+#define JG_GO(W, L)                                                                                                   \
+    hipLaunchKernelGGL((spmm_merge<VEC, NT, U, W, L>), grid, block, 0, st, off, idx, w, x, out, partial, chunk_row, R, \
+                       C, E, F, s.chunk, s.nchunks)
+    if (narrow && lds) JG_GO(false, true);
+    else if (narrow) JG_GO(false, false);
+    else if (lds) JG_GO(true, true);
+    else JG_GO(true, false);
+#undef JG_GO
     if (k1) (void)hipEventRecord(k1, st);
     const int ngroups = (int)ceil_div(s.nchunks, kGroup);
     if (ngroups > 1)
