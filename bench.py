@@ -29,7 +29,7 @@ HBM_PEAK_GBPS = 8000.0
 F = 128
 # FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 per spmm_merge launch on this exact (seeded) workload;
 # factors from a plain 1 GiB copy in the same counter runs.
-PROFILED_TRAFFIC_BYTES = 7.077e9
+PROFILED_TRAFFIC_BYTES = 7.074e9
 
 
 def spmm_bytes(R, E, feat):
