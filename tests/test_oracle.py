@@ -271,3 +271,24 @@ def test_gat_forward_matches_dense_fp64():
                                       np.stack([a[C:], a[C:]]))
     np.testing.assert_allclose(o8[:, 0], out, rtol=1e-6, atol=1e-7)
     assert a8.shape == (E, 2)
+
+
+# ------------------------------------------------------ committed vectors ---
+
+def test_oracle_reproduces_committed_vectors():
+    """tests/golden/oracle_vectors_v64.npz was written by make_oracle_vectors.py;
+    a change in oracle.c that alters any output shows up here."""
+    import importlib.util
+    here = os.path.join(os.path.dirname(__file__), "golden")
+    spec = importlib.util.spec_from_file_location("make_oracle_vectors", os.path.join(here, "make_oracle_vectors.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    fresh = mod.build()
+    gold = np.load(os.path.join(here, "oracle_vectors_v64.npz"))
+    assert set(gold.files) == set(fresh)
+    for k in gold.files:
+        a, b = gold[k], np.asarray(fresh[k])
+        if a.dtype.kind in "iu":
+            assert np.array_equal(a, b), k
+        else:
+            np.testing.assert_allclose(b, a, rtol=1e-6, atol=1e-7, err_msg=k)
