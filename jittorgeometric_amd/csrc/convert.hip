@@ -11,18 +11,23 @@
 //                         (bucket = key >> shift, <= 2048 buckets).
 //   2. scan             : the (bucket, block) table -> each block's write
 //                         cursor in each bucket (and every bucket's extent).
-//   3. partition        : every block re-reads its edges and writes them, as
-//                         12/16-byte records, to their bucket in input order.
-//   4. sub-block plan   : buckets are cut into sub-blocks of <= 32768
-//                         records, so a hub's bucket is many blocks' work.
+//   3. partition        : every block re-reads its edges, sorts its tile by
+//                         bucket inside LDS and writes 12/16-byte records,
+//                         one contiguous run per (block, bucket), in input
+//                         order.
+//   4. sub-block plan   : buckets are cut into sub-blocks of <= 8192 records
+//                         (one tile), so a hub's bucket is many blocks' work.
 //   5. sub-block count  : LDS counts per key of the bucket (<= 2048 keys).
 //   6. bucket offsets   : per bucket, prefix over its sub-blocks and keys ->
 //                         the final offsets array and every sub-block's
 //                         first output slot per key.
-//   7. sub-block scatter: records are walked in order and placed at
-//                         cursor[key] + (rank among equal keys so far); a
-//                         bucket's output window is a few hundred KB, so the
-//                         scattered 4-byte stores combine in L2.
+//   7. sub-block scatter: the tile is sorted by key inside LDS and leaves as
+//                         one contiguous run per (sub-block, key).
+//
+// Both scatters go through LDS because lanes that store 64 unrelated
+// addresses leave partly written cache lines behind: with ~1000 bins times
+// ~500 resident blocks the write frontier does not fit in L2 and every short
+// store is written back on its own (2.7-3x the bytes on the counters).
 //
 // Two levels of at most 2048 bins each cover V <= 2^22 vertices.  Above that
 // the records are sorted by plain LSD passes of the same stable partition
@@ -86,38 +91,112 @@ __global__ __launch_bounds__(kPartThreads) void csx_bucket_histogram(const int32
     if (blockIdx.x == 0 && threadIdx.x == 0) table[(int64_t)nbins * nblocks] = 0;
 }
 
-// ------------------------------------------------------- stable tile rank ---
+// ------------------------------------------------------- stable tile sort ---
 // The block's tile is kTile consecutive items; wave w owns the kWaveSpan
 // consecutive items starting at w*kWaveSpan and visits them in rounds of 64
 // (lane l = item r*64 + l), so (wave, round, lane) is the input order.
-// cnt is [kPartWaves][nbins] in LDS.  On entry cnt is undefined; `cursor(b)`
-// gives the position of the first item of bin b in this tile.  On exit
-// pos[r] is the destination of this thread's item of round r (bin[r] < 0:
-// item absent).  `after(b, end)` is called once per bin with the position
-// one past the tile's last item of bin b.
-template <typename Cursor, typename After>
-__device__ __forceinline__ void tile_rank(int *cnt, int nbins, int nbits, const int (&bin)[kItems],
-                                          int (&pos)[kItems], Cursor cursor, After after)
+//
+// tile_sort gives every item its position in the tile sorted stably by bin:
+//   start[bin] + (items of that bin in earlier waves)
+//              + (same wave, earlier rounds) + (same round, lower lanes).
+// Per-wave counters are 16 bits wide (a wave holds 1024 items, a tile 8192
+// positions), two waves to a word.  tile_emit then moves the records through
+// an LDS window of kStage records so that consecutive lanes hold consecutive
+// sorted records, and hands each one to `emit` with its global position
+// gbase(bin) + (position - start[bin]).  The window takes what is left of
+// kTileLdsBytes after the per-bin arrays, so two blocks fit a CU's 160 KB.
+constexpr size_t kTileLdsBytes = 78 * 1024;
+
+struct TileLds {
+    uint32_t *cnt;    // [kPartWaves / 2][nbins]
+    int *start;       // [nbins] tile-local first position of the bin
+    int *delta;       // [nbins] global minus tile-local position
+    int *misc;        // [kPartWaves] wave totals, [kPartWaves] tile total
+    uint32_t *stage;  // stage_n records
+    int stage_n;
+};
+constexpr int kTileMisc = 16;
+inline size_t tile_bins_bytes(int nbins) { return ((size_t)(kPartWaves / 2 + 2) * nbins + kTileMisc) * 4; }
+// records per trip through LDS: a multiple of the block size, at most a tile
+inline int tile_stage_records(int nbins, size_t rec_bytes)
 {
+    size_t n = (kTileLdsBytes - tile_bins_bytes(nbins)) / rec_bytes;
+    n = n / kPartThreads * kPartThreads;
+    return (int)(n > (size_t)kTile ? (size_t)kTile : n);
+}
+inline size_t tile_lds_bytes(int nbins, size_t rec_bytes)
+{
+    return tile_bins_bytes(nbins) + (size_t)tile_stage_records(nbins, rec_bytes) * rec_bytes;
+}
+template <typename Rec, typename Base>
+__device__ __forceinline__ int tile_sort(uint32_t *raw, int stage_n, TileLds &L, int nbins, int nbits,
+                                         const int (&bin)[kItems], int (&lp)[kItems], Base gbase)
+{
+    L.stage = raw;
+    L.stage_n = stage_n;
+    L.cnt = raw + stage_n * (sizeof(Rec) / 4);
+    L.start = reinterpret_cast<int *>(L.cnt + (kPartWaves / 2) * nbins);
+    L.delta = L.start + nbins;
+    L.misc = L.delta + nbins;
+
     const int w = threadIdx.x >> 6;
     const int lane = lane_id();
-    int *mine = cnt + w * nbins;
-    for (int b = threadIdx.x; b < nbins * kPartWaves; b += kPartThreads) cnt[b] = 0;
+    const int half = (w & 1) * 16;
+    uint32_t *mine = L.cnt + (w >> 1) * nbins;
+    for (int i = threadIdx.x; i < (kPartWaves / 2) * nbins; i += kPartThreads) L.cnt[i] = 0;
+    // bins b0 .. b0+K-1 belong to this thread in the per-bin phase; their
+    // global bases are fetched now so the latency hides behind the counting
+    constexpr int kMaxK = kMaxBins / kPartThreads;
+    const int K = (nbins + kPartThreads - 1) / kPartThreads;
+    const int b0 = threadIdx.x * K;
+    int gb[kMaxK];
+#pragma unroll
+    for (int i = 0; i < kMaxK; i++) gb[i] = (i < K && b0 + i < nbins) ? gbase(b0 + i) : 0;
     __syncthreads();
 #pragma unroll
     for (int r = 0; r < kItems; r++)
-        if (bin[r] >= 0) atomicAdd(&mine[bin[r]], 1);
+        if (bin[r] >= 0) atomicAdd(&mine[bin[r]], 1u << half);
     __syncthreads();
-    for (int b = threadIdx.x; b < nbins; b += kPartThreads) {
-        int run = cursor(b);
+    uint32_t pk[kMaxK][kPartWaves / 2];
+    int tot[kMaxK];
+    int mysum = 0;
 #pragma unroll
-        for (int v = 0; v < kPartWaves; v++) {
-            int c = cnt[v * nbins + b];
-            cnt[v * nbins + b] = run;
-            run += c;
+    for (int i = 0; i < kMaxK; i++) {
+        tot[i] = 0;
+        if (i < K && b0 + i < nbins) {
+            int run = 0;
+#pragma unroll
+            for (int v = 0; v < kPartWaves / 2; v++) {
+                const uint32_t c = L.cnt[v * nbins + b0 + i];
+                const int lo = c & 0xffff, hi = c >> 16;
+                pk[i][v] = (uint32_t)run | ((uint32_t)(run + lo) << 16);
+                run += lo + hi;
+            }
+            tot[i] = run;
+            mysum += run;
         }
-        after(b, run);
     }
+    int inc = mysum;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        const int t = __shfl_up(inc, d, kWave);
+        if (lane >= d) inc += t;
+    }
+    if (lane == kWave - 1) L.misc[w] = inc;
+    __syncthreads();
+    int base = inc - mysum;
+    for (int v = 0; v < w; v++) base += L.misc[v];
+#pragma unroll
+    for (int i = 0; i < kMaxK; i++)
+        if (i < K && b0 + i < nbins) {
+            L.start[b0 + i] = base;
+            L.delta[b0 + i] = gb[i] - base;
+            const uint32_t both = (uint32_t)base | ((uint32_t)base << 16);
+#pragma unroll
+            for (int v = 0; v < kPartWaves / 2; v++) L.cnt[v * nbins + b0 + i] = pk[i][v] + both;
+            base += tot[i];
+        }
+    if (threadIdx.x == kPartThreads - 1) L.misc[kPartWaves] = base;
     __syncthreads();
     const uint64_t below = lane == 0 ? 0ull : (~0ull >> (kWave - lane));
 #pragma unroll
@@ -133,10 +212,31 @@ __device__ __forceinline__ void tile_rank(int *cnt, int nbins, int nbits, const 
         // peers: valid lanes of this round with the same bin as this lane
         const int leader = __ffsll((unsigned long long)peers) - 1;
         const int rank = __popcll(peers & below);
-        int start = 0;
-        if (valid && lane == leader) start = atomicAdd(&mine[b], __popcll(peers));
-        start = __shfl(start, leader < 0 ? 0 : leader, kWave);
-        pos[r] = start + rank;
+        uint32_t old = 0;
+        if (valid && lane == leader) old = atomicAdd(&mine[b], (uint32_t)__popcll(peers) << half);
+        old = __shfl(old, leader < 0 ? 0 : leader, kWave);
+        lp[r] = (int)((old >> half) & 0xffff) + rank;
+    }
+    return L.misc[kPartWaves];
+}
+
+template <typename Rec, typename Emit>
+__device__ __forceinline__ void tile_emit(const TileLds &L, int total, int shift, int mask, const Rec (&rec)[kItems],
+                                          const int (&bin)[kItems], const int (&lp)[kItems], Emit emit)
+{
+    Rec *stage = reinterpret_cast<Rec *>(L.stage);
+    for (int h0 = 0; h0 < total; h0 += L.stage_n) {
+#pragma unroll
+        for (int r = 0; r < kItems; r++)
+            if (bin[r] >= 0 && (unsigned)(lp[r] - h0) < (unsigned)L.stage_n) stage[lp[r] - h0] = rec[r];
+        __syncthreads();
+        const int n = min(total - h0, L.stage_n);
+#pragma unroll 4
+        for (int j = threadIdx.x; j < n; j += kPartThreads) {
+            const Rec q = stage[j];
+            emit(L.delta[(q.key >> shift) & mask] + h0 + j, q);
+        }
+        __syncthreads();
     }
 }
 
@@ -222,25 +322,23 @@ __global__ void csx_unpack_sorted(const Rec *__restrict__ recs, const int32_t *_
 template <typename Rec, typename Loader>
 __global__ __launch_bounds__(kPartThreads) void csx_partition(Loader in, int shift, int mask, int nbins,
                                                               int nbits, const int32_t *__restrict__ table,
-                                                              int nblocks, Rec *__restrict__ out)
+                                                              int nblocks, Rec *__restrict__ out, int stage_n)
 {
-    extern __shared__ int cnt[];
+    extern __shared__ uint32_t lds_raw[];
     const int w = threadIdx.x >> 6;
     const int64_t base = (int64_t)blockIdx.x * kTile + (int64_t)w * kWaveSpan + lane_id();
     Rec rec[kItems];
-    int bin[kItems], pos[kItems];
+    int bin[kItems], lp[kItems];
 #pragma unroll
     for (int r = 0; r < kItems; r++) in.load(base + (int64_t)r * kWave, rec[r]);
 #pragma unroll
     for (int r = 0; r < kItems; r++)
         bin[r] = in.valid(base + (int64_t)r * kWave, rec[r]) ? ((rec[r].key >> shift) & mask) : -1;
     const int blk = blockIdx.x;
-    tile_rank(
-        cnt, nbins, nbits, bin, pos, [&](int b) { return table[(int64_t)b * nblocks + blk]; },
-        [](int, int) {});
-#pragma unroll
-    for (int r = 0; r < kItems; r++)
-        if (bin[r] >= 0) out[pos[r]] = rec[r];
+    TileLds L;
+    const int total = tile_sort<Rec>(lds_raw, stage_n, L, nbins, nbits, bin, lp,
+                                     [&](int b) { return table[(int64_t)b * nblocks + blk]; });
+    tile_emit(L, total, shift, mask, rec, bin, lp, [&](int pos, const Rec &q) { out[pos] = q; });
 }
 
 // ---------------------------------------------------------------- step 4 ---
@@ -248,7 +346,7 @@ __global__ __launch_bounds__(kPartThreads) void csx_partition(Loader in, int shi
 // Cuts every bucket into sub-blocks of at most kSubRecords records (at least
 // one per bucket): sub_first[b] = first sub-block of b, sub_bucket[s] = bucket
 // of sub-block s (-1 for the unused tail of the max_sub launch slots).
-constexpr int kSubRecords = 4 * kTile;
+constexpr int kSubRecords = kTile;
 
 __global__ __launch_bounds__(1024) void csx_plan_subblocks(const int32_t *__restrict__ table, int nblocks,
                                                            int nbuckets, int max_sub,
@@ -256,20 +354,37 @@ __global__ __launch_bounds__(1024) void csx_plan_subblocks(const int32_t *__rest
                                                            int32_t *__restrict__ sub_first)
 {
     __shared__ int first[kMaxBins + 1];
-    for (int b = threadIdx.x; b < nbuckets; b += 1024) {
-        const int size = table[(int64_t)(b + 1) * nblocks] - table[(int64_t)b * nblocks];
-        first[b] = size <= kSubRecords ? 1 : (size + kSubRecords - 1) / kSubRecords;
-    }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        int run = 0;
-        for (int b = 0; b < nbuckets; b++) {
-            const int n = first[b];
-            first[b] = run;
-            run += n;
+    __shared__ int wave_tot[16];
+    // thread t owns buckets 2t and 2t+1
+    int n[2], mysum = 0;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int b = 2 * threadIdx.x + i;
+        n[i] = 0;
+        if (b < nbuckets) {
+            const int size = table[(int64_t)(b + 1) * nblocks] - table[(int64_t)b * nblocks];
+            n[i] = size <= kSubRecords ? 1 : (size + kSubRecords - 1) / kSubRecords;
         }
-        first[nbuckets] = run;
+        mysum += n[i];
     }
+    int inc = mysum;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        const int t = __shfl_up(inc, d, kWave);
+        if (lane_id() >= d) inc += t;
+    }
+    const int w = threadIdx.x >> 6;
+    if (lane_id() == kWave - 1) wave_tot[w] = inc;
+    __syncthreads();
+    int run = inc - mysum;
+    for (int v = 0; v < w; v++) run += wave_tot[v];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int b = 2 * threadIdx.x + i;
+        if (b < nbuckets) first[b] = run;
+        run += n[i];
+    }
+    if (threadIdx.x == 1023) first[nbuckets] = run;   // buckets past the last count 0: the total
     __syncthreads();
     for (int b = threadIdx.x; b <= nbuckets; b += 1024) sub_first[b] = first[b];
     for (int b = threadIdx.x; b < nbuckets; b += 1024)
@@ -345,12 +460,10 @@ __global__ __launch_bounds__(kPartThreads) void csx_bucket_offsets(const int32_t
     for (int kb = 0; kb < nkeys; kb += kPartThreads) {
         const int k = kb + threadIdx.x;
         int total = 0;
-        if (k < nkeys)
-            for (int s = s0; s < s1; s++) {
-                const int c = cnt2[(int64_t)s * nkeys + k];
-                cnt2[(int64_t)s * nkeys + k] = total;
-                total += c;
-            }
+        if (k < nkeys) {
+#pragma unroll 8
+            for (int s = s0; s < s1; s++) total += cnt2[(int64_t)s * nkeys + k];
+        }
         // block-exclusive scan of `total` in key order
         int inc = total;
 #pragma unroll
@@ -366,7 +479,13 @@ __global__ __launch_bounds__(kPartThreads) void csx_bucket_offsets(const int32_t
         const int key_base = before + inc - total;
         if (k < nkeys) {
             if (k0 + k < V) off[k0 + k] = key_base;
-            for (int s = s0; s < s1; s++) cnt2[(int64_t)s * nkeys + k] += key_base;
+            int run = key_base;
+#pragma unroll 8
+            for (int s = s0; s < s1; s++) {
+                const int c = cnt2[(int64_t)s * nkeys + k];
+                cnt2[(int64_t)s * nkeys + k] = run;
+                run += c;
+            }
         }
         __syncthreads();
         if (threadIdx.x == kPartThreads - 1) carry = key_base + total;
@@ -376,8 +495,8 @@ __global__ __launch_bounds__(kPartThreads) void csx_bucket_offsets(const int32_t
 }
 
 // ---------------------------------------------------------------- step 7 ---
-// One block per sub-block: chunks of kTile records are ranked in order;
-// cursor[] (LDS) carries each key's next free slot from one chunk to the next.
+// One block per sub-block (one tile of records): sorted by key inside LDS,
+// then every key's run goes to cnt2[sub][key] onwards.
 template <typename Rec, bool PERM>
 __global__ __launch_bounds__(kPartThreads) void csx_sub_scatter(const Rec *__restrict__ recs,
                                                                 const int32_t *__restrict__ table, int nblocks,
@@ -386,38 +505,28 @@ __global__ __launch_bounds__(kPartThreads) void csx_sub_scatter(const Rec *__res
                                                                 const int32_t *__restrict__ cnt2, int shift,
                                                                 int32_t *__restrict__ out_idx,
                                                                 uint32_t *__restrict__ out_w,
-                                                                int32_t *__restrict__ out_perm)
+                                                                int32_t *__restrict__ out_perm, int stage_n)
 {
-    extern __shared__ int lds[];
-    const SubRange sr = sub_range(table, nblocks, sub_bucket, sub_first, blockIdx.x);
+    extern __shared__ uint32_t lds_raw[];
+    const int sub = blockIdx.x;
+    const SubRange sr = sub_range(table, nblocks, sub_bucket, sub_first, sub);
     if (sr.bucket < 0) return;
-    const int nkeys = 1 << shift;
-    int *cursor = lds;               // [nkeys]
-    int *cnt = lds + nkeys;          // [kPartWaves][nkeys]
-    for (int k = threadIdx.x; k < nkeys; k += kPartThreads) cursor[k] = cnt2[(int64_t)blockIdx.x * nkeys + k];
-    __syncthreads();
-    const int w = threadIdx.x >> 6;
-    const int mask = nkeys - 1;
-    for (int chunk = sr.begin; chunk < sr.end; chunk += kTile) {
-        const int base = chunk + w * kWaveSpan + lane_id();
-        Rec rec[kItems];
-        int bin[kItems], pos[kItems];
+    const int nkeys = 1 << shift, mask = nkeys - 1;
+    const int base = sr.begin + (threadIdx.x >> 6) * kWaveSpan + lane_id();
+    Rec rec[kItems];
+    int bin[kItems], lp[kItems];
 #pragma unroll
-        for (int r = 0; r < kItems; r++) rec[r] = recs[min(base + r * kWave, sr.end - 1)];
+    for (int r = 0; r < kItems; r++) rec[r] = recs[min(base + r * kWave, sr.end - 1)];
 #pragma unroll
-        for (int r = 0; r < kItems; r++) bin[r] = base + r * kWave < sr.end ? (rec[r].key & mask) : -1;
-        tile_rank(
-            cnt, nkeys, shift, bin, pos, [&](int b) { return cursor[b]; },
-            [&](int b, int next) { cursor[b] = next; });
-#pragma unroll
-        for (int r = 0; r < kItems; r++)
-            if (bin[r] >= 0) {
-                out_idx[pos[r]] = rec[r].other;
-                if (out_w) out_w[pos[r]] = rec[r].w;
-                if (PERM) out_perm[pos[r]] = get_id(rec[r]);
-            }
-        __syncthreads();
-    }
+    for (int r = 0; r < kItems; r++) bin[r] = base + r * kWave < sr.end ? (rec[r].key & mask) : -1;
+    TileLds L;
+    const int total = tile_sort<Rec>(lds_raw, stage_n, L, nkeys, shift, bin, lp,
+                                     [&](int k) { return cnt2[(int64_t)sub * nkeys + k]; });
+    tile_emit(L, total, 0, mask, rec, bin, lp, [&](int pos, const Rec &q) {
+        out_idx[pos] = q.other;
+        if (out_w) out_w[pos] = q.w;
+        if (PERM) out_perm[pos] = get_id(q);
+    });
 }
 
 // Expands compressed offsets into one row id per entry (for the transpose).
@@ -517,7 +626,8 @@ static int32_t convert(const int32_t *keys, const int32_t *others, const float *
         // V > 2^22: LSD passes over 11-bit digits; sub_first doubles as the record count
         Rec *bufs[2] = {recs, carve.take<Rec>((size_t)E)};
         int32_t *count = sub_first;
-        const size_t lds = (size_t)kPartWaves * kMaxBins * sizeof(int);
+        const size_t lds = tile_lds_bytes(kMaxBins, sizeof(Rec));
+        const int stage_n = tile_stage_records(kMaxBins, sizeof(Rec));
         for (int d = 0; d < p.digits; d++) {
             const int shift = d * kMaxBinBits;
             Rec *dst = bufs[d & 1];
@@ -530,7 +640,7 @@ static int32_t convert(const int32_t *keys, const int32_t *others, const float *
                 auto part = csx_partition<Rec, CooLoader<Rec>>;
                 allow_lds(part, lds);
                 hipLaunchKernelGGL(part, dim3(nb), dim3(kPartThreads), lds, s, in, shift, kMaxBins - 1, kMaxBins,
-                                   kMaxBinBits, table, nblk, dst);
+                                   kMaxBinBits, table, nblk, dst, stage_n);
             } else {
                 RecLoader<Rec> in{bufs[(d - 1) & 1], count, E};
                 hipLaunchKernelGGL((csx_digit_histogram<Rec, RecLoader<Rec>>), dim3(nb), dim3(kPartThreads), 0, s, in,
@@ -539,7 +649,7 @@ static int32_t convert(const int32_t *keys, const int32_t *others, const float *
                 auto part = csx_partition<Rec, RecLoader<Rec>>;
                 allow_lds(part, lds);
                 hipLaunchKernelGGL(part, dim3(nb), dim3(kPartThreads), lds, s, in, shift, kMaxBins - 1, kMaxBins,
-                                   kMaxBinBits, table, nblk, dst);
+                                   kMaxBinBits, table, nblk, dst, stage_n);
             }
         }
         hipLaunchKernelGGL((csx_unpack_sorted<Rec, PERM>), dim3((unsigned)ceil_div(E + 1, 256)), dim3(256), 0, s,
@@ -556,10 +666,10 @@ static int32_t convert(const int32_t *keys, const int32_t *others, const float *
 
     CooLoader<Rec> in{keys, others, reinterpret_cast<const uint32_t *>(w), E, V};
     auto part = csx_partition<Rec, CooLoader<Rec>>;
-    const size_t part_lds = (size_t)kPartWaves * p.nbuckets * sizeof(int);
+    const size_t part_lds = tile_lds_bytes(p.nbuckets, sizeof(Rec));
     allow_lds(part, part_lds);
     hipLaunchKernelGGL(part, dim3(nb), dim3(kPartThreads), part_lds, s, in, p.shift, 0x7fffffff, p.nbuckets, bbits,
-                       table, nblk, recs);
+                       table, nblk, recs, tile_stage_records(p.nbuckets, sizeof(Rec)));
 
     hipLaunchKernelGGL(csx_plan_subblocks, dim3(1), dim3(1024), 0, s, table, nblk, p.nbuckets, p.max_sub, sub_bucket,
                        sub_first);
@@ -569,10 +679,11 @@ static int32_t convert(const int32_t *keys, const int32_t *others, const float *
                        p.nbuckets, sub_first, p.shift, V, cnt2, out_off);
     const int nkeys = 1 << p.shift;
     auto scat = csx_sub_scatter<Rec, PERM>;
-    const size_t scat_lds = (size_t)(kPartWaves + 1) * nkeys * sizeof(int);
+    const size_t scat_lds = tile_lds_bytes(nkeys, sizeof(Rec));
     allow_lds(scat, scat_lds);
     hipLaunchKernelGGL(scat, dim3((unsigned)p.max_sub), dim3(kPartThreads), scat_lds, s, recs, table, nblk,
-                       sub_bucket, sub_first, cnt2, p.shift, out_idx, reinterpret_cast<uint32_t *>(out_w), out_perm);
+                       sub_bucket, sub_first, cnt2, p.shift, out_idx, reinterpret_cast<uint32_t *>(out_w), out_perm,
+                       tile_stage_records(nkeys, sizeof(Rec)));
     return launch_status("coo_to_csx");
 }
 
