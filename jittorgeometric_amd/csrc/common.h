@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 #include <stddef.h>
 #include <stdint.h>
+#include <string.h>
 
 #include "../../include/jgamd.h"
 
@@ -43,6 +44,13 @@ int32_t exclusive_scan_i32(const int32_t *in, int32_t *out, int64_t n, int32_t *
 size_t spmm_ws_bytes(int32_t R, int64_t E, int32_t F);
 int32_t spmm_enqueue(const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out, int32_t R,
                      int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, hipStream_t s);
+
+// ---- tile-based edge softmax for 1, 2, 4 or 8 heads (edge_softmax_flat.hip) --
+// fwd: a = x, b unused; bwd: a = y, b = g.  Needs V > 0, E > 0, off[V] == E.
+bool edge_softmax_flat_supported(int H);
+size_t edge_softmax_flat_ws_bytes(int64_t E);
+void edge_softmax_flat_enqueue(bool fwd, const int32_t *off, const float *a, const float *b, float *out, int32_t V,
+                               int64_t E, int32_t H, void *ws, hipStream_t s);
 
 #ifdef __HIPCC__
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }

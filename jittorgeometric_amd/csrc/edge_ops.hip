@@ -341,7 +341,14 @@ static int long_capacity(int32_t V, int64_t E)
     const int64_t c = E / kLongColumn + 1;
     return (int)(c < (int64_t)V ? c : (int64_t)V);
 }
-static size_t softmax_ws_bytes(int32_t V, int64_t E) { return 256 + carve_bytes((size_t)long_capacity(V, E), 4); }
+static size_t group_ws_bytes(int32_t V, int64_t E) { return 256 + carve_bytes((size_t)long_capacity(V, E), 4); }
+static size_t softmax_ws_bytes(int32_t V, int64_t E) { return group_ws_bytes(V, E) + edge_softmax_flat_ws_bytes(E); }
+// JGAMD_SOFTMAX=groups keeps the lane-group-per-column kernels for 1-8 heads too
+static bool use_flat(int H)
+{
+    const char *e = getenv("JGAMD_SOFTMAX");
+    return edge_softmax_flat_supported(H) && !(e && strcmp(e, "groups") == 0);
+}
 
 static int32_t check_softmax_ws(const char *who, const void *ws, size_t have, int32_t V, int64_t E)
 {
@@ -384,6 +391,10 @@ JG_EXPORT int32_t jgamd_edge_softmax_fwd(const int32_t *off, const float *x, flo
         return launch_status("edge_softmax_fwd");
     }
     if (int32_t rc = check_softmax_ws("edge_softmax_fwd", ws, ws_bytes, V, E)) return rc;
+    if (use_flat(H)) {
+        edge_softmax_flat_enqueue(true, off, x, nullptr, y, V, E, H, static_cast<char *>(ws) + group_ws_bytes(V, E), s);
+        return launch_status("edge_softmax_fwd");
+    }
     switch (pick_group(E, V, H)) {
     case 1: case 2: case 4: launch_groups(edge_softmax_fwd_k<4>, 4, V, s, off, x, y, V, H); break;
     case 8: launch_groups(edge_softmax_fwd_k<8>, 8, V, s, off, x, y, V, H); break;
@@ -410,6 +421,10 @@ JG_EXPORT int32_t jgamd_edge_softmax_bwd(const int32_t *off, const float *y, con
         return launch_status("edge_softmax_bwd");
     }
     if (int32_t rc = check_softmax_ws("edge_softmax_bwd", ws, ws_bytes, V, E)) return rc;
+    if (use_flat(H)) {
+        edge_softmax_flat_enqueue(false, off, y, g, dx, V, E, H, static_cast<char *>(ws) + group_ws_bytes(V, E), s);
+        return launch_status("edge_softmax_bwd");
+    }
     switch (pick_group(E, V, H)) {
     case 1: case 2: case 4: launch_groups(edge_softmax_bwd_k<4>, 4, V, s, off, y, g, dx, V, H); break;
     case 8: launch_groups(edge_softmax_bwd_k<8>, 8, V, s, off, y, g, dx, V, H); break;

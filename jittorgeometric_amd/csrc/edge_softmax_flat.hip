@@ -1,0 +1,696 @@
+// Edge softmax over fixed tiles of entries, for H in {1, 2, 4, 8} heads.
+//
+// The reference (ops/cpp/edgesoftmax_op.cc:48-65, edgesoftmaxbackward_op.cc:45-51)
+// walks every destination column three times.  Columns of a power-law graph
+// run from one entry to millions, so here the unit of work is not a column
+// but a tile of T consecutive entries of the [E,H] array:
+//
+//   1. tile kernel  : a lane holds K consecutive entries (all H heads, loaded
+//                     as vectors).  Each entry's column is found from the
+//                     offsets staged in LDS; per-column totals (max, then sum
+//                     of exp; or sum of y*g) come from a lane-local reduction
+//                     over runs of equal columns plus one segmented scan over
+//                     the block's lanes, in a fixed order (no float atomics).
+//                     Columns that lie inside the tile are finished from
+//                     registers: x is read once, y written once.  A column
+//                     that crosses a tile edge leaves a piece per tile.
+//   2. merge kernel : one wavefront per column that crosses tile edges folds
+//                     its pieces (tail piece of the tile it starts in, then
+//                     the head pieces of the following tiles).
+//   3. finish kernel: the entries of crossing columns are computed from the
+//                     inputs with the merged totals.
+//
+// A column's slot in a tile is the position of its first entry inside the
+// tile (0 for the column that began in an earlier tile), so slots are unique
+// and below T.
+#include "common.h"
+
+namespace jg {
+
+constexpr int kFlatThreads = 256;
+constexpr int kFlatWaves = kFlatThreads / kWave;
+
+template <int H> struct FlatShape {
+    static constexpr int K = H <= 2 ? 8 : 4;        // entries per lane
+    static constexpr int T = kFlatThreads * K;      // entries per tile
+};
+
+struct FlatMeta {
+    int head_open;   // the tile's first column began in an earlier tile
+    int head_cs, head_ce;
+    int tail_open;   // the tile's last column continues in the next tile
+    int tail_cs, tail_ce;
+    int pad0, pad1;
+};
+
+// The tile's T*H floats pass through LDS twice: loaded with consecutive lanes
+// on consecutive 16-byte vectors (whole cache lines per instruction), read
+// back as K*H consecutive floats per lane, and the other way round for the
+// result.  Four floats of padding per 32 keep the per-lane reads off each
+// other's banks.  The same memory then holds the per-column totals.
+__host__ __device__ constexpr int flat_pad(int f) { return f + (f >> 5) * 4; }
+
+template <int H, int T> struct FlatLds {
+    int off[T + 2];
+    __attribute__((aligned(16))) float tot[flat_pad(T * H)];
+    float carry[kFlatWaves * H];
+    int wflag[kFlatWaves];
+    int wlast[kFlatWaves];
+    int wfirst[kFlatWaves];
+};
+
+struct OpMax {
+    __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); }
+};
+struct OpAdd {
+    __device__ __forceinline__ float operator()(float a, float b) const { return a + b; }
+};
+
+// tile_first[i] / tile_last[i] = column of the first / last entry of tile i.
+// One thread per column: it owns the entries [off[c], off[c+1]) and marks the
+// tiles whose first or last entry falls among them.
+__global__ void esm_tile_columns(const int32_t *__restrict__ off, int V, int E, int T, int ntiles,
+                                 int32_t *__restrict__ tile_first, int32_t *__restrict__ tile_last)
+{
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= V) return;
+    const int s = off[c], e = min(off[c + 1], E);
+    if (e <= s) return;
+    for (int i = (s + T - 1) / T; i < ntiles && (int64_t)i * T < e; i++) tile_first[i] = c;
+    for (int i = s / T + 1; i <= ntiles && (int64_t)i * T <= e; i++) tile_last[i - 1] = c;   // last entry i*T - 1
+    if (e == E) tile_last[ntiles - 1] = c;
+}
+
+// What a tile knows about its entries' columns.
+template <int K> struct LaneColumns {
+    int slot[K];
+    unsigned closed;   // bit k: entry k is valid and its column lies inside the tile
+    int tail_slot;     // slot of the tile's last column
+    int closed_lo, closed_hi;   // the valid entries of columns inside the tile, relative to t0
+};
+
+// Stages the offsets of the tile's columns [c_lo, c_hi] and resolves the column
+// of each of this lane's K entries (entries past the tile's end take the
+// column of the tile's last entry).  Thread 0 records the tile's metadata.
+template <int H, int K, int T>
+__device__ __forceinline__ void resolve_columns(const int32_t *__restrict__ off, int c_lo, int c_hi, int t0, int n,
+                                                FlatLds<H, T> &L, LaneColumns<K> &cols, FlatMeta *meta_out)
+{
+    const int ncol = c_hi - c_lo + 1;
+    const bool staged = ncol + 1 <= T + 2;
+    if (staged)
+        for (int i = threadIdx.x; i <= ncol; i += kFlatThreads) L.off[i] = off[c_lo + i];
+    __syncthreads();
+    auto offv = [&](int c) { return staged ? L.off[c - c_lo] : off[c]; };
+    const int last = t0 + n - 1;
+    const int j0 = t0 + threadIdx.x * K;
+    const int jc = min(j0, last);
+    int lo = c_lo, hi = c_hi;
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (offv(mid) <= jc) lo = mid;
+        else hi = mid - 1;
+    }
+    int c = lo, cs = offv(c), ce = offv(c + 1);
+    cols.closed = 0;
+#pragma unroll
+    for (int k = 0; k < K; k++) {
+        const int j = min(j0 + k, last);
+        while (ce <= j && c < c_hi) {      // c < c_hi only matters if off[V] != E
+            c++;
+            cs = ce;
+            ce = offv(c + 1);
+        }
+        cols.slot[k] = max(cs - t0, 0);
+        if (j0 + k <= last && cs >= t0 && ce <= t0 + n) cols.closed |= 1u << k;
+    }
+    cols.tail_slot = max(offv(c_hi) - t0, 0);
+    cols.closed_lo = offv(c_lo) < t0 ? min(offv(c_lo + 1) - t0, n) : 0;
+    cols.closed_hi = offv(c_hi + 1) > t0 + n ? max(offv(c_hi) - t0, cols.closed_lo) : n;
+    if (threadIdx.x == 0) {
+        FlatMeta m;
+        m.head_cs = offv(c_lo);
+        m.head_ce = offv(c_lo + 1);
+        m.head_open = m.head_cs < t0;
+        m.tail_cs = offv(c_hi);
+        m.tail_ce = offv(c_hi + 1);
+        m.tail_open = m.tail_ce > t0 + n;
+        m.pad0 = m.pad1 = 0;
+        *meta_out = m;
+    }
+}
+
+// One step of an inclusive segmented scan over the wavefront: lanes that the
+// move reaches and that have seen no segment start yet fold the moved value in.
+// CTRL: row_shr:n = 0x110+n, row_bcast:15 = 0x142, row_bcast:31 = 0x143; lanes
+// without a source (or outside ROWS) receive the identity and no flag.
+template <int CTRL, int ROWS, int H, typename Op>
+__device__ __forceinline__ void seg_scan_step(float (&v)[H], int &fl, Op op, float ident)
+{
+    const int fu = __builtin_amdgcn_update_dpp(0, fl, CTRL, ROWS, 0xf, false);
+#pragma unroll
+    for (int h = 0; h < H; h++) {
+        const float up = __int_as_float(
+            __builtin_amdgcn_update_dpp(__float_as_int(ident), __float_as_int(v[h]), CTRL, ROWS, 0xf, false));
+        v[h] = fl ? v[h] : op(up, v[h]);
+    }
+    fl |= fu;
+}
+
+// The H totals of one slot.
+template <int H> __device__ __forceinline__ void read_totals(const float *tot, int slot, float (&t)[H])
+{
+    if constexpr (H >= 4) {
+#pragma unroll
+        for (int q = 0; q < H / 4; q++) {
+            const float4 v = *reinterpret_cast<const float4 *>(tot + slot * H + 4 * q);
+            t[4 * q] = v.x;
+            t[4 * q + 1] = v.y;
+            t[4 * q + 2] = v.z;
+            t[4 * q + 3] = v.w;
+        }
+    } else if constexpr (H == 2) {
+        const float2 v = *reinterpret_cast<const float2 *>(tot + slot * 2);
+        t[0] = v.x;
+        t[1] = v.y;
+    } else {
+        t[0] = tot[slot];
+    }
+}
+
+// Per-column totals of val over the tile -> L.tot[slot*H + h].  Entries that
+// do not count must hold the identity.  Starts and ends with a barrier.
+template <int H, int K, int T, typename Op>
+__device__ __forceinline__ void segment_totals(const float (&val)[K][H], const int (&slot)[K], FlatLds<H, T> &L, Op op,
+                                               float ident)
+{
+    const int lane = lane_id();
+    const int w = threadIdx.x >> 6;
+    __syncthreads();
+    // runs of equal columns inside the lane: the first and the last may go on
+    // in the neighbouring lanes, the ones between are complete
+    float acc[H], headv[H];
+    bool multi = false;
+#pragma unroll
+    for (int h = 0; h < H; h++) acc[h] = val[0][h];
+#pragma unroll
+    for (int k = 1; k < K; k++) {
+        if (slot[k] != slot[k - 1]) {
+            if (!multi) {
+#pragma unroll
+                for (int h = 0; h < H; h++) headv[h] = acc[h];
+                multi = true;
+            } else {
+#pragma unroll
+                for (int h = 0; h < H; h++) L.tot[slot[k - 1] * H + h] = acc[h];
+            }
+#pragma unroll
+            for (int h = 0; h < H; h++) acc[h] = val[k][h];
+        } else {
+#pragma unroll
+            for (int h = 0; h < H; h++) acc[h] = op(acc[h], val[k][h]);
+        }
+    }
+    if (!multi) {
+#pragma unroll
+        for (int h = 0; h < H; h++) headv[h] = acc[h];
+    }
+    const int firstslot = slot[0], lastslot = slot[K - 1];
+    if (lane == kWave - 1) L.wlast[w] = lastslot;
+    if (lane == 0) L.wfirst[w] = firstslot;
+    __syncthreads();
+    int prevlast = __shfl_up(lastslot, 1, kWave);
+    if (lane == 0) prevlast = w > 0 ? L.wlast[w - 1] : -1;
+    int nextfirst = __shfl_down(firstslot, 1, kWave);
+    if (lane == kWave - 1) nextfirst = w < kFlatWaves - 1 ? L.wfirst[w + 1] : -2;
+    // inclusive segmented scan of the last runs: a lane starts a new segment
+    // if a column begins inside it or at its first entry
+    int fl = (multi || firstslot != prevlast) ? 1 : 0;
+    float v[H];
+#pragma unroll
+    for (int h = 0; h < H; h++) v[h] = acc[h];
+    // rows of 16 lanes with row shifts, then lane 15 -> next row (rows 1, 3)
+    // and lane 31 -> rows 2, 3: all data-parallel moves on the vector ALU
+    // (a step changes nothing once every lane has seen a segment start)
+    seg_scan_step<0x111, 0xf>(v, fl, op, ident);
+    seg_scan_step<0x112, 0xf>(v, fl, op, ident);
+    if (__ballot(fl == 0)) {
+        seg_scan_step<0x114, 0xf>(v, fl, op, ident);
+        seg_scan_step<0x118, 0xf>(v, fl, op, ident);
+        if (__ballot(fl == 0)) {
+            seg_scan_step<0x142, 0xa>(v, fl, op, ident);
+            seg_scan_step<0x143, 0xc>(v, fl, op, ident);
+        }
+    }
+    if (lane == kWave - 1) {
+#pragma unroll
+        for (int h = 0; h < H; h++) L.carry[w * H + h] = v[h];
+        L.wflag[w] = fl;
+    }
+    __syncthreads();
+    float carry[H];
+#pragma unroll
+    for (int h = 0; h < H; h++) carry[h] = ident;
+    for (int u = 0; u < w; u++) {
+        const bool cut = L.wflag[u] != 0;
+#pragma unroll
+        for (int h = 0; h < H; h++) carry[h] = cut ? L.carry[u * H + h] : op(carry[h], L.carry[u * H + h]);
+    }
+#pragma unroll
+    for (int h = 0; h < H; h++) {
+        if (!fl) v[h] = op(carry[h], v[h]);
+        // total of the previous lane's last column up to that lane
+        float prev = __shfl_up(v[h], 1, kWave);
+        if (lane == 0) prev = carry[h];
+        if (multi) L.tot[firstslot * H + h] = firstslot == prevlast ? op(prev, headv[h]) : headv[h];
+        if (nextfirst != lastslot) L.tot[lastslot * H + h] = v[h];
+    }
+    __syncthreads();
+}
+
+template <int N> struct __attribute__((aligned(16))) FloatVec {
+    float f[N];
+};
+
+// Lane's K*H consecutive floats starting at entry j0: one vector access when
+// the arrays are 16-byte aligned and the lane is inside the array, else
+// element by element with the entry index clamped.
+template <int H, int K>
+__device__ __forceinline__ void load_lane(const float *__restrict__ a, bool aligned, int j0, int E, float (&v)[K][H])
+{
+    if (aligned && j0 + K <= E) {
+        const FloatVec<K * H> t = *reinterpret_cast<const FloatVec<K * H> *>(a + (int64_t)j0 * H);
+#pragma unroll
+        for (int k = 0; k < K; k++)
+#pragma unroll
+            for (int h = 0; h < H; h++) v[k][h] = t.f[k * H + h];
+    } else {
+#pragma unroll
+        for (int k = 0; k < K; k++) {
+            const int64_t j = min(j0 + k, E - 1);
+#pragma unroll
+            for (int h = 0; h < H; h++) v[k][h] = a[j * H + h];
+        }
+    }
+}
+
+template <int H, int K>
+__device__ __forceinline__ void store_lane(float *__restrict__ a, bool aligned, int j0, unsigned mask,
+                                           const float (&v)[K][H])
+{
+    if (aligned && mask == (1u << K) - 1) {
+        FloatVec<K * H> t;
+#pragma unroll
+        for (int k = 0; k < K; k++)
+#pragma unroll
+            for (int h = 0; h < H; h++) t.f[k * H + h] = v[k][h];
+        *reinterpret_cast<FloatVec<K * H> *>(a + (int64_t)j0 * H) = t;
+    } else {
+#pragma unroll
+        for (int k = 0; k < K; k++)
+            if (mask >> k & 1) {
+#pragma unroll
+                for (int h = 0; h < H; h++) a[(int64_t)(j0 + k) * H + h] = v[k][h];
+            }
+    }
+}
+
+// Tile [t0, t0+T) of a[E][H] -> v, through LDS (see FlatLds).  Needs a 16-byte
+// aligned array; positions past the array's end repeat its last element.
+// Ends with the lanes' reads still in flight on `buf`: a barrier must follow
+// before buf is written again.
+template <int H, int K>
+__device__ __forceinline__ void load_tile(const float *__restrict__ a, int t0, int E, float *buf, float (&v)[K][H])
+{
+    constexpr int NV = K * H / 4;
+    const int64_t total = (int64_t)E * H;
+    float4 q[NV];
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int f = (i * kFlatThreads + threadIdx.x) * 4;
+        const int64_t g = (int64_t)t0 * H + f;
+        if (g + 4 <= total) {
+            q[i] = *reinterpret_cast<const float4 *>(a + g);
+        } else {
+            q[i].x = a[min(g, total - 1)];
+            q[i].y = a[min(g + 1, total - 1)];
+            q[i].z = a[min(g + 2, total - 1)];
+            q[i].w = a[min(g + 3, total - 1)];
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int f = (i * kFlatThreads + threadIdx.x) * 4;
+        *reinterpret_cast<float4 *>(buf + flat_pad(f)) = q[i];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const float4 t = *reinterpret_cast<const float4 *>(buf + flat_pad((int)threadIdx.x * K * H + 4 * i));
+        const float c[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+        for (int j = 0; j < 4; j++) v[(4 * i + j) / H][(4 * i + j) % H] = c[j];
+    }
+}
+
+// v -> out for the entries [lo, hi) of the tile (relative to t0), through LDS.
+// Starts with a barrier (buf may still be read as totals).
+template <int H, int K>
+__device__ __forceinline__ void store_tile(float *__restrict__ out, int t0, int lo, int hi, float *buf,
+                                           const float (&v)[K][H])
+{
+    constexpr int NV = K * H / 4;
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        float4 t;
+        t.x = v[(4 * i) / H][(4 * i) % H];
+        t.y = v[(4 * i + 1) / H][(4 * i + 1) % H];
+        t.z = v[(4 * i + 2) / H][(4 * i + 2) % H];
+        t.w = v[(4 * i + 3) / H][(4 * i + 3) % H];
+        *reinterpret_cast<float4 *>(buf + flat_pad((int)threadIdx.x * K * H + 4 * i)) = t;
+    }
+    __syncthreads();
+    const int flo = lo * H, fhi = hi * H;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int f = (i * kFlatThreads + threadIdx.x) * 4;
+        const float4 t = *reinterpret_cast<const float4 *>(buf + flat_pad(f));
+        float *dst = out + (int64_t)t0 * H + f;
+        if (f >= flo && f + 4 <= fhi) {
+            *reinterpret_cast<float4 *>(dst) = t;
+        } else {
+            if (f >= flo && f < fhi) dst[0] = t.x;
+            if (f + 1 >= flo && f + 1 < fhi) dst[1] = t.y;
+            if (f + 2 >= flo && f + 2 < fhi) dst[2] = t.z;
+            if (f + 3 >= flo && f + 3 < fhi) dst[3] = t.w;
+        }
+    }
+}
+
+__device__ __forceinline__ bool both_aligned(const void *a, const void *b)
+{
+    return (((uintptr_t)a | (uintptr_t)b) & 15) == 0;
+}
+
+// pieces: [ntiles][2][2H] floats; index 0 = head column, 1 = tail column;
+// forward: H maxima then H sums (relative to those maxima); backward: H sums.
+template <int H> __device__ __forceinline__ float *piece(float *pieces, int tile, int which)
+{
+    return pieces + ((int64_t)tile * 2 + which) * 2 * H;
+}
+
+template <int H>
+__global__ __launch_bounds__(kFlatThreads) void esm_fwd_tile(const int32_t *__restrict__ off,
+                                                             const float *__restrict__ x, float *__restrict__ y,
+                                                             const int32_t *__restrict__ tile_first,
+                                                             const int32_t *__restrict__ tile_last, int V, int E,
+                                                             FlatMeta *__restrict__ meta, float *__restrict__ pieces,
+                                                             int staged)
+{
+    constexpr int K = FlatShape<H>::K, T = FlatShape<H>::T;
+    __shared__ FlatLds<H, T> L;
+    const int tile = blockIdx.x;
+    // the clamps only matter if off[] and E disagree (tiles no column claimed)
+    const int c_lo = min(max(tile_first[tile], 0), V - 1);
+    const int c_hi = min(max(tile_last[tile], c_lo), V - 1);
+    const int t0 = tile * T;
+    const int n = min(T, E - t0);
+    const int j0 = t0 + threadIdx.x * K;
+    const bool aligned = both_aligned(x, y);
+    const bool through_lds = aligned && staged;
+    float v[K][H];
+    if (through_lds) load_tile<H, K>(x, t0, E, L.tot, v);
+    else load_lane<H, K>(x, aligned, j0, E, v);
+    LaneColumns<K> cols;
+    resolve_columns<H, K, T>(off, c_lo, c_hi, t0, n, L, cols, meta + tile);
+#pragma unroll
+    for (int k = 0; k < K; k++)
+        if (j0 + k >= t0 + n) {
+#pragma unroll
+            for (int h = 0; h < H; h++) v[k][h] = -INFINITY;
+        }
+    segment_totals<H, K, T>(v, cols.slot, L, OpMax(), -INFINITY);
+    const int tail_slot = cols.tail_slot;
+    if (threadIdx.x < H) {
+        piece<H>(pieces, tile, 0)[threadIdx.x] = L.tot[threadIdx.x];
+        piece<H>(pieces, tile, 1)[threadIdx.x] = L.tot[tail_slot * H + threadIdx.x];
+    }
+#pragma unroll
+    for (int k = 0; k < K; k++) {
+        float m[H];
+        read_totals<H>(L.tot, cols.slot[k], m);
+#pragma unroll
+        for (int h = 0; h < H; h++) v[k][h] = j0 + k < t0 + n ? __expf(v[k][h] - m[h]) : 0.f;
+    }
+    segment_totals<H, K, T>(v, cols.slot, L, OpAdd(), 0.f);
+    if (threadIdx.x < H) {
+        piece<H>(pieces, tile, 0)[H + threadIdx.x] = L.tot[threadIdx.x];
+        piece<H>(pieces, tile, 1)[H + threadIdx.x] = L.tot[tail_slot * H + threadIdx.x];
+    }
+#pragma unroll
+    for (int k = 0; k < K; k++) {
+        float t[H];
+        read_totals<H>(L.tot, cols.slot[k], t);
+#pragma unroll
+        for (int h = 0; h < H; h++) v[k][h] = v[k][h] * __frcp_rn(t[h]);
+    }
+    if (through_lds) store_tile<H, K>(y, t0, cols.closed_lo, cols.closed_hi, L.tot, v);
+    else store_lane<H, K>(y, aligned, j0, cols.closed, v);
+}
+
+template <int H>
+__global__ __launch_bounds__(kFlatThreads) void esm_bwd_tile(const int32_t *__restrict__ off,
+                                                             const float *__restrict__ y, const float *__restrict__ g,
+                                                             float *__restrict__ dx,
+                                                             const int32_t *__restrict__ tile_first,
+                                                             const int32_t *__restrict__ tile_last, int V, int E,
+                                                             FlatMeta *__restrict__ meta, float *__restrict__ pieces,
+                                                             int staged)
+{
+    constexpr int K = FlatShape<H>::K, T = FlatShape<H>::T;
+    __shared__ FlatLds<H, T> L;
+    const int tile = blockIdx.x;
+    // the clamps only matter if off[] and E disagree (tiles no column claimed)
+    const int c_lo = min(max(tile_first[tile], 0), V - 1);
+    const int c_hi = min(max(tile_last[tile], c_lo), V - 1);
+    const int t0 = tile * T;
+    const int n = min(T, E - t0);
+    const int j0 = t0 + threadIdx.x * K;
+    const bool aligned = both_aligned(y, g) && ((uintptr_t)dx & 15) == 0;
+    const bool through_lds = aligned && staged;
+    float yv[K][H], yg[K][H];
+    if (through_lds) {
+        load_tile<H, K>(y, t0, E, L.tot, yv);
+        __syncthreads();
+        load_tile<H, K>(g, t0, E, L.tot, yg);
+    } else {
+        load_lane<H, K>(y, aligned, j0, E, yv);
+        load_lane<H, K>(g, aligned, j0, E, yg);
+    }
+    LaneColumns<K> cols;
+    resolve_columns<H, K, T>(off, c_lo, c_hi, t0, n, L, cols, meta + tile);
+#pragma unroll
+    for (int k = 0; k < K; k++)
+#pragma unroll
+        for (int h = 0; h < H; h++) yg[k][h] = j0 + k < t0 + n ? yv[k][h] * yg[k][h] : 0.f;
+    segment_totals<H, K, T>(yg, cols.slot, L, OpAdd(), 0.f);
+    const int tail_slot = cols.tail_slot;
+    if (threadIdx.x < H) {
+        piece<H>(pieces, tile, 0)[threadIdx.x] = L.tot[threadIdx.x];
+        piece<H>(pieces, tile, 1)[threadIdx.x] = L.tot[tail_slot * H + threadIdx.x];
+    }
+#pragma unroll
+    for (int k = 0; k < K; k++) {
+        float t[H];
+        read_totals<H>(L.tot, cols.slot[k], t);
+#pragma unroll
+        for (int h = 0; h < H; h++) yg[k][h] = yg[k][h] - yv[k][h] * t[h];
+    }
+    if (through_lds) store_tile<H, K>(dx, t0, cols.closed_lo, cols.closed_hi, L.tot, yg);
+    else store_lane<H, K>(dx, aligned, j0, cols.closed, yg);
+}
+
+// One wavefront per tile in which a crossing column begins: folds the tail
+// piece of that tile and the head pieces of the tiles the column runs
+// through into stat[tile] (forward: H maxima, H sums; backward: H sums).
+template <int H, int T, bool FWD>
+__global__ __launch_bounds__(kFlatThreads) void esm_merge(const FlatMeta *__restrict__ meta,
+                                                          float *__restrict__ pieces, float *__restrict__ stat,
+                                                          int ntiles)
+{
+    const int tile = blockIdx.x * kFlatWaves + (threadIdx.x >> 6);
+    if (tile >= ntiles) return;
+    const FlatMeta m = meta[tile];
+    if (!m.tail_open || m.tail_cs < tile * T) return;
+    const int last_tile = (m.tail_ce - 1) / T;
+    const int lane = lane_id();
+    float mx[H], sum[H];
+#pragma unroll
+    for (int h = 0; h < H; h++) {
+        mx[h] = -INFINITY;
+        sum[h] = 0.f;
+    }
+    auto fold = [&](int h, float m2, float s2) {
+        if (FWD) {
+            const float mm = fmaxf(mx[h], m2);
+            sum[h] = (mx[h] == -INFINITY ? 0.f : sum[h] * expf(mx[h] - mm)) + (m2 == -INFINITY ? 0.f : s2 * expf(m2 - mm));
+            mx[h] = mm;
+        } else {
+            sum[h] += s2;
+        }
+    };
+    // lane 0 starts from the tail piece of this tile; head pieces of the
+    // following tiles are dealt round-robin, each lane keeping tile order.
+    // Most crossing columns end in the next tile: short chains are folded by
+    // lane 0 alone and skip the exchange between lanes.
+    const bool chain_short = last_tile - tile < 4;
+    if (chain_short) {
+        if (lane == 0)
+            for (int j = tile; j <= last_tile; j++) {
+                const float *p = piece<H>(pieces, j, j == tile ? 1 : 0);
+#pragma unroll
+                for (int h = 0; h < H; h++) fold(h, FWD ? p[h] : 0.f, FWD ? p[H + h] : p[h]);
+            }
+    } else {
+        for (int j = tile + lane; j <= last_tile; j += kWave) {
+            const float *p = piece<H>(pieces, j, j == tile ? 1 : 0);
+#pragma unroll
+            for (int h = 0; h < H; h++) fold(h, FWD ? p[h] : 0.f, FWD ? p[H + h] : p[h]);
+        }
+#pragma unroll
+        for (int o = 1; o < kWave; o <<= 1) {
+#pragma unroll
+            for (int h = 0; h < H; h++) {
+                const float m2 = FWD ? __shfl_xor(mx[h], o, kWave) : 0.f;
+                const float s2 = __shfl_xor(sum[h], o, kWave);
+                fold(h, m2, s2);
+            }
+        }
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int h = 0; h < H; h++) {
+            if (FWD) {
+                stat[(int64_t)tile * 2 * H + h] = mx[h];
+                stat[(int64_t)tile * 2 * H + H + h] = sum[h];
+            } else {
+                stat[(int64_t)tile * 2 * H + h] = sum[h];
+            }
+        }
+    }
+}
+
+// Entries of crossing columns.  a = x (forward) or y (backward); b = g.
+template <int H, int T, bool FWD>
+__global__ __launch_bounds__(kFlatThreads) void esm_finish(const FlatMeta *__restrict__ meta,
+                                                           const float *__restrict__ stat, const float *__restrict__ a,
+                                                           const float *__restrict__ b, float *__restrict__ out, int E)
+{
+    const int tile = blockIdx.x;
+    const int t0 = tile * T;
+    const int n = min(T, E - t0);
+    const FlatMeta m = meta[tile];
+#pragma unroll
+    for (int part = 0; part < 2; part++) {
+        int src, s, e;
+        if (part == 0) {
+            if (!m.head_open) continue;
+            src = m.head_cs / T;
+            s = t0;
+            e = min(m.head_ce, t0 + n);
+        } else {
+            if (!m.tail_open || m.tail_cs < t0) continue;
+            src = tile;
+            s = m.tail_cs;
+            e = t0 + n;
+        }
+        const float *st = stat + (int64_t)src * 2 * H;
+        // kFlatThreads % H == 0: a thread stays on one head
+        const int h = (int)(((int64_t)s * H + threadIdx.x) % H);
+        const float s0 = st[h], s1 = FWD ? st[H + h] : 0.f;
+        const int64_t end = (int64_t)e * H;
+        constexpr int kBatch = 4;
+        for (int64_t p0 = (int64_t)s * H + threadIdx.x; p0 < end; p0 += (int64_t)kBatch * kFlatThreads) {
+            float va[kBatch], vb[kBatch];
+#pragma unroll
+            for (int i = 0; i < kBatch; i++) {
+                const int64_t p = min(p0 + (int64_t)i * kFlatThreads, end - 1);
+                va[i] = a[p];
+                vb[i] = FWD ? 0.f : b[p];
+            }
+#pragma unroll
+            for (int i = 0; i < kBatch; i++) {
+                const int64_t p = p0 + (int64_t)i * kFlatThreads;
+                if (p < end) out[p] = FWD ? expf(va[i] - s0) / s1 : va[i] * vb[i] - va[i] * s0;
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------ host ---
+static int flat_tiles(int64_t E, int H)
+{
+    const int T = H <= 2 ? FlatShape<1>::T : FlatShape<4>::T;
+    return (int)ceil_div(E, T);
+}
+
+bool edge_softmax_flat_supported(int H) { return H == 1 || H == 2 || H == 4 || H == 8; }
+
+size_t edge_softmax_flat_ws_bytes(int64_t E)
+{
+    // sized for the smallest tile and the widest pieces (H = 8)
+    const size_t tiles = (size_t)ceil_div(E > 0 ? E : 1, (int64_t)FlatShape<8>::T);
+    return carve_bytes(tiles, sizeof(FlatMeta)) + carve_bytes(tiles * 4 * 8, 4) + carve_bytes(tiles * 2 * 8, 4) +
+           2 * carve_bytes(tiles, 4);
+}
+
+template <int H>
+static void flat_launch(bool fwd, const int32_t *off, const float *a, const float *b, float *out, int32_t V, int64_t E,
+                        void *ws, hipStream_t s)
+{
+    constexpr int T = FlatShape<H>::T;
+    const int ntiles = flat_tiles(E, H);
+    Carver carve(ws);
+    const size_t cap = (size_t)ceil_div(E, (int64_t)FlatShape<8>::T);
+    FlatMeta *meta = carve.take<FlatMeta>(cap);
+    float *pieces = carve.take<float>(cap * 4 * 8);
+    float *stat = carve.take<float>(cap * 2 * 8);
+    int32_t *tile_first = carve.take<int32_t>(cap);
+    int32_t *tile_last = carve.take<int32_t>(cap);
+    // Through LDS pays once a lane's K*H floats span 64 bytes or more (measured:
+    // 1 head 42 vs 44 us direct, 8 heads 390 vs 319 us); JGAMD_SOFTMAX_STAGE=0/1 overrides.
+    const char *env = getenv("JGAMD_SOFTMAX_STAGE");
+    const int staged = env ? atoi(env) : (H >= 2 ? 1 : 0);
+    hipLaunchKernelGGL(esm_tile_columns, dim3((unsigned)ceil_div(V, 256)), dim3(256), 0, s, off, V, (int)E, T, ntiles,
+                       tile_first, tile_last);
+    if (fwd) {
+        hipLaunchKernelGGL(esm_fwd_tile<H>, dim3(ntiles), dim3(kFlatThreads), 0, s, off, a, out, tile_first, tile_last,
+                           V, (int)E, meta, pieces, staged);
+        hipLaunchKernelGGL((esm_merge<H, T, true>), dim3((unsigned)ceil_div(ntiles, kFlatWaves)), dim3(kFlatThreads), 0, s,
+                           meta, pieces, stat, ntiles);
+        hipLaunchKernelGGL((esm_finish<H, T, true>), dim3(ntiles), dim3(kFlatThreads), 0, s, meta, stat, a, a, out,
+                           (int)E);
+    } else {
+        hipLaunchKernelGGL(esm_bwd_tile<H>, dim3(ntiles), dim3(kFlatThreads), 0, s, off, a, b, out, tile_first,
+                           tile_last, V, (int)E, meta, pieces, staged);
+        hipLaunchKernelGGL((esm_merge<H, T, false>), dim3((unsigned)ceil_div(ntiles, kFlatWaves)), dim3(kFlatThreads), 0,
+                           s, meta, pieces, stat, ntiles);
+        hipLaunchKernelGGL((esm_finish<H, T, false>), dim3(ntiles), dim3(kFlatThreads), 0, s, meta, stat, a, b, out,
+                           (int)E);
+    }
+}
+
+// fwd: a = x, b unused; bwd: a = y, b = g.  V > 0, E > 0, off[V] == E.
+void edge_softmax_flat_enqueue(bool fwd, const int32_t *off, const float *a, const float *b, float *out, int32_t V,
+                               int64_t E, int32_t H, void *ws, hipStream_t s)
+{
+    switch (H) {
+    case 1: flat_launch<1>(fwd, off, a, b, out, V, E, ws, s); break;
+    case 2: flat_launch<2>(fwd, off, a, b, out, V, E, ws, s); break;
+    case 4: flat_launch<4>(fwd, off, a, b, out, V, E, ws, s); break;
+    default: flat_launch<8>(fwd, off, a, b, out, V, E, ws, s); break;
+    }
+}
+
+}  // namespace jg

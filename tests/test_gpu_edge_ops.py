@@ -43,6 +43,10 @@ def test_edgesoftmax_reference_fixture_and_gradient():
     (1, 0, 1, 0, 0), (1, 300, 1, 0, 1), (300, 2000, 1, 2, 2), (300, 2000, 2, 2, 3), (5000, 40000, 8, 3, 4),
     (2000, 300000, 1, 2, 5), (2000, 100000, 4, 1, 6), (700, 9000, 3, 2, 7), (700, 9000, 16, 2, 8),
     (20000, 30000, 64, 0, 9), (100, 5000, 128, 1, 10),
+    # tile edge cases of the 1/2/4/8-head path: E a multiple of the tile (2048 and 1024 entries),
+    # one entry more, mostly empty columns (more columns than entries in a tile), one column only
+    (300, 4096, 1, 1, 11), (300, 4097, 2, 1, 12), (50, 3072, 4, 0, 13), (50, 2049, 8, 1, 14),
+    (200000, 5000, 1, 0, 15), (300000, 3000, 8, 2, 16), (1, 70000, 2, 0, 17), (3, 40000, 8, 0, 18),
 ])
 def test_edgesoftmax_forward_backward(V, E, H, hubs, seed):
     from jittorgeometric_amd.ops import EdgeSoftmax
@@ -89,6 +93,43 @@ def test_edgesoftmax_reference_shapes_E_and_E1():
     assert y1.shape == (E,) and y2.shape == (E, 1)
     assert torch.equal(y1, y2[:, 0])
     assert_close(y1.cpu().numpy(), oracle.edgesoftmax(x, off), rtol=1e-5, atol=1e-7)
+
+
+@pytest.mark.parametrize("H", [1, 4])
+@pytest.mark.parametrize("variant", ["misaligned", "groups", "stage0", "stage1"])
+def test_edgesoftmax_code_paths_agree(H, variant, monkeypatch):
+    """Arrays that are not 16-byte aligned, the lane-group kernels, and both ways of
+    moving a tile (direct / through LDS) give the default path's results."""
+    from jittorgeometric_amd.ops import EdgeSoftmax
+    rng = np.random.default_rng(40 + H)
+    V, E = 3000, 50000
+    ei, w = rand_graph(rng, V, E, 2)
+    csc, (row, off, _) = make_csc(ei, w, V)
+    x = rng.standard_normal((E, H)).astype(np.float32)
+    g = rng.standard_normal((E, H)).astype(np.float32)
+    xt = to_gpu(x).requires_grad_(True)
+    y = EdgeSoftmax(xt, csc)
+    y.backward(to_gpu(g))
+    if variant == "misaligned":
+        pad = torch.zeros(E * H + 1, device=dev())
+        pad[1:] = to_gpu(x).reshape(-1)
+        x2 = pad[1:].reshape(E, H).requires_grad_(True)
+        assert x2.data_ptr() % 16 != 0
+        gpad = torch.zeros(E * H + 1, device=dev())
+        gpad[1:] = to_gpu(g).reshape(-1)
+        g2 = gpad[1:].reshape(E, H)
+    else:
+        if variant == "groups":
+            monkeypatch.setenv("JGAMD_SOFTMAX", "groups")
+        else:
+            monkeypatch.setenv("JGAMD_SOFTMAX_STAGE", variant[-1])
+        x2 = to_gpu(x).requires_grad_(True)
+        g2 = to_gpu(g)
+    y2 = EdgeSoftmax(x2, csc)
+    y2.backward(g2)
+    assert_close(y2.detach().cpu().numpy(), y.detach().cpu().numpy(), rtol=2e-6, atol=1e-8, what=variant)
+    gref = xt.grad.cpu().numpy()
+    assert_close(x2.grad.cpu().numpy(), gref, scale=np.abs(gref) + 1e-3, rtol=1e-5, what=variant + " backward")
 
 
 def test_edgesoftmax_large_logits_stay_finite():
