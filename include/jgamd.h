@@ -86,6 +86,13 @@ int32_t jgamd_csx_transpose(const int32_t *off, const int32_t *idx, const float 
                             float *out_w, int32_t *out_perm, void *ws, size_t ws_bytes,
                             void *stream);
 
+/* inv[perm[i]] = i for a permutation of [0,n) (entries outside the range are
+ * skipped).  No reference counterpart: it turns the out_perm of
+ * jgamd_csx_transpose (transposed slot -> original slot) into the map
+ * original slot -> transposed slot that jgamd_gat_bwd gathers through.
+ */
+int32_t jgamd_invert_permutation(const int32_t *perm, int64_t n, int32_t *inv, void *stream);
+
 /* ------------------------------------------------------------------------
  * Weighted row-gather SpMM:  out[r,:] = sum_{j in [off[r],off[r+1])} w[j] * x[idx[j],:]
  * Replaces AggregateOp::jit_run (ops/cpp/aggregate_op.cc:26-71 CPU,
@@ -178,8 +185,9 @@ int32_t jgamd_gat_fwd(const int32_t *off, const int32_t *idx, const float *h,
                       void *stream);
 
 /* Backward of jgamd_gat_fwd.  Needs both orders of the graph: (off, idx) are
- * the CSC arrays used forward, (t_off, t_idx, t_perm) their transpose as
- * produced by jgamd_csx_transpose (t_perm[j] = CSC slot of transposed slot j).
+ * the CSC arrays used forward, (t_off, t_idx) their transpose as produced by
+ * jgamd_csx_transpose, and t_inv[j] = transposed slot of CSC slot j, i.e. the
+ * inverse of that call's out_perm (jgamd_invert_permutation).
  * With H > 1 the head width D must span a power-of-two number of lanes
  * (D in {1,2,4,...,256}); other shapes return JGAMD_ERR_UNSUPPORTED and are
  * served by the unfused operator chain.
@@ -190,7 +198,7 @@ int32_t jgamd_gat_fwd(const int32_t *off, const int32_t *idx, const float *h,
  */
 int32_t jgamd_gat_bwd_workspace(int32_t V, int64_t E, int32_t H, int32_t D, size_t *bytes);
 int32_t jgamd_gat_bwd(const int32_t *off, const int32_t *idx, const int32_t *t_off,
-                      const int32_t *t_idx, const int32_t *t_perm, const float *h, const float *a_src,
+                      const int32_t *t_idx, const int32_t *t_inv, const float *h, const float *a_src,
                       const float *a_dst, float slope, const float *el, const float *er,
                       const float *smax, const float *ssum, const float *out,
                       const float *g_out, float *g_h, float *g_a_src, float *g_a_dst,

@@ -541,6 +541,15 @@ __global__ void csx_expand_rows(const int32_t *__restrict__ off, int32_t R, int3
     }
 }
 
+// inv[perm[i]] = i; entries of perm outside [0,n) are skipped.
+__global__ void csx_invert_permutation(const int32_t *__restrict__ perm, int64_t n, int32_t *__restrict__ inv)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int32_t p = perm[i];
+    if ((uint64_t)p < (uint64_t)n) inv[p] = (int32_t)i;
+}
+
 __global__ void fill_i32(int32_t *p, int64_t n, int32_t v)
 {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -768,4 +777,14 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_csx_transpose(co
     }
     return out_perm ? convert<true>(idx, rows, w, E, C, out_idx, out_off, out_w, out_perm, inner, s)
                     : convert<false>(idx, rows, w, E, C, out_idx, out_off, out_w, out_perm, inner, s);
+}
+
+extern "C" __attribute__((visibility("default"))) int32_t jgamd_invert_permutation(const int32_t *perm, int64_t n, int32_t *inv, void *stream)
+{
+    if (n < 0 || n >= ((int64_t)1 << 31)) return fail(JGAMD_ERR_SIZE, "invert_permutation: n=%lld out of range", (long long)n);
+    if (n == 0) return 0;
+    if (!perm || !inv) return fail(JGAMD_ERR_NULL, "invert_permutation: NULL array");
+    hipLaunchKernelGGL(csx_invert_permutation, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), perm, n, inv);
+    return launch_status("invert_permutation");
 }

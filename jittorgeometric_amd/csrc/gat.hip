@@ -24,6 +24,7 @@ namespace jg {
 
 constexpr int kGatThreads = 256;
 constexpr int kGatWaves = kGatThreads / kWave;
+constexpr int kGzHeads = 16;   // heads whose logit gradients are staged in LDS by the backward pass
 // gathers in flight per wavefront, bounded by the registers they land in
 constexpr int gat_unroll(int regs) { return regs >= 16 ? 2 : regs >= 8 ? 4 : 8; }
 
@@ -512,20 +513,28 @@ __global__ __launch_bounds__(256) void gat_bwd_node_stats_vec(const float *__res
 //   alpha  = exp(lrelu(el[r]+er[c]) - smax[c]) / ssum[c]
 //   galpha = g_out[c,k,:].h[r,k,:]                     (reduced over the head's lanes)
 //   gz     = alpha (galpha - g_out[c,k,:].out[c,k,:]) * lrelu'(z)
-//   g_h[r,:] += alpha g_out[c,:];  g_el[r,k] += gz;  gz_csc[perm[j],k] = gz
+//   g_h[r,:] += alpha g_out[c,:];  g_el[r,k] += gz;  gz_t[j,k] = gz  (transposed order: consecutive
+//   entries store consecutive addresses; the destination-side sum gathers them through t_inv)
 // lph = lanes per head (power of two) when H > 1; for H == 1 the whole
 // wavefront (all tiles) reduces into the single head.
 template <int VEC, int NT>
 __global__ __launch_bounds__(kGatThreads) void gat_bwd_merge(
-    const int32_t *__restrict__ t_off, const int32_t *__restrict__ t_idx, const int32_t *__restrict__ t_perm,
+    const int32_t *__restrict__ t_off, const int32_t *__restrict__ t_idx,
     const float *__restrict__ h, const float *__restrict__ el, const float4 *__restrict__ stat,
     const float *__restrict__ g_out, float slope, float *__restrict__ g_h, float *__restrict__ g_el,
-    float *__restrict__ gz_csc, float *__restrict__ partial, float *__restrict__ pel,
+    float *__restrict__ gz_t, float *__restrict__ partial, float *__restrict__ pel,
     const int32_t *__restrict__ chunk_row, int R, int E, int H, int D, int lph, int chunk, int nchunks)
 {
     constexpr int kGatUnroll = gat_unroll(VEC * NT);
+    // The logit gradients of a group of 64 entries wait in LDS and leave as one contiguous
+    // block when the group is done: a global store inside the gather loop makes every wait
+    // for a gathered row wait for the stores in flight as well (loads and stores share one
+    // counter and do not complete in order with each other).
+    __shared__ float gz_stage[kGatWaves][kWave * kGzHeads];
     const int k = blockIdx.x * kGatWaves + wave_in_block();
     if (k >= nchunks) return;
+    float *gzbuf = gz_stage[wave_in_block()];
+    const bool staged = H <= kGzHeads;
     const int lane = lane_id();
     const int F = H * D;
     const int f0 = lane * VEC;
@@ -597,11 +606,10 @@ __global__ __launch_bounds__(kGatThreads) void gat_bwd_merge(
 
     for (int jb = j0; jb < j1; jb += kWave) {
         const int n = min(kWave, j1 - jb);
-        int my_c = -1, my_p = 0;
+        int my_c = -1;
         if (lane < n) {
             my_c = t_idx[jb + lane];
-            my_p = t_perm[jb + lane];
-            if ((unsigned)my_c >= (unsigned)R || (unsigned)my_p >= (unsigned)E) my_c = -1;
+            if ((unsigned)my_c >= (unsigned)R) my_c = -1;
         }
         for (int i0 = 0; i0 < n; i0 += kGatUnroll) {
             float gv[kGatUnroll][NT][VEC];
@@ -624,7 +632,6 @@ __global__ __launch_bounds__(kGatThreads) void gat_bwd_merge(
                     while (jj == row_end && r < r1) flush_row();
                     const int c = bcast_i(my_c, i0 + u);
                     if (c >= 0) {
-                        const int slot = bcast_i(my_p, i0 + u);
                         float dot[NT];
 #pragma unroll
                         for (int t = 0; t < NT; t++) {
@@ -654,11 +661,26 @@ __global__ __launch_bounds__(kGatThreads) void gat_bwd_merge(
                                 gel[t] += gz;
 #pragma unroll
                                 for (int v = 0; v < VEC; v++) acc[t][v] = fmaf(alpha, gv[u][t][v], acc[t][v]);
-                                if (lead[t]) gz_csc[(uint32_t)slot * (uint32_t)H + (uint32_t)head[t]] = gz;
+                                if (lead[t]) {
+                                    if (staged) gzbuf[(i0 + u) * H + head[t]] = gz;
+                                    else gz_t[(uint32_t)jj * (uint32_t)H + (uint32_t)head[t]] = gz;
+                                }
+                            }
+                    } else {
+                        // destination out of range: the edge counts for nothing on either side
+#pragma unroll
+                        for (int t = 0; t < NT; t++)
+                            if (act[t] && lead[t]) {
+                                if (staged) gzbuf[(i0 + u) * H + head[t]] = 0.f;
+                                else gz_t[(uint32_t)jj * (uint32_t)H + (uint32_t)head[t]] = 0.f;
                             }
                     }
                 }
             }
+        }
+        if (staged) {
+            float *dst = gz_t + (size_t)jb * H;
+            for (int i = lane; i < n * H; i += kWave) dst[i] = gzbuf[i];
         }
     }
     while (r < r1) flush_row();
@@ -992,7 +1014,7 @@ JG_EXPORT int32_t jgamd_gat_bwd_workspace(int32_t V, int64_t E, int32_t H, int32
 }
 
 JG_EXPORT int32_t jgamd_gat_bwd(const int32_t *off, const int32_t *idx, const int32_t *t_off, const int32_t *t_idx,
-                                const int32_t *t_perm, const float *h, const float *a_src, const float *a_dst,
+                                const int32_t *t_inv, const float *h, const float *a_src, const float *a_dst,
                                 float slope, const float *el, const float *er, const float *smax, const float *ssum,
                                 const float *out, const float *g_out, float *g_h, float *g_a_src, float *g_a_dst,
                                 int32_t V, int64_t E, int32_t H, int32_t D, void *ws, size_t ws_bytes, void *stream)
@@ -1013,7 +1035,7 @@ JG_EXPORT int32_t jgamd_gat_bwd(const int32_t *off, const int32_t *idx, const in
     }
     if (!off || !t_off || !h || !a_src || !a_dst || !el || !er || !smax || !ssum || !out || !g_out || !g_h)
         return fail(JGAMD_ERR_NULL, "gat_bwd: NULL array");
-    if (E > 0 && (!t_idx || !t_perm)) return fail(JGAMD_ERR_NULL, "gat_bwd: transposed arrays are NULL with E > 0");
+    if (E > 0 && (!t_idx || !t_inv)) return fail(JGAMD_ERR_NULL, "gat_bwd: transposed arrays are NULL with E > 0");
     if ((((uintptr_t)h | (uintptr_t)g_out | (uintptr_t)g_h) & 15) != 0)
         return fail(JGAMD_ERR_ALIGN, "gat_bwd: h/g_out/g_h not 16-byte aligned");
     const size_t need = gat_bwd_ws(V, E, H, D);
@@ -1047,7 +1069,7 @@ JG_EXPORT int32_t jgamd_gat_bwd(const int32_t *off, const int32_t *idx, const in
     dim3 grid((unsigned)ceil_div(s.nchunks, kGatWaves)), block(kGatThreads);
 #define JG_BWD(VV, NN)                                                                                             \
     case VV * 16 + NN:                                                                                             \
-        hipLaunchKernelGGL((gat_bwd_merge<VV, NN>), grid, block, 0, st, t_off, t_idx, t_perm, h, el, stat, g_out,  \
+        hipLaunchKernelGGL((gat_bwd_merge<VV, NN>), grid, block, 0, st, t_off, t_idx, h, el, stat, g_out,          \
                            slope, g_h, g_el, gz, partial, pel, chunk_row, V, (int)E, H, D, s.lph, s.chunk,         \
                            s.nchunks);                                                                             \
         if (ngroups > 1)                                                                                           \
@@ -1058,9 +1080,9 @@ JG_EXPORT int32_t jgamd_gat_bwd(const int32_t *off, const int32_t *idx, const in
         break;
     JG_GAT_DISPATCH(JG_BWD)
 #undef JG_BWD
-    // g_er[c,k] = sum of gz over the (contiguous) CSC slots of column c: the row-gather SpMM
-    // with identity indices and unit weights on the [E,H] array
-    if (int32_t rc = spmm_enqueue(off, nullptr, nullptr, gz, g_er, V, (int32_t)E, E, H, spmm_ws,
+    // g_er[c,k] = sum of gz over the CSC slots of column c: the row-gather SpMM with unit
+    // weights; slot j's row of the [E,H] array sits at its transposed position t_inv[j]
+    if (int32_t rc = spmm_enqueue(off, t_inv, nullptr, gz, g_er, V, (int32_t)E, E, H, spmm_ws,
                                   spmm_ws_bytes(V, E, H), st))
         return rc;
     hipLaunchKernelGGL(gat_bwd_finish, dim3((unsigned)nred), dim3(256), 0, st, h, a_src, a_dst, g_el, g_er, g_h, red,

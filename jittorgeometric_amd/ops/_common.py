@@ -40,6 +40,20 @@ def transposed(holder, off, idx, w, R, C):
     return off_t, idx_t, w_t, perm
 
 
+def transposed_inverse(holder, perm):
+    """inv with inv[perm[j]] = j (original slot -> transposed slot) for the perm
+    that `transposed` returned for `holder`; built once and kept beside it."""
+    cached = getattr(holder, "_jgamd_transposed_inv", None)
+    if cached is not None and cached[1] is perm:
+        return cached[0]
+    lib = _lib.load()
+    dev = _lib.require_gpu(perm)
+    inv = torch.empty_like(perm)
+    _lib.check(lib.jgamd_invert_permutation(_lib.ptr(perm), perm.shape[0], _lib.ptr(inv), _lib.stream_ptr(dev)))
+    holder._jgamd_transposed_inv = (inv, perm)
+    return inv
+
+
 def spmm(off, idx, w, x, R):
     """out[r,:] = sum_j w[j] * x[idx[j],:]; idx/w may be None (identity / ones)."""
     lib = _lib.load()

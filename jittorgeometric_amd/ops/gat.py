@@ -6,7 +6,7 @@ EdgeSoftmax -> multiply -> ScatterToVertex of GATConv.propagate
 import torch
 
 from .. import _lib
-from ._common import as_f32, transposed
+from ._common import as_f32, transposed, transposed_inverse
 
 
 def fused_supported(H, D, backward=True):
@@ -61,12 +61,13 @@ class GatFusedFunc(torch.autograd.Function):
         V, H, D = h.shape
         E = csc.row_indices.shape[0]
         off_t, idx_t, _, perm = transposed(csc, csc.column_offset, csc.row_indices, csc.edge_weight, V, V)
+        inv = transposed_inverse(csc, perm)
         g_h = torch.empty_like(h)
         g_as, g_ad = torch.empty_like(a_src), torch.empty_like(a_dst)
         nbytes = _lib.query(lib.jgamd_gat_bwd_workspace, V, E, H, D)
         ws = _lib.workspace(nbytes, dev)
         _lib.check(lib.jgamd_gat_bwd(_lib.ptr(csc.column_offset), _lib.ptr(csc.row_indices), _lib.ptr(off_t),
-                                     _lib.ptr(idx_t), _lib.ptr(perm), _lib.ptr(h), _lib.ptr(a_src), _lib.ptr(a_dst),
+                                     _lib.ptr(idx_t), _lib.ptr(inv), _lib.ptr(h), _lib.ptr(a_src), _lib.ptr(a_dst),
                                      float(ctx.slope), _lib.ptr(el), _lib.ptr(er), _lib.ptr(smax), _lib.ptr(ssum),
                                      _lib.ptr(out), _lib.ptr(g_out), _lib.ptr(g_h), _lib.ptr(g_as), _lib.ptr(g_ad),
                                      V, E, H, D, _lib.ptr(ws), nbytes, _lib.stream_ptr(dev)))
