@@ -114,6 +114,13 @@ def test_permutation_output_and_transpose():
     assert np.array_equal(idx_t.cpu().numpy(), row)
     assert np.array_equal(w_t.cpu().numpy(), cw)
     assert np.array_equal(perm_t.cpu().numpy(), np.argsort(dst_sorted, kind="stable"))
+    # the inverse map (original slot -> transposed slot), cached beside the transpose
+    from jittorgeometric_amd.ops._common import transposed_inverse
+    inv = transposed_inverse(holder, perm_t)
+    assert transposed_inverse(holder, perm_t) is inv
+    want_inv = np.empty(E, np.int32)
+    want_inv[perm_t.cpu().numpy()] = np.arange(E, dtype=np.int32)
+    assert np.array_equal(inv.cpu().numpy(), want_inv)
 
 
 def test_int64_edge_index_is_narrowed_like_the_reference_data_class():
