@@ -121,6 +121,19 @@ int32_t jgamd_spmm_csx(const int32_t *off, const int32_t *idx, const float *w, c
                        float *out, int32_t R, int32_t C, int64_t E, int32_t F, void *ws,
                        size_t ws_bytes, void *stream);
 
+/* jgamd_spmm_csx with a row finish:
+ *   out[r,:] = beta * sum_j w[j] * x[idx[j],:] + alpha * h[r,:]
+ * h is [R,F] (NULL or alpha == 0 drops the term) and may be x itself; out must
+ * not overlap x or h.  One call is one hop of the reference's polynomial
+ * propagation layers, whose Python loop runs the product and then two
+ * element-wise passes (nn/conv/appnp_conv.py:42-51: x = propagate(x);
+ * x = x * (1 - alpha); x = x + alpha * h).  Same workspace as jgamd_spmm_csx.
+ */
+int32_t jgamd_spmm_csx_axpby(const int32_t *off, const int32_t *idx, const float *w,
+                             const float *x, float *out, float beta, float alpha,
+                             const float *h, int32_t R, int32_t C, int64_t E, int32_t F,
+                             void *ws, size_t ws_bytes, void *stream);
+
 /* Benchmark support; no counterpart in the reference.  Runs jgamd_spmm_csx
  * `iters` times on `stream`, with one hipEvent pair around each launch of the
  * gather kernel (spmm_merge) and one around each whole call (three launches),

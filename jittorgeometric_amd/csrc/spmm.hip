@@ -89,14 +89,24 @@ __global__ void spmm_chunk_rows(const int32_t *__restrict__ off, int R, int chun
 // WIDE = false: every row of x starts less than 4 GiB from x, so a gathered
 // row is addressed as (scalar base) + (32-bit byte offset): one readlane and
 // one vector add per entry.  WIDE = true keeps 64-bit row arithmetic.
-template <int VEC, int NT, int UNROLL, bool WIDE, bool LDS>
+//
+// EPI = true finishes every row as beta * sum + alpha * h[row,:] (h == nullptr
+// drops the second term).  The row of h is fetched when the row begins.  A
+// row that began in an earlier chunk is stored raw: spmm_fixup adds its
+// pieces and applies the same finish.
+struct RowFinish {
+    float beta, alpha;
+    const float *h;
+};
+
+template <int VEC, int NT, int UNROLL, bool WIDE, bool LDS, bool EPI>
 __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__restrict__ off,
                                                            const int32_t *__restrict__ idx,
                                                            const float *__restrict__ w,
                                                            const float *__restrict__ x, float *__restrict__ out,
                                                            float *__restrict__ partial,
                                                            const int32_t *__restrict__ chunk_row, int R, int C,
-                                                           int E, int F, int chunk, int nchunks)
+                                                           int E, int F, int chunk, int nchunks, RowFinish fin)
 {
     static_assert(kWave % UNROLL == 0, "groups tile a 64-entry batch");
     __shared__ int2 staged_all[LDS ? kSpmmThreads : 1];
@@ -141,8 +151,38 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__rest
 #pragma unroll
         for (int v = 0; v < VEC; v++) acc[t][v] = 0.f;
 
+    // EPI: h row of the current row; raw_row = the chunk's first row when it began earlier
+    float hrow[EPI ? NT : 1][EPI ? VEC : 1];
+    int raw_row = -1;
+    auto fetch_h = [&]() {
+        if constexpr (EPI) {
+            if (fin.h) {
+                const float *src = fin.h + (size_t)min(r, R - 1) * F;
+#pragma unroll
+                for (int t = 0; t < NT; t++) vload<VEC>(hrow[t], src + fo[t]);
+            } else {
+#pragma unroll
+                for (int t = 0; t < NT; t++)
+#pragma unroll
+                    for (int v = 0; v < VEC; v++) hrow[t][v] = 0.f;
+            }
+        }
+    };
+    if constexpr (EPI) {
+        if (r < r1 && uniform(off[r]) + r < p0) raw_row = r;
+        fetch_h();
+    }
+
     auto flush_row = [&]() {
         float *dst = out + (size_t)r * F + f0;
+        if constexpr (EPI) {
+            if (r != raw_row) {
+#pragma unroll
+                for (int t = 0; t < NT; t++)
+#pragma unroll
+                    for (int v = 0; v < VEC; v++) acc[t][v] = fmaf(fin.alpha, hrow[t][v], fin.beta * acc[t][v]);
+            }
+        }
 #pragma unroll
         for (int t = 0; t < NT; t++) {
             if (act[t]) vstore_stream<VEC>(dst + t * kWave * VEC, acc[t]);
@@ -150,6 +190,7 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__rest
             for (int v = 0; v < VEC; v++) acc[t][v] = 0.f;
         }
         r++;
+        if constexpr (EPI) fetch_h();
         if (r - rb == kWave) {
             rb = r;
             ends = (rb + lane < R) ? off[rb + 1 + lane] : kNever;
@@ -316,12 +357,12 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_group_sums(const int32_t *_
 // One wavefront per chunk b: if the first row of b started in an earlier
 // chunk a and ends in b, out[row] = (pieces a .. b-1, in order) + out[row];
 // whole groups between a and b come from group_sum.
-template <int VEC, int NT>
+template <int VEC, int NT, bool EPI>
 __global__ __launch_bounds__(kSpmmThreads) void spmm_fixup(const int32_t *__restrict__ off, float *__restrict__ out,
                                                            const float *__restrict__ partial,
                                                            const float *__restrict__ group_sum,
                                                            const int32_t *__restrict__ chunk_row, int F, int chunk,
-                                                           int nchunks)
+                                                           int nchunks, RowFinish fin)
 {
     const int k = blockIdx.x * kSpmmWaves + wave_in_block();
     if (k >= nchunks) return;
@@ -349,9 +390,34 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_fixup(const int32_t *__rest
     }
     float *dst = out + (size_t)r0 * F;
     add_pieces<VEC, NT>(acc, dst, 0, 1, F, f0);
+    if constexpr (EPI) {
+#pragma unroll
+        for (int t = 0; t < NT; t++)
+#pragma unroll
+            for (int v = 0; v < VEC; v++) acc[t][v] *= fin.beta;
+        if (fin.h) {
+            float hv[NT][VEC];
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                const int f = f0 + t * kWave * VEC;
+                vload<VEC>(hv[t], fin.h + (size_t)r0 * F + (f < F ? f : 0));
+#pragma unroll
+                for (int v = 0; v < VEC; v++) acc[t][v] = fmaf(fin.alpha, hv[t][v], acc[t][v]);
+            }
+        }
+    }
 #pragma unroll
     for (int t = 0; t < NT; t++)
         if (f0 + t * kWave * VEC < F) vstore<VEC>(dst + f0 + t * kWave * VEC, acc[t]);
+}
+
+// out = beta * out + alpha * h, element-wise (the finish as a pass of its own, for the
+// shapes the fused kernels do not cover).
+__global__ void spmm_finish_rows(float *__restrict__ out, const float *__restrict__ h, int64_t n, float beta,
+                                 float alpha)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = fmaf(alpha, h ? h[i] : 0.f, beta * out[i]);
 }
 
 // ------------------------------------------------------------------ host ---
@@ -407,7 +473,8 @@ size_t spmm_ws_bytes(int32_t R, int64_t E, int32_t F)
 template <int VEC, int NT>
 static void launch_spmm(const SpmmShape &s, const int32_t *off, const int32_t *idx, const float *w, const float *x,
                         float *out, float *partial, float *group_sum, const int32_t *chunk_row, int R, int C, int E,
-                        int F, hipStream_t st, hipEvent_t k0 = nullptr, hipEvent_t k1 = nullptr)
+                        int F, hipStream_t st, hipEvent_t k0 = nullptr, hipEvent_t k1 = nullptr,
+                        const RowFinish *fin = nullptr)
 {
     dim3 grid((unsigned)ceil_div(s.nchunks, kSpmmWaves), (unsigned)s.slabs), block(kSpmmThreads);
     // gathers in flight per wavefront: bounded by the registers they land in
@@ -421,21 +488,36 @@ static void launch_spmm(const SpmmShape &s, const int32_t *off, const int32_t *i
     }();
     const bool lds = stage_env ? stage_env == 1 : F >= kLdsStageMinWidth;
     const bool narrow = (uint64_t)C * (uint64_t)F * 4u < ((uint64_t)1 << 32);
-#define JG_GO(W, L)                                                                                                   \
-    hipLaunchKernelGGL((spmm_merge<VEC, NT, U, W, L>), grid, block, 0, st, off, idx, w, x, out, partial, chunk_row, R, \
-                       C, E, F, s.chunk, s.nchunks)
-    if (narrow && lds) JG_GO(false, true);
-    else if (narrow) JG_GO(false, false);
-    else if (lds) JG_GO(true, true);
-    else JG_GO(true, false);
+    // the fused row finish exists for 32-bit offsets only; wide shapes finish in a pass of their own
+    const bool fused = fin && narrow;
+    const RowFinish none{1.f, 0.f, nullptr};
+    const RowFinish f = fused ? *fin : none;
+#define JG_GO(W, L, P)                                                                                              \
+    hipLaunchKernelGGL((spmm_merge<VEC, NT, U, W, L, P>), grid, block, 0, st, off, idx, w, x, out, partial,         \
+                       chunk_row, R, C, E, F, s.chunk, s.nchunks, f)
+    if (fused && lds) JG_GO(false, true, true);
+    else if (fused) JG_GO(false, false, true);
+    else if (narrow && lds) JG_GO(false, true, false);
+    else if (narrow) JG_GO(false, false, false);
+    else if (lds) JG_GO(true, true, false);
+    else JG_GO(true, false, false);
 #undef JG_GO
     if (k1) (void)hipEventRecord(k1, st);
     const int ngroups = (int)ceil_div(s.nchunks, kGroup);
     if (ngroups > 1)
         hipLaunchKernelGGL((spmm_group_sums<VEC, NT>), dim3((unsigned)ceil_div(ngroups, kSpmmWaves), (unsigned)s.slabs),
                            block, 0, st, off, partial, group_sum, chunk_row, R, F, s.chunk, s.nchunks);
-    hipLaunchKernelGGL((spmm_fixup<VEC, NT>), grid, block, 0, st, off, out, partial, group_sum, chunk_row, F, s.chunk,
-                       s.nchunks);
+    if (fused)
+        hipLaunchKernelGGL((spmm_fixup<VEC, NT, true>), grid, block, 0, st, off, out, partial, group_sum, chunk_row, F,
+                           s.chunk, s.nchunks, f);
+    else
+        hipLaunchKernelGGL((spmm_fixup<VEC, NT, false>), grid, block, 0, st, off, out, partial, group_sum, chunk_row, F,
+                           s.chunk, s.nchunks, f);
+    if (fin && !fused) {
+        const int64_t n = (int64_t)R * F;
+        hipLaunchKernelGGL(spmm_finish_rows, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, st, out, fin->h, n,
+                           fin->beta, fin->alpha);
+    }
 }
 
 }  // namespace jg
@@ -460,7 +542,7 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_workspa
 
 static int32_t spmm_call(const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out,
                          int32_t R, int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, void *stream,
-                         hipEvent_t k0, hipEvent_t k1)
+                         hipEvent_t k0, hipEvent_t k1, const RowFinish *fin = nullptr)
 {
     if (int32_t rc = check_spmm_sizes(R, E, F)) return rc;
     if (C < 0) return fail(JGAMD_ERR_SIZE, "spmm_csx: negative C");
@@ -474,7 +556,8 @@ static int32_t spmm_call(const int32_t *off, const int32_t *idx, const float *w,
         return fail(JGAMD_ERR_WORKSPACE, "spmm_csx: workspace %zu < %zu bytes", ws ? ws_bytes : (size_t)0, need);
     if (((uintptr_t)ws & 255) != 0) return fail(JGAMD_ERR_ALIGN, "spmm_csx: workspace not 256-byte aligned");
 
-    const uintptr_t bits = (uintptr_t)x | (uintptr_t)out;
+    // h is read with x's vector width: its alignment counts too
+    const uintptr_t bits = (uintptr_t)x | (uintptr_t)out | (uintptr_t)(fin ? fin->h : nullptr);
     const SpmmShape s = spmm_shape(R, E, F, (bits & 15) == 0, (bits & 7) == 0);
     Carver carve(ws);
     int32_t *chunk_row = carve.take<int32_t>((size_t)s.nchunks + 1);
@@ -486,7 +569,7 @@ static int32_t spmm_call(const int32_t *off, const int32_t *idx, const float *w,
                        s.chunk, s.nchunks, chunk_row);
 #define JG_CASE(V, N)                                                                                \
     if (s.vec == V && s.nt == N) {                                                                   \
-        launch_spmm<V, N>(s, off, idx, w, x, out, partial, group_sum, chunk_row, R, C, (int)E, F, st, k0, k1); \
+        launch_spmm<V, N>(s, off, idx, w, x, out, partial, group_sum, chunk_row, R, C, (int)E, F, st, k0, k1, fin); \
         return launch_status("spmm_csx");                                                            \
     }
 #define JG_CASES(V) JG_CASE(V, 1) JG_CASE(V, 2) JG_CASE(V, 3) JG_CASE(V, 4) JG_CASE(V, 5) JG_CASE(V, 6) JG_CASE(V, 8)
@@ -504,6 +587,15 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx(const i
                                                                          void *ws, size_t ws_bytes, void *stream)
 {
     return spmm_call(off, idx, w, x, out, R, C, E, F, ws, ws_bytes, stream, nullptr, nullptr);
+}
+
+extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_axpby(
+    const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out, float beta, float alpha,
+    const float *h, int32_t R, int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, void *stream)
+{
+    if (h && (((uintptr_t)h & 3) != 0)) return fail(JGAMD_ERR_ALIGN, "spmm_csx_axpby: h not 4-byte aligned");
+    const RowFinish fin{beta, alpha, alpha != 0.f ? h : nullptr};
+    return spmm_call(off, idx, w, x, out, R, C, E, F, ws, ws_bytes, stream, nullptr, nullptr, &fin);
 }
 
 namespace jg {

@@ -67,3 +67,43 @@ def spmm(off, idx, w, x, R):
     _lib.check(lib.jgamd_spmm_csx(_lib.ptr(off), _lib.ptr(idx), _lib.ptr(w), _lib.ptr(x), _lib.ptr(out), R, C, E, F,
                                   _lib.ptr(ws), nbytes, _lib.stream_ptr(dev)))
     return out
+
+
+def spmm_axpby(off, idx, w, x, R, beta, alpha, h):
+    """out[r,:] = beta * sum_j w[j] * x[idx[j],:] + alpha * h[r,:]  (h may be None)."""
+    lib = _lib.load()
+    dev = _lib.require_gpu(off, x, idx, w, h)
+    x = as_f32(x, "x")
+    h = as_f32(h, "h") if h is not None else None
+    C, F = x.shape
+    if h is not None and tuple(h.shape) != (R, F):
+        raise ValueError("h must be [%d, %d], got %s" % (R, F, tuple(h.shape)))
+    E = int(idx.shape[0]) if idx is not None else C
+    out = torch.empty((R, F), dtype=torch.float32, device=dev)
+    nbytes = _lib.query(lib.jgamd_spmm_csx_workspace, R, E, F)
+    ws = _lib.workspace(nbytes, dev)
+    _lib.check(lib.jgamd_spmm_csx_axpby(_lib.ptr(off), _lib.ptr(idx), _lib.ptr(w), _lib.ptr(x), _lib.ptr(out),
+                                        float(beta), float(alpha), _lib.ptr(h), R, C, E, F, _lib.ptr(ws), nbytes,
+                                        _lib.stream_ptr(dev)))
+    return out
+
+
+def both_orders(csc, csr):
+    """((off, idx, w) gathering into destinations, (off, idx, w) gathering into
+    sources) from whichever of the CSC / CSR objects is given; the missing one is
+    the cached transpose of the other."""
+    if csc is None and csr is None:
+        raise ValueError("need a CSC or a CSR")
+    if csc is not None:
+        fwd = (as_i32(csc.column_offset, "column_offset"), as_i32(csc.row_indices, "row_indices"),
+               as_f32(csc.edge_weight, "edge_weight"))
+    if csr is not None:
+        bwd = (as_i32(csr.row_offset, "row_offset"), as_i32(csr.column_indices, "column_indices"),
+               as_f32(csr.edge_weight, "edge_weight"))
+    if csc is None:
+        V = bwd[0].shape[0] - 1
+        fwd = transposed(csr, bwd[0], bwd[1], bwd[2], V, V)[:3]
+    if csr is None:
+        V = fwd[0].shape[0] - 1
+        bwd = transposed(csc, fwd[0], fwd[1], fwd[2], V, V)[:3]
+    return fwd, bwd

@@ -8,7 +8,15 @@ the benchmark import this package; the shipped library never does.
 
 Functions with no independent pin (see oracle.c header for the pins of the
 rest): none of the arithmetic.  The cuSPARSE-internal summation order behind
-the reference's SpmmCsr is "parity unpinned" (third-party, jittor==1.3.9.14).
+the reference's SpmmCsr and SpmmCoo is "parity unpinned" (third-party,
+jittor==1.3.9.14).  Pins of the numpy restatements at the end of this file:
+  spmmcoo       hand-derived fixture of tests/test_spmmcoo.py, dense fp64 product
+  toundirected  hand-derived fixture of tests/test_undirected.py, brute force over
+                Python sets; which of several equal (row, col) pairs survives is
+                "parity unpinned" (the reference's std::sort leaves it open)
+  appnp         K = 1 closed form, fp64 power iteration, the personalised
+                PageRank limit alpha * (I - (1 - alpha) A)^-1 h on a small graph
+  sgconv        dense fp64 A^K x W
 """
 import ctypes
 import os
@@ -261,3 +269,54 @@ def gat_forward_heads(h, csc, a_src, a_dst, slope=0.2):
         outs.append(o)
         alphas.append(al[:, 0])
     return np.stack(outs, axis=1), np.stack(alphas, axis=1)
+
+
+def spmmcoo(x, edge_index, edge_weight, trans_A=True):
+    """ops/spmmcoo.py:21-33: cuSPARSE COO product op(A) x with A = (row, col, w);
+    trans_A=True -> out[col] += w * x[row].  The library's summation order is not
+    specified; this restatement adds in edge order, in fp32."""
+    x = _f32(x)
+    row, col = np.asarray(edge_index[0]), np.asarray(edge_index[1])
+    w = _f32(edge_weight)
+    out = np.zeros_like(x)
+    dst, src = (col, row) if trans_A else (row, col)
+    for e in range(row.shape[0]):
+        out[dst[e]] = (out[dst[e]] + w[e] * x[src[e]]).astype(np.float32)
+    return out
+
+
+def toundirected(edge_index, edge_attr):
+    """ops/cpp/toundirected_op.cc:35-60: append (r, c, a) and (c, r, a) per edge, sort by
+    (row, col), keep the first of each run of equal pairs.  The sort here is stable."""
+    ei = np.asarray(edge_index)
+    attr = np.asarray(edge_attr).reshape(-1)
+    E = ei.shape[1]
+    rows = np.stack([ei[0], ei[1]], axis=1).reshape(-1)
+    cols = np.stack([ei[1], ei[0]], axis=1).reshape(-1)
+    data = np.repeat(attr, 2)
+    order = np.lexsort((cols, rows))            # stable; last key is the primary one
+    rows, cols, data = rows[order], cols[order], data[order]
+    keep = np.ones(2 * E, bool)
+    keep[1:] = (rows[1:] != rows[:-1]) | (cols[1:] != cols[:-1])
+    return np.stack([rows[keep], cols[keep]]).astype(np.int32), data[keep].reshape(1, -1)
+
+
+def appnp(x, csc, K, alpha):
+    """nn/conv/appnp_conv.py:42-51: K times x = propagate(x); x = x * (1 - alpha);
+    x = x + alpha * h, all in fp32."""
+    h = _f32(x)
+    x = h
+    for _ in range(K):
+        x = aggregate_with_weight(x, csc)
+        x = (x * np.float32(1 - alpha)).astype(np.float32)
+        x = (x + np.float32(alpha) * h).astype(np.float32)
+    return x
+
+
+def sgconv(x, csc, K, weight, bias=None):
+    """nn/conv/sg_conv.py:62-69: K products, then the linear layer (weight is [in, out])."""
+    x = _f32(x)
+    for _ in range(K):
+        x = aggregate_with_weight(x, csc)
+    out = (x.astype(np.float64) @ np.asarray(weight, np.float64)).astype(np.float32)
+    return out if bias is None else (out + _f32(bias)).astype(np.float32)

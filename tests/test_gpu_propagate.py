@@ -1,0 +1,200 @@
+"""Callers either side of the SpMM path on the GPU against the CPU oracle: the
+product with a fused row finish, APPNP / SGConv built on it, SpmmCoo and
+toUndirected.  fp32, 1e-5 relative to the sum of absolute terms."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from util import assert_close, dev, rand_graph, to_gpu
+
+pytestmark = pytest.mark.gpu
+GOLD = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_fixtures.json")))
+
+
+def graphs(V, E, hubs, seed):
+    from jittorgeometric_amd.ops import cootocsc, cootocsr
+    rng = np.random.default_rng(seed)
+    ei, _ = rand_graph(rng, V, E, hubs)
+    ei = ei[:, ei[0] != ei[1]]
+    ei, w = oracle.gcn_norm(ei, None, V)
+    ei = ei.astype(np.int32)
+    csc_o, csr_o = oracle.cootocsc(ei, w, V), oracle.cootocsr(ei, w, V)
+    return rng, ei, w, csc_o, csr_o, cootocsc(to_gpu(ei), to_gpu(w), V), cootocsr(to_gpu(ei), to_gpu(w), V)
+
+
+def abs_prod(x, csx):
+    """sum_j |w_j| |x[idx_j]| per output element, widened for long rows: the oracle adds a row's
+    terms one after the other in fp32, so its own sum carries about deg * 2^-24 of this."""
+    deg = np.diff(csx[1]).reshape(-1, 1).astype(np.float64)
+    return oracle.aggregate(np.abs(x), csx[0], csx[1], np.abs(csx[2])).astype(np.float64) * (1 + deg * 6e-3)
+
+
+@pytest.mark.parametrize("V,E,F,hubs,seed", [(1, 0, 4, 0, 0), (50, 0, 3, 0, 1), (300, 4000, 7, 0, 2),
+                                             (3000, 60000, 64, 2, 3), (2000, 150000, 128, 1, 4),
+                                             (5000, 40000, 33, 3, 5), (800, 30000, 256, 2, 6)])
+def test_product_with_row_finish(V, E, F, hubs, seed):
+    """beta * A x + alpha * h in one call; hub rows are cut into pieces, so the finish must be
+    applied exactly once to them too."""
+    from jittorgeometric_amd.ops._common import spmm_axpby
+    rng, ei, w, csc_o, csr_o, csc, csr = graphs(V, E, hubs, seed)
+    x = rng.standard_normal((V, F)).astype(np.float32)
+    h = rng.standard_normal((V, F)).astype(np.float32)
+    base = oracle.aggregate_with_weight(x, csc_o).astype(np.float64)
+    scale = abs_prod(x, csc_o)
+    args = (csc.column_offset, csc.row_indices, csc.edge_weight, to_gpu(x), V)
+    for beta, alpha, hh in ((0.9, 0.1, h), (1.0, 0.0, None), (-2.0, 0.5, h), (0.25, 0.0, h), (1.0, 1.0, x)):
+        got = spmm_axpby(*args, beta, alpha, None if hh is None else to_gpu(hh)).cpu().numpy()
+        want = beta * base + (alpha * hh.astype(np.float64) if hh is not None else 0.0)
+        assert_close(got, want, scale=abs(beta) * scale + (abs(alpha) * np.abs(hh) if hh is not None else 0.0) + 1e-30,
+                     what="beta=%g alpha=%g" % (beta, alpha))
+
+
+def test_row_finish_with_unaligned_h():
+    from jittorgeometric_amd.ops._common import spmm_axpby
+    V, F = 700, 64
+    rng, ei, w, csc_o, csr_o, csc, csr = graphs(V, 9000, 1, 11)
+    x = rng.standard_normal((V, F)).astype(np.float32)
+    h = rng.standard_normal((V, F)).astype(np.float32)
+    pad = torch.zeros(V * F + 1, device=dev())
+    pad[1:] = to_gpu(h).reshape(-1)
+    h_dev = pad[1:].reshape(V, F)
+    assert h_dev.data_ptr() % 16 != 0
+    got = spmm_axpby(csc.column_offset, csc.row_indices, csc.edge_weight, to_gpu(x), V, 0.8, 0.2, h_dev).cpu().numpy()
+    want = 0.8 * oracle.aggregate_with_weight(x, csc_o).astype(np.float64) + 0.2 * h
+    assert_close(got, want, scale=0.8 * abs_prod(x, csc_o) + 0.2 * np.abs(h))
+
+
+@pytest.mark.parametrize("spmm", [True, False])
+@pytest.mark.parametrize("V,E,F,K,hubs,seed", [(400, 5000, 16, 1, 0, 20), (3000, 50000, 41, 4, 2, 21),
+                                               (1500, 80000, 128, 10, 1, 22)])
+def test_appnp_forward_backward(V, E, F, K, hubs, seed, spmm):
+    from jittorgeometric_amd.nn import APPNP
+    alpha = 0.1
+    rng, ei, w, csc_o, csr_o, csc, csr = graphs(V, E, hubs, seed)
+    x = rng.standard_normal((V, F)).astype(np.float32)
+    g = rng.standard_normal((V, F)).astype(np.float32)
+    want = oracle.appnp(x, csc_o, K, alpha)
+    # magnitude of the terms: the same recursion on absolute values
+    mag = oracle.appnp(np.abs(x), (csc_o[0], csc_o[1], np.abs(csc_o[2])), K, alpha).astype(np.float64)
+    mag = mag * (1 + np.diff(csc_o[1]).reshape(-1, 1) * 6e-3)
+    outs = []
+    for fused in (True, False):
+        xt = to_gpu(x).requires_grad_(True)
+        layer = APPNP(K, alpha, spmm=spmm, fused=fused)
+        out = layer(xt, csc, csr)
+        out.backward(to_gpu(g))
+        assert_close(out.detach().cpu().numpy(), want, scale=mag, rtol=3e-5, what="forward fused=%s" % fused)
+        outs.append((out.detach().cpu().numpy(), xt.grad.cpu().numpy()))
+    # gradient: the transposed recursion, g_x = M^K g + alpha * sum_{i<K} M^i g with M = (1-alpha) A^T,
+    # restated with the oracle's CSR aggregation in fp64
+    v = g.astype(np.float64)
+    gmag = np.abs(g).astype(np.float64)
+    for _ in range(K):
+        v = (1 - alpha) * oracle.aggregate(v.astype(np.float32), *csr_o).astype(np.float64) + alpha * g
+        gmag = (1 - alpha) * oracle.aggregate(gmag.astype(np.float32), csr_o[0], csr_o[1], np.abs(csr_o[2])) + alpha * np.abs(g)
+    for (_, grad), name in zip(outs, ("fused", "chain")):
+        assert_close(grad, v, scale=gmag, rtol=5e-5, what="gradient " + name)
+    assert_close(outs[0][0], outs[1][0], scale=mag, rtol=2e-5, what="fused vs chain")
+
+
+def test_propagate_axpby_gradients():
+    from jittorgeometric_amd.ops import propagate_axpby
+    V, F = 500, 24
+    rng, ei, w, csc_o, csr_o, csc, csr = graphs(V, 6000, 1, 30)
+    x = rng.standard_normal((V, F)).astype(np.float32)
+    h = rng.standard_normal((V, F)).astype(np.float32)
+    g = rng.standard_normal((V, F)).astype(np.float32)
+    xt, ht = to_gpu(x).requires_grad_(True), to_gpu(h).requires_grad_(True)
+    out = propagate_axpby(xt, ht, csc, csr, beta=0.7, alpha=0.3)
+    out.backward(to_gpu(g))
+    assert_close(out.detach().cpu().numpy(), 0.7 * oracle.aggregate_with_weight(x, csc_o).astype(np.float64) + 0.3 * h,
+                 scale=0.7 * abs_prod(x, csc_o) + 0.3 * np.abs(h))
+    assert_close(xt.grad.cpu().numpy(), 0.7 * oracle.aggregate_with_weight_grad(g, csr_o).astype(np.float64),
+                 scale=0.7 * abs_prod(g, csr_o) + 1e-30)
+    assert_close(ht.grad.cpu().numpy(), 0.3 * g.astype(np.float64))
+    # only one of the two orders given: the other is the cached transpose
+    out2 = propagate_axpby(to_gpu(x), to_gpu(h), None, csr, beta=0.7, alpha=0.3)
+    assert_close(out2.cpu().numpy(), out.detach().cpu().numpy(), scale=0.7 * abs_prod(x, csc_o) + 0.3 * np.abs(h))
+
+
+@pytest.mark.parametrize("spmm", [True, False])
+def test_sgconv_forward_backward(spmm):
+    from jittorgeometric_amd.nn import SGConv
+    V, Fin, Fout, K = 1200, 48, 7, 3
+    rng, ei, w, csc_o, csr_o, csc, csr = graphs(V, 20000, 1, 40)
+    x = rng.standard_normal((V, Fin)).astype(np.float32)
+    layer = SGConv(Fin, Fout, K=K, spmm=spmm).to(dev())
+    with torch.no_grad():
+        layer.bias.copy_(to_gpu(rng.standard_normal(Fout).astype(np.float32)))
+    W, b = layer.weight.detach().cpu().numpy(), layer.bias.detach().cpu().numpy()
+    xt = to_gpu(x).requires_grad_(True)
+    out = layer(xt, csc, csr)
+    want = oracle.sgconv(x, csc_o, K, W, b)
+    assert_close(out.detach().cpu().numpy(), want, scale=np.abs(want) + 1.0, rtol=1e-4)
+    g = rng.standard_normal((V, Fout)).astype(np.float32)
+    out.backward(to_gpu(g))
+    # d/dx = (A^T)^K (g W^T), d/dW = (A^K x)^T g
+    v = (g.astype(np.float64) @ W.T.astype(np.float64)).astype(np.float32)
+    ak = x
+    for _ in range(K):
+        v = oracle.aggregate_with_weight_grad(v, csr_o)
+        ak = oracle.aggregate_with_weight(ak, csc_o)
+    assert_close(xt.grad.cpu().numpy(), v, scale=np.abs(v) + 1.0, rtol=1e-4)
+    gw = ak.astype(np.float64).T @ g.astype(np.float64)
+    assert_close(layer.weight.grad.cpu().numpy(), gw, scale=np.abs(gw) + 1.0, rtol=1e-4)
+    assert_close(layer.bias.grad.cpu().numpy(), g.astype(np.float64).sum(0), scale=np.abs(g).sum(0), rtol=1e-5)
+
+
+def test_spmmcoo_reference_fixture_and_random():
+    from jittorgeometric_amd.ops import SpmmCoo
+    f = GOLD["spmmcoo_v3"]
+    x = torch.tensor(f["x"], device=dev())
+    ei = torch.tensor(f["edge_index"], dtype=torch.int32, device=dev())
+    w = torch.tensor(f["edge_weight"], device=dev())
+    assert SpmmCoo(x, ei, w).tolist() == f["out"]
+    assert SpmmCoo(x, ei, w, trans_A=False).tolist() == f["out_no_trans"]
+    rng = np.random.default_rng(50)
+    V, E, F = 4000, 70000, 40
+    ein, wn = rand_graph(rng, V, E, 2)
+    xn = rng.standard_normal((V, F)).astype(np.float32)
+    gn = rng.standard_normal((V, F)).astype(np.float32)
+    for trans in (True, False):
+        xt = to_gpu(xn).requires_grad_(True)
+        out = SpmmCoo(xt, to_gpu(ein), to_gpu(wn), trans_A=trans)
+        out.backward(to_gpu(gn))
+        want = oracle.spmmcoo(xn, ein, wn, trans_A=trans)
+        scale = oracle.spmmcoo(np.abs(xn), ein, np.abs(wn), trans_A=trans).astype(np.float64)
+        # the oracle adds in edge order, one fp32 rounding per edge: hub rows carry deg * 2^-24
+        deg = np.bincount(ein[1] if trans else ein[0], minlength=V).reshape(V, 1)
+        assert_close(out.detach().cpu().numpy(), want, scale=scale * (1 + deg * 6e-3), what="trans_A=%s" % trans)
+        wantg = oracle.spmmcoo(gn, ein, wn, trans_A=not trans)
+        gscale = oracle.spmmcoo(np.abs(gn), ein, np.abs(wn), trans_A=not trans).astype(np.float64)
+        degg = np.bincount(ein[0] if trans else ein[1], minlength=V).reshape(V, 1)
+        assert_close(xt.grad.cpu().numpy(), wantg, scale=gscale * (1 + degg * 6e-3), what="grad trans_A=%s" % trans)
+    with pytest.raises(Exception):
+        SpmmCoo(x, ei, w, trans_B=True)
+
+
+@pytest.mark.parametrize("V,E,seed", [(3, 0, 0), (1, 5, 1), (8, 40, 2), (2000, 30000, 3), (50000, 200000, 4)])
+def test_toundirected(V, E, seed):
+    from jittorgeometric_amd.ops import toUndirected
+    rng = np.random.default_rng(seed)
+    ei = rng.integers(0, V, (2, E)).astype(np.int32)
+    attr = rng.standard_normal(E).astype(np.float32)
+    ni, na = toUndirected(to_gpu(ei), to_gpu(attr), V)
+    wi, wa = oracle.toundirected(ei, attr)
+    assert np.array_equal(ni.cpu().numpy(), wi)
+    assert np.array_equal(na.cpu().numpy().view(np.int32), wa.view(np.int32))
+    assert tuple(na.shape) == (1, wi.shape[1])
+
+
+def test_toundirected_reference_fixture():
+    from jittorgeometric_amd.ops import toUndirected
+    f = GOLD["toundirected_v3"]
+    ni, na = toUndirected(torch.tensor(f["edge_index"], device=dev()), torch.tensor(f["edge_attr"], device=dev()),
+                          f["num_nodes"])
+    assert ni.tolist() == f["new_edge_index"] and na.tolist() == f["new_edge_attr"]

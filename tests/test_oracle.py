@@ -292,3 +292,76 @@ def test_oracle_reproduces_committed_vectors():
             assert np.array_equal(a, b), k
         else:
             np.testing.assert_allclose(b, a, rtol=1e-6, atol=1e-7, err_msg=k)
+
+
+# ------------------------------------------- callers either side of the path ---
+
+def test_spmmcoo_reference_fixture_and_dense_product():
+    g = GOLD["spmmcoo_v3"]
+    x = np.array(g["x"], np.float32)
+    ei = np.array(g["edge_index"], np.int32)
+    w = np.array(g["edge_weight"], np.float32)
+    assert oracle.spmmcoo(x, ei, w).tolist() == g["out"]
+    assert oracle.spmmcoo(x, ei, w, trans_A=False).tolist() == g["out_no_trans"]
+    rng = np.random.default_rng(70)
+    ei, w = rand_graph(rng, 60, 700)
+    x = rng.standard_normal((60, 9)).astype(np.float32)
+    A = sp.coo_matrix((w.astype(np.float64), (ei[0], ei[1])), shape=(60, 60)).tocsr()
+    np.testing.assert_allclose(oracle.spmmcoo(x, ei, w), A.T @ x.astype(np.float64), rtol=1e-5, atol=2e-5)
+    np.testing.assert_allclose(oracle.spmmcoo(x, ei, w, trans_A=False), A @ x.astype(np.float64), rtol=1e-5, atol=2e-5)
+    # same quantity as the CSC aggregation (tests/test_mp_spmm.py:28-36 prints them side by side)
+    np.testing.assert_allclose(oracle.spmmcoo(x, ei, w), oracle.aggregate_with_weight(x, oracle.cootocsc(ei, w, 60)),
+                               rtol=1e-5, atol=2e-5)
+
+
+def test_toundirected_reference_fixture_and_bruteforce():
+    g = GOLD["toundirected_v3"]
+    ni, na = oracle.toundirected(np.array(g["edge_index"], np.int32), np.array(g["edge_attr"], np.float32))
+    assert ni.tolist() == g["new_edge_index"] and na.tolist() == g["new_edge_attr"]
+    rng = np.random.default_rng(71)
+    for _ in range(10):
+        V, E = int(rng.integers(1, 8)), int(rng.integers(0, 25))
+        ei = rng.integers(0, V, (2, E)).astype(np.int32)
+        attr = rng.integers(0, 100, E).astype(np.float32)
+        ni, na = oracle.toundirected(ei, attr)
+        first = {}
+        for e in range(E):                      # append order: forward, then reversed
+            for pair in ((int(ei[0, e]), int(ei[1, e])), (int(ei[1, e]), int(ei[0, e]))):
+                first.setdefault(pair, float(attr[e]))
+        want = sorted(first)
+        assert [tuple(p) for p in ni.T.tolist()] == want
+        assert na.reshape(-1).tolist() == [first[p] for p in want]
+        assert na.shape == (1, len(want))
+
+
+def test_appnp_closed_forms():
+    rng = np.random.default_rng(72)
+    V = 40
+    ei, _ = rand_graph(rng, V, 300, loops=False)
+    ei, w = oracle.gcn_norm(ei, None, V)
+    csc = oracle.cootocsc(ei, w, V)
+    A = sp.coo_matrix((w.astype(np.float64), (ei[1], ei[0])), shape=(V, V)).toarray()
+    h = rng.standard_normal((V, 5)).astype(np.float32)
+    alpha = 0.1
+    np.testing.assert_allclose(oracle.appnp(h, csc, 1, alpha), (1 - alpha) * (A @ h) + alpha * h, rtol=1e-5, atol=1e-6)
+    x = h.astype(np.float64)
+    for _ in range(7):
+        x = (1 - alpha) * (A @ x) + alpha * h
+    np.testing.assert_allclose(oracle.appnp(h, csc, 7, alpha), x, rtol=1e-5, atol=1e-5)
+    limit = alpha * np.linalg.solve(np.eye(V) - (1 - alpha) * A, h.astype(np.float64))
+    np.testing.assert_allclose(oracle.appnp(h, csc, 300, alpha), limit, rtol=1e-4, atol=1e-5)
+    assert np.array_equal(oracle.appnp(h, csc, 0, alpha), h)
+
+
+def test_sgconv_dense_closed_form():
+    rng = np.random.default_rng(73)
+    V = 30
+    ei, _ = rand_graph(rng, V, 200, loops=False)
+    ei, w = oracle.gcn_norm(ei, None, V)
+    csc = oracle.cootocsc(ei, w, V)
+    A = sp.coo_matrix((w.astype(np.float64), (ei[1], ei[0])), shape=(V, V)).toarray()
+    x = rng.standard_normal((V, 6)).astype(np.float32)
+    W = rng.standard_normal((6, 4)).astype(np.float32)
+    b = rng.standard_normal(4).astype(np.float32)
+    want = np.linalg.matrix_power(A, 3) @ x.astype(np.float64) @ W.astype(np.float64) + b
+    np.testing.assert_allclose(oracle.sgconv(x, csc, 3, W, b), want, rtol=1e-5, atol=1e-5)
