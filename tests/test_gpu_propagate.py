@@ -198,3 +198,22 @@ def test_toundirected_reference_fixture():
     ni, na = toUndirected(torch.tensor(f["edge_index"], device=dev()), torch.tensor(f["edge_attr"], device=dev()),
                           f["num_nodes"])
     assert ni.tolist() == f["new_edge_index"] and na.tolist() == f["new_edge_attr"]
+
+
+def test_row_finish_on_wide_rows_runs_as_its_own_pass():
+    """x larger than 4 GiB: the product takes the 64-bit address kernels, which have no fused
+    finish; the blend then runs as a separate pass with the same result."""
+    from jittorgeometric_amd.ops._common import spmm, spmm_axpby
+    rng = np.random.default_rng(46)
+    C, F, R, E = 4_300_000, 256, 3000, 40000
+    x = torch.empty((C, F), dtype=torch.float32, device=dev())
+    x.normal_()
+    src = rng.integers(0, C, E).astype(np.int32)
+    dst = rng.integers(0, R, E).astype(np.int32)
+    w = rng.standard_normal(E).astype(np.float32)
+    row, off, cw = oracle.cootocsc(np.stack([src, dst]), w, R)
+    h = torch.randn(R, F, device=dev())
+    plain = spmm(to_gpu(off), to_gpu(row), to_gpu(cw), x, R)
+    got = spmm_axpby(to_gpu(off), to_gpu(row), to_gpu(cw), x, R, 0.75, 0.25, h)
+    want = 0.75 * plain.double() + 0.25 * h.double()
+    assert_close(got.cpu().numpy(), want.cpu().numpy(), scale=(0.75 * plain.abs() + 0.25 * h.abs()).cpu().numpy() + 1e-6)
