@@ -123,16 +123,18 @@ int32_t jgamd_spmm_csx(const int32_t *off, const int32_t *idx, const float *w, c
 
 /* jgamd_spmm_csx with a row finish:
  *   out[r,:] = beta * sum_j w[j] * x[idx[j],:] + alpha * h[r,:]
- * h is [R,F] (NULL or alpha == 0 drops the term) and may be x itself; out must
- * not overlap x or h.  One call is one hop of the reference's polynomial
+ * h is [h_rows,F] with h_rows = R, or 1 for one row added to every output row
+ * (a layer's bias: nn/conv/gcn_conv.py:109-110 adds it after the product);
+ * NULL or alpha == 0 drops the term.  h may be x itself; out must not overlap
+ * x or h.  One call is one hop of the reference's polynomial
  * propagation layers, whose Python loop runs the product and then two
  * element-wise passes (nn/conv/appnp_conv.py:42-51: x = propagate(x);
  * x = x * (1 - alpha); x = x + alpha * h).  Same workspace as jgamd_spmm_csx.
  */
 int32_t jgamd_spmm_csx_axpby(const int32_t *off, const int32_t *idx, const float *w,
                              const float *x, float *out, float beta, float alpha,
-                             const float *h, int32_t R, int32_t C, int64_t E, int32_t F,
-                             void *ws, size_t ws_bytes, void *stream);
+                             const float *h, int32_t h_rows, int32_t R, int32_t C, int64_t E,
+                             int32_t F, void *ws, size_t ws_bytes, void *stream);
 
 /* Benchmark support; no counterpart in the reference.  Runs jgamd_spmm_csx
  * `iters` times on `stream`, with one hipEvent pair around each launch of the

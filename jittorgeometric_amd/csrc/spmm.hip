@@ -97,6 +97,7 @@ __global__ void spmm_chunk_rows(const int32_t *__restrict__ off, int R, int chun
 struct RowFinish {
     float beta, alpha;
     const float *h;
+    int h_stride;   // floats between the rows of h: F, or 0 when one row serves every output row
 };
 
 template <int VEC, int NT, int UNROLL, bool WIDE, bool LDS, bool EPI>
@@ -157,7 +158,7 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__rest
     auto fetch_h = [&]() {
         if constexpr (EPI) {
             if (fin.h) {
-                const float *src = fin.h + (size_t)min(r, R - 1) * F;
+                const float *src = fin.h + (size_t)min(r, R - 1) * fin.h_stride;
 #pragma unroll
                 for (int t = 0; t < NT; t++) vload<VEC>(hrow[t], src + fo[t]);
             } else {
@@ -400,7 +401,7 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_fixup(const int32_t *__rest
 #pragma unroll
             for (int t = 0; t < NT; t++) {
                 const int f = f0 + t * kWave * VEC;
-                vload<VEC>(hv[t], fin.h + (size_t)r0 * F + (f < F ? f : 0));
+                vload<VEC>(hv[t], fin.h + (size_t)r0 * fin.h_stride + (f < F ? f : 0));
 #pragma unroll
                 for (int v = 0; v < VEC; v++) acc[t][v] = fmaf(fin.alpha, hv[t][v], acc[t][v]);
             }
@@ -413,11 +414,11 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_fixup(const int32_t *__rest
 
 // out = beta * out + alpha * h, element-wise (the finish as a pass of its own, for the
 // shapes the fused kernels do not cover).
-__global__ void spmm_finish_rows(float *__restrict__ out, const float *__restrict__ h, int64_t n, float beta,
-                                 float alpha)
+__global__ void spmm_finish_rows(float *__restrict__ out, const float *__restrict__ h, int64_t n, int F,
+                                 int h_stride, float beta, float alpha)
 {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) out[i] = fmaf(alpha, h ? h[i] : 0.f, beta * out[i]);
+    if (i < n) out[i] = fmaf(alpha, h ? h[h_stride ? i : i % F] : 0.f, beta * out[i]);
 }
 
 // ------------------------------------------------------------------ host ---
@@ -490,7 +491,7 @@ static void launch_spmm(const SpmmShape &s, const int32_t *off, const int32_t *i
     const bool narrow = (uint64_t)C * (uint64_t)F * 4u < ((uint64_t)1 << 32);
     // the fused row finish exists for 32-bit offsets only; wide shapes finish in a pass of their own
     const bool fused = fin && narrow;
-    const RowFinish none{1.f, 0.f, nullptr};
+    const RowFinish none{1.f, 0.f, nullptr, 0};
     const RowFinish f = fused ? *fin : none;
 #define JG_GO(W, L, P)                                                                                              \
     hipLaunchKernelGGL((spmm_merge<VEC, NT, U, W, L, P>), grid, block, 0, st, off, idx, w, x, out, partial,         \
@@ -515,8 +516,8 @@ static void launch_spmm(const SpmmShape &s, const int32_t *off, const int32_t *i
                            s.chunk, s.nchunks, f);
     if (fin && !fused) {
         const int64_t n = (int64_t)R * F;
-        hipLaunchKernelGGL(spmm_finish_rows, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, st, out, fin->h, n,
-                           fin->beta, fin->alpha);
+        hipLaunchKernelGGL(spmm_finish_rows, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, st, out, fin->h, n, F,
+                           fin->h_stride, fin->beta, fin->alpha);
     }
 }
 
@@ -591,10 +592,13 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx(const i
 
 extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_axpby(
     const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out, float beta, float alpha,
-    const float *h, int32_t R, int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, void *stream)
+    const float *h, int32_t h_rows, int32_t R, int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes,
+    void *stream)
 {
     if (h && (((uintptr_t)h & 3) != 0)) return fail(JGAMD_ERR_ALIGN, "spmm_csx_axpby: h not 4-byte aligned");
-    const RowFinish fin{beta, alpha, alpha != 0.f ? h : nullptr};
+    if (h && h_rows != 1 && h_rows != R)
+        return fail(JGAMD_ERR_SIZE, "spmm_csx_axpby: h has %d rows, expected %d or 1", h_rows, R);
+    const RowFinish fin{beta, alpha, alpha != 0.f ? h : nullptr, h_rows == 1 ? 0 : F};
     return spmm_call(off, idx, w, x, out, R, C, E, F, ws, ws_bytes, stream, nullptr, nullptr, &fin);
 }
 

@@ -4,6 +4,7 @@ import torch
 from torch import nn
 
 from ...ops import SpmmCsr, aggregateWithWeight, cootocsc
+from ...ops.propagate import aggregate_bias
 from ...utils import add_remaining_self_loops
 from ...utils.num_nodes import maybe_num_nodes
 from ..dense import add_bias, xw
@@ -66,6 +67,9 @@ class GCNConv(nn.Module):
 
     def forward(self, x, csc, csr):
         x = xw(x, self.weight)
+        if self.bias is not None and x.is_cuda and x.dim() == 2:
+            # product and bias in one kernel; spmm=True only needs the CSR (:96-97)
+            return aggregate_bias(x, self.bias, None if self.spmm and csr is not None else csc, csr)
         if self.spmm:
             out = self.propagate_spmm(x=x, csr=csr)
         else:

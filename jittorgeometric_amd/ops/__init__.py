@@ -7,7 +7,7 @@ from .edgesoftmax import EdgeSoftmax  # noqa: F401
 from .gat import gat_aggregate  # noqa: F401
 from .scatterToEdge import ScatterToEdge  # noqa: F401
 from .scatterToVertex import ScatterToVertex  # noqa: F401
-from .propagate import appnp_propagate, propagate_axpby  # noqa: F401
+from .propagate import aggregate_bias, appnp_propagate, propagate_axpby  # noqa: F401
 from .spmmcoo import SpmmCoo  # noqa: F401
 from .spmmcsr import SpmmCsr  # noqa: F401
 from .toundirected import toUndirected  # noqa: F401

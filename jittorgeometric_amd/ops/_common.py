@@ -70,20 +70,25 @@ def spmm(off, idx, w, x, R):
 
 
 def spmm_axpby(off, idx, w, x, R, beta, alpha, h):
-    """out[r,:] = beta * sum_j w[j] * x[idx[j],:] + alpha * h[r,:]  (h may be None)."""
+    """out[r,:] = beta * sum_j w[j] * x[idx[j],:] + alpha * h[r,:]; h is [R,F], or [F] / [1,F]
+    for one row added to every output row, or None."""
     lib = _lib.load()
     dev = _lib.require_gpu(off, x, idx, w, h)
     x = as_f32(x, "x")
     h = as_f32(h, "h") if h is not None else None
     C, F = x.shape
-    if h is not None and tuple(h.shape) != (R, F):
-        raise ValueError("h must be [%d, %d], got %s" % (R, F, tuple(h.shape)))
+    h_rows = R
+    if h is not None:
+        if h.dim() == 1 or (h.dim() == 2 and h.shape[0] == 1 and R != 1):
+            h_rows = 1
+        if h.numel() != h_rows * F:
+            raise ValueError("h must be [%d, %d] or [%d], got %s" % (R, F, F, tuple(h.shape)))
     E = int(idx.shape[0]) if idx is not None else C
     out = torch.empty((R, F), dtype=torch.float32, device=dev)
     nbytes = _lib.query(lib.jgamd_spmm_csx_workspace, R, E, F)
     ws = _lib.workspace(nbytes, dev)
     _lib.check(lib.jgamd_spmm_csx_axpby(_lib.ptr(off), _lib.ptr(idx), _lib.ptr(w), _lib.ptr(x), _lib.ptr(out),
-                                        float(beta), float(alpha), _lib.ptr(h), R, C, E, F, _lib.ptr(ws), nbytes,
+                                        float(beta), float(alpha), _lib.ptr(h), h_rows, R, C, E, F, _lib.ptr(ws), nbytes,
                                         _lib.stream_ptr(dev)))
     return out
 

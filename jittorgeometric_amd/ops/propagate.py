@@ -32,6 +32,31 @@ def propagate_axpby(x, h, csc, csr, beta=1.0, alpha=0.0):
     return HopFunc.apply(x, h, fwd, bwd, float(beta), float(alpha))
 
 
+class AggregateBiasFunc(torch.autograd.Function):
+    """A x + bias with the bias added in the product's row store
+    (nn/conv/gcn_conv.py:102-110 adds it in a pass of its own)."""
+
+    @staticmethod
+    def forward(ctx, x, bias, fwd, bwd):
+        ctx.bwd = bwd
+        return spmm_axpby(fwd[0], fwd[1], fwd[2], x, x.shape[0], 1.0, 1.0, bias)
+
+    @staticmethod
+    def backward(ctx, g):
+        from ..nn.dense import column_sum
+        g = g.contiguous()
+        off, idx, w = ctx.bwd
+        gx = spmm_axpby(off, idx, w, g, g.shape[0], 1.0, 0.0, None) if ctx.needs_input_grad[0] else None
+        gb = column_sum(g) if ctx.needs_input_grad[1] else None
+        return gx, gb, None, None
+
+
+def aggregate_bias(x, bias, csc, csr):
+    """aggregateWithWeight(x, csc, csr) + bias in one pass; either of csc / csr may be None."""
+    fwd, bwd = both_orders(csc, csr)
+    return AggregateBiasFunc.apply(x.contiguous(), bias, fwd, bwd)
+
+
 class AppnpFunc(torch.autograd.Function):
     """K hops x <- (1 - alpha) A x + alpha h with x_0 = h.  With M = (1 - alpha) A^T the
     gradient is M^K g + alpha * (M^(K-1) + ... + M + I) g, evaluated by the same hop:

@@ -217,3 +217,21 @@ def test_row_finish_on_wide_rows_runs_as_its_own_pass():
     got = spmm_axpby(to_gpu(off), to_gpu(row), to_gpu(cw), x, R, 0.75, 0.25, h)
     want = 0.75 * plain.double() + 0.25 * h.double()
     assert_close(got.cpu().numpy(), want.cpu().numpy(), scale=(0.75 * plain.abs() + 0.25 * h.abs()).cpu().numpy() + 1e-6)
+
+
+@pytest.mark.parametrize("F", [7, 64, 130])
+def test_aggregate_with_bias_row(F):
+    """One row of h added to every output row (a layer's bias), and its gradients."""
+    from jittorgeometric_amd.ops import aggregate_bias
+    V = 2500
+    rng, ei, w, csc_o, csr_o, csc, csr = graphs(V, 40000, 2, 60 + F)
+    x = rng.standard_normal((V, F)).astype(np.float32)
+    b = rng.standard_normal(F).astype(np.float32)
+    g = rng.standard_normal((V, F)).astype(np.float32)
+    xt, bt = to_gpu(x).requires_grad_(True), to_gpu(b).requires_grad_(True)
+    out = aggregate_bias(xt, bt, csc, csr)
+    out.backward(to_gpu(g))
+    want = oracle.aggregate_with_weight(x, csc_o).astype(np.float64) + b
+    assert_close(out.detach().cpu().numpy(), want, scale=abs_prod(x, csc_o) + np.abs(b))
+    assert_close(xt.grad.cpu().numpy(), oracle.aggregate_with_weight_grad(g, csr_o), scale=abs_prod(g, csr_o) + 1e-30)
+    assert_close(bt.grad.cpu().numpy(), g.astype(np.float64).sum(0), scale=np.abs(g).sum(0))
