@@ -209,7 +209,7 @@ def main():
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": args.traffic_bytes,
                      "traffic_source": "profiles/bench_workload_mi355x.txt",
                      "traffic_rate_gbps": round(args.traffic_bytes / (k_ms.value * 1e-3) / 1e9, 1) if args.traffic_bytes else None,
-                     "kernel": "spmm_merge<2,1,16,false,true>", "kernel_ms": round(k_ms.value, 4),
+                     "kernel": "spmm_merge<2,1,16,false,true,false>", "kernel_ms": round(k_ms.value, 4),
                      "call_ms": round(c_ms.value, 4), "algorithmic_bytes": bytes_step},
         "cpu_baseline": cpu,
     }
