@@ -1,1 +1,1 @@
-from .conv import APPNP, GATConv, GCNConv, MessagePassingNts, SAGEConv, SGConv, gcn_norm, sage_norm  # noqa: F401
+from .conv import APPNP, GATConv, GCNConv, GPRGNN, MessagePassingNts, SAGEConv, SGConv, gcn_norm, sage_norm  # noqa: F401

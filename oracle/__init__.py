@@ -17,6 +17,7 @@ jittor==1.3.9.14).  Pins of the numpy restatements at the end of this file:
   appnp         K = 1 closed form, fp64 power iteration, the personalised
                 PageRank limit alpha * (I - (1 - alpha) A)^-1 h on a small graph
   sgconv        dense fp64 A^K x W
+  gprgnn        dense fp64 sum_k temp[k] A^k x
 """
 import ctypes
 import os
@@ -320,3 +321,14 @@ def sgconv(x, csc, K, weight, bias=None):
         x = aggregate_with_weight(x, csc)
     out = (x.astype(np.float64) @ np.asarray(weight, np.float64)).astype(np.float32)
     return out if bias is None else (out + _f32(bias)).astype(np.float32)
+
+
+def gprgnn(x, csc, temp):
+    """nn/conv/gpr_conv.py:80-88: out = x * temp[0]; K times x = propagate(x); out = out + temp[k+1] * x."""
+    x = _f32(x)
+    temp = _f32(temp)
+    out = (x * temp[0]).astype(np.float32)
+    for k in range(temp.shape[0] - 1):
+        x = aggregate_with_weight(x, csc)
+        out = (out + temp[k + 1] * x).astype(np.float32)
+    return out

@@ -235,3 +235,34 @@ def test_aggregate_with_bias_row(F):
     assert_close(out.detach().cpu().numpy(), want, scale=abs_prod(x, csc_o) + np.abs(b))
     assert_close(xt.grad.cpu().numpy(), oracle.aggregate_with_weight_grad(g, csr_o), scale=abs_prod(g, csr_o) + 1e-30)
     assert_close(bt.grad.cpu().numpy(), g.astype(np.float64).sum(0), scale=np.abs(g).sum(0))
+
+
+@pytest.mark.parametrize("init", ["PPR", "SGC", "NPPR", "WS"])
+def test_gprgnn_forward_backward(init):
+    from jittorgeometric_amd.nn import GPRGNN
+    V, F, K = 1500, 20, 4
+    rng, ei, w, csc_o, csr_o, csc, csr = graphs(V, 25000, 1, 80)
+    x = rng.standard_normal((V, F)).astype(np.float32)
+    g = rng.standard_normal((V, F)).astype(np.float32)
+    layer = GPRGNN(K, 0.1, init, spmm=False, Gamma=[0.5, -0.2, 0.1, 0.3, 0.05]).to(dev())
+    temp = layer.temp.detach().cpu().numpy()
+    if init == "PPR":
+        assert np.allclose(temp, [0.1, 0.09, 0.081, 0.0729, 0.6561])
+    xt = to_gpu(x).requires_grad_(True)
+    out = layer(xt, csc, csr)
+    out.backward(to_gpu(g))
+    want = oracle.gprgnn(x, csc_o, temp)
+    mag = oracle.gprgnn(np.abs(x), (csc_o[0], csc_o[1], np.abs(csc_o[2])), np.abs(temp)).astype(np.float64)
+    mag = mag * (1 + np.diff(csc_o[1]).reshape(-1, 1) * 6e-3)
+    assert_close(out.detach().cpu().numpy(), want, scale=mag + 1e-30, rtol=3e-5)
+    # d/dtemp[k] = <g, A^k x>;  d/dx = sum_k temp[k] (A^T)^k g
+    xs, gs = [x], [g]
+    for _ in range(K):
+        xs.append(oracle.aggregate_with_weight(xs[-1], csc_o))
+        gs.append(oracle.aggregate_with_weight_grad(gs[-1], csr_o))
+    gt = np.array([(g.astype(np.float64) * xk).sum() for xk in xs])
+    gts = np.array([(np.abs(g).astype(np.float64) * np.abs(xk)).sum() for xk in xs])
+    assert_close(layer.temp.grad.cpu().numpy(), gt, scale=gts, rtol=1e-4)
+    gx = sum(float(temp[k]) * gs[k].astype(np.float64) for k in range(K + 1))
+    gxs = sum(abs(float(temp[k])) * np.abs(gs[k]).astype(np.float64) for k in range(K + 1))
+    assert_close(xt.grad.cpu().numpy(), gx, scale=gxs + 1e-3, rtol=1e-4)

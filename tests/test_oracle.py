@@ -365,3 +365,16 @@ def test_sgconv_dense_closed_form():
     b = rng.standard_normal(4).astype(np.float32)
     want = np.linalg.matrix_power(A, 3) @ x.astype(np.float64) @ W.astype(np.float64) + b
     np.testing.assert_allclose(oracle.sgconv(x, csc, 3, W, b), want, rtol=1e-5, atol=1e-5)
+
+
+def test_gprgnn_dense_closed_form():
+    rng = np.random.default_rng(74)
+    V = 30
+    ei, _ = rand_graph(rng, V, 200, loops=False)
+    ei, w = oracle.gcn_norm(ei, None, V)
+    csc = oracle.cootocsc(ei, w, V)
+    A = sp.coo_matrix((w.astype(np.float64), (ei[1], ei[0])), shape=(V, V)).toarray()
+    x = rng.standard_normal((V, 6)).astype(np.float32)
+    temp = rng.standard_normal(5).astype(np.float32)
+    want = sum(float(temp[k]) * np.linalg.matrix_power(A, k) @ x.astype(np.float64) for k in range(5))
+    np.testing.assert_allclose(oracle.gprgnn(x, csc, temp), want, rtol=1e-5, atol=1e-5)
