@@ -230,6 +230,23 @@ int32_t jgamd_column_sum_workspace(int64_t R, int32_t F, size_t *bytes);
 int32_t jgamd_column_sum(const float *x, float *out, int64_t R, int32_t F, void *ws,
                          size_t ws_bytes, void *stream);
 
+/* ------------------------------------------------------------------------
+ * Neighbour sampling for one layer of a sampled subgraph: for destination
+ * dst[i] (a column of the global CSC arrays g_off / g_idx with g_nodes
+ * columns) write its neighbours to out[layer_off[i] .. layer_off[i+1]): all of
+ * them, in order, when it has at most `fanout` (or fanout < 0), else `fanout`
+ * distinct ones, in the order they have in g_idx.  Replaces
+ * sampleprocessing_op.sampleprocessing(fanout, dst, column_offset,
+ * row_indices, global_column_offset, global_row_indices)
+ * (ops/sampleprocessing.py:34, ops/cpp/sampleprocessing_op.cc:47-84,88-160).
+ * The reference draws from rand() / a clock-seeded curand state; here the
+ * draw is a pure function of (seed, destination id).  fanout <= 1024.
+ */
+int32_t jgamd_sample_neighbors(const int32_t *dst, const int32_t *layer_off, const int32_t *g_off,
+                               const int32_t *g_idx, int32_t n_dst, int32_t g_nodes,
+                               int32_t fanout, int64_t out_len, uint64_t seed, int32_t *out,
+                               void *stream);
+
 #ifdef __cplusplus
 }
 #endif

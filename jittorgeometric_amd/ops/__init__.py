@@ -3,8 +3,12 @@
 from .aggregateWithWeight import aggregateWithWeight  # noqa: F401
 from .cootocsc import cootocsc  # noqa: F401
 from .cootocsr import cootocsr  # noqa: F401
+from .csctocsr import csctocsr  # noqa: F401
 from .edgesoftmax import EdgeSoftmax  # noqa: F401
 from .gat import gat_aggregate  # noqa: F401
+from .getweight import getweight  # noqa: F401
+from .gpuinitco import gpuinitco  # noqa: F401
+from .sampleprocessing import sampleprocessing  # noqa: F401
 from .scatterToEdge import ScatterToEdge  # noqa: F401
 from .scatterToVertex import ScatterToVertex  # noqa: F401
 from .propagate import aggregate_bias, appnp_propagate, propagate_axpby  # noqa: F401

@@ -18,6 +18,12 @@ jittor==1.3.9.14).  Pins of the numpy restatements at the end of this file:
                 PageRank limit alpha * (I - (1 - alpha) A)^-1 h on a small graph
   sgconv        dense fp64 A^K x W
   gprgnn        dense fp64 sum_k temp[k] A^k x
+  gpuinitco / getweight / csctocsr  brute-force Python loops on small graphs,
+                the README's CSC -> CSR known answer
+  sampleprocessing  "parity unpinned": the reference draws with rand() /
+                clock-seeded curand, so no output of it can be reproduced.  Pinned
+                here: the copy branch exactly, and for the sampled branch the
+                invariants (distinct, subset, count, order) and uniformity
 """
 import ctypes
 import os
@@ -331,4 +337,68 @@ def gprgnn(x, csc, temp):
     for k in range(temp.shape[0] - 1):
         x = aggregate_with_weight(x, csc)
         out = (out + temp[k + 1] * x).astype(np.float32)
+    return out
+
+
+def gpuinitco(dst_size, fanout_i, csc_layer_dst, csc_global_column_offset):
+    """ops/cpp/gpuinitco_op.cc:37-50 (the GPU branch; the CPU branch :27-32 leaves zeros):
+    out[i+1] = min(degree of dst[i], fanout); not a running sum."""
+    dst = np.asarray(csc_layer_dst)
+    g = np.asarray(csc_global_column_offset)
+    out = np.zeros(dst_size + 1, np.int32)
+    out[1:] = np.minimum(g[dst + 1] - g[dst], fanout_i)
+    return out
+
+
+def getweight(vtx_size, csc_layer_dst, csc_layer_src, csc_layer_column_offset, csc_layer_row_indices):
+    """ops/cpp/getweight_op.cc:36-82: in-degree of dst[i] += size of column i, out-degree
+    of every row index += 1, weight = 1 / (sqrtf(out[src]) * sqrtf(in[dst]))."""
+    dst = np.asarray(csc_layer_dst)
+    off = np.asarray(csc_layer_column_offset)
+    row = np.asarray(csc_layer_row_indices)
+    ins = np.zeros(vtx_size, np.int32)
+    outs = np.zeros(vtx_size, np.int32)
+    w = np.zeros(off[-1], np.float32)
+    for i in range(dst.shape[0]):
+        ins[dst[i]] += off[i + 1] - off[i]
+        for j in range(off[i], off[i + 1]):
+            outs[row[j]] += 1
+    for i in range(dst.shape[0]):
+        for j in range(off[i], off[i + 1]):
+            w[j] = np.float32(1) / (np.sqrt(np.float32(outs[row[j]])) * np.sqrt(np.float32(ins[dst[i]])))
+    return w
+
+
+def csctocsr(column_offset, row_indices, dst, src):
+    """ops/cpp/csctocsr_op.cc:36-78: rows are the positions of `src`; an entry whose row
+    index is not in `src` is dropped; column indices hold dst ids; stable in column order."""
+    off, row = np.asarray(column_offset), np.asarray(row_indices)
+    dst, src = np.asarray(dst), np.asarray(src)
+    where = {int(s): i for i, s in enumerate(src)}
+    r_o = np.zeros(src.shape[0] + 1, np.int32)
+    for j in range(off[-1]):
+        if int(row[j]) in where:
+            r_o[where[int(row[j])] + 1] += 1
+    r_o = np.cumsum(r_o).astype(np.int32)
+    c_i = np.zeros(off[-1], np.int32)
+    ptr = r_o[:-1].copy()
+    for i in range(dst.shape[0]):
+        for j in range(off[i], off[i + 1]):
+            k = where.get(int(row[j]))
+            if k is not None:
+                c_i[ptr[k]] = dst[i]
+                ptr[k] += 1
+    return r_o, c_i
+
+
+def sampleprocessing(fanout_i, csc_layer_dst, csc_layer_column_offset, csc_global_column_offset,
+                     csc_global_row_indices, seed=0):
+    """ops/cpp/sampleprocessing_op.cc:47-84 with a seeded draw (see oracle.c)."""
+    dst = _i32(csc_layer_dst)
+    loff = _i32(csc_layer_column_offset)
+    goff = _i32(csc_global_column_offset)
+    gidx = _i32(csc_global_row_indices)
+    out = np.zeros(int(loff[-1]), np.int32)
+    lib().orc_sample_neighbors(_p(dst), _p(loff), _p(goff), _p(gidx), ctypes.c_int32(dst.shape[0]),
+                               ctypes.c_int32(int(fanout_i)), ctypes.c_uint64(int(seed) & (2**64 - 1)), _p(out))
     return out

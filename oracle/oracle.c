@@ -230,3 +230,54 @@ void orc_edgetovertex(float *out, const float *x, const int32_t *indices,
                     out[(size_t)node * feature_dim + j] + x[(size_t)i * feature_dim + j];
         }
 }
+
+/* Seeded restatement of ops/cpp/sampleprocessing_op.cc:47-84: all neighbours
+ * of dst[i] when it has at most `fanout` (or fanout < 0), else `fanout`
+ * distinct ones.  The reference draws them with rand() (:66-69), which fixes
+ * no answer; the draw here is Floyd's subset algorithm on a 64-bit mix of
+ * (seed, destination, step), and the picks keep their order in g_idx. */
+static uint32_t orc_sample_mix(uint64_t seed, uint32_t node, uint32_t step)
+{
+    uint64_t z = seed + 0x9E3779B97F4A7C15ull * (((uint64_t)node << 32) | step);
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z ^= z >> 31;
+    return (uint32_t)(z >> 32);
+}
+
+int orc_sample_neighbors(const int32_t *dst, const int32_t *layer_off, const int32_t *g_off,
+                         const int32_t *g_idx, int32_t n_dst, int32_t fanout, uint64_t seed,
+                         int32_t *out)
+{
+    for (int32_t i = 0; i < n_dst; i++) {
+        int32_t pos = layer_off[i];
+        int32_t cap = layer_off[i + 1] - pos;
+        int32_t node = dst[i];
+        int32_t start = g_off[node];
+        int32_t deg = g_off[node + 1] - start;
+        if (cap <= 0 || deg <= 0) continue;
+        if (fanout < 0 || deg <= fanout) {
+            for (int32_t j = 0; j < deg && j < cap; j++) out[pos + j] = g_idx[start + j];
+            continue;
+        }
+        int32_t k = fanout < cap ? fanout : cap;
+        int32_t *mine = out + pos;
+        int32_t have = 0;
+        for (int32_t j = deg - k; j < deg; j++) {
+            uint32_t r = orc_sample_mix(seed, (uint32_t)node, (uint32_t)(j - (deg - k)));
+            int32_t t = (int32_t)(((uint64_t)r * (uint64_t)(j + 1)) >> 32);
+            int taken = 0;
+            for (int32_t q = 0; q < have; q++) taken |= mine[q] == t;
+            if (taken) t = j;
+            int32_t q = have;
+            while (q > 0 && mine[q - 1] > t) {
+                mine[q] = mine[q - 1];
+                q--;
+            }
+            mine[q] = t;
+            have++;
+        }
+        for (int32_t q = 0; q < k; q++) mine[q] = g_idx[start + mine[q]];
+    }
+    return 0;
+}

@@ -378,3 +378,74 @@ def test_gprgnn_dense_closed_form():
     temp = rng.standard_normal(5).astype(np.float32)
     want = sum(float(temp[k]) * np.linalg.matrix_power(A, k) @ x.astype(np.float64) for k in range(5))
     np.testing.assert_allclose(oracle.gprgnn(x, csc, temp), want, rtol=1e-5, atol=1e-5)
+
+
+# -------------------------------------------------- sampled-subgraph operators ---
+
+def _global_csc(rng, V, E):
+    ei, w = rand_graph(rng, V, E)
+    row, off, _ = oracle.cootocsc(ei, w, V)
+    return off, row
+
+
+def test_gpuinitco_and_getweight_small_cases():
+    rng = np.random.default_rng(80)
+    goff, grow = _global_csc(rng, 30, 200)
+    dst = rng.permutation(30)[:12].astype(np.int32)
+    out = oracle.gpuinitco(12, 5, dst, goff)
+    assert out[0] == 0 and out[1:].tolist() == [min(int(goff[d + 1] - goff[d]), 5) for d in dst]
+    # getweight on a full small graph equals 1/sqrt(outdeg[src] * indeg[dst]) from bincounts
+    ids = np.arange(30, dtype=np.int32)
+    w = oracle.getweight(30, ids, ids, goff, grow)
+    indeg = np.diff(goff)
+    outdeg = np.bincount(grow, minlength=30)
+    col = np.repeat(ids, indeg)
+    np.testing.assert_allclose(w, 1.0 / np.sqrt(outdeg[grow].astype(np.float64) * indeg[col]), rtol=3e-7)
+
+
+def test_csctocsr_readme_known_answer_and_dropped_sources():
+    g = GOLD["csctocsr_readme_v4"]
+    ids = np.arange(4, dtype=np.int32)
+    r_o, c_i = oracle.csctocsr(np.array(g["column_offset"]), np.array(g["row_indices"]), ids, ids)
+    assert r_o.tolist() == g["row_offset"] and c_i.tolist() == g["column_indices"]
+    # a layer: dst ids are global, src lists only some of the row indices
+    off = np.array([0, 2, 3, 6]); row = np.array([7, 9, 7, 4, 9, 5]); dst = np.array([20, 21, 22]); src = np.array([9, 7, 5])
+    r_o, c_i = oracle.csctocsr(off, row, dst, src)
+    assert r_o.tolist() == [0, 2, 4, 5]                      # 9: cols 20, 22; 7: cols 20, 21; 5: col 22; 4 dropped
+    assert c_i.tolist() == [20, 22, 20, 21, 22, 0]
+
+
+def test_sampleprocessing_invariants_and_uniformity():
+    rng = np.random.default_rng(81)
+    V = 60
+    goff, grow = _global_csc(rng, V, 1500)
+    dst = rng.permutation(V)[:40].astype(np.int32)
+    for fanout in (-1, 3, 10, 1000):
+        cnt = np.diff(goff)[dst] if fanout < 0 else np.minimum(np.diff(goff)[dst], fanout)
+        loff = np.concatenate([[0], np.cumsum(cnt)]).astype(np.int32)
+        a = oracle.sampleprocessing(fanout, dst, loff, goff, grow, seed=5)
+        assert np.array_equal(a, oracle.sampleprocessing(fanout, dst, loff, goff, grow, seed=5))
+        for i, d in enumerate(dst):
+            nb = grow[goff[d]:goff[d + 1]]
+            got = a[loff[i]:loff[i + 1]]
+            if fanout < 0 or len(nb) <= fanout:
+                assert np.array_equal(got, nb)                       # the copy branch of the reference, exactly
+            else:
+                # a sub-sequence of the neighbour list with `fanout` distinct positions
+                pos, it = [], 0
+                for v in got:
+                    while nb[it] != v:
+                        it += 1
+                    pos.append(it)
+                    it += 1
+                assert len(pos) == fanout and len(set(pos)) == fanout
+    # uniformity: one destination with 12 distinct neighbours, fanout 4, many seeds
+    goff1 = np.array([0, 12], np.int32); grow1 = np.arange(100, 112, dtype=np.int32)
+    hits = np.zeros(12)
+    n = 6000
+    for s in range(n):
+        hits[oracle.sampleprocessing(4, np.array([0], np.int32), np.array([0, 4], np.int32), goff1, grow1, seed=s) - 100] += 1
+    expect = n * 4 / 12
+    assert np.all(np.abs(hits - expect) < 5 * np.sqrt(expect))
+    assert len({tuple(oracle.sampleprocessing(4, np.array([0], np.int32), np.array([0, 4], np.int32), goff1, grow1,
+                                              seed=s)) for s in range(300)}) > 150
