@@ -152,6 +152,14 @@ def main():
     gat_fb_ms = timed(gat_step, 20, 3)
     gat_bytes = gE * (4 + 4 * H * D) + gV * (4 + 8 * H + 4 * H * D) + gV * H * D * 4 + 2 * gV * H * 4
 
+    # ---- edge softmax (the reference's [E,1] shape) and one APPNP hop on the main graph ----
+    from jittorgeometric_amd.ops import EdgeSoftmax
+    from jittorgeometric_amd.ops._common import spmm_axpby
+    logits = torch.randn(E, 1, device=dev)
+    esm_fwd_ms = timed(lambda: EdgeSoftmax(logits, csc), 20, 3)
+    hop_ms = timed(lambda: spmm_axpby(csc.column_offset, csc.row_indices, csc.edge_weight, x, V, 0.9, 0.1, x), 10, 2)
+    del logits
+
     # ---- CPU baseline: the reference's single-threaded loop (oracle port) ----
     cpu = None
     if not args.no_cpu_baseline:
@@ -205,6 +213,9 @@ def main():
         "gat_fused_fwd_bwd_ms": round(gat_fb_ms, 4),
         "gat_fused_fwd_algorithmic_gbps": round(gat_bytes / (gat_fwd_ms * 1e-3) / 1e9, 1),
         "gat_shape": "V=%d, E=%d (power-law exp 2.3 + self-loops), 8 heads x 16" % (gV, gE),
+        "edge_softmax_fwd_ms": round(esm_fwd_ms, 4),
+        "edge_softmax_fwd_algorithmic_gbps": round((8 * E + 4 * (V + 1)) / (esm_fwd_ms * 1e-3) / 1e9, 1),
+        "appnp_hop_f128_ms": round(hop_ms, 4),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": args.traffic_bytes,
                      "traffic_source": "profiles/bench_workload_mi355x.txt",
