@@ -52,6 +52,12 @@ size_t edge_softmax_flat_ws_bytes(int64_t E);
 void edge_softmax_flat_enqueue(bool fwd, const int32_t *off, const float *a, const float *b, float *out, int32_t V,
                                int64_t E, int32_t H, void *ws, hipStream_t s);
 
+// ---- gather-sum for rows of 1, 2, 4 or 8 floats (edge_softmax_flat.hip) ----------
+// Same result as the wide-row product; shares edge_softmax_flat_ws_bytes(E) of workspace.
+bool narrow_spmm_supported(int F, const void *x);
+void narrow_spmm_enqueue(const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out, int32_t R,
+                         int32_t C, int64_t E, int32_t F, void *ws, hipStream_t s);
+
 #ifdef __HIPCC__
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
 // Wave index inside the block as a wave-uniform (scalar) value.

@@ -40,7 +40,8 @@ struct FlatMeta {
     int head_cs, head_ce;
     int tail_open;   // the tile's last column continues in the next tile
     int tail_cs, tail_ce;
-    int pad0, pad1;
+    int tail_col;    // id of the tile's last column
+    int pad1;
 };
 
 // The tile's T*H floats pass through LDS twice: loaded with consecutive lanes
@@ -87,6 +88,7 @@ template <int K> struct LaneColumns {
     unsigned closed;   // bit k: entry k is valid and its column lies inside the tile
     int tail_slot;     // slot of the tile's last column
     int closed_lo, closed_hi;   // the valid entries of columns inside the tile, relative to t0
+    bool staged;                // the tile's offsets are in L.off (else read from memory)
 };
 
 // Stages the offsets of the tile's columns [c_lo, c_hi] and resolves the column
@@ -124,6 +126,7 @@ __device__ __forceinline__ void resolve_columns(const int32_t *__restrict__ off,
         cols.slot[k] = max(cs - t0, 0);
         if (j0 + k <= last && cs >= t0 && ce <= t0 + n) cols.closed |= 1u << k;
     }
+    cols.staged = staged;
     cols.tail_slot = max(offv(c_hi) - t0, 0);
     cols.closed_lo = offv(c_lo) < t0 ? min(offv(c_lo + 1) - t0, n) : 0;
     cols.closed_hi = offv(c_hi + 1) > t0 + n ? max(offv(c_hi) - t0, cols.closed_lo) : n;
@@ -135,7 +138,8 @@ __device__ __forceinline__ void resolve_columns(const int32_t *__restrict__ off,
         m.tail_cs = offv(c_hi);
         m.tail_ce = offv(c_hi + 1);
         m.tail_open = m.tail_ce > t0 + n;
-        m.pad0 = m.pad1 = 0;
+        m.tail_col = c_hi;
+        m.pad1 = 0;
         *meta_out = m;
     }
 }
@@ -268,7 +272,7 @@ __device__ __forceinline__ void segment_totals(const float (&val)[K][H], const i
     __syncthreads();
 }
 
-template <int N> struct __attribute__((aligned(16))) FloatVec {
+template <int N> struct __attribute__((aligned(N >= 4 ? 16 : 4 * N))) FloatVec {
     float f[N];
 };
 
@@ -511,19 +515,95 @@ __global__ __launch_bounds__(kFlatThreads) void esm_bwd_tile(const int32_t *__re
     else store_lane<H, K>(dx, aligned, j0, cols.closed, yg);
 }
 
+// ---- narrow-row gather-sum on the same tiles ---------------------------------
+// out[c,:] = sum over the entries j of column c of w[j] * x[idx[j],:] for rows of
+// H = 1, 2, 4 or 8 floats (idx == nullptr: x[j,:], w == nullptr: weight one).  The
+// wide-row kernel gives a whole wavefront to one entry; with a handful of floats
+// per row that leaves most lanes idle, so here a lane gathers K entries and the
+// per-column totals come from the segmented scan.  Columns inside the tile are
+// written by the tile kernel, crossing ones by esm_merge; out is zeroed first
+// (empty columns belong to no tile).
+__global__ void esm_fill_zero(float *__restrict__ p, int64_t n)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0.f;
+}
+
+template <int H>
+__global__ __launch_bounds__(kFlatThreads) void esm_colsum_tile(const int32_t *__restrict__ off,
+                                                                const int32_t *__restrict__ idx,
+                                                                const float *__restrict__ w,
+                                                                const float *__restrict__ x, float *__restrict__ out,
+                                                                const int32_t *__restrict__ tile_first,
+                                                                const int32_t *__restrict__ tile_last, int V, int C,
+                                                                int E, FlatMeta *__restrict__ meta,
+                                                                float *__restrict__ pieces)
+{
+    constexpr int K = FlatShape<H>::K, T = FlatShape<H>::T;
+    __shared__ FlatLds<H, T> L;
+    const int tile = blockIdx.x;
+    const int c_lo = min(max(tile_first[tile], 0), V - 1);
+    const int c_hi = min(max(tile_last[tile], c_lo), V - 1);
+    const int t0 = tile * T;
+    const int n = min(T, E - t0);
+    const int j0 = t0 + threadIdx.x * K;
+    // gathers first: (row, weight) of the lane's K entries, then the rows themselves
+    int row[K];
+    float wk[K];
+#pragma unroll
+    for (int k = 0; k < K; k++) {
+        const int j = min(j0 + k, E - 1);
+        row[k] = idx ? idx[j] : j;
+        wk[k] = w ? w[j] : 1.f;
+        if (j0 + k >= t0 + n || (unsigned)row[k] >= (unsigned)C) {
+            row[k] = 0;
+            wk[k] = 0.f;
+        }
+    }
+    float v[K][H];
+#pragma unroll
+    for (int k = 0; k < K; k++) {
+        const FloatVec<H> r = *reinterpret_cast<const FloatVec<H> *>(x + (int64_t)row[k] * H);
+#pragma unroll
+        for (int h = 0; h < H; h++) v[k][h] = r.f[h];
+    }
+    LaneColumns<K> cols;
+    resolve_columns<H, K, T>(off, c_lo, c_hi, t0, n, L, cols, meta + tile);
+#pragma unroll
+    for (int k = 0; k < K; k++)
+#pragma unroll
+        for (int h = 0; h < H; h++) v[k][h] *= wk[k];
+    segment_totals<H, K, T>(v, cols.slot, L, OpAdd(), 0.f);
+    if (threadIdx.x < H) {
+        piece<H>(pieces, tile, 0)[threadIdx.x] = L.tot[threadIdx.x];
+        piece<H>(pieces, tile, 1)[threadIdx.x] = L.tot[cols.tail_slot * H + threadIdx.x];
+    }
+    // the columns that lie inside the tile: one thread each
+    for (int c = c_lo + (int)threadIdx.x; c <= c_hi; c += kFlatThreads) {
+        const int cs = cols.staged ? L.off[c - c_lo] : off[c];
+        const int ce = cols.staged ? L.off[c - c_lo + 1] : off[c + 1];
+        if (ce > cs && cs >= t0 && ce <= t0 + n) {
+            float t[H];
+            read_totals<H>(L.tot, cs - t0, t);
+#pragma unroll
+            for (int h = 0; h < H; h++) out[(int64_t)c * H + h] = t[h];
+        }
+    }
+}
+
 // One wavefront per tile in which a crossing column begins: folds the tail
 // piece of that tile and the head pieces of the tiles the column runs
 // through into stat[tile] (forward: H maxima, H sums; backward: H sums).
 template <int H, int T, bool FWD>
 __global__ __launch_bounds__(kFlatThreads) void esm_merge(const FlatMeta *__restrict__ meta,
                                                           float *__restrict__ pieces, float *__restrict__ stat,
-                                                          int ntiles)
+                                                          int ntiles, float *__restrict__ column_out = nullptr)
 {
     const int tile = blockIdx.x * kFlatWaves + (threadIdx.x >> 6);
     if (tile >= ntiles) return;
     const FlatMeta m = meta[tile];
     if (!m.tail_open || m.tail_cs < tile * T) return;
-    const int last_tile = (m.tail_ce - 1) / T;
+    const int last_tile = min((m.tail_ce - 1) / T, ntiles - 1);   // the clamp only matters for offsets past E
     const int lane = lane_id();
     float mx[H], sum[H];
 #pragma unroll
@@ -574,6 +654,8 @@ __global__ __launch_bounds__(kFlatThreads) void esm_merge(const FlatMeta *__rest
             if (FWD) {
                 stat[(int64_t)tile * 2 * H + h] = mx[h];
                 stat[(int64_t)tile * 2 * H + H + h] = sum[h];
+            } else if (column_out) {
+                column_out[(int64_t)m.tail_col * H + h] = sum[h];     // column sums: the total is the result
             } else {
                 stat[(int64_t)tile * 2 * H + h] = sum[h];
             }
@@ -678,6 +760,48 @@ static void flat_launch(bool fwd, const int32_t *off, const float *a, const floa
                            s, meta, pieces, stat, ntiles);
         hipLaunchKernelGGL((esm_finish<H, T, false>), dim3(ntiles), dim3(kFlatThreads), 0, s, meta, stat, a, b, out,
                            (int)E);
+    }
+}
+
+template <int H>
+static void colsum_launch(const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out, int32_t R,
+                          int32_t C, int64_t E, void *ws, hipStream_t s)
+{
+    constexpr int T = FlatShape<H>::T;
+    const int ntiles = flat_tiles(E, H);
+    Carver carve(ws);
+    const size_t cap = (size_t)ceil_div(E, (int64_t)FlatShape<8>::T);
+    FlatMeta *meta = carve.take<FlatMeta>(cap);
+    float *pieces = carve.take<float>(cap * 4 * 8);
+    float *stat = carve.take<float>(cap * 2 * 8);
+    int32_t *tile_first = carve.take<int32_t>(cap);
+    int32_t *tile_last = carve.take<int32_t>(cap);
+    const int64_t n_out = (int64_t)R * H;
+    hipLaunchKernelGGL(esm_fill_zero, dim3((unsigned)ceil_div(n_out, 256)), dim3(256), 0, s, out, n_out);
+    hipLaunchKernelGGL(esm_tile_columns, dim3((unsigned)ceil_div(R, 256)), dim3(256), 0, s, off, R, (int)E, T, ntiles,
+                       tile_first, tile_last);
+    hipLaunchKernelGGL(esm_colsum_tile<H>, dim3(ntiles), dim3(kFlatThreads), 0, s, off, idx, w, x, out, tile_first,
+                       tile_last, R, C, (int)E, meta, pieces);
+    hipLaunchKernelGGL((esm_merge<H, T, false>), dim3((unsigned)ceil_div(ntiles, kFlatWaves)), dim3(kFlatThreads), 0, s,
+                       meta, pieces, stat, ntiles, out);
+}
+
+// out[r,:] = sum_j w[j] * x[idx[j],:] for rows of F = 1, 2, 4 or 8 floats.  Needs R > 0,
+// E > 0, off[0] == 0, off[R] == E, x rows aligned to min(16, 4F) bytes.
+bool narrow_spmm_supported(int F, const void *x)
+{
+    if (!(F == 1 || F == 2 || F == 4 || F == 8)) return false;
+    return ((uintptr_t)x & (uintptr_t)((F >= 4 ? 16 : 4 * F) - 1)) == 0;
+}
+
+void narrow_spmm_enqueue(const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out, int32_t R,
+                         int32_t C, int64_t E, int32_t F, void *ws, hipStream_t s)
+{
+    switch (F) {
+    case 1: colsum_launch<1>(off, idx, w, x, out, R, C, E, ws, s); break;
+    case 2: colsum_launch<2>(off, idx, w, x, out, R, C, E, ws, s); break;
+    case 4: colsum_launch<4>(off, idx, w, x, out, R, C, E, ws, s); break;
+    default: colsum_launch<8>(off, idx, w, x, out, R, C, E, ws, s); break;
     }
 }
 

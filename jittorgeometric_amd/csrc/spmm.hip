@@ -464,11 +464,15 @@ static SpmmShape spmm_shape(int32_t R, int64_t E, int32_t F, bool aligned16, boo
     return s;
 }
 
+static bool narrow_width(int32_t F) { return F == 1 || F == 2 || F == 4 || F == 8; }
+
 size_t spmm_ws_bytes(int32_t R, int64_t E, int32_t F)
 {
     SpmmShape s = spmm_shape(R, E, F, true, true);
-    return carve_bytes((size_t)s.nchunks + 1, 4) + carve_bytes((size_t)s.nchunks * (size_t)F, 4) +
-           carve_bytes((size_t)ceil_div(s.nchunks, kGroup) * (size_t)F, 4);
+    const size_t wide = carve_bytes((size_t)s.nchunks + 1, 4) + carve_bytes((size_t)s.nchunks * (size_t)F, 4) +
+                        carve_bytes((size_t)ceil_div(s.nchunks, kGroup) * (size_t)F, 4);
+    const size_t narrow = narrow_width(F) ? edge_softmax_flat_ws_bytes(E) : 0;
+    return wide > narrow ? wide : narrow;
 }
 
 template <int VEC, int NT>
@@ -556,6 +560,17 @@ static int32_t spmm_call(const int32_t *off, const int32_t *idx, const float *w,
     if (!ws || ws_bytes < need)
         return fail(JGAMD_ERR_WORKSPACE, "spmm_csx: workspace %zu < %zu bytes", ws ? ws_bytes : (size_t)0, need);
     if (((uintptr_t)ws & 255) != 0) return fail(JGAMD_ERR_ALIGN, "spmm_csx: workspace not 256-byte aligned");
+
+    // Rows of 1, 2, 4 or 8 floats: a lane per entry and a segmented scan instead of a wavefront
+    // per entry (JGAMD_SPMM_NARROW=merge keeps the wide-row kernels).  Entries must tile [0, E).
+    static const bool narrow_off = [] {
+        const char *e = getenv("JGAMD_SPMM_NARROW");
+        return e && e[0] == 'm';
+    }();
+    if (!fin && !k0 && !narrow_off && E > 0 && narrow_width(F) && narrow_spmm_supported(F, x)) {
+        narrow_spmm_enqueue(off, idx, w, x, out, R, C, E, F, ws, static_cast<hipStream_t>(stream));
+        return launch_status("spmm_csx");
+    }
 
     // h is read with x's vector width: its alignment counts too
     const uintptr_t bits = (uintptr_t)x | (uintptr_t)out | (uintptr_t)(fin ? fin->h : nullptr);
