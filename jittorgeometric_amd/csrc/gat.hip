@@ -854,7 +854,19 @@ __global__ __launch_bounds__(1024) void gat_bwd_reduce(const float *__restrict__
     float s = 0.f;
     if (col < 2 * F) {
         const int which = col / F, f = col % F;
-        for (int b = grp; b < nblocks; b += 16) s += red[((size_t)b * 2 + which) * F + f];
+        // eight partials fetched together, added in the same order as one by one
+        constexpr int kB = 8;
+        for (int b0 = grp; b0 < nblocks; b0 += 16 * kB) {
+            float v[kB];
+#pragma unroll
+            for (int i = 0; i < kB; i++) {
+                const int b = min(b0 + 16 * i, nblocks - 1);
+                v[i] = red[((size_t)b * 2 + which) * F + f];
+            }
+#pragma unroll
+            for (int i = 0; i < kB; i++)
+                if (b0 + 16 * i < nblocks) s += v[i];
+        }
     }
     part[grp][threadIdx.x & 63] = s;
     __syncthreads();
