@@ -45,15 +45,15 @@ size_t spmm_ws_bytes(int32_t R, int64_t E, int32_t F);
 int32_t spmm_enqueue(const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out, int32_t R,
                      int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, hipStream_t s);
 
-// ---- tile-based edge softmax for 1, 2, 4 or 8 heads (edge_softmax_flat.hip) --
+// ---- tile-based edge softmax for 1, 2, 4 or 8 heads (entry_tiles.hip) --
 // fwd: a = x, b unused; bwd: a = y, b = g.  Needs V > 0, E > 0, off[V] == E.
 bool edge_softmax_flat_supported(int H);
-size_t edge_softmax_flat_ws_bytes(int64_t E);
+size_t entry_tiles_ws_bytes(int64_t E);
 void edge_softmax_flat_enqueue(bool fwd, const int32_t *off, const float *a, const float *b, float *out, int32_t V,
                                int64_t E, int32_t H, void *ws, hipStream_t s);
 
-// ---- gather-sum for rows of 1, 2, 4 or 8 floats (edge_softmax_flat.hip) ----------
-// Same result as the wide-row product; shares edge_softmax_flat_ws_bytes(E) of workspace.
+// ---- gather-sum for rows of 1, 2, 4 or 8 floats (entry_tiles.hip) ----------
+// Same result as the wide-row product; shares entry_tiles_ws_bytes(E) of workspace.
 bool narrow_spmm_supported(int F, const void *x);
 void narrow_spmm_enqueue(const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out, int32_t R,
                          int32_t C, int64_t E, int32_t F, void *ws, hipStream_t s);

@@ -342,7 +342,7 @@ static int long_capacity(int32_t V, int64_t E)
     return (int)(c < (int64_t)V ? c : (int64_t)V);
 }
 static size_t group_ws_bytes(int32_t V, int64_t E) { return 256 + carve_bytes((size_t)long_capacity(V, E), 4); }
-static size_t softmax_ws_bytes(int32_t V, int64_t E) { return group_ws_bytes(V, E) + edge_softmax_flat_ws_bytes(E); }
+static size_t softmax_ws_bytes(int32_t V, int64_t E) { return group_ws_bytes(V, E) + entry_tiles_ws_bytes(E); }
 // JGAMD_SOFTMAX=groups keeps the lane-group-per-column kernels for 1-8 heads too
 static bool use_flat(int H)
 {

@@ -1,4 +1,5 @@
-// Edge softmax over fixed tiles of entries, for H in {1, 2, 4, 8} heads.
+// Per-column work over fixed tiles of entries: edge softmax for H in {1, 2, 4, 8}
+// heads, and the gather-sum for rows of 1, 2, 4 or 8 floats (further down).
 //
 // The reference (ops/cpp/edgesoftmax_op.cc:48-65, edgesoftmaxbackward_op.cc:45-51)
 // walks every destination column three times.  Columns of a power-law graph
@@ -719,7 +720,7 @@ static int flat_tiles(int64_t E, int H)
 
 bool edge_softmax_flat_supported(int H) { return H == 1 || H == 2 || H == 4 || H == 8; }
 
-size_t edge_softmax_flat_ws_bytes(int64_t E)
+size_t entry_tiles_ws_bytes(int64_t E)
 {
     // sized for the smallest tile and the widest pieces (H = 8)
     const size_t tiles = (size_t)ceil_div(E > 0 ? E : 1, (int64_t)FlatShape<8>::T);

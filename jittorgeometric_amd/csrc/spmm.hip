@@ -471,7 +471,7 @@ size_t spmm_ws_bytes(int32_t R, int64_t E, int32_t F)
     SpmmShape s = spmm_shape(R, E, F, true, true);
     const size_t wide = carve_bytes((size_t)s.nchunks + 1, 4) + carve_bytes((size_t)s.nchunks * (size_t)F, 4) +
                         carve_bytes((size_t)ceil_div(s.nchunks, kGroup) * (size_t)F, 4);
-    const size_t narrow = narrow_width(F) ? edge_softmax_flat_ws_bytes(E) : 0;
+    const size_t narrow = narrow_width(F) ? entry_tiles_ws_bytes(E) : 0;
     return wide > narrow ? wide : narrow;
 }
 
