@@ -124,11 +124,11 @@ __device__ __forceinline__ void resolve_columns(const int32_t *__restrict__ off,
             cs = ce;
             ce = offv(c + 1);
         }
-        cols.slot[k] = max(cs - t0, 0);
+        cols.slot[k] = min(max(cs - t0, 0), T - 1);     // the upper clamp only matters for inconsistent offsets
         if (j0 + k <= last && cs >= t0 && ce <= t0 + n) cols.closed |= 1u << k;
     }
     cols.staged = staged;
-    cols.tail_slot = max(offv(c_hi) - t0, 0);
+    cols.tail_slot = min(max(offv(c_hi) - t0, 0), T - 1);
     cols.closed_lo = offv(c_lo) < t0 ? min(offv(c_lo + 1) - t0, n) : 0;
     cols.closed_hi = offv(c_hi + 1) > t0 + n ? max(offv(c_hi) - t0, cols.closed_lo) : n;
     if (threadIdx.x == 0) {
@@ -679,7 +679,7 @@ __global__ __launch_bounds__(kFlatThreads) void esm_finish(const FlatMeta *__res
         int src, s, e;
         if (part == 0) {
             if (!m.head_open) continue;
-            src = m.head_cs / T;
+            src = min(max(m.head_cs, 0) / T, tile);
             s = t0;
             e = min(m.head_ce, t0 + n);
         } else {
