@@ -1,0 +1,58 @@
+"""The entry points neither allocate, nor synchronise, nor clear memory with memset calls, so a
+sequence of them can be recorded into a HIP graph and replayed.  Every replay is checked against
+the eager result, with eager work and synchronisations between the replays."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from util import assert_close, dev, rand_graph, to_gpu
+
+pytestmark = pytest.mark.gpu
+
+
+def test_two_layer_gcn_and_appnp_replay_as_a_graph():
+    from jittorgeometric_amd.nn import APPNP, GCNConv
+    from jittorgeometric_amd.ops import cootocsc, cootocsr
+    rng = np.random.default_rng(5)
+    V, F = 2708, 64
+    ei, _ = rand_graph(rng, V, 10556, 1)
+    ei = ei[:, ei[0] != ei[1]]
+    ei, w = oracle.gcn_norm(ei, None, V)
+    csc = cootocsc(to_gpu(ei.astype(np.int32)), to_gpu(w), V)
+    csr = cootocsr(to_gpu(ei.astype(np.int32)), to_gpu(w), V)
+    l1, l2 = GCNConv(F, 32, spmm=False).to(dev()), GCNConv(32, 7, spmm=False).to(dev())
+    prop = APPNP(4, 0.1, spmm=False)
+
+    def model(x):
+        with torch.no_grad():
+            return prop(l2(torch.relu(l1(x, csc, csr)), csc, csr), csc, csr)
+
+    static_x = torch.randn(V, F, device=dev())
+    # warm-up on a side stream, as graph capture requires
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        for _ in range(3):
+            model(static_x)
+    torch.cuda.current_stream().wait_stream(s)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_out = model(static_x)
+    for trial in range(4):
+        x = torch.randn(V, F, device=dev())
+        want = model(x)                      # eager work between the replays
+        torch.cuda.synchronize()
+        static_x.copy_(x)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_out, want), "replay %d differs from the eager result" % trial
+    # the eager result itself against the oracle
+    W1, b1 = l1.weight.detach().cpu().numpy(), l1.bias.detach().cpu().numpy()
+    W2, b2 = l2.weight.detach().cpu().numpy(), l2.bias.detach().cpu().numpy()
+    csc_o = oracle.cootocsc(ei.astype(np.int32), w, V)
+    xh = x.cpu().numpy()
+    h = np.maximum(oracle.aggregate_with_weight((xh @ W1).astype(np.float32), csc_o) + b1, 0).astype(np.float32)
+    z = (oracle.aggregate_with_weight((h @ W2).astype(np.float32), csc_o) + b2).astype(np.float32)
+    ref = oracle.appnp(z, csc_o, 4, 0.1)
+    assert_close(want.cpu().numpy(), ref, scale=np.abs(ref) + 1.0, rtol=1e-4)
