@@ -402,3 +402,11 @@ def sampleprocessing(fanout_i, csc_layer_dst, csc_layer_column_offset, csc_globa
     lib().orc_sample_neighbors(_p(dst), _p(loff), _p(goff), _p(gidx), ctypes.c_int32(dst.shape[0]),
                                ctypes.c_int32(int(fanout_i)), ctypes.c_uint64(int(seed) & (2**64 - 1)), _p(out))
     return out
+
+
+def from_nodes(offset, indices, nodes):
+    """ops/saparse_ops.py:9-39 (and :42-71 with the CSR arrays): the neighbour lists of `nodes`,
+    concatenated in the order given."""
+    off, idx = np.asarray(offset), np.asarray(indices)
+    parts = [idx[off[n]:off[n + 1]] for n in np.asarray(nodes).reshape(-1)]
+    return np.concatenate(parts).astype(np.int32) if parts else np.zeros(0, np.int32)

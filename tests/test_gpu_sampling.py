@@ -118,3 +118,19 @@ def test_two_layer_sampled_subgraph_end_to_end():
     w = getweight(V, to_gpu(dst), src.to(torch.int32), loff, rows).cpu().numpy()
     want = oracle.getweight(V, dst, src.cpu().numpy(), loff.cpu().numpy(), rows.cpu().numpy())
     assert np.array_equal(w.view(np.int32), want.view(np.int32))
+
+
+def test_from_nodes_and_to_nodes():
+    from jittorgeometric_amd.ops import cootocsc, cootocsr, from_nodes, to_nodes
+    rng = np.random.default_rng(21)
+    V = 3000
+    ei, w = rand_graph(rng, V, 40000, 2)
+    csc, csr = cootocsc(to_gpu(ei), to_gpu(w), V), cootocsr(to_gpu(ei), to_gpu(w), V)
+    row, coff, _ = oracle.cootocsc(ei, w, V)
+    col, roff, _ = oracle.cootocsr(ei, w, V)
+    nodes = np.concatenate([rng.integers(0, V, 500), [0, 0, V - 1]]).astype(np.int32)     # hubs, repeats, last node
+    assert np.array_equal(from_nodes(csc, to_gpu(nodes)).cpu().numpy(), oracle.from_nodes(coff, row, nodes))
+    assert np.array_equal(to_nodes(csr, to_gpu(nodes)).cpu().numpy(), oracle.from_nodes(roff, col, nodes))
+    assert from_nodes(csc, to_gpu(np.zeros(0, np.int32))).numel() == 0
+    with pytest.raises(ValueError):
+        from_nodes(None, to_gpu(nodes))
