@@ -199,6 +199,11 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__rest
         row_end = r < r1 ? bcast_i(ends, r - rb) : kNever;
     };
 
+    // (index, weight) of the batch after the current one are fetched while the current one is
+    // worked on; the index is clamped, what lies past the chunk is discarded when it is used
+    const int jlast = max(j1 - 1, 0);
+    int nxt_c = idx ? load_stream(idx + min(j0 + lane, jlast)) : 0;
+    float nxt_w = w ? load_stream(w + min(j0 + lane, jlast)) : 1.f;
     for (int jb = j0; jb < j1; jb += kWave) {
         const int n = min(kWave, j1 - jb);
         int my_c;
@@ -206,8 +211,10 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__rest
         {
             const bool ok = lane < n;
             const int jj = jb + lane;
-            my_c = idx ? (ok ? load_stream(idx + jj) : 0) : jj;
-            my_w = ok ? (w ? load_stream(w + jj) : 1.f) : 0.f;
+            my_c = idx ? (ok ? nxt_c : 0) : jj;
+            my_w = ok ? nxt_w : 0.f;
+            if (idx) nxt_c = load_stream(idx + min(jj + kWave, jlast));
+            if (w) nxt_w = load_stream(w + min(jj + kWave, jlast));
             if ((unsigned)my_c >= (unsigned)C) {
                 my_c = 0;
                 my_w = 0.f;
