@@ -247,6 +247,32 @@ int32_t jgamd_sample_neighbors(const int32_t *dst, const int32_t *layer_off, con
                                int32_t fanout, int64_t out_len, uint64_t seed, int32_t *out,
                                void *stream);
 
+/* ------------------------------------------------------------------------
+ * Graph preprocessing in front of the conversion.
+ *
+ * jgamd_add_remaining_self_loops: utils/loop.py:98-136 — the input's
+ * self-loops are dropped, the other edges keep their order, one loop per
+ * node is appended; a node's loop takes the weight of its last dropped loop,
+ * else `fill`.  out_index must hold 2*(E+N) int32, out_weight E+N floats;
+ * *out_kept (device) receives the number of kept edges K, and the result is
+ * out_index[0..K+N) (rows) followed directly by out_index[K+N..2(K+N)) (cols),
+ * out_weight[0..K+N).  edge_weight may be NULL (weights of one).
+ *
+ * jgamd_degree_power: out[v] = deg[v]^power with inf -> 0
+ * (nn/conv/gcn_conv.py:35-36).  jgamd_scale_edge_weights:
+ * out[e] = by_row[row[e]] * w[e] * by_col[col[e]] (either factor array may be
+ * NULL) — gcn_conv.py:37, sage_conv.py:40.
+ */
+int32_t jgamd_add_remaining_self_loops_workspace(int64_t E, int32_t N, size_t *bytes);
+int32_t jgamd_add_remaining_self_loops(const int32_t *edge_index, const float *edge_weight,
+                                       int64_t E, int32_t N, float fill, int32_t *out_index,
+                                       float *out_weight, int32_t *out_kept, void *ws,
+                                       size_t ws_bytes, void *stream);
+int32_t jgamd_degree_power(const float *deg, int32_t N, float power, float *out, void *stream);
+int32_t jgamd_scale_edge_weights(const int32_t *edge_index, const float *edge_weight,
+                                 const float *by_row, const float *by_col, int64_t E, int32_t N,
+                                 float *out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

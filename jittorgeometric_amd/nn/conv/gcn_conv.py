@@ -32,11 +32,31 @@ def _degree_norm(edge_index, edge_weight, num_nodes, improved, add_self_loops, p
         edge_weight = torch.ones((edge_index.size(1),), dtype=torch.float32, device=edge_index.device)
     if add_self_loops:
         edge_index, edge_weight = add_remaining_self_loops(edge_index, edge_weight, fill_value, num_nodes)
-    row, col = edge_index[0].long(), edge_index[1].long()
     deg = _degree_by_col(edge_index, edge_weight, num_nodes)
+    if deg.is_cuda and deg.dtype == torch.float32 and edge_index.dtype == torch.int32:
+        # deg^power (inf -> 0) and the per-edge products as library kernels
+        from ... import _lib
+        lib = _lib.load()
+        dinv = torch.empty_like(deg)
+        _lib.check(lib.jgamd_degree_power(_lib.ptr(deg), num_nodes, float(power), _lib.ptr(dinv),
+                                          _lib.stream_ptr(deg.device)))
+        return edge_index, edge_weight, dinv, None, None
+    row, col = edge_index[0].long(), edge_index[1].long()
     dinv = deg.pow(power)
     dinv.masked_fill_(dinv == float("inf"), 0)
     return edge_index, edge_weight, dinv, row, col
+
+
+def _scale(edge_index, edge_weight, by_row, by_col, num_nodes):
+    """by_row[row] * w * by_col[col] on the GPU (either factor may be None)."""
+    from ... import _lib
+    lib = _lib.load()
+    ei = edge_index.contiguous()
+    w = edge_weight.contiguous()
+    out = torch.empty_like(w)
+    _lib.check(lib.jgamd_scale_edge_weights(_lib.ptr(ei), _lib.ptr(w), _lib.ptr(by_row), _lib.ptr(by_col), ei.shape[1],
+                                            num_nodes, _lib.ptr(out), _lib.stream_ptr(w.device)))
+    return out
 
 
 def gcn_norm(edge_index, edge_weight=None, num_nodes=None, improved=False, add_self_loops=True, dtype=None):
@@ -44,6 +64,8 @@ def gcn_norm(edge_index, edge_weight=None, num_nodes=None, improved=False, add_s
     degree summed by column (nn/conv/gcn_conv.py:18-37)."""
     edge_index, edge_weight, dis, row, col = _degree_norm(edge_index, edge_weight, num_nodes, improved,
                                                           add_self_loops, -0.5)
+    if row is None:
+        return edge_index, _scale(edge_index, edge_weight, dis, dis, dis.shape[0])
     return edge_index, dis[row] * edge_weight * dis[col]
 
 

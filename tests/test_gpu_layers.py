@@ -156,3 +156,47 @@ def test_gcn_norm_with_hub_destination_matches_oracle():
         assert np.array_equal(gi.cpu().numpy(), oi)
         # degrees of 10^5-edge hubs are float sums in different orders
         assert_close(gw.cpu().numpy(), ow, rtol=2e-4, atol=0, what=fn.__name__)
+
+
+@pytest.mark.parametrize("V,E,with_w,fill,seed", [(4, 0, True, 1.0, 0), (7, 30, True, 1.0, 1), (7, 30, False, 2.0, 2),
+                                                  (5000, 80000, True, 2.0, 3), (3000, 2048, True, 1.0, 4),
+                                                  (3000, 2049, False, 1.0, 5), (1, 5, True, 1.0, 6)])
+def test_add_remaining_self_loops_kernels(V, E, with_w, fill, seed):
+    """Kept edges in input order, one loop per node appended, a dropped loop's weight kept (at most
+    one loop per node in the input: with several the reference keeps whichever its indexed assignment
+    writes last)."""
+    from jittorgeometric_amd.utils import add_remaining_self_loops
+    rng = np.random.default_rng(seed)
+    ei = rng.integers(0, V, (2, E)).astype(np.int32)
+    ei = ei[:, ei[0] != ei[1]]
+    loops = rng.permutation(V)[:max(V // 3, 1)].astype(np.int32)          # distinct nodes with a loop
+    ei = np.concatenate([ei, np.stack([loops, loops])], axis=1)
+    ei = ei[:, rng.permutation(ei.shape[1])]
+    w = (rng.random(ei.shape[1]).astype(np.float32) + 0.5) if with_w else None
+    gi, gw = add_remaining_self_loops(to_gpu(ei), to_gpu(w) if with_w else None, fill, V)
+    oi, ow = oracle.add_remaining_self_loops(ei, w, fill, V)
+    assert gi.dtype == torch.int32 and np.array_equal(gi.cpu().numpy(), oi)
+    if with_w:
+        assert np.array_equal(gw.cpu().numpy().view(np.int32), ow.view(np.int32))
+    else:
+        assert gw is None and ow is None
+    # int64 indices come back as int64
+    gi64, _ = add_remaining_self_loops(to_gpu(ei).long(), None, fill, V)
+    assert gi64.dtype == torch.int64 and np.array_equal(gi64.cpu().numpy(), oi)
+
+
+def test_norms_with_existing_weighted_loops_and_flags():
+    from jittorgeometric_amd.nn import gcn_norm, sage_norm
+    rng = np.random.default_rng(17)
+    V, E = 3000, 50000
+    ei = rng.integers(0, V, (2, E)).astype(np.int32)
+    ei = ei[:, ei[0] != ei[1]]
+    loops = rng.permutation(V)[:700].astype(np.int32)
+    ei = np.concatenate([ei[:, :20000], np.stack([loops, loops]), ei[:, 20000:]], axis=1)
+    w = rng.random(ei.shape[1]).astype(np.float32) + 0.5
+    for kwargs in ({}, {"improved": True}, {"add_self_loops": False}):
+        for fn, ofn in ((gcn_norm, oracle.gcn_norm), (sage_norm, oracle.sage_norm)):
+            gi, gw = fn(to_gpu(ei), to_gpu(w), V, **kwargs)
+            oi, ow = ofn(ei, w, V, **kwargs)
+            assert np.array_equal(gi.cpu().numpy(), oi)
+            assert_close(gw.cpu().numpy(), ow, rtol=2e-5, atol=1e-7, what="%s %s" % (fn.__name__, kwargs))
