@@ -13,60 +13,53 @@ from ..inits import glorot, zeros
 
 def _degree_by_col(edge_index, edge_weight, num_nodes):
     """deg[v] = sum of the weights of the edges whose destination is v
-    (jt.scatter(..., reduce='add') by col in gcn_conv.py:33-34).  On the GPU it
-    is the column sum of the CSC arrays: conversion + gather-sum, in a fixed
-    order and without the same-address atomics a hub destination causes."""
-    if edge_weight.is_cuda and edge_weight.dtype == torch.float32 and edge_index.shape[1] > 0:
-        from ...ops._common import spmm
-        csc = cootocsc(edge_index.contiguous(), edge_weight, num_nodes)
-        return spmm(csc.column_offset, None, None, csc.edge_weight.view(-1, 1), num_nodes).view(-1)
-    deg = torch.zeros((num_nodes,), dtype=edge_weight.dtype, device=edge_weight.device)
-    deg.scatter_add_(0, edge_index[1].long(), edge_weight)
-    return deg
-
-
-def _degree_norm(edge_index, edge_weight, num_nodes, improved, add_self_loops, power):
-    fill_value = 2.0 if improved else 1.0
-    num_nodes = maybe_num_nodes(edge_index, num_nodes)
-    if edge_weight is None:
-        edge_weight = torch.ones((edge_index.size(1),), dtype=torch.float32, device=edge_index.device)
-    if add_self_loops:
-        edge_index, edge_weight = add_remaining_self_loops(edge_index, edge_weight, fill_value, num_nodes)
-    deg = _degree_by_col(edge_index, edge_weight, num_nodes)
-    if deg.is_cuda and deg.dtype == torch.float32 and edge_index.dtype == torch.int32:
-        # deg^power (inf -> 0) and the per-edge products as library kernels
-        from ... import _lib
-        lib = _lib.load()
-        dinv = torch.empty_like(deg)
-        _lib.check(lib.jgamd_degree_power(_lib.ptr(deg), num_nodes, float(power), _lib.ptr(dinv),
-                                          _lib.stream_ptr(deg.device)))
-        return edge_index, edge_weight, dinv, None, None
-    row, col = edge_index[0].long(), edge_index[1].long()
-    dinv = deg.pow(power)
-    dinv.masked_fill_(dinv == float("inf"), 0)
-    return edge_index, edge_weight, dinv, row, col
+    (jt.scatter(..., reduce='add') by col in gcn_conv.py:33-34): the column sum
+    of the CSC arrays, i.e. conversion + gather-sum, in a fixed order and
+    without the same-address atomics a hub destination causes."""
+    from ...ops._common import spmm
+    if edge_index.shape[1] == 0:
+        return torch.zeros((num_nodes,), dtype=torch.float32, device=edge_weight.device)
+    csc = cootocsc(edge_index.contiguous(), edge_weight, num_nodes)
+    return spmm(csc.column_offset, None, None, csc.edge_weight.view(-1, 1), num_nodes).view(-1)
 
 
 def _scale(edge_index, edge_weight, by_row, by_col, num_nodes):
-    """by_row[row] * w * by_col[col] on the GPU (either factor may be None)."""
+    """by_row[row] * w * by_col[col] (either factor may be None)."""
     from ... import _lib
     lib = _lib.load()
-    ei = edge_index.contiguous()
+    dev = _lib.require_gpu(edge_index, edge_weight)
+    ei = (edge_index if edge_index.dtype == torch.int32 else edge_index.to(torch.int32)).contiguous()
     w = edge_weight.contiguous()
     out = torch.empty_like(w)
     _lib.check(lib.jgamd_scale_edge_weights(_lib.ptr(ei), _lib.ptr(w), _lib.ptr(by_row), _lib.ptr(by_col), ei.shape[1],
-                                            num_nodes, _lib.ptr(out), _lib.stream_ptr(w.device)))
+                                            num_nodes, _lib.ptr(out), _lib.stream_ptr(dev)))
     return out
+
+
+def _degree_norm(edge_index, edge_weight, num_nodes, improved, add_self_loops, power):
+    """(edge_index, edge_weight, deg^power with inf -> 0) after the optional self-loop step."""
+    from ... import _lib
+    lib = _lib.load()
+    dev = _lib.require_gpu(edge_index, edge_weight)
+    fill_value = 2.0 if improved else 1.0
+    num_nodes = int(maybe_num_nodes(edge_index, num_nodes))
+    if edge_weight is None:
+        edge_weight = torch.ones((edge_index.size(1),), dtype=torch.float32, device=dev)
+    elif edge_weight.dtype != torch.float32:
+        edge_weight = edge_weight.to(torch.float32)
+    if add_self_loops:
+        edge_index, edge_weight = add_remaining_self_loops(edge_index, edge_weight, fill_value, num_nodes)
+    deg = _degree_by_col(edge_index, edge_weight, num_nodes)
+    dinv = torch.empty_like(deg)
+    _lib.check(lib.jgamd_degree_power(_lib.ptr(deg), num_nodes, float(power), _lib.ptr(dinv), _lib.stream_ptr(dev)))
+    return edge_index, edge_weight, dinv
 
 
 def gcn_norm(edge_index, edge_weight=None, num_nodes=None, improved=False, add_self_loops=True, dtype=None):
     """Symmetric normalisation w = d^-1/2[row] * w * d^-1/2[col] with the
     degree summed by column (nn/conv/gcn_conv.py:18-37)."""
-    edge_index, edge_weight, dis, row, col = _degree_norm(edge_index, edge_weight, num_nodes, improved,
-                                                          add_self_loops, -0.5)
-    if row is None:
-        return edge_index, _scale(edge_index, edge_weight, dis, dis, dis.shape[0])
-    return edge_index, dis[row] * edge_weight * dis[col]
+    edge_index, edge_weight, dis = _degree_norm(edge_index, edge_weight, num_nodes, improved, add_self_loops, -0.5)
+    return edge_index, _scale(edge_index, edge_weight, dis, dis, dis.shape[0])
 
 
 class GCNConv(nn.Module):
@@ -89,7 +82,7 @@ class GCNConv(nn.Module):
 
     def forward(self, x, csc, csr):
         x = xw(x, self.weight)
-        if self.bias is not None and x.is_cuda and x.dim() == 2:
+        if self.bias is not None and x.dim() == 2:
             # product and bias in one kernel; spmm=True only needs the CSR (:96-97)
             return aggregate_bias(x, self.bias, None if self.spmm and csr is not None else csc, csr)
         if self.spmm:

@@ -11,11 +11,8 @@ from .gcn_conv import _degree_norm, _scale
 
 def sage_norm(edge_index, edge_weight=None, num_nodes=None, improved=False, add_self_loops=True, dtype=None):
     """Mean weights w * d^-1[col] (nn/conv/sage_conv.py:16-40)."""
-    edge_index, edge_weight, dinv, row, col = _degree_norm(edge_index, edge_weight, num_nodes, improved,
-                                                           add_self_loops, -1.0)
-    if col is None:
-        return edge_index, _scale(edge_index, edge_weight, None, dinv, dinv.shape[0])
-    return edge_index, edge_weight * dinv[col]
+    edge_index, edge_weight, dinv = _degree_norm(edge_index, edge_weight, num_nodes, improved, add_self_loops, -1.0)
+    return edge_index, _scale(edge_index, edge_weight, None, dinv, dinv.shape[0])
 
 
 class SAGEConv(nn.Module):

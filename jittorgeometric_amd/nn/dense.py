@@ -66,7 +66,7 @@ class _AddBias(torch.autograd.Function):
     def backward(ctx, g):
         gb = None
         if ctx.needs_input_grad[1]:
-            if g.is_cuda and g.dim() == 2 and g.dtype == torch.float32:
+            if g.dim() == 2 and g.dtype == torch.float32:
                 gb = column_sum(g.contiguous())
             else:
                 gb = g.sum(0)

@@ -200,3 +200,13 @@ def test_norms_with_existing_weighted_loops_and_flags():
             oi, ow = ofn(ei, w, V, **kwargs)
             assert np.array_equal(gi.cpu().numpy(), oi)
             assert_close(gw.cpu().numpy(), ow, rtol=2e-5, atol=1e-7, what="%s %s" % (fn.__name__, kwargs))
+
+
+def test_preprocessing_refuses_cpu_tensors():
+    from jittorgeometric_amd import _lib
+    from jittorgeometric_amd.nn import gcn_norm, sage_norm
+    from jittorgeometric_amd.utils import add_remaining_self_loops
+    ei = torch.tensor([[0, 1], [1, 0]], dtype=torch.int32)
+    for fn in (lambda: gcn_norm(ei, None, 2), lambda: sage_norm(ei, None, 2), lambda: add_remaining_self_loops(ei, None, 1.0, 2)):
+        with pytest.raises(_lib.JgamdError):
+            fn()
