@@ -84,6 +84,10 @@ def test_feature_widths(F):
     (1, 0, 0, 4, 0), (1, 50, 0, 128, 1), (3, 0, 0, 64, 2), (50, 7, 0, 128, 3),
     (4000, 200000, 2, 128, 4), (4000, 200000, 2, 32, 5), (100000, 50000, 0, 16, 6),
     (30000, 600000, 4, 64, 7), (20000, 300000, 1, 256, 8),
+    # rows of 1-8 floats take the tile kernels: mostly empty rows (more rows than entries in a tile),
+    # hubs that cross many tiles, entry counts around the tile sizes
+    (200000, 5000, 0, 1, 9), (300000, 3000, 2, 8, 10), (4000, 200000, 2, 1, 11), (4000, 200000, 2, 4, 12),
+    (500, 2048, 0, 2, 13), (500, 2049, 1, 8, 14), (3, 70000, 0, 1, 15), (1, 30000, 0, 8, 16),
 ])
 def test_shapes_empty_rows_and_hubs(V, E, hubs, F, seed):
     rng = np.random.default_rng(seed)
