@@ -6,6 +6,8 @@
 // run from one entry to millions, so here the unit of work is not a column
 // but a tile of T consecutive entries of the [E,H] array:
 //
+//   0. tile columns : one thread per column records, for every tile, the
+//                     column of its first and of its last entry.
 //   1. tile kernel  : a lane holds K consecutive entries (all H heads, loaded
 //                     as vectors).  Each entry's column is found from the
 //                     offsets staged in LDS; per-column totals (max, then sum
