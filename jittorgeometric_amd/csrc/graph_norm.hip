@@ -58,7 +58,8 @@ __global__ __launch_bounds__(kLoopThreads) void loops_count(const int32_t *__res
 }
 
 // Kept edges of tile b go to positions base[b] + (rank inside the tile, input order).
-// A thread owns kLoopItems CONSECUTIVE edges so that its ranks are consecutive.
+// Edge (round i, thread t) = base + i*256 + t, so loads and stores of a round are coalesced; its
+// rank = kept edges of earlier rounds + of earlier wavefronts in the round + of lower lanes.
 __global__ __launch_bounds__(kLoopThreads) void loops_scatter(const int32_t *__restrict__ row,
                                                               const int32_t *__restrict__ col,
                                                               const float *__restrict__ w, int64_t E,
@@ -67,42 +68,48 @@ __global__ __launch_bounds__(kLoopThreads) void loops_scatter(const int32_t *__r
                                                               int32_t *__restrict__ out_index,
                                                               float *__restrict__ out_w)
 {
-    __shared__ int wave_sum[kLoopThreads / kWave];
-    const int64_t first = (int64_t)blockIdx.x * kLoopTile + (int64_t)threadIdx.x * kLoopItems;
-    int r[kLoopItems], c[kLoopItems];
+    constexpr int kWaves = kLoopThreads / kWave;
+    __shared__ int cnt[kLoopItems][kWaves];
+    const int64_t first = (int64_t)blockIdx.x * kLoopTile + threadIdx.x;
+    const int wv = threadIdx.x >> 6, lane = lane_id();
+    const uint64_t below = lane == 0 ? 0ull : (~0ull >> (kWave - lane));
+    int r[kLoopItems], c[kLoopItems], rank[kLoopItems];
     float ww[kLoopItems];
-    int mine = 0;
 #pragma unroll
     for (int i = 0; i < kLoopItems; i++) {
-        const int64_t e = first + i;
+        const int64_t e = first + (int64_t)i * kLoopThreads;
         const int64_t ec = e < E ? e : E - 1;
         r[i] = row[ec];
         c[i] = col[ec];
         ww[i] = w ? w[ec] : 1.f;
         if (e >= E) r[i] = c[i];        // past the end: treated as dropped
-        mine += r[i] != c[i];
     }
-    // exclusive scan of `mine` over the block
-    int inc = mine;
 #pragma unroll
-    for (int d = 1; d < kWave; d <<= 1) {
-        const int t = __shfl_up(inc, d, kWave);
-        if (lane_id() >= d) inc += t;
+    for (int i = 0; i < kLoopItems; i++) {
+        const uint64_t keep = __ballot(r[i] != c[i]);
+        rank[i] = __popcll(keep & below);
+        if (lane == 0) cnt[i][wv] = __popcll(keep);
     }
-    if (lane_id() == kWave - 1) wave_sum[threadIdx.x >> 6] = inc;
     __syncthreads();
-    int before = inc - mine;
-    for (int v = 0; v < (int)(threadIdx.x >> 6); v++) before += wave_sum[v];
     const int64_t out_E = (int64_t)*total_kept + N;     // row 1 of out_index starts here
-    int64_t pos = (int64_t)base[blockIdx.x] + before;
+    int64_t pos = base[blockIdx.x];
 #pragma unroll
-    for (int i = 0; i < kLoopItems; i++)
-        if (r[i] != c[i]) {
-            out_index[pos] = r[i];
-            out_index[out_E + pos] = c[i];
-            out_w[pos] = ww[i];
-            pos++;
+    for (int i = 0; i < kLoopItems; i++) {
+        int before = 0, round_total = 0;
+#pragma unroll
+        for (int v = 0; v < kWaves; v++) {
+            const int n = cnt[i][v];
+            before += v < wv ? n : 0;
+            round_total += n;
         }
+        if (r[i] != c[i]) {
+            const int64_t p = pos + before + rank[i];
+            out_index[p] = r[i];
+            out_index[out_E + p] = c[i];
+            out_w[p] = ww[i];
+        }
+        pos += round_total;
+    }
 }
 
 __global__ void loops_append(const float *__restrict__ w, const int32_t *__restrict__ last_loop,
