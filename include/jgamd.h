@@ -136,6 +136,25 @@ int32_t jgamd_spmm_csx_axpby(const int32_t *off, const int32_t *idx, const float
                              const float *h, int32_t h_rows, int32_t R, int32_t C, int64_t E,
                              int32_t F, void *ws, size_t ws_bytes, void *stream);
 
+/* jgamd_spmm_csx without a workspace argument.  No counterpart in the
+ * reference: it is for callers that cannot allocate device memory or own a
+ * workspace (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc).  Same kernels, same result bit for bit; the scratch
+ * (chunk rows, row pieces, group sums) is a fixed 64 MiB device array inside
+ * the library, one copy per GPU, held until the process ends.
+ *   - Shapes whose jgamd_spmm_csx_workspace() exceeds 64 MiB are rejected with
+ *     JGAMD_ERR_SIZE and nothing is enqueued (the 1M-node / 17M-entry graph at
+ *     F = 128 needs 36 MiB).
+ *   - Calls no hipMalloc / hipFree or allocating routine.  The first call on
+ *     a device looks up the array's address (hipGetSymbolAddress) with that
+ *     device current and keeps it; make that call outside a stream capture.
+ *   - All calls on one GPU share the array: two calls that overlap in time on
+ *     one GPU (different streams) race.  Calls on one stream are ordered.
+ */
+int32_t jgamd_spmm_csx_noalloc(const int32_t *off, const int32_t *idx, const float *w,
+                               const float *x, float *out, int32_t R, int32_t C, int64_t E,
+                               int32_t F, void *stream);
+
 /* Benchmark support; no counterpart in the reference.  Runs jgamd_spmm_csx
  * `iters` times on `stream`, with one hipEvent pair around each launch of the
  * gather kernel (spmm_merge) and one around each whole call (three launches),

@@ -24,6 +24,7 @@ SIGNATURES = {
     "jgamd_sample_neighbors": [_P, _P, _P, _P, _I32, _I32, _I32, _I64, _c.c_uint64, _P, _P],
     "jgamd_spmm_csx_workspace": [_I32, _I64, _I32, _SZP],
     "jgamd_spmm_csx": [_P, _P, _P, _P, _P, _I32, _I32, _I64, _I32, _P, _c.c_size_t, _P],
+    "jgamd_spmm_csx_noalloc": [_P, _P, _P, _P, _P, _I32, _I32, _I64, _I32, _P],
     "jgamd_spmm_csx_axpby": [_P, _P, _P, _P, _P, _c.c_float, _c.c_float, _P, _I32, _I32, _I32, _I64, _I32, _P,
                              _c.c_size_t, _P],
     "jgamd_spmm_csx_timed": [_P, _P, _P, _P, _P, _I32, _I32, _I64, _I32, _P, _c.c_size_t, _P, _I32,

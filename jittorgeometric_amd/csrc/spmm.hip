@@ -20,6 +20,8 @@
 // does not change from run to run.
 #include <stdlib.h>
 
+#include <mutex>
+
 #include "common.h"
 
 namespace jg {
@@ -662,4 +664,61 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_timed(
     *kernel_ms = (float)(ksum / iters);
     *call_ms = (float)(csum / iters);
     return rc;
+}
+
+// ---- the product without a workspace argument --------------------------------
+// For callers that can neither allocate nor own a workspace: chunk_row, partial
+// and group_sum live in a fixed device array that is part of the code object.
+// Every GPU the library runs on holds its own copy of the array, at its own
+// address, until the process ends; the array's name is only a handle on the
+// host, so its device address is resolved once per device and kept.
+constexpr size_t kStaticScratchBytes = (size_t)64 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_lock;
+void *g_scratch_ptr[kMaxDevices];   // device address of `scratch` on each device, once known
+
+int32_t static_scratch(void **out)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail((int32_t)e, "spmm_csx_noalloc: hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices)
+        return fail(JGAMD_ERR_UNSUPPORTED, "spmm_csx_noalloc: device %d outside [0, %d)", dev, kMaxDevices);
+    std::lock_guard<std::mutex> hold(g_scratch_lock);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            (void)hipGetLastError();
+            return fail(e != hipSuccess ? (int32_t)e : JGAMD_ERR_UNSUPPORTED,
+                        "spmm_csx_noalloc: hipGetSymbolAddress: %s", hipGetErrorString(e));
+        }
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return 0;
+}
+}  // namespace
+
+extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_noalloc(const int32_t *off, const int32_t *idx,
+                                                                                 const float *w, const float *x,
+                                                                                 float *out, int32_t R, int32_t C,
+                                                                                 int64_t E, int32_t F, void *stream)
+{
+    if (int32_t rc = check_spmm_sizes(R, E, F)) return rc;
+    if (R == 0 || F == 0) return 0;
+    const size_t need = spmm_ws_bytes(R, E, F);
+    if (need > kStaticScratchBytes)
+        return fail(JGAMD_ERR_SIZE,
+                    "spmm_csx_noalloc: R=%d E=%lld F=%d needs %zu bytes of scratch, the fixed array holds %zu; "
+                    "use jgamd_spmm_csx with a workspace",
+                    R, (long long)E, F, need, kStaticScratchBytes);
+    void *ws = nullptr;
+    if (int32_t rc = static_scratch(&ws)) return rc;
+    // Nothing in the scratch has to start at zero: every word a kernel reads was written by an
+    // earlier kernel of the same call (chunk rows; a piece is read only for chunks that stored one).
+    return spmm_call(off, idx, w, x, out, R, C, E, F, ws, kStaticScratchBytes, stream, nullptr, nullptr);
 }
