@@ -62,7 +62,8 @@ const char *jgamd_last_error(void);
  * Result is bit-identical to the reference: a stable counting sort, i.e.
  * inside a row the edges keep their input order; weights are copied.
  * Edges whose key is outside [0,V) are dropped (the reference would write out
- * of bounds); the tail of out_idx/out_w is then left untouched.
+ * of bounds); out_off[V] is then below E and the slots of out_idx / out_w /
+ * out_perm from out_off[V] on are set to zero.
  * Limits: 0 <= E < 2^31 - 2^20, 0 <= V < 2^31 - 1 (V <= 2^22 takes the
  * two-level path, larger V plain radix passes over the same records).
  */

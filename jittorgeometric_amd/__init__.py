@@ -6,6 +6,7 @@ hand-written gfx950 kernels of libjgamd.so, reached through ctypes with raw
 device pointers.  There is no CPU implementation behind these operators:
 calling them on CPU tensors, or without the built library, raises.
 """
+from ._lib import JgamdError  # noqa: F401
 from .data import CSC, CSR  # noqa: F401
 from . import ops  # noqa: F401
 

@@ -556,6 +556,29 @@ __global__ void fill_i32(int32_t *p, int64_t n, int32_t v)
     if (i < n) p[i] = v;
 }
 
+// Edges with a key outside [0,V) were dropped, so off[V] may be below E: the slots past
+// off[V] are zeroed (the reference hands zero-filled arrays to the op, ops/cootocsr.py:30-32).
+// Nothing to do in the usual case, which costs one read of off[V] per thread.
+__global__ void csx_zero_tail(const int32_t *__restrict__ off_end, int64_t E, int32_t *__restrict__ out_idx,
+                              uint32_t *__restrict__ out_w, int32_t *__restrict__ out_perm)
+{
+    const int64_t first = *off_end;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = first + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < E; i += step) {
+        out_idx[i] = 0;
+        if (out_w) out_w[i] = 0u;
+        if (out_perm) out_perm[i] = 0;
+    }
+}
+
+static void zero_tail(const int32_t *out_off, int32_t V, int64_t E, int32_t *out_idx, float *out_w,
+                      int32_t *out_perm, hipStream_t s)
+{
+    const unsigned blocks = (unsigned)(ceil_div(E, 256) < 1024 ? ceil_div(E, 256) : 1024);
+    hipLaunchKernelGGL(csx_zero_tail, dim3(blocks), dim3(256), 0, s, out_off + V, E, out_idx,
+                       reinterpret_cast<uint32_t *>(out_w), out_perm);
+}
+
 // ------------------------------------------------------------------ host ---
 struct ConvPlan {
     int shift;        // low key bits handled inside a bucket
@@ -664,6 +687,7 @@ static int32_t convert(const int32_t *keys, const int32_t *others, const float *
         hipLaunchKernelGGL((csx_unpack_sorted<Rec, PERM>), dim3((unsigned)ceil_div(E + 1, 256)), dim3(256), 0, s,
                            bufs[(p.digits - 1) & 1], count, E, V, out_off, out_idx,
                            reinterpret_cast<uint32_t *>(out_w), out_perm);
+        zero_tail(out_off, V, E, out_idx, out_w, out_perm, s);
         return launch_status("coo_to_csx(lsd)");
     }
 
@@ -693,6 +717,7 @@ static int32_t convert(const int32_t *keys, const int32_t *others, const float *
     hipLaunchKernelGGL(scat, dim3((unsigned)p.max_sub), dim3(kPartThreads), scat_lds, s, recs, table, nblk,
                        sub_bucket, sub_first, cnt2, p.shift, out_idx, reinterpret_cast<uint32_t *>(out_w), out_perm,
                        tile_stage_records(nkeys, sizeof(Rec)));
+    zero_tail(out_off, V, E, out_idx, out_w, out_perm, s);
     return launch_status("coo_to_csx");
 }
 

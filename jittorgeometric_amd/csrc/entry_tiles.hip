@@ -70,6 +70,12 @@ struct OpAdd {
     __device__ __forceinline__ float operator()(float a, float b) const { return a + b; }
 };
 
+// Entries the offsets cover: off[V], clamped to the length of the per-entry arrays.
+__device__ __forceinline__ int covered_entries(const int32_t *__restrict__ off, int V, int E)
+{
+    return min(max(off[V], 0), E);
+}
+
 // tile_first[i] / tile_last[i] = column of the first / last entry of tile i.
 // One thread per column: it owns the entries [off[c], off[c+1]) and marks the
 // tiles whose first or last entry falls among them.
@@ -78,11 +84,37 @@ __global__ void esm_tile_columns(const int32_t *__restrict__ off, int V, int E, 
 {
     const int c = blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= V) return;
-    const int s = off[c], e = min(off[c + 1], E);
+    // entries past off[V] belong to no column (offsets of a conversion that dropped keys):
+    // only the tiles that hold covered entries get a first and a last column
+    const int covered = covered_entries(off, V, E);
+    const int s = off[c], e = min(off[c + 1], covered);
     if (e <= s) return;
+    ntiles = (covered + T - 1) / T;
     for (int i = (s + T - 1) / T; i < ntiles && (int64_t)i * T < e; i++) tile_first[i] = c;
     for (int i = s / T + 1; i <= ntiles && (int64_t)i * T <= e; i++) tile_last[i - 1] = c;   // last entry i*T - 1
-    if (e == E) tile_last[ntiles - 1] = c;
+    if (e == covered) tile_last[ntiles - 1] = c;
+}
+
+// A tile that holds no covered entry: no column is open in it, and (zero_out) its slots of the
+// per-entry result are zero.  Returns true if the calling block has nothing else to do.
+template <int H, int T>
+__device__ __forceinline__ bool skip_uncovered_tile(int t0, int covered, int E, FlatMeta *meta_out, float *out)
+{
+    // slots past the covered entries, in this tile
+    if (out) {
+        const int64_t lo = (int64_t)max(t0, covered) * H, hi = (int64_t)min(t0 + T, E) * H;
+        for (int64_t p = lo + threadIdx.x; p < hi; p += kFlatThreads) out[p] = 0.f;
+    }
+    if (t0 < covered) return false;
+    if (threadIdx.x == 0) {
+        FlatMeta m;
+        m.head_open = m.tail_open = 0;
+        m.head_cs = m.head_ce = m.tail_cs = m.tail_ce = covered;
+        m.tail_col = 0;
+        m.pad1 = 0;
+        *meta_out = m;
+    }
+    return true;
 }
 
 // What a tile knows about its entries' columns.
@@ -418,11 +450,13 @@ __global__ __launch_bounds__(kFlatThreads) void esm_fwd_tile(const int32_t *__re
     constexpr int K = FlatShape<H>::K, T = FlatShape<H>::T;
     __shared__ FlatLds<H, T> L;
     const int tile = blockIdx.x;
-    // the clamps only matter if off[] and E disagree (tiles no column claimed)
+    const int t0 = tile * T;
+    const int covered = covered_entries(off, V, E);
+    if (skip_uncovered_tile<H, T>(t0, covered, E, meta + tile, y)) return;
+    // the clamps only matter for offsets that are not monotone
     const int c_lo = min(max(tile_first[tile], 0), V - 1);
     const int c_hi = min(max(tile_last[tile], c_lo), V - 1);
-    const int t0 = tile * T;
-    const int n = min(T, E - t0);
+    const int n = min(T, covered - t0);
     const int j0 = t0 + threadIdx.x * K;
     const bool aligned = both_aligned(x, y);
     const bool through_lds = aligned && staged;
@@ -478,11 +512,13 @@ __global__ __launch_bounds__(kFlatThreads) void esm_bwd_tile(const int32_t *__re
     constexpr int K = FlatShape<H>::K, T = FlatShape<H>::T;
     __shared__ FlatLds<H, T> L;
     const int tile = blockIdx.x;
-    // the clamps only matter if off[] and E disagree (tiles no column claimed)
+    const int t0 = tile * T;
+    const int covered = covered_entries(off, V, E);
+    if (skip_uncovered_tile<H, T>(t0, covered, E, meta + tile, dx)) return;
+    // the clamps only matter for offsets that are not monotone
     const int c_lo = min(max(tile_first[tile], 0), V - 1);
     const int c_hi = min(max(tile_last[tile], c_lo), V - 1);
-    const int t0 = tile * T;
-    const int n = min(T, E - t0);
+    const int n = min(T, covered - t0);
     const int j0 = t0 + threadIdx.x * K;
     const bool aligned = both_aligned(y, g) && ((uintptr_t)dx & 15) == 0;
     const bool through_lds = aligned && staged;
@@ -545,10 +581,12 @@ __global__ __launch_bounds__(kFlatThreads) void esm_colsum_tile(const int32_t *_
     constexpr int K = FlatShape<H>::K, T = FlatShape<H>::T;
     __shared__ FlatLds<H, T> L;
     const int tile = blockIdx.x;
+    const int t0 = tile * T;
+    const int covered = covered_entries(off, V, E);
+    if (skip_uncovered_tile<H, T>(t0, covered, E, meta + tile, nullptr)) return;
     const int c_lo = min(max(tile_first[tile], 0), V - 1);
     const int c_hi = min(max(tile_last[tile], c_lo), V - 1);
-    const int t0 = tile * T;
-    const int n = min(T, E - t0);
+    const int n = min(T, covered - t0);
     const int j0 = t0 + threadIdx.x * K;
     // gathers first: (row, weight) of the lane's K entries, then the rows themselves
     int row[K];

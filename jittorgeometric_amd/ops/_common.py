@@ -18,11 +18,58 @@ def as_f32(t, name):
     return t.contiguous()
 
 
+def _stamp(t):
+    """Identity and in-place version of a tensor: changes whenever the holder's
+    attribute is rebound or written in place."""
+    return None if t is None else (id(t), t._version)
+
+
+def _holder_arrays(holder, names, what):
+    """(off, idx, w) of a CSC / CSR object as contiguous int32 / int32 / float32
+    device arrays.  Holders built by hand carry whatever torch.tensor([...]) gave
+    them (int64 indices, float64 weights, as in the reference's own test scripts,
+    tests/test_aggregate.py:43-54); the kernels read int32 / float32 only, so
+    anything else is converted here, once, and kept on the holder until one of
+    its arrays is rebound or written in place."""
+    src = tuple(getattr(holder, n, None) for n in names)
+    off, idx, w = src
+    if off is None or idx is None:
+        raise _lib.JgamdError("%s: %s and %s must be set" % (what, names[0], names[1]))
+    stamp = tuple(_stamp(t) for t in src)
+    cached = getattr(holder, "_jgamd_arrays", None)
+    if cached is not None and cached[0] == stamp and all(a is b for a, b in zip(cached[1], src)):
+        return cached[2]
+    for n, t in zip(names, src):
+        if t is not None and not isinstance(t, torch.Tensor):
+            raise _lib.JgamdError("%s.%s must be a torch tensor, got %s" % (what, n, type(t).__name__))
+    _lib.require_gpu(off, idx, w)
+    out = (as_i32(off, names[0]).reshape(-1), as_i32(idx, names[1]).reshape(-1),
+           as_f32(w, names[2]).reshape(-1) if w is not None else None)
+    if out[0].shape[0] < 1:
+        raise _lib.JgamdError("%s.%s is empty (needs V+1 entries)" % (what, names[0]))
+    if out[2] is not None and out[2].shape[0] != out[1].shape[0]:
+        raise _lib.JgamdError("%s: %d weights for %d indices" % (what, out[2].shape[0], out[1].shape[0]))
+    holder._jgamd_arrays = (stamp, src, out)
+    return out
+
+
+def csc_arrays(csc):
+    """(column_offset, row_indices, edge_weight) ready for the C ABI."""
+    return _holder_arrays(csc, ("column_offset", "row_indices", "edge_weight"), "CSC")
+
+
+def csr_arrays(csr):
+    """(row_offset, column_indices, edge_weight) ready for the C ABI."""
+    return _holder_arrays(csr, ("row_offset", "column_indices", "edge_weight"), "CSR")
+
+
 def transposed(holder, off, idx, w, R, C):
     """(off_t, idx_t, w_t, perm) of a compressed structure, built on first use
-    and kept on the CSR/CSC object it belongs to."""
+    and kept on the CSR/CSC object it belongs to; rebuilt when any of the three
+    arrays is another tensor or has been written in place since."""
+    stamp = (_stamp(off), _stamp(idx), _stamp(w))
     cached = getattr(holder, "_jgamd_transposed", None)
-    if cached is not None and cached[4] is off and cached[5] is idx and cached[6] is w:
+    if cached is not None and cached[7] == stamp and cached[4] is off and cached[5] is idx and cached[6] is w:
         return cached[:4]
     lib = _lib.load()
     dev = _lib.require_gpu(off, idx, w)
@@ -36,7 +83,7 @@ def transposed(holder, off, idx, w, R, C):
     _lib.check(lib.jgamd_csx_transpose(_lib.ptr(off), _lib.ptr(idx), _lib.ptr(w), R, C, E, _lib.ptr(off_t),
                                        _lib.ptr(idx_t), _lib.ptr(w_t), _lib.ptr(perm), _lib.ptr(ws), nbytes,
                                        _lib.stream_ptr(dev)))
-    holder._jgamd_transposed = (off_t, idx_t, w_t, perm, off, idx, w)
+    holder._jgamd_transposed = (off_t, idx_t, w_t, perm, off, idx, w, stamp)
     return off_t, idx_t, w_t, perm
 
 
@@ -54,11 +101,27 @@ def transposed_inverse(holder, perm):
     return inv
 
 
+def _raw_arrays(off, idx, w, R):
+    """Last line of defence in front of the pointer hand-over: dtype, layout and the
+    length of the offsets (no copy when the arrays already are what the kernels read)."""
+    off = as_i32(off, "off")
+    idx = as_i32(idx, "idx") if idx is not None else None
+    w = as_f32(w, "w") if w is not None else None
+    if off.numel() != R + 1:
+        raise _lib.JgamdError("offsets have %d entries for %d rows" % (off.numel(), R))
+    if idx is not None and w is not None and idx.numel() != w.numel():
+        raise _lib.JgamdError("%d weights for %d indices" % (w.numel(), idx.numel()))
+    return off, idx, w
+
+
 def spmm(off, idx, w, x, R):
     """out[r,:] = sum_j w[j] * x[idx[j],:]; idx/w may be None (identity / ones)."""
     lib = _lib.load()
     dev = _lib.require_gpu(off, x, idx, w)
     x = as_f32(x, "x")
+    off, idx, w = _raw_arrays(off, idx, w, R)
+    if x.dim() != 2:
+        raise _lib.JgamdError("x must be [rows, F], got %s" % (tuple(x.shape),))
     C, F = x.shape
     E = int(idx.shape[0]) if idx is not None else C
     out = torch.empty((R, F), dtype=torch.float32, device=dev)
@@ -75,6 +138,7 @@ def spmm_axpby(off, idx, w, x, R, beta, alpha, h):
     lib = _lib.load()
     dev = _lib.require_gpu(off, x, idx, w, h)
     x = as_f32(x, "x")
+    off, idx, w = _raw_arrays(off, idx, w, R)
     h = as_f32(h, "h") if h is not None else None
     C, F = x.shape
     h_rows = R
@@ -100,11 +164,9 @@ def both_orders(csc, csr):
     if csc is None and csr is None:
         raise ValueError("need a CSC or a CSR")
     if csc is not None:
-        fwd = (as_i32(csc.column_offset, "column_offset"), as_i32(csc.row_indices, "row_indices"),
-               as_f32(csc.edge_weight, "edge_weight"))
+        fwd = csc_arrays(csc)
     if csr is not None:
-        bwd = (as_i32(csr.row_offset, "row_offset"), as_i32(csr.column_indices, "column_indices"),
-               as_f32(csr.edge_weight, "edge_weight"))
+        bwd = csr_arrays(csr)
     if csc is None:
         V = bwd[0].shape[0] - 1
         fwd = transposed(csr, bwd[0], bwd[1], bwd[2], V, V)[:3]

@@ -3,7 +3,7 @@ jittor_geometric.ops.aggregateWithWeight (ops/aggregateWithWeight.py:19-54);
 the loops of ops/cpp/aggregate_op.cc run as csrc/spmm.hip."""
 import torch
 
-from ._common import spmm
+from ._common import csc_arrays, csr_arrays, spmm
 
 
 class AggregateFunc(torch.autograd.Function):
@@ -11,15 +11,19 @@ class AggregateFunc(torch.autograd.Function):
     def forward(ctx, x, csc, csr, edge_weight):
         ctx.csr = csr
         ctx.weight = edge_weight
-        w = edge_weight if isinstance(edge_weight, torch.Tensor) else csc.edge_weight
+        off, idx, w = csc_arrays(csc)
+        if isinstance(edge_weight, torch.Tensor):
+            w = edge_weight.reshape(-1)
         # the reference sizes the output like x (zeros_like, :28)
-        return spmm(csc.column_offset, csc.row_indices, w, x, x.shape[0])
+        return spmm(off, idx, w, x, x.shape[0])
 
     @staticmethod
     def backward(ctx, grad_output):
         csr = ctx.csr
-        w = ctx.weight if isinstance(ctx.weight, torch.Tensor) else csr.edge_weight
-        g = spmm(csr.row_offset, csr.column_indices, w, grad_output.contiguous(), grad_output.shape[0])
+        off, idx, w = csr_arrays(csr)
+        if isinstance(ctx.weight, torch.Tensor):
+            w = ctx.weight.reshape(-1)
+        g = spmm(off, idx, w, grad_output, grad_output.shape[0])
         return g, None, None, None
 
 

@@ -19,8 +19,8 @@ def _convert(edge_index, edge_weight, v_num, key_row, with_perm=False):
     if edge_weight.shape[0] != E:
         raise _lib.JgamdError("edge_weight has %d entries for %d edges" % (edge_weight.shape[0], E))
     v_num = int(v_num)
-    # the reference hands zero-filled outputs to the op (ops/cootocsr.py:30-32);
-    # the kernels overwrite every slot, so plain allocations do
+    # the reference hands zero-filled outputs to the op (ops/cootocsr.py:30-32); the library
+    # writes every slot (slots past off[V], left over when keys were dropped, as zeros)
     idx = torch.empty(E, dtype=torch.int32, device=dev)
     off = torch.empty(v_num + 1, dtype=torch.int32, device=dev)
     w = torch.empty(E, dtype=torch.float32, device=dev)

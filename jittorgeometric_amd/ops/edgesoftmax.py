@@ -6,7 +6,7 @@ independent heads."""
 import torch
 
 from .. import _lib
-from ._common import as_f32
+from ._common import as_f32, csc_arrays
 
 
 def _heads(x):
@@ -19,9 +19,11 @@ class EdgeSoftmaxFunc(torch.autograd.Function):
         lib = _lib.load()
         dev = _lib.require_gpu(x, csc.column_offset)
         x = as_f32(x, "x")
-        off = csc.column_offset
+        off = csc_arrays(csc)[0]
         V, E, H = off.shape[0] - 1, x.shape[0], _heads(x)
-        y = torch.empty_like(x)
+        if x.dim() > 2:
+            raise _lib.JgamdError("EdgeSoftmax: x must be [E] or [E,H], got %s" % (tuple(x.shape),))
+        y = torch.empty(x.shape, dtype=torch.float32, device=dev)
         nbytes = _lib.query(lib.jgamd_edge_softmax_workspace, V, E)
         ws = _lib.workspace(nbytes, dev)
         _lib.check(lib.jgamd_edge_softmax_fwd(_lib.ptr(off), _lib.ptr(x), _lib.ptr(y), V, E, H, _lib.ptr(ws), nbytes,
@@ -34,11 +36,11 @@ class EdgeSoftmaxFunc(torch.autograd.Function):
     def backward(ctx, grad_output):
         lib = _lib.load()
         (y,) = ctx.saved_tensors
-        off = ctx.csc.column_offset
+        off = csc_arrays(ctx.csc)[0]
         g = as_f32(grad_output, "grad")
         dev = _lib.require_gpu(g, y)
         V, E, H = off.shape[0] - 1, y.shape[0], _heads(y)
-        dx = torch.empty_like(y)
+        dx = torch.empty(y.shape, dtype=torch.float32, device=dev)
         nbytes = _lib.query(lib.jgamd_edge_softmax_workspace, V, E)
         ws = _lib.workspace(nbytes, dev)
         _lib.check(lib.jgamd_edge_softmax_bwd(_lib.ptr(off), _lib.ptr(y), _lib.ptr(g), _lib.ptr(dx), V, E, H,

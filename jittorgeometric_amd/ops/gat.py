@@ -6,7 +6,7 @@ EdgeSoftmax -> multiply -> ScatterToVertex of GATConv.propagate
 import torch
 
 from .. import _lib
-from ._common import as_f32, transposed, transposed_inverse
+from ._common import as_f32, csc_arrays, transposed, transposed_inverse
 
 
 def fused_supported(H, D, backward=True):
@@ -28,14 +28,20 @@ def gat_forward_raw(h, csc, a_src, a_dst, slope=0.2, want_alpha=False):
     lib = _lib.load()
     dev = _lib.require_gpu(h, csc.row_indices, csc.column_offset, a_src, a_dst)
     h, a_src, a_dst = as_f32(h, "h"), as_f32(a_src, "a_src"), as_f32(a_dst, "a_dst")
+    off, idx, _ = csc_arrays(csc)
+    if h.dim() != 3 or tuple(a_src.shape) != tuple(h.shape[1:]) or tuple(a_dst.shape) != tuple(h.shape[1:]):
+        raise _lib.JgamdError("gat: h must be [V,H,D] and a_src/a_dst [H,D], got %s, %s, %s"
+                              % (tuple(h.shape), tuple(a_src.shape), tuple(a_dst.shape)))
     V, H, D = h.shape
-    E = csc.row_indices.shape[0]
+    if off.shape[0] != V + 1:
+        raise _lib.JgamdError("gat: %d column offsets for %d nodes" % (off.shape[0], V))
+    E = idx.shape[0]
     mk = lambda *s: torch.empty(s, dtype=torch.float32, device=dev)
     out, el, er, smax, ssum = mk(V, H, D), mk(V, H), mk(V, H), mk(V, H), mk(V, H)
     alpha = mk(E, H) if want_alpha else None
     nbytes = _lib.query(lib.jgamd_gat_fwd_workspace, V, E, H, D)
     ws = _lib.workspace(nbytes, dev)
-    _lib.check(lib.jgamd_gat_fwd(_lib.ptr(csc.column_offset), _lib.ptr(csc.row_indices), _lib.ptr(h),
+    _lib.check(lib.jgamd_gat_fwd(_lib.ptr(off), _lib.ptr(idx), _lib.ptr(h),
                                  _lib.ptr(a_src), _lib.ptr(a_dst), float(slope), _lib.ptr(el), _lib.ptr(er),
                                  _lib.ptr(smax), _lib.ptr(ssum), _lib.ptr(alpha), _lib.ptr(out), V, E, H, D,
                                  _lib.ptr(ws), nbytes, _lib.stream_ptr(dev)))
@@ -45,6 +51,8 @@ def gat_forward_raw(h, csc, a_src, a_dst, slope=0.2, want_alpha=False):
 class GatFusedFunc(torch.autograd.Function):
     @staticmethod
     def forward(ctx, h, a_src, a_dst, csc, slope):
+        # what backward reads must be what forward read: dense fp32 copies, not the caller's views
+        h, a_src, a_dst = as_f32(h, "h"), as_f32(a_src, "a_src"), as_f32(a_dst, "a_dst")
         r = gat_forward_raw(h, csc, a_src, a_dst, slope)
         ctx.save_for_backward(h, a_src, a_dst, r["el"], r["er"], r["smax"], r["ssum"], r["out"])
         ctx.csc = csc
@@ -59,14 +67,16 @@ class GatFusedFunc(torch.autograd.Function):
         g_out = as_f32(g_out, "g_out")
         dev = _lib.require_gpu(g_out, h)
         V, H, D = h.shape
-        E = csc.row_indices.shape[0]
-        off_t, idx_t, _, perm = transposed(csc, csc.column_offset, csc.row_indices, csc.edge_weight, V, V)
+        off, idx, w = csc_arrays(csc)
+        E = idx.shape[0]
+        off_t, idx_t, _, perm = transposed(csc, off, idx, w, V, V)
         inv = transposed_inverse(csc, perm)
-        g_h = torch.empty_like(h)
-        g_as, g_ad = torch.empty_like(a_src), torch.empty_like(a_dst)
+        g_h = torch.empty((V, H, D), dtype=torch.float32, device=dev)
+        g_as = torch.empty((H, D), dtype=torch.float32, device=dev)
+        g_ad = torch.empty((H, D), dtype=torch.float32, device=dev)
         nbytes = _lib.query(lib.jgamd_gat_bwd_workspace, V, E, H, D)
         ws = _lib.workspace(nbytes, dev)
-        _lib.check(lib.jgamd_gat_bwd(_lib.ptr(csc.column_offset), _lib.ptr(csc.row_indices), _lib.ptr(off_t),
+        _lib.check(lib.jgamd_gat_bwd(_lib.ptr(off), _lib.ptr(idx), _lib.ptr(off_t),
                                      _lib.ptr(idx_t), _lib.ptr(inv), _lib.ptr(h), _lib.ptr(a_src), _lib.ptr(a_dst),
                                      float(ctx.slope), _lib.ptr(el), _lib.ptr(er), _lib.ptr(smax), _lib.ptr(ssum),
                                      _lib.ptr(out), _lib.ptr(g_out), _lib.ptr(g_h), _lib.ptr(g_as), _lib.ptr(g_ad),

@@ -4,6 +4,7 @@ jittor_geometric.ops.ScatterToVertex (ops/scatterToVertex.py:23-50): whatever
 (edgetovertex flag 1, scatterToVertex.py:38), and so does this."""
 import torch
 
+from ._common import csc_arrays
 from .scatterToEdge import edge_to_vertex, scatter_to_edge
 
 
@@ -11,12 +12,12 @@ class ScatterToVertexFunc(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, csc, flow):
         ctx.csc = csc
-        v_num = csc.column_offset.shape[0] - 1
-        return edge_to_vertex(x.contiguous(), csc, 1, v_num)
+        v_num = csc_arrays(csc)[0].shape[0] - 1
+        return edge_to_vertex(x, csc, 1, v_num)
 
     @staticmethod
     def backward(ctx, grad_output):
-        return scatter_to_edge(grad_output.contiguous(), ctx.csc, 1), None, None
+        return scatter_to_edge(grad_output, ctx.csc, 1), None, None
 
 
 def ScatterToVertex(x, csc, flow):

@@ -5,7 +5,7 @@ out[c] = sum over entries (r, c) of w * x[r]."""
 import torch
 
 from .. import _lib
-from ._common import as_f32, as_i32, spmm, transposed
+from ._common import csr_arrays, spmm, transposed
 
 # False: backward is the exact transpose of forward (the true gradient).
 # True: backward re-applies the forward product, as the reference does
@@ -15,15 +15,11 @@ REFERENCE_GRAD = False
 
 
 def _product(x, csr, trans_A):
-    col = as_i32(csr.column_indices, "column_indices")
-    off = as_i32(csr.row_offset, "row_offset")
-    w = as_f32(csr.edge_weight, "edge_weight")
+    off, col, w = csr_arrays(csr)
     v_num = off.shape[0] - 1
     if trans_A:
         # the transposed product is run as a gather over the transposed arrays,
         # built once per CSR object (stable, so the result is reproducible)
-        if col is not csr.column_indices or off is not csr.row_offset or w is not csr.edge_weight:
-            csr.column_indices, csr.row_offset, csr.edge_weight = col, off, w
         off_t, idx_t, w_t, _ = transposed(csr, off, col, w, v_num, v_num)
         return spmm(off_t, idx_t, w_t, x, v_num)
     return spmm(off, col, w, x, v_num)
@@ -41,7 +37,7 @@ class SpmmCsrFunc(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output):
         trans = ctx.trans_A if REFERENCE_GRAD else not ctx.trans_A
-        return _product(grad_output.contiguous(), ctx.csr, trans), None, None, None
+        return _product(grad_output, ctx.csr, trans), None, None, None
 
 
 def SpmmCsr(x, csr, trans_A=True, trans_B=False):
