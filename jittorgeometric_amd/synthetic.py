@@ -8,15 +8,36 @@ self-loops removed (gcn_norm appends one per node afterwards).
 import numpy as np
 
 
-def _sample_endpoints(rng, weights, n_edges, chunk=1 << 24):
-    """n_edges draws with P(i) proportional to weights[i]."""
+def _sample_endpoints(rng, weights, n_edges, chunk=1 << 22, threads=8):
+    """n_edges draws with P(i) proportional to weights[i].  The uniforms come from
+    `rng` in one sequence; the table look-ups (the slow part, and independent of
+    one another) are spread over a few threads."""
+    from concurrent.futures import ThreadPoolExecutor
     cdf = np.cumsum(weights, dtype=np.float64)
     cdf /= cdf[-1]
     out = np.empty(n_edges, np.int32)
-    for s in range(0, n_edges, chunk):
-        e = min(n_edges, s + chunk)
-        out[s:e] = np.searchsorted(cdf, rng.random(e - s), side="right").astype(np.int32)
-    np.minimum(out, len(weights) - 1, out=out)
+    top = len(weights) - 1
+
+    def look_up(args):
+        s, u = args
+        out[s:s + len(u)] = np.minimum(np.searchsorted(cdf, u, side="right"), top)
+
+    def chunks():
+        for s in range(0, n_edges, chunk):
+            yield s, rng.random(min(n_edges, s + chunk) - s)
+
+    if n_edges <= chunk:
+        for c in chunks():
+            look_up(c)
+        return out
+    with ThreadPoolExecutor(max_workers=threads) as pool:
+        pending = []
+        for c in chunks():
+            pending.append(pool.submit(look_up, c))
+            if len(pending) >= 2 * threads:          # bounds the uniforms held at once
+                pending.pop(0).result()
+        for f in pending:
+            f.result()
     return out
 
 

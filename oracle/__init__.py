@@ -116,6 +116,48 @@ def aggregate(x, indices, offset, weight, scalar=False):
     return out
 
 
+def _sub_rows(indices, offset, weight, rows):
+    """Compressed arrays of the chosen rows only, each row's entries in their order."""
+    rows = np.asarray(rows, dtype=np.int64)
+    lens = (offset[rows + 1] - offset[rows]).astype(np.int64)
+    sub_off = np.zeros(rows.shape[0] + 1, np.int64)
+    np.cumsum(lens, out=sub_off[1:])
+    assert sub_off[-1] < 2 ** 31
+    take = np.repeat(offset[rows].astype(np.int64) - sub_off[:-1], lens) + np.arange(sub_off[-1], dtype=np.int64)
+    return _i32(indices[take]), _i32(sub_off), _f32(weight[take])
+
+
+def aggregate_rows_f64(x, indices, offset, weight, rows):
+    """(exact, terms) for the chosen rows: sum_j w[j] * x[indices[j],:] accumulated in
+    float64 and the sum of the absolute terms.  Not the reference's arithmetic: the
+    value its sequential fp32 loop approximates, used to arbitrate on rows so long
+    that the loop itself has drifted."""
+    x = _f32(x)
+    indices, offset, weight = _i32(indices), _i32(offset), _f32(weight)
+    sub_idx, sub_off, sub_w = _sub_rows(indices, offset, weight, rows)
+    n = sub_off.shape[0] - 1
+    out = np.empty((n, x.shape[1]), np.float64)
+    terms = np.empty((n, x.shape[1]), np.float64)
+    lib().orc_aggregate_f64(_p(out), _p(terms), _p(x), _p(sub_idx), _p(sub_off), _p(sub_w), ctypes.c_int32(n),
+                            ctypes.c_int32(x.shape[1]))
+    return out, terms
+
+
+def aggregate_rows(x, indices, offset, weight, rows):
+    """Rows `rows` of aggregate(x, indices, offset, weight), by the same C loop run on the
+    compressed arrays of those rows only (each chosen row keeps its entries in their order),
+    so that a sample of rows of a graph with 10^8 entries costs seconds.  The loop takes
+    its row count from the offsets it is given and never looks at how many rows x has."""
+    x = _f32(x)
+    indices, offset, weight = _i32(indices), _i32(offset), _f32(weight)
+    sub_idx, sub_off, sub_w = _sub_rows(indices, offset, weight, rows)
+    n = sub_off.shape[0] - 1
+    out = np.empty((n, x.shape[1]), np.float32)
+    lib().orc_aggregate(_p(out), _p(x), _p(sub_idx), _p(sub_off), _p(sub_w), ctypes.c_int32(n),
+                        ctypes.c_int32(x.shape[1]))
+    return out
+
+
 def edgesoftmax(x, offset):
     """ops/cpp/edgesoftmax_op.cc:36-66.  x is [E], [E,1] (reference shapes) or
     [E,H] (independent heads)."""

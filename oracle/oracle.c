@@ -128,6 +128,30 @@ void orc_aggregate_scalar(float *out, const float *x, const int32_t *indices,
                     x[(size_t)indices[j] * feature_dim + k] * weight[j];
 }
 
+/* Not a restatement of the reference: the same row sums with double accumulators,
+ * i.e. the exact value of sum_j w[j] * x[indices[j],:] up to fp64 rounding.  The
+ * reference's sequential fp32 sum drifts from it by up to (deg - 1) * 2^-24 of the sum
+ * of the absolute terms (0.5 % on a row of 3.8 million same-sign terms); this is the
+ * arbiter the tests hold both that loop and the kernels against.  terms (optional)
+ * receives the sums of the absolute terms.  Pinned by scipy's fp64 sparse product. */
+void orc_aggregate_f64(double *out, double *terms, const float *x, const int32_t *indices,
+                       const int32_t *offset, const float *weight, int32_t v_num,
+                       int32_t feature_dim)
+{
+    for (int32_t i = 0; i < v_num; i++) {
+        double *o = out + (size_t)i * feature_dim;
+        double *t = terms ? terms + (size_t)i * feature_dim : NULL;
+        for (int32_t k = 0; k < feature_dim; k++) o[k] = 0.0;
+        if (t) for (int32_t k = 0; k < feature_dim; k++) t[k] = 0.0;
+        for (int32_t j = offset[i]; j < offset[i + 1]; j++) {
+            const float *xr = x + (size_t)indices[j] * feature_dim;
+            const double w = (double)weight[j];
+            for (int32_t k = 0; k < feature_dim; k++) o[k] += w * (double)xr[k];
+            if (t) for (int32_t k = 0; k < feature_dim; k++) t[k] += fabs(w) * fabs((double)xr[k]);
+        }
+    }
+}
+
 /* ops/cpp/edgesoftmax_op.cc:36-66.  One scalar per edge (x is [E] or [E,1]).
  * `exp` on a float argument resolves to the float overload in the
  * reference's C++ translation unit, hence expf here.  The reference reads

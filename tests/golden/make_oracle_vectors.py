@@ -32,6 +32,10 @@ def build():
         out["x%d" % F] = x
         out["agg_fwd%d" % F] = oracle.aggregate(x, row, coff, cw)
         out["agg_bwd%d" % F] = oracle.aggregate(x, col, roff, rw)
+        # sum of the absolute terms of every output element: what a difference in the order
+        # of summation scales with (the tolerance of the GPU tests is relative to it)
+        out["agg_fwd_terms%d" % F] = oracle.aggregate(np.abs(x), row, coff, np.abs(cw))
+        out["agg_bwd_terms%d" % F] = oracle.aggregate(np.abs(x), col, roff, np.abs(rw))
     E = ei.shape[1]
     for H in (1, 2):
         z = (2 * rng.standard_normal((E, H))).astype(np.float32)
@@ -43,7 +47,9 @@ def build():
     xe = rng.standard_normal((E, 5)).astype(np.float32)
     out.update(sc_x=xv, sc_xe=xe, sc_src=oracle.scattertoedge(xv, row, coff, 0),
                sc_dst=oracle.scattertoedge(xv, row, coff, 1), ev_src=oracle.edgetovertex(xe, row, coff, 0),
-               ev_dst=oracle.edgetovertex(xe, row, coff, 1))
+               ev_dst=oracle.edgetovertex(xe, row, coff, 1),
+               ev_src_terms=oracle.edgetovertex(np.abs(xe), row, coff, 0),
+               ev_dst_terms=oracle.edgetovertex(np.abs(xe), row, coff, 1))
     h = np.maximum(rng.standard_normal((V, 2, 6)), 0).astype(np.float32)
     a_src = (rng.standard_normal((2, 6)) / 2).astype(np.float32)
     a_dst = (rng.standard_normal((2, 6)) / 2).astype(np.float32)
@@ -51,6 +57,10 @@ def build():
     o1, al1, _ = oracle.gat_forward(np.ascontiguousarray(h[:, 0, :]), (row, coff, cw),
                                     np.concatenate([a_src[0], a_dst[0]]), 0.2)
     out.update(gat_h=h, gat_a_src=a_src, gat_a_dst=a_dst, gat_out2=o2, gat_alpha2=al2, gat_out1=o1, gat_alpha1=al1)
+    # sum over a destination's in-edges of alpha * |h[src]|, per head and feature
+    terms = np.zeros_like(o2, dtype=np.float64)
+    np.add.at(terms, np.repeat(np.arange(V), np.diff(coff)), al2[:, :, None].astype(np.float64) * np.abs(h[row]))
+    out["gat_terms2"] = terms.astype(np.float32)
     return out
 
 

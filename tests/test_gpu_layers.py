@@ -115,11 +115,13 @@ def test_spmmcsr_reference_grad_switch():
     g = rng.standard_normal((V, F)).astype(np.float32)
     ocsr, ocsc = oracle.cootocsr(ei, w, V), oracle.cootocsc(ei, w, V)
     try:
-        for flag, want in ((False, oracle.aggregate(g, *ocsr)), (True, oracle.aggregate(g, *ocsc))):
+        for flag, arrays in ((False, ocsr), (True, ocsc)):
+            want = oracle.aggregate(g, *arrays)
+            terms = oracle.aggregate(np.abs(g), arrays[0], arrays[1], np.abs(arrays[2]))
             spmmcsr.REFERENCE_GRAD = flag
             xt = to_gpu(x).requires_grad_(True)
             SpmmCsr(xt, csr).backward(to_gpu(g))
-            assert_close(xt.grad.cpu().numpy(), want, np.abs(want) + 1.0, what="REFERENCE_GRAD=%s" % flag)
+            assert_close(xt.grad.cpu().numpy(), want, terms, what="REFERENCE_GRAD=%s" % flag)
     finally:
         spmmcsr.REFERENCE_GRAD = False
 

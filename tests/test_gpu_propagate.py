@@ -134,18 +134,28 @@ def test_sgconv_forward_backward(spmm):
     xt = to_gpu(x).requires_grad_(True)
     out = layer(xt, csc, csr)
     want = oracle.sgconv(x, csc_o, K, W, b)
-    assert_close(out.detach().cpu().numpy(), want, scale=np.abs(want) + 1.0, rtol=1e-4)
+    # K products and one dense product in a row, each good to 1e-5 of its sum of absolute
+    # terms; the bound is carried through the chain by running it on absolute values
+    steps = (K + 1) * 1e-5
+    abs_csc = (csc_o[0], csc_o[1], np.abs(csc_o[2]))
+    abs_csr = (csr_o[0], csr_o[1], np.abs(csr_o[2]))
+    assert_close(out.detach().cpu().numpy(), want, scale=oracle.sgconv(np.abs(x), abs_csc, K, np.abs(W), np.abs(b)),
+                 rtol=steps)
     g = rng.standard_normal((V, Fout)).astype(np.float32)
     out.backward(to_gpu(g))
     # d/dx = (A^T)^K (g W^T), d/dW = (A^K x)^T g
     v = (g.astype(np.float64) @ W.T.astype(np.float64)).astype(np.float32)
-    ak = x
+    va = (np.abs(g).astype(np.float64) @ np.abs(W).T.astype(np.float64)).astype(np.float32)
+    ak, aka = x, np.abs(x)
     for _ in range(K):
         v = oracle.aggregate_with_weight_grad(v, csr_o)
+        va = oracle.aggregate_with_weight_grad(va, abs_csr)
         ak = oracle.aggregate_with_weight(ak, csc_o)
-    assert_close(xt.grad.cpu().numpy(), v, scale=np.abs(v) + 1.0, rtol=1e-4)
+        aka = oracle.aggregate_with_weight(aka, abs_csc)
+    assert_close(xt.grad.cpu().numpy(), v, scale=va, rtol=steps)
     gw = ak.astype(np.float64).T @ g.astype(np.float64)
-    assert_close(layer.weight.grad.cpu().numpy(), gw, scale=np.abs(gw) + 1.0, rtol=1e-4)
+    assert_close(layer.weight.grad.cpu().numpy(), gw, scale=aka.astype(np.float64).T @ np.abs(g).astype(np.float64),
+                 rtol=steps)
     assert_close(layer.bias.grad.cpu().numpy(), g.astype(np.float64).sum(0), scale=np.abs(g).sum(0), rtol=1e-5)
 
 

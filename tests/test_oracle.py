@@ -144,6 +144,30 @@ def test_aggregate_vs_scipy_fp64_and_transpose_identity(V, E, F, seed):
 
 # ----------------------------------------------------------- edge softmax ---
 
+def test_aggregate_rows_equals_the_full_loop_on_those_rows():
+    """aggregate_rows is the same C loop on a sub-structure: bit-identical to the
+    rows of the full result (empty rows, a hub and repeated rows included)."""
+    rng = np.random.default_rng(77)
+    V, E, F = 300, 5000, 13
+    ei = np.stack([rng.integers(0, V, E), rng.integers(0, V, E)]).astype(np.int32)
+    ei[1, :900] = 5
+    w = rng.standard_normal(E).astype(np.float32)
+    x = rng.standard_normal((V, F)).astype(np.float32)
+    row, off, cw = oracle.cootocsc(ei, w, V)
+    full = oracle.aggregate(x, row, off, cw)
+    rows = np.array([5, 0, 299, 17, 17, 123] + list(np.flatnonzero(np.diff(off) == 0)[:3]))
+    assert np.array_equal(oracle.aggregate_rows(x, row, off, cw, rows), full[rows])
+    # the float64 arbiter against scipy's sparse product in float64, and its bound on the fp32 loop
+    import scipy.sparse as sp
+    A = sp.csr_matrix((cw.astype(np.float64), row, off), shape=(V, V))
+    exact, terms = oracle.aggregate_rows_f64(x, row, off, cw, rows)
+    np.testing.assert_allclose(exact, (A @ x.astype(np.float64))[rows], rtol=1e-12, atol=1e-13)
+    A_abs = sp.csr_matrix((np.abs(cw).astype(np.float64), row, off), shape=(V, V))      # duplicates add as |w|
+    np.testing.assert_allclose(terms, (A_abs @ np.abs(x).astype(np.float64))[rows], rtol=1e-12)
+    deg = np.diff(off)[rows][:, None]
+    assert np.all(np.abs(full[rows] - exact) <= (deg + 1) * 2.0 ** -24 * terms + 1e-30)
+
+
 def test_edgesoftmax_reference_fixture():
     g = GOLD["edgesoftmax_v3"]
     y = oracle.edgesoftmax(np.array(g["x"], np.float32), np.array(g["column_offset"], np.int32))
