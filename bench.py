@@ -1,24 +1,38 @@
 #!/usr/bin/env python3
 """Benchmark of the sparse message-passing hot path on one MI355X.
 
-Workload: weighted CSR/CSC SpMM at F=128 on the 1M-node power-law graph
-(Chung-Lu, exponent 2.1, 16M directed edges, degree cap 20,000, self-loops
-appended, gcn_norm weights, edges in random order), plus the COO->CSR/CSC
-conversion of the same graph and a GCN layer forward+backward on it.  One
-"step" is one SpMM pass (out[dst] = sum w * x[src]) over the whole graph.
-Inputs are synthetic and resident in HBM before the timed region.
+Default workload (--config 2): weighted CSR/CSC SpMM at F=128 on the 1M-node
+power-law graph (Chung-Lu, exponent 2.1, 16M directed edges, degree cap 20,000,
+self-loops appended, gcn_norm weights, edges in random order), plus the
+COO->CSR/CSC conversion of the same graph, a GCN layer forward+backward, edge
+softmax and one fused propagation hop on it.  One "step" is one SpMM pass
+(out[dst] = sum w * x[src]) over the whole graph.  --config 1, 3, 4, 5 run the
+other benchmark configurations with the same one-line JSON shape.  Inputs are
+synthetic and resident in HBM before the timed region.
 
-Prints ONE JSON line.  `value` is algorithmic bytes per step / time per step
-(bytes = 4(R+1) + 8E + 4EF + 4RF: offsets, (idx,w) per entry, one F-row
-gather per entry, the output).  Gathered rows that hit the L2 / Infinity
-Cache never reach HBM, so this figure can exceed what the HBM moved; the
-`roofline.traffic` field holds the measured HBM bytes when a counter run has
-supplied them.
+The line's `value` is algorithmic bytes per step / time per step
+(SpMM: 4(R+1) + 8E + 4EF + 4RF: offsets, (idx,w) per entry, one F-row gather per
+entry, the output) or the step time for the time-like configurations.
+
+`roofline` describes the dominant kernel of the step:
+  traffic           bytes one launch moves between L2 and the memory fabric, from the rocprofv3
+                    counter summary under profiles/ (FETCH_SIZE and WRITE_SIZE, each scaled by
+                    what it reads for a plain copy of known size); the summary must describe this
+                    very workload (V, E, F are compared) or the run stops
+  achieved, frac    traffic / the kernel's mean launch time measured in this run with HIP events
+                    on the launch stream, and that rate over the 8 TB/s HBM peak.  A gathered row
+                    that L2 serves is not memory traffic, so this -- not the algorithmic figure --
+                    is what is held against the memory roofline.  Hits in the memory-side Infinity
+                    Cache cannot be told from HBM reads by any counter the GPU exposes, so `frac`
+                    is an upper bound of the HBM share; `compulsory_frac` (every array once) is
+                    the lower bound
+  effective         algorithmic bytes / kernel time (can exceed the peak: it counts rows L2 serves)
 """
 import argparse
 import ctypes
 import json
 import os
+import re
 import sys
 import time
 
@@ -26,54 +40,68 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-F = 128
-# FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 per spmm_merge launch on this exact (seeded) workload;
-# factors from a plain 1 GiB copy in the same counter runs.
-PROFILED_TRAFFIC_BYTES = 7.074e9
 
 
 def spmm_bytes(R, E, feat):
     return 4 * (R + 1) + 8 * E + 4 * E * feat + 4 * R * feat
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the single-thread CPU timing")
-    ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run one plain 1 GiB device copy (known traffic, for scaling rocprof counters)")
-    ap.add_argument("--traffic-bytes", type=float, default=PROFILED_TRAFFIC_BYTES,
-                    help="bytes moved between L2 and the fabric per spmm_merge launch, from the separate "
-                         "rocprofv3 --pmc runs summarised under profiles/ (counters cannot be read in-process)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py: this build runs on one GPU only; --gpus %d is not supported "
-                 "(no collectives or sharding are part of it)" % args.gpus)
+def spmm_compulsory_bytes(R, C, E, feat):
+    return 4 * (R + 1) + 8 * E + 4 * C * feat + 4 * R * feat
 
-    import numpy as np
-    import torch
-    from jittorgeometric_amd import _lib, synthetic
-    from jittorgeometric_amd.nn import GCNConv, gcn_norm
-    from jittorgeometric_amd.ops import cootocsc, cootocsr
-    from jittorgeometric_amd.ops._common import spmm
 
-    if not torch.cuda.is_available():
-        sys.exit("bench.py: no GPU visible")
-    lib = _lib.load()
-    dev = torch.device("cuda:0")
-    torch.manual_seed(0)
+def read_profile(name, expect):
+    """Key figures of a rocprofv3 summary under profiles/ ('@key value' lines).  The summary
+    must have been taken on the workload of this run."""
+    path = os.path.join(ROOT, "profiles", name)
+    if not os.path.exists(path):
+        return None
+    vals = {}
+    for line in open(path):
+        m = re.match(r"@(\w+)\s+(\S+)", line)
+        if m:
+            vals[m.group(1)] = m.group(2)
+    for key, want in expect.items():
+        if key not in vals or int(float(vals[key])) != int(want):
+            sys.exit("bench.py: %s describes %s=%s, this run has %s=%s; take the counters again "
+                     "(the command is in the file's header)" % (path, key, vals.get(key), key, want))
+    return vals
 
-    # ---- inputs (host generation, then resident on the device) -------------
-    ei_np, V = synthetic.make("powerlaw_1m")
-    ei = torch.from_numpy(ei_np).to(dev)
-    ei, w = gcn_norm(ei, None, V)
-    ei = ei.contiguous()
-    E = ei.shape[1]
-    x = torch.randn(V, F, device=dev)
 
-    def timed(fn, iters, warm):
+def roofline(profile_name, expect, kernel, kernel_ms, algorithmic, compulsory, timing):
+    prof = read_profile(profile_name, expect)
+    traffic = float(prof["traffic_bytes"]) if prof and "traffic_bytes" in prof else None
+    rate = lambda b: round(b / (kernel_ms * 1e-3) / 1e9, 1)
+    out = {"bound": "hbm", "peak": HBM_PEAK_GBPS, "unit": "GB/s", "kernel": kernel, "kernel_ms": round(kernel_ms, 4),
+           "kernel_ms_source": timing, "traffic": traffic,
+           "traffic_source": ("profiles/" + profile_name) if traffic else None,
+           "algorithmic_bytes": algorithmic, "compulsory_bytes": compulsory,
+           "effective": rate(algorithmic), "compulsory_frac": round(rate(compulsory) / HBM_PEAK_GBPS, 4)}
+    if traffic:
+        out["achieved"], out["achieved_basis"] = rate(traffic), "counted L2<->fabric bytes / kernel time"
+    else:
+        out["achieved"], out["achieved_basis"] = rate(algorithmic), "algorithmic bytes / kernel time (no counter summary)"
+    out["frac"] = round(out["achieved"] / HBM_PEAK_GBPS, 4)
+    if prof:
+        for k in ("l2_hit_rate", "profile_kernel_us"):
+            if k in prof:
+                out[k] = float(prof[k])
+    return out
+
+
+class Bench:
+    def __init__(self, args):
+        import torch
+        from jittorgeometric_amd import _lib
+        self.args = args
+        self.torch = torch
+        self._lib = _lib
+        self.lib = _lib.load()
+        self.dev = torch.device("cuda:0")
+        torch.manual_seed(0)
+
+    def timed(self, fn, iters, warm):
+        torch = self.torch
         for _ in range(warm):
             fn()
         torch.cuda.synchronize()
@@ -83,57 +111,131 @@ def main():
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / iters * 1e3
 
-    if args.calibrate_copy:
-        a = torch.empty(1 << 28, dtype=torch.float32, device=dev).fill_(1.0)
+    def graph(self, name, norm="gcn"):
+        """(edge_index, weights, V, CSC, CSR, conversion times) of a configuration after the
+        normalisation with self-loops, converted on the device."""
+        from jittorgeometric_amd import synthetic
+        from jittorgeometric_amd.nn import gcn_norm, sage_norm
+        from jittorgeometric_amd.ops import cootocsc, cootocsr
+        ei_np, V = synthetic.make(name)
+        ei = self.torch.from_numpy(ei_np).to(self.dev)
+        ei, w = (gcn_norm if norm == "gcn" else sage_norm)(ei, None, V)
+        ei = ei.contiguous()
+        csr_ms = self.timed(lambda: cootocsr(ei, w, V), 10, 2)
+        csc_ms = self.timed(lambda: cootocsc(ei, w, V), 10, 2)
+        return ei, w, V, cootocsc(ei, w, V), cootocsr(ei, w, V), csr_ms, csc_ms
+
+    def spmm_kernel_ms(self, off, idx, w, x, R, iters):
+        """Mean duration of the gather kernel (spmm_merge) and of the whole call, from HIP events
+        recorded on the launch stream inside the library."""
+        torch, _lib, lib = self.torch, self._lib, self.lib
+        C, F = x.shape
+        E = idx.shape[0]
+        out = torch.empty(R, F, device=self.dev)
+        nbytes = _lib.query(lib.jgamd_spmm_csx_workspace, R, E, F)
+        ws = _lib.workspace(nbytes, self.dev)
+        k_ms, c_ms = ctypes.c_float(), ctypes.c_float()
+        torch.cuda.synchronize()
+        _lib.check(lib.jgamd_spmm_csx_timed(off.data_ptr(), idx.data_ptr(), w.data_ptr(), x.data_ptr(), out.data_ptr(),
+                                            R, C, E, F, ws.data_ptr(), nbytes, _lib.stream_ptr(self.dev), iters,
+                                            ctypes.byref(k_ms), ctypes.byref(c_ms)))
+        return k_ms.value, c_ms.value
+
+    def calibrate_copy(self):
+        torch = self.torch
+        a = torch.empty(1 << 28, dtype=torch.float32, device=self.dev).fill_(1.0)
         b = torch.empty_like(a)
         torch.cuda.synchronize()
         b.copy_(a)                      # reads 1 GiB, writes 1 GiB
         torch.cuda.synchronize()
-        del a, b
 
-    # ---- conversion ---------------------------------------------------------
-    conv_csr_ms = timed(lambda: cootocsr(ei, w, V), 10, 2)
-    conv_csc_ms = timed(lambda: cootocsc(ei, w, V), 10, 2)
-    csr = cootocsr(ei, w, V)
-    csc = cootocsc(ei, w, V)
+    def cpu_spmm_baseline(self, csc, x, step, bytes_step, conv_inputs, what):
+        """The reference's single-threaded loops (oracle port) on this host, bounded to about
+        10-30 s, and the GPU result of the same step held against them."""
+        import numpy as np
+        import oracle
+        col, off, wv = (t.cpu().numpy() for t in (csc.row_indices, csc.column_offset, csc.edge_weight))
+        xh = x.cpu().numpy()
+        V, F = xh.shape
+        passes, t0 = 0, time.perf_counter()
+        while passes < 1 or (time.perf_counter() - t0 < 10.0 and passes < 64):
+            ref = oracle.aggregate(xh, col, off, wv)
+            passes += 1
+        cpu_s = (time.perf_counter() - t0) / passes
+        # Tolerance of the path: 1e-5 of the sum of absolute terms + 1e-6, held against the exact
+        # (float64) row sums.  The reference's loop adds a row in fp32 one term after the other and
+        # is itself only good to (entries - 1) * 2^-24 of that sum, which the comparison with it allows.
+        exact, terms = oracle.aggregate_f64(xh, col, off, wv)
+        deg = np.diff(off).astype(np.float64)[:, None]
+        got = step().cpu().numpy().astype(np.float64)
+        err_exact = float(np.max(np.abs(got - exact) / (1e-6 + 1e-5 * terms)))
+        err_loop = float(np.max(np.abs(got - ref) / (1e-6 + (1e-5 + deg * 2.0 ** -24) * terms)))
+        err = max(err_exact, err_loop)
+        ei, w = conv_inputs
+        t0 = time.perf_counter()
+        oracle.cootocsr(ei.cpu().numpy(), w.cpu().numpy(), V)
+        cpu_conv_s = time.perf_counter() - t0
+        return {"value": round(bytes_step / cpu_s / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": "%d full passes of %s, %.2f s each" % (passes, what, cpu_s),
+                "cpu_model": cpu_model(), "host_cores_available": os.cpu_count(),
+                "coo_to_csr_edges_per_s": round(ei.shape[1] / cpu_conv_s),
+                "gpu_vs_exact_max_scaled_err": round(err_exact, 4),
+                "gpu_vs_cpu_max_scaled_err": round(err_loop, 4)}, err
 
-    # ---- the timed steps: SpMM over the CSC arrays at F=128 ------------------
+
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def base_line(args, metric, value, unit, ms, higher, workload, extra_config):
+    cfg = {"workload": workload}
+    cfg.update(extra_config)
+    return {"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(ms, 4), "higher_is_better": higher, "scaling": "weak", "vs_baseline": None,
+            "dtype": "f32", "data": "synthetic", "config": cfg}
+
+
+# --------------------------------------------------------------------------------- config 2
+def config2(b):
+    from jittorgeometric_amd import synthetic
+    from jittorgeometric_amd.nn import GCNConv
+    from jittorgeometric_amd.ops import EdgeSoftmax, cootocsc, gat_aggregate
+    from jittorgeometric_amd.ops._common import spmm, spmm_axpby
+    from jittorgeometric_amd.ops.gat import gat_forward_raw
+    from jittorgeometric_amd.utils import add_remaining_self_loops
+    torch, args, dev = b.torch, b.args, b.dev
+    F = 128
+    ei, w, V, csc, csr, conv_csr_ms, conv_csc_ms = b.graph("powerlaw_1m")
+    E = ei.shape[1]
+    x = torch.randn(V, F, device=dev)
+    if args.calibrate_copy:
+        b.calibrate_copy()
+
     step = lambda: spmm(csc.column_offset, csc.row_indices, csc.edge_weight, x, V)
-    ms_per_step = timed(step, args.steps, args.warmup)
+    ms_per_step = b.timed(step, args.steps, args.warmup)
     bytes_step = spmm_bytes(V, E, F)
     value = bytes_step / (ms_per_step * 1e-3) / 1e9
+    bwd_ms = b.timed(lambda: spmm(csr.row_offset, csr.column_indices, csr.edge_weight, x, V), 20, 3)
+    k_ms, c_ms = b.spmm_kernel_ms(csc.column_offset, csc.row_indices, csc.edge_weight, x, V, max(args.steps, 10))
 
-    # backward direction (CSR arrays), same kernel
-    bwd_ms = timed(lambda: spmm(csr.row_offset, csr.column_indices, csr.edge_weight, x, V), 20, 3)
-
-    # ---- dominant kernel alone: hipEvents around each spmm_merge launch ------
-    out = torch.empty(V, F, device=dev)
-    nbytes = _lib.query(lib.jgamd_spmm_csx_workspace, V, E, F)
-    ws = _lib.workspace(nbytes, dev)
-    k_ms, c_ms = ctypes.c_float(), ctypes.c_float()
-    torch.cuda.synchronize()
-    _lib.check(lib.jgamd_spmm_csx_timed(csc.column_offset.data_ptr(), csc.row_indices.data_ptr(),
-                                        csc.edge_weight.data_ptr(), x.data_ptr(), out.data_ptr(), V, V, E, F,
-                                        ws.data_ptr(), nbytes, _lib.stream_ptr(dev), max(args.steps, 10),
-                                        ctypes.byref(k_ms), ctypes.byref(c_ms)))
-    achieved = bytes_step / (k_ms.value * 1e-3) / 1e9
-
-    # ---- one GCN layer forward + backward on the same graph ------------------
+    # one GCN layer forward + backward on the same graph
     layer = GCNConv(F, F, spmm=False).to(dev)
     xg = x.clone().requires_grad_(True)
-
     g_up = torch.randn(V, F, device=dev)
 
     def layer_step():
         layer.zero_grad(set_to_none=True)
         xg.grad = None
         layer(xg, csc, csr).backward(g_up)
-    gcn_ms = timed(layer_step, 10, 2)
+    gcn_ms = b.timed(layer_step, 10, 2)
 
-    # ---- fused GAT layer core on the 169k-node configuration ----------------------
-    from jittorgeometric_amd.ops import gat_aggregate
-    from jittorgeometric_amd.ops.gat import gat_forward_raw
-    from jittorgeometric_amd.utils import add_remaining_self_loops
+    # fused GAT layer core on the 169k-node configuration
     gei_np, gV = synthetic.make("gat_169k")
     gei, _ = add_remaining_self_loops(torch.from_numpy(gei_np).to(dev), None, 1.0, gV)
     gei = gei.contiguous()
@@ -144,68 +246,42 @@ def main():
     ga_s = (torch.randn(H, D, device=dev) / 4).requires_grad_(True)
     ga_d = (torch.randn(H, D, device=dev) / 4).requires_grad_(True)
     gg = torch.randn(gV, H, D, device=dev)
-    gat_fwd_ms = timed(lambda: gat_forward_raw(gh.detach(), gcsc, ga_s.detach(), ga_d.detach(), 0.2), 20, 3)
+    gat_fwd_ms = b.timed(lambda: gat_forward_raw(gh.detach(), gcsc, ga_s.detach(), ga_d.detach(), 0.2), 20, 3)
 
     def gat_step():
         gh.grad = ga_s.grad = ga_d.grad = None
         gat_aggregate(gh, gcsc, ga_s, ga_d, 0.2).backward(gg)
-    gat_fb_ms = timed(gat_step, 20, 3)
+    gat_fb_ms = b.timed(gat_step, 20, 3)
     gat_bytes = gE * (4 + 4 * H * D) + gV * (4 + 8 * H + 4 * H * D) + gV * H * D * 4 + 2 * gV * H * 4
 
-    # ---- edge softmax (the reference's [E,1] shape) and one APPNP hop on the main graph ----
-    from jittorgeometric_amd.ops import EdgeSoftmax
-    from jittorgeometric_amd.ops._common import spmm_axpby
-    logits = torch.randn(E, 1, device=dev)
-    esm_fwd_ms = timed(lambda: EdgeSoftmax(logits, csc), 20, 3)
-    hop_ms = timed(lambda: spmm_axpby(csc.column_offset, csc.row_indices, csc.edge_weight, x, V, 0.9, 0.1, x), 10, 2)
-    del logits
+    # edge softmax (the reference's [E,1] shape, and 8 heads) and one propagation hop
+    logits = torch.randn(E, 1, device=dev, requires_grad=True)
+    esm_fwd_ms = b.timed(lambda: EdgeSoftmax(logits.detach(), csc), 20, 3)
+    y1 = EdgeSoftmax(logits, csc)
+    g1 = torch.randn(E, 1, device=dev)
+    esm_bwd_ms = b.timed(lambda: torch.autograd.grad(y1, logits, g1, retain_graph=True), 20, 3)
+    del y1, g1, logits
+    logits8 = torch.randn(E, 8, device=dev)
+    esm8_fwd_ms = b.timed(lambda: EdgeSoftmax(logits8, csc), 10, 2)
+    del logits8
+    hop_ms = b.timed(lambda: spmm_axpby(csc.column_offset, csc.row_indices, csc.edge_weight, x, V, 0.9, 0.1, x), 10, 2)
 
-    # ---- CPU baseline: the reference's single-threaded loop (oracle port) ----
-    cpu = None
+    cpu, err = (None, 0.0)
     if not args.no_cpu_baseline:
-        import oracle
-        col = csc.row_indices.cpu().numpy()
-        off = csc.column_offset.cpu().numpy()
-        wv = csc.edge_weight.cpu().numpy()
-        xh = x.cpu().numpy()
-        passes, t0 = 0, time.perf_counter()
-        while passes < 3 or (time.perf_counter() - t0 < 10.0 and passes < 64):
-            ref = oracle.aggregate(xh, col, off, wv)
-            passes += 1
-        cpu_s = (time.perf_counter() - t0) / passes
-        got = step().cpu().numpy()
-        err = float(np.max(np.abs(got - ref) / (1e-6 + 1e-5 * np.abs(ref) + 1e-5)))
-        t0 = time.perf_counter()
-        oracle.cootocsr(ei.cpu().numpy(), w.cpu().numpy(), V)
-        cpu_conv_s = time.perf_counter() - t0
-        cpu = {"value": round(bytes_step / cpu_s / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
-               "sample": "%d full SpMM passes of the same workload (V=%d, E=%d, F=%d), %.2f s each"
-                         % (passes, V, E, F, cpu_s),
-               "host_cores_available": os.cpu_count(),
-               "coo_to_csr_edges_per_s": round(E / cpu_conv_s),
-               "gpu_vs_cpu_max_scaled_err": round(err, 4)}
+        cpu, err = b.cpu_spmm_baseline(csc, x, step, bytes_step, (ei, w),
+                                       "the same SpMM workload (V=%d, E=%d, F=%d)" % (V, E, F))
 
-    line = {
-        "metric": "spmm_f128_algorithmic_bandwidth",
-        "value": round(value, 1),
-        "unit": "GB/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4),
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "f32",
-        "data": "synthetic",
-        "config": {"workload": "weighted CSC SpMM, V=1,000,000 Chung-Lu power-law (exp 2.1, cap 20000) "
-                               "+ self-loops, gcn_norm weights, F=128", "V": V, "E": E, "F": F,
-                   "bytes_per_step": bytes_step},
-        "pct_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
+    line = base_line(args, "spmm_f128_algorithmic_bandwidth", round(value, 1), "GB/s", ms_per_step, True,
+                     "config 2: weighted CSC SpMM, V=1,000,000 Chung-Lu power-law (exp 2.1, cap 20000) "
+                     "+ self-loops, gcn_norm weights, F=128", {"V": V, "E": E, "F": F, "bytes_per_step": bytes_step})
+    esm_b = lambda h, per: (per * E * h + 4 * (V + 1))
+    line.update({
+        "pct_hbm_peak_algorithmic": round(100 * value / HBM_PEAK_GBPS, 2),
         "spmm_csr_backward_ms": round(bwd_ms, 4),
         "coo_to_csr_edges_per_s": round(E / (conv_csr_ms * 1e-3)),
         "coo_to_csc_edges_per_s": round(E / (conv_csc_ms * 1e-3)),
         "coo_to_csr_ms": round(conv_csr_ms, 4),
+        "coo_to_csr_algorithmic_gbps": round((24 * E + 8 * (V + 1)) / (conv_csr_ms * 1e-3) / 1e9, 1),
         "gcn_layer_fwd_bwd_ms": round(gcn_ms, 4),
         "gcn_layer_shape": "GCNConv(128->128) on the same graph, aggregateWithWeight path: x@W, SpMM, bias; "
                            "backward SpMM, W.grad, x.grad",
@@ -214,17 +290,249 @@ def main():
         "gat_fused_fwd_algorithmic_gbps": round(gat_bytes / (gat_fwd_ms * 1e-3) / 1e9, 1),
         "gat_shape": "V=%d, E=%d (power-law exp 2.3 + self-loops), 8 heads x 16" % (gV, gE),
         "edge_softmax_fwd_ms": round(esm_fwd_ms, 4),
-        "edge_softmax_fwd_algorithmic_gbps": round((8 * E + 4 * (V + 1)) / (esm_fwd_ms * 1e-3) / 1e9, 1),
+        "edge_softmax_fwd_algorithmic_gbps": round(esm_b(1, 8) / (esm_fwd_ms * 1e-3) / 1e9, 1),
+        "edge_softmax_bwd_ms": round(esm_bwd_ms, 4),
+        "edge_softmax_bwd_algorithmic_gbps": round(esm_b(1, 12) / (esm_bwd_ms * 1e-3) / 1e9, 1),
+        "edge_softmax_h8_fwd_ms": round(esm8_fwd_ms, 4),
+        "edge_softmax_h8_fwd_algorithmic_gbps": round(esm_b(8, 8) / (esm8_fwd_ms * 1e-3) / 1e9, 1),
         "appnp_hop_f128_ms": round(hop_ms, 4),
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": args.traffic_bytes,
-                     "traffic_source": "profiles/bench_workload_mi355x.txt",
-                     "traffic_rate_gbps": round(args.traffic_bytes / (k_ms.value * 1e-3) / 1e9, 1) if args.traffic_bytes else None,
-                     "kernel": "spmm_merge<2,1,16,false,true,false>", "kernel_ms": round(k_ms.value, 4),
-                     "call_ms": round(c_ms.value, 4), "algorithmic_bytes": bytes_step},
+        "roofline": roofline("spmm_merge_powerlaw_1m_f128.txt", {"V": V, "E": E, "F": F}, "spmm_merge", k_ms,
+                             bytes_step, spmm_compulsory_bytes(V, V, E, F), "hipEvents in this run"),
+        "spmm_call_ms": round(c_ms, 4),
         "cpu_baseline": cpu,
-    }
+    })
+    return line, err
+
+
+# --------------------------------------------------------------------------------- config 1
+def config1(b):
+    """2-layer GCN forward + backward on the 2,708-node graph (1433 -> 256 -> 7)."""
+    import numpy as np
+    from jittorgeometric_amd.nn import GCNConv
+    from jittorgeometric_amd.ops._common import spmm
+    torch, args, dev = b.torch, b.args, b.dev
+    ei, w, V, csc, csr, conv_csr_ms, conv_csc_ms = b.graph("cora_like")
+    E = ei.shape[1]
+    rng = np.random.default_rng(1)
+    xh = (rng.random((V, 1433)) < 0.013).astype(np.float32)
+    xh /= np.maximum(xh.sum(1, keepdims=True), 1)
+    x = torch.from_numpy(xh).to(dev)
+    y = torch.from_numpy(rng.integers(0, 7, V)).to(dev)
+    l1, l2 = GCNConv(1433, 256, spmm=False).to(dev), GCNConv(256, 7, spmm=False).to(dev)
+
+    def step():
+        l1.zero_grad(set_to_none=True)
+        l2.zero_grad(set_to_none=True)
+        out = l2(torch.relu(l1(x, csc, csr)), csc, csr)
+        torch.nn.functional.cross_entropy(out, y).backward()
+    ms = b.timed(step, args.steps, args.warmup)
+    h = torch.randn(V, 256, device=dev)
+    k_ms, _ = b.spmm_kernel_ms(csc.column_offset, csc.row_indices, csc.edge_weight, h, V, 50)
+    cpu = None
+    if not args.no_cpu_baseline:
+        import oracle
+        W1, W2 = l1.weight.detach().cpu().numpy(), l2.weight.detach().cpu().numpy()
+        oc = tuple(t.cpu().numpy() for t in (csc.row_indices, csc.column_offset, csc.edge_weight))
+        orr = tuple(t.cpu().numpy() for t in (csr.column_indices, csr.row_offset, csr.edge_weight))
+        n, t0 = 0, time.perf_counter()
+        while n < 3 or time.perf_counter() - t0 < 3.0:
+            a1 = oracle.aggregate(xh @ W1, *oc)
+            a2 = oracle.aggregate(np.maximum(a1, 0) @ W2, *oc)
+            g2 = oracle.aggregate(a2, *orr)                       # stand-in upstream gradient of the same shape
+            g1 = oracle.aggregate((g2 @ W2.T) * (a1 > 0), *orr)
+            _ = xh.T @ g1
+            n += 1
+        cpu = {"value": round((time.perf_counter() - t0) / n * 1e3, 3), "unit": "ms", "cores": 1, "kind": "port",
+               "sample": "%d passes of the four aggregations and the dense products of the step (numpy + oracle loops)" % n,
+               "cpu_model": cpu_model()}
+    line = base_line(args, "gcn2_fwd_bwd_ms", round(ms, 4), "ms", ms, False,
+                     "config 1: 2-layer GCN forward+backward, V=2708, 10556 directed edges + self-loops, 1433->256->7",
+                     {"V": V, "E": E})
+    line.update({"coo_to_csr_ms": round(conv_csr_ms, 4),
+                 "roofline": roofline("spmm_merge_cora_like_f256.txt", {"V": V, "E": E, "F": 256}, "spmm_merge", k_ms,
+                                      spmm_bytes(V, E, 256), spmm_compulsory_bytes(V, V, E, 256), "hipEvents in this run"),
+                 "note": "launch-bound at this size: 13k entries are one launch of a few microseconds",
+                 "cpu_baseline": cpu})
+    return line, 0.0
+
+
+# --------------------------------------------------------------------------------- config 3
+def config3(b):
+    """Fused GAT core (edge softmax + weighted aggregation), 8 heads x 16, forward and backward."""
+    from jittorgeometric_amd import synthetic
+    from jittorgeometric_amd.ops import cootocsc, gat_aggregate
+    from jittorgeometric_amd.ops.gat import gat_forward_raw
+    from jittorgeometric_amd.utils import add_remaining_self_loops
+    torch, args, dev = b.torch, b.args, b.dev
+    ei_np, V = synthetic.make("gat_169k")
+    ei, _ = add_remaining_self_loops(torch.from_numpy(ei_np).to(dev), None, 1.0, V)
+    ei = ei.contiguous()
+    E = ei.shape[1]
+    csc = cootocsc(ei, torch.ones(E, device=dev), V)
+    H, D = 8, 16
+    h = torch.randn(V, H, D, device=dev, requires_grad=True)
+    a_s = (torch.randn(H, D, device=dev) / 4).requires_grad_(True)
+    a_d = (torch.randn(H, D, device=dev) / 4).requires_grad_(True)
+    g = torch.randn(V, H, D, device=dev)
+    fwd_ms = b.timed(lambda: gat_forward_raw(h.detach(), csc, a_s.detach(), a_d.detach(), 0.2), 20, 3)
+
+    def step():
+        h.grad = a_s.grad = a_d.grad = None
+        gat_aggregate(h, csc, a_s, a_d, 0.2).backward(g)
+    ms = b.timed(step, args.steps, args.warmup)
+    fwd_bytes = E * (4 + 4 * H * D) + V * (4 + 8 * H + 4 * H * D) + V * H * D * 4 + 2 * V * H * 4
+    compulsory = 8 * E + 4 * (V + 1) + 2 * V * H * D * 4 + 4 * V * H * 4
+    cpu = None
+    if not args.no_cpu_baseline:
+        import oracle
+        row, off = csc.row_indices.cpu().numpy(), csc.column_offset.cpu().numpy()
+        hh, s, d = h.detach().cpu().numpy(), a_s.detach().cpu().numpy(), a_d.detach().cpu().numpy()
+        n, t0 = 0, time.perf_counter()
+        while n < 1 or time.perf_counter() - t0 < 5.0:
+            oracle.gat_forward_heads(hh, (row, off, None), s, d, 0.2)
+            n += 1
+        cpu = {"value": round((time.perf_counter() - t0) / n * 1e3, 2), "unit": "ms (forward only)", "cores": 1,
+               "kind": "port", "sample": "%d forward passes of the reference's operator chain (oracle loops), all heads" % n,
+               "cpu_model": cpu_model()}
+    prof = read_profile("gat_merge_gat_169k_h8x16.txt", {"V": V, "E": E, "F": H * D})
+    k_ms = float(prof["profile_kernel_us"]) / 1e3 if prof and "profile_kernel_us" in prof else fwd_ms
+    line = base_line(args, "gat_fused_fwd_bwd_ms", round(ms, 4), "ms", ms, False,
+                     "config 3: fused GAT core fwd+bwd, V=169,343, power-law exp 2.3 + self-loops, 8 heads x 16",
+                     {"V": V, "E": E, "H": H, "D": D})
+    line.update({"gat_fused_fwd_ms": round(fwd_ms, 4),
+                 "gat_fused_fwd_algorithmic_gbps": round(fwd_bytes / (fwd_ms * 1e-3) / 1e9, 1),
+                 "roofline": roofline("gat_merge_gat_169k_h8x16.txt", {"V": V, "E": E, "F": H * D}, "gat_fwd_merge", k_ms,
+                                      fwd_bytes, compulsory,
+                                      "rocprofv3 summary" if prof else "whole forward call in this run (4 launches)"),
+                 "cpu_baseline": cpu})
+    return line, 0.0
+
+
+# --------------------------------------------------------------------------------- config 4
+def config4(b):
+    """Dense-degree aggregation at F = 602, 256, 41 and the conversion of the 114.6M-edge list."""
+    from jittorgeometric_amd.ops._common import spmm
+    torch, args, dev = b.torch, b.args, b.dev
+    ei, w, V, csc, csr, conv_csr_ms, conv_csc_ms = b.graph("dense_233k")
+    E = ei.shape[1]
+    res = {}
+    for F in (602, 256, 41):
+        x = torch.randn(V, F, device=dev)
+        step = lambda: spmm(csc.column_offset, csc.row_indices, csc.edge_weight, x, V)
+        ms = b.timed(step, args.steps if F == 602 else 10, args.warmup if F == 602 else 2)
+        k_ms, _ = b.spmm_kernel_ms(csc.column_offset, csc.row_indices, csc.edge_weight, x, V, 10)
+        res[F] = (ms, k_ms, x, step)
+    ms, k_ms, x, step = res[602]
+    bytes_step = spmm_bytes(V, E, 602)
+    cpu, err = (None, 0.0)
+    if not args.no_cpu_baseline:
+        x41 = res[41][2]
+        cpu, err = b.cpu_spmm_baseline(csc, x41, res[41][3], spmm_bytes(V, E, 41), (ei, w),
+                                       "the F=41 product of this graph (V=%d, E=%d)" % (V, E))
+    line = base_line(args, "spmm_f602_algorithmic_bandwidth", round(bytes_step / (ms * 1e-3) / 1e9, 1), "GB/s", ms, True,
+                     "config 4: weighted CSC SpMM, V=232,965, lognormal degrees (mean 492) + self-loops, F=602",
+                     {"V": V, "E": E, "F": 602, "bytes_per_step": bytes_step})
+    line.update({"spmm_f256_ms": round(res[256][0], 4),
+                 "spmm_f256_algorithmic_gbps": round(spmm_bytes(V, E, 256) / (res[256][0] * 1e-3) / 1e9, 1),
+                 "spmm_f41_ms": round(res[41][0], 4),
+                 "spmm_f41_algorithmic_gbps": round(spmm_bytes(V, E, 41) / (res[41][0] * 1e-3) / 1e9, 1),
+                 "coo_to_csr_ms": round(conv_csr_ms, 4), "coo_to_csr_edges_per_s": round(E / (conv_csr_ms * 1e-3)),
+                 "coo_to_csc_edges_per_s": round(E / (conv_csc_ms * 1e-3)),
+                 "roofline": roofline("spmm_merge_dense_233k_f602.txt", {"V": V, "E": E, "F": 602}, "spmm_merge", k_ms,
+                                      bytes_step, spmm_compulsory_bytes(V, V, E, 602), "hipEvents in this run"),
+                 "cpu_baseline": cpu})
+    return line, err
+
+
+# --------------------------------------------------------------------------------- config 5
+def config5(b):
+    """Full-graph 3-layer GCN and GraphSAGE-mean forward + backward (100 -> 256 -> 256 -> 47)."""
+    from jittorgeometric_amd.nn import GCNConv, SAGEConv
+    from jittorgeometric_amd.ops import cootocsc, cootocsr
+    from jittorgeometric_amd.ops._common import spmm
+    torch, args, dev = b.torch, b.args, b.dev
+    ei, w, V, csc, csr, conv_csr_ms, conv_csc_ms = b.graph("powerlaw_2m4")
+    E = ei.shape[1]
+    dims = [100, 256, 256, 47]
+    x = torch.randn(V, 100, device=dev)
+    y = torch.randint(0, 47, (V,), device=dev)
+
+    def model_step(layers, call):
+        for layer in layers:
+            layer.zero_grad(set_to_none=True)
+        hcur = x
+        for i, layer in enumerate(layers):
+            hcur = call(layer, hcur)
+            if i < 2:
+                hcur = torch.relu(hcur)
+        torch.nn.functional.cross_entropy(hcur, y).backward()
+
+    gcn = [GCNConv(dims[i], dims[i + 1], spmm=False).to(dev) for i in range(3)]
+    gcn_ms = b.timed(lambda: model_step(gcn, lambda l, t: l(t, csc, csr)), args.steps, args.warmup)
+    from jittorgeometric_amd.nn import sage_norm
+    sei, sw = sage_norm(ei[:, :E - V].contiguous(), None, V)       # same edges, mean weights
+    sei = sei.contiguous()
+    scsc, scsr = cootocsc(sei, sw, V), cootocsr(sei, sw, V)
+    sage = [SAGEConv(dims[i], dims[i + 1], root_weight=False, spmm=False).to(dev) for i in range(3)]
+    sage_ms = b.timed(lambda: model_step(sage, lambda l, t: l(t, None, None, scsc, scsr)), args.steps, args.warmup)
+    prod = {}
+    for F in (100, 256, 47):
+        xf = torch.randn(V, F, device=dev)
+        prod[F] = (b.timed(lambda: spmm(csc.column_offset, csc.row_indices, csc.edge_weight, xf, V), 10, 2),
+                   b.spmm_kernel_ms(csc.column_offset, csc.row_indices, csc.edge_weight, xf, V, 10)[0], xf)
+    cpu, err = (None, 0.0)
+    if not args.no_cpu_baseline:
+        xf = prod[47][2]
+        cpu, err = b.cpu_spmm_baseline(csc, xf, lambda: spmm(csc.column_offset, csc.row_indices, csc.edge_weight, xf, V),
+                                       spmm_bytes(V, E, 47), (ei, w),
+                                       "the F=47 product of this graph (V=%d, E=%d)" % (V, E))
+    line = base_line(args, "gcn3_fullgraph_fwd_bwd_ms", round(gcn_ms, 3), "ms", gcn_ms, False,
+                     "config 5: 3-layer GCN full-graph forward+backward, V=2,449,029 power-law (exp 2.1, mean 50) "
+                     "+ self-loops, 100->256->256->47", {"V": V, "E": E})
+    line.update({"sage3_fullgraph_fwd_bwd_ms": round(sage_ms, 3),
+                 "coo_to_csr_ms": round(conv_csr_ms, 4), "coo_to_csr_edges_per_s": round(E / (conv_csr_ms * 1e-3)),
+                 "coo_to_csc_edges_per_s": round(E / (conv_csc_ms * 1e-3))})
+    for F in (100, 256, 47):
+        line["spmm_f%d_ms" % F] = round(prod[F][0], 4)
+        line["spmm_f%d_algorithmic_gbps" % F] = round(spmm_bytes(V, E, F) / (prod[F][0] * 1e-3) / 1e9, 1)
+    line["roofline"] = roofline("spmm_merge_powerlaw_2m4_f256.txt", {"V": V, "E": E, "F": 256}, "spmm_merge", prod[256][1],
+                                spmm_bytes(V, E, 256), spmm_compulsory_bytes(V, V, E, 256), "hipEvents in this run")
+    line["cpu_baseline"] = cpu
+    return line, err
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=None)
+    ap.add_argument("--config", type=int, default=2, choices=[1, 2, 3, 4, 5],
+                    help="benchmark configuration; 2 (the headline SpMM workload) is the default")
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the single-thread CPU timing")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain 1 GiB device copy (known traffic, for scaling rocprof counters)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only; --gpus %d is not supported "
+                 "(no collectives or sharding are part of it)" % args.gpus)
+    defaults = {1: (200, 20), 2: (50, 5), 3: (50, 5), 4: (10, 2), 5: (5, 1)}
+    if args.steps is None:
+        args.steps = defaults[args.config][0]
+    if args.warmup is None:
+        args.warmup = defaults[args.config][1]
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    b = Bench(args)
+    if args.calibrate_copy and args.config != 2:
+        b.calibrate_copy()
+    line, err = {1: config1, 2: config2, 3: config3, 4: config4, 5: config5}[args.config](b)
     print(json.dumps(line))
+    if err > 1.0:
+        sys.exit("bench.py: the GPU result is %.2f times the tolerance away from the CPU result "
+                 "(1e-5 of the sum of absolute terms + 1e-6 against the exact row sums; against the "
+                 "reference's fp32 loop its own sequential rounding is allowed on top)" % err)
 
 
 if __name__ == "__main__":

@@ -143,6 +143,18 @@ def aggregate_rows_f64(x, indices, offset, weight, rows):
     return out, terms
 
 
+def aggregate_f64(x, indices, offset, weight):
+    """aggregate_rows_f64 for every row (no copy of the compressed arrays)."""
+    x = _f32(x)
+    indices, offset, weight = _i32(indices), _i32(offset), _f32(weight)
+    n = offset.shape[0] - 1
+    out = np.empty((n, x.shape[1]), np.float64)
+    terms = np.empty((n, x.shape[1]), np.float64)
+    lib().orc_aggregate_f64(_p(out), _p(terms), _p(x), _p(indices), _p(offset), _p(weight), ctypes.c_int32(n),
+                            ctypes.c_int32(x.shape[1]))
+    return out, terms
+
+
 def aggregate_rows(x, indices, offset, weight, rows):
     """Rows `rows` of aggregate(x, indices, offset, weight), by the same C loop run on the
     compressed arrays of those rows only (each chosen row keeps its entries in their order),
