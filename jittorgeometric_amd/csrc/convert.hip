@@ -12,9 +12,12 @@
 //   2. scan             : the (bucket, block) table -> each block's write
 //                         cursor in each bucket (and every bucket's extent).
 //   3. partition        : every block re-reads its edges, sorts its tile by
-//                         bucket inside LDS and writes 12/16-byte records,
+//                         bucket inside LDS and writes one record per edge,
 //                         one contiguous run per (block, bucket), in input
-//                         order.
+//                         order.  A record is packed into 8 bytes (12 with the
+//                         permutation) when a node id and the key bits left for
+//                         the second level fit one word, else it is the plain
+//                         12/16-byte (key, other, weight[, position]).
 //   4. sub-block plan   : buckets are cut into sub-blocks of <= 8192 records
 //                         (one tile), so a hub's bucket is many blocks' work.
 //   5. sub-block count  : LDS counts per key of the bucket (<= 2048 keys).
@@ -33,6 +36,8 @@
 // the records are sorted by plain LSD passes of the same stable partition
 // (11-bit digits, least significant first), the offsets are read off the
 // sorted keys, and the records are unpacked.
+#include <type_traits>
+
 #include "common.h"
 
 namespace jg {
@@ -53,6 +58,79 @@ struct __attribute__((aligned(16))) Rec4 {
     int32_t key, other;
     uint32_t w;
     int32_t id;
+};
+
+// Between the two levels a record is packed: inside a bucket only the low `shift` bits of the
+// key matter, so a = (key low bits << obits) | other endpoint and b = the weight's bits.  An
+// endpoint that does not fit the obits = 32 - shift bits left (never the case for node ids
+// below V, whatever the graph) is replaced by the all-ones field and b by the edge's position
+// in the input; the last step then fetches endpoint and weight from the input arrays.  With
+// out_perm the record carries the edge's position as a third word.
+struct __attribute__((aligned(8))) Pack2 {
+    uint32_t a, b;
+};
+struct Pack3 {
+    uint32_t a, b;
+    int32_t id;
+};
+template <bool PERM> struct PackOf { using type = Pack2; };
+template <> struct PackOf<true> { using type = Pack3; };
+__device__ __forceinline__ int32_t get_id(const Pack2 &) { return 0; }
+__device__ __forceinline__ int32_t get_id(const Pack3 &r) { return r.id; }
+struct PackRule {
+    int shift;          // low key bits kept in a record
+    int obits;          // bits of the endpoint field (32 - shift)
+    uint32_t omask;     // all ones in that field = "look the edge up"
+};
+__device__ __forceinline__ uint32_t key_low_of(uint32_t a, const PackRule &p) { return p.shift ? a >> p.obits : 0u; }
+__device__ __forceinline__ Pack2 pack(const Rec3 &r, const PackRule &p)
+{
+    // an endpoint that does not fit was replaced by -1 when the record was loaded, with its
+    // edge's position in the weight word
+    Pack2 q;
+    q.a = ((uint32_t)r.other >= p.omask ? p.omask : (uint32_t)r.other) | (p.shift ? ((uint32_t)r.key << p.obits) : 0u);
+    q.b = r.w;
+    return q;
+}
+__device__ __forceinline__ Pack3 pack(const Rec4 &r, const PackRule &p)
+{
+    Pack3 q;
+    q.a = ((uint32_t)r.other >= p.omask ? p.omask : (uint32_t)r.other) | (p.shift ? ((uint32_t)r.key << p.obits) : 0u);
+    q.b = r.w;
+    q.id = r.id;
+    return q;
+}
+
+// How the second level reads a record of either form.
+struct PackedView {
+    PackRule rule;
+    template <typename R> __device__ __forceinline__ int key_low(const R &q) const { return (int)key_low_of(q.a, rule); }
+    template <bool PERM, typename R>
+    __device__ __forceinline__ void unpack(const R &q, const int32_t *others_in, const uint32_t *w_in, int32_t &other,
+                                           uint32_t &wv, int32_t &id) const
+    {
+        uint32_t o = rule.shift ? (q.a & rule.omask) : q.a;
+        wv = q.b;
+        id = get_id(q);
+        if (o == rule.omask) {       // endpoint kept in the input arrays
+            if (!PERM) id = (int32_t)wv;
+            o = (uint32_t)others_in[id];
+            wv = w_in ? w_in[id] : 0u;
+        }
+        other = (int32_t)o;
+    }
+};
+struct PlainView {
+    int mask;
+    template <typename R> __device__ __forceinline__ int key_low(const R &q) const { return q.key & mask; }
+    template <bool PERM, typename R>
+    __device__ __forceinline__ void unpack(const R &q, const int32_t *, const uint32_t *, int32_t &other, uint32_t &wv,
+                                           int32_t &id) const
+    {
+        other = q.other;
+        wv = q.w;
+        id = get_id(q);
+    }
 };
 
 template <bool PERM> struct RecOf { using type = Rec3; };
@@ -220,8 +298,8 @@ __device__ __forceinline__ int tile_sort(uint32_t *raw, int stage_n, TileLds &L,
     return L.misc[kPartWaves];
 }
 
-template <typename Rec, typename Emit>
-__device__ __forceinline__ void tile_emit(const TileLds &L, int total, int shift, int mask, const Rec (&rec)[kItems],
+template <typename Rec, typename BinOfRec, typename Emit>
+__device__ __forceinline__ void tile_emit(const TileLds &L, int total, BinOfRec bin_of_rec, const Rec (&rec)[kItems],
                                           const int (&bin)[kItems], const int (&lp)[kItems], Emit emit)
 {
     Rec *stage = reinterpret_cast<Rec *>(L.stage);
@@ -234,7 +312,7 @@ __device__ __forceinline__ void tile_emit(const TileLds &L, int total, int shift
 #pragma unroll 4
         for (int j = threadIdx.x; j < n; j += kPartThreads) {
             const Rec q = stage[j];
-            emit(L.delta[(q.key >> shift) & mask] + h0 + j, q);
+            emit(L.delta[bin_of_rec(q)] + h0 + j, q);
         }
         __syncthreads();
     }
@@ -242,12 +320,15 @@ __device__ __forceinline__ void tile_emit(const TileLds &L, int total, int shift
 
 // ---------------------------------------------------------------- step 3 ---
 // Loader for the first partition: items come from the COO arrays.
+__device__ __forceinline__ void keep_position(Rec3 &r, int32_t c) { r.w = (uint32_t)c; }
+__device__ __forceinline__ void keep_position(Rec4 &, int32_t) {}      // has it already (id)
 template <typename Rec> struct CooLoader {
     const int32_t *keys;
     const int32_t *others;
     const uint32_t *w;
     int64_t n;
     int32_t V;
+    uint32_t omask;     // endpoints from this value up do not pack (0: nothing is packed, LSD passes)
     // Branch-free: the index is clamped, validity is judged afterwards.
     __device__ __forceinline__ void load(int64_t e, Rec &r) const
     {
@@ -256,6 +337,14 @@ template <typename Rec> struct CooLoader {
         r.other = others[c];
         r.w = w ? w[c] : 0u;
         set_id(r, (int32_t)c);
+        // an endpoint that does not pack is looked up again from its position at the end; no
+        // lane of a wavefront has one in any graph whose node ids are below V
+        if (omask && __ballot((uint32_t)r.other >= omask) != 0ull) {
+            if ((uint32_t)r.other >= omask) {
+                r.other = -1;
+                keep_position(r, (int32_t)c);
+            }
+        }
     }
     __device__ __forceinline__ bool valid(int64_t e, const Rec &r) const
     {
@@ -338,7 +427,31 @@ __global__ __launch_bounds__(kPartThreads) void csx_partition(Loader in, int shi
     TileLds L;
     const int total = tile_sort<Rec>(lds_raw, stage_n, L, nbins, nbits, bin, lp,
                                      [&](int b) { return table[(int64_t)b * nblocks + blk]; });
-    tile_emit(L, total, shift, mask, rec, bin, lp, [&](int pos, const Rec &q) { out[pos] = q; });
+    tile_emit(L, total, [&](const Rec &q) { return (q.key >> shift) & mask; }, rec, bin, lp,
+              [&](int pos, const Rec &q) { out[pos] = q; });
+}
+
+// The first partition of the two-level path: same tile sort, the records leave packed.
+template <typename Rec, typename Out>
+__global__ __launch_bounds__(kPartThreads) void csx_partition_pack(CooLoader<Rec> in, PackRule rule, int nbins, int nbits,
+                                                                   const int32_t *__restrict__ table, int nblocks,
+                                                                   Out *__restrict__ out, int stage_n)
+{
+    extern __shared__ uint32_t lds_raw[];
+    const int w = threadIdx.x >> 6;
+    const int64_t base = (int64_t)blockIdx.x * kTile + (int64_t)w * kWaveSpan + lane_id();
+    Rec rec[kItems];
+    int bin[kItems], lp[kItems];
+#pragma unroll
+    for (int r = 0; r < kItems; r++) in.load(base + (int64_t)r * kWave, rec[r]);
+#pragma unroll
+    for (int r = 0; r < kItems; r++) bin[r] = in.valid(base + (int64_t)r * kWave, rec[r]) ? (rec[r].key >> rule.shift) : -1;
+    const int blk = blockIdx.x;
+    TileLds L;
+    const int total = tile_sort<Rec>(lds_raw, stage_n, L, nbins, nbits, bin, lp,
+                                     [&](int b) { return table[(int64_t)b * nblocks + blk]; });
+    tile_emit(L, total, [&](const Rec &q) { return q.key >> rule.shift; }, rec, bin, lp,
+              [&](int pos, const Rec &q) { out[pos] = pack(q, rule); });
 }
 
 // ---------------------------------------------------------------- step 4 ---
@@ -412,27 +525,27 @@ __device__ __forceinline__ SubRange sub_range(const int32_t *table, int nblocks,
 
 // ---------------------------------------------------------------- step 5 ---
 // cnt2[s][key] = records of sub-block s whose low key bits are `key`.
-template <typename Rec>
+template <typename Rec, typename View>
 __global__ __launch_bounds__(kPartThreads) void csx_sub_count(const Rec *__restrict__ recs,
                                                               const int32_t *__restrict__ table, int nblocks,
                                                               const int32_t *__restrict__ sub_bucket,
-                                                              const int32_t *__restrict__ sub_first, int shift,
+                                                              const int32_t *__restrict__ sub_first, View view, int shift,
                                                               int32_t *__restrict__ cnt2)
 {
     __shared__ int bins[kMaxBins];
     const SubRange r = sub_range(table, nblocks, sub_bucket, sub_first, blockIdx.x);
     if (r.bucket < 0) return;
-    const int nkeys = 1 << shift, mask = nkeys - 1;
+    const int nkeys = 1 << shift;
     for (int k = threadIdx.x; k < nkeys; k += kPartThreads) bins[k] = 0;
     __syncthreads();
     constexpr int kBatch = 8;
     for (int e0 = r.begin + threadIdx.x; e0 < r.end; e0 += kBatch * kPartThreads) {
-        int32_t k[kBatch];
+        int k[kBatch];
 #pragma unroll
-        for (int i = 0; i < kBatch; i++) k[i] = recs[min(e0 + i * kPartThreads, r.end - 1)].key;
+        for (int i = 0; i < kBatch; i++) k[i] = view.key_low(recs[min(e0 + i * kPartThreads, r.end - 1)]);
 #pragma unroll
         for (int i = 0; i < kBatch; i++)
-            if (e0 + i * kPartThreads < r.end) atomicAdd(&bins[k[i] & mask], 1);
+            if (e0 + i * kPartThreads < r.end) atomicAdd(&bins[k[i]], 1);
     }
     __syncthreads();
     for (int k = threadIdx.x; k < nkeys; k += kPartThreads) cnt2[(int64_t)blockIdx.x * nkeys + k] = bins[k];
@@ -496,13 +609,15 @@ __global__ __launch_bounds__(kPartThreads) void csx_bucket_offsets(const int32_t
 
 // ---------------------------------------------------------------- step 7 ---
 // One block per sub-block (one tile of records): sorted by key inside LDS,
-// then every key's run goes to cnt2[sub][key] onwards.
-template <typename Rec, bool PERM>
+// then every key's run goes to cnt2[sub][key] onwards, unpacked.
+template <typename Rec, bool PERM, typename View>
 __global__ __launch_bounds__(kPartThreads) void csx_sub_scatter(const Rec *__restrict__ recs,
                                                                 const int32_t *__restrict__ table, int nblocks,
                                                                 const int32_t *__restrict__ sub_bucket,
                                                                 const int32_t *__restrict__ sub_first,
-                                                                const int32_t *__restrict__ cnt2, int shift,
+                                                                const int32_t *__restrict__ cnt2, View view, int shift,
+                                                                const int32_t *__restrict__ others_in,
+                                                                const uint32_t *__restrict__ w_in,
                                                                 int32_t *__restrict__ out_idx,
                                                                 uint32_t *__restrict__ out_w,
                                                                 int32_t *__restrict__ out_perm, int stage_n)
@@ -511,21 +626,24 @@ __global__ __launch_bounds__(kPartThreads) void csx_sub_scatter(const Rec *__res
     const int sub = blockIdx.x;
     const SubRange sr = sub_range(table, nblocks, sub_bucket, sub_first, sub);
     if (sr.bucket < 0) return;
-    const int nkeys = 1 << shift, mask = nkeys - 1;
+    const int nkeys = 1 << shift;
     const int base = sr.begin + (threadIdx.x >> 6) * kWaveSpan + lane_id();
     Rec rec[kItems];
     int bin[kItems], lp[kItems];
 #pragma unroll
     for (int r = 0; r < kItems; r++) rec[r] = recs[min(base + r * kWave, sr.end - 1)];
 #pragma unroll
-    for (int r = 0; r < kItems; r++) bin[r] = base + r * kWave < sr.end ? (rec[r].key & mask) : -1;
+    for (int r = 0; r < kItems; r++) bin[r] = base + r * kWave < sr.end ? view.key_low(rec[r]) : -1;
     TileLds L;
     const int total = tile_sort<Rec>(lds_raw, stage_n, L, nkeys, shift, bin, lp,
                                      [&](int k) { return cnt2[(int64_t)sub * nkeys + k]; });
-    tile_emit(L, total, 0, mask, rec, bin, lp, [&](int pos, const Rec &q) {
-        out_idx[pos] = q.other;
-        if (out_w) out_w[pos] = q.w;
-        if (PERM) out_perm[pos] = get_id(q);
+    tile_emit(L, total, [&](const Rec &q) { return view.key_low(q); }, rec, bin, lp, [&](int pos, const Rec &q) {
+        int32_t other, id;
+        uint32_t wv;
+        view.template unpack<PERM>(q, others_in, w_in, other, wv, id);
+        out_idx[pos] = other;
+        if (out_w) out_w[pos] = wv;
+        if (PERM) out_perm[pos] = id;
     });
 }
 
@@ -615,6 +733,8 @@ static size_t conv_ws_bytes(int64_t E, int32_t V, bool perm)
     size_t b = 0;
     b += carve_bytes(table_n, 4);
     b += carve_bytes(scan_ws_ints((int64_t)table_n), 4);
+    // LSD passes keep two buffers of unpacked records; the two-level path one of packed records
+    // (the array is carved at the unpacked size either way, which the LSD fallback needs)
     b += carve_bytes((size_t)E, perm ? sizeof(Rec4) : sizeof(Rec3)) * (p.digits > 0 ? 2 : 1);
     b += carve_bytes((size_t)p.max_sub, 4);
     b += carve_bytes((size_t)p.nbuckets + 1, 4);
@@ -664,7 +784,7 @@ static int32_t convert(const int32_t *keys, const int32_t *others, const float *
             const int shift = d * kMaxBinBits;
             Rec *dst = bufs[d & 1];
             if (d == 0) {
-                CooLoader<Rec> in{keys, others, reinterpret_cast<const uint32_t *>(w), E, V};
+                CooLoader<Rec> in{keys, others, reinterpret_cast<const uint32_t *>(w), E, V, 0u};
                 hipLaunchKernelGGL((csx_digit_histogram<Rec, CooLoader<Rec>>), dim3(nb), dim3(kPartThreads), 0, s, in,
                                    shift, kMaxBins - 1, kMaxBins, table, nblk);
                 if ((rc = exclusive_scan_i32(table, table, (int64_t)table_n, sums, s))) return rc;
@@ -697,26 +817,51 @@ static int32_t convert(const int32_t *keys, const int32_t *others, const float *
                        table, nblk);
     if ((rc = exclusive_scan_i32(table, table, (int64_t)table_n, sums, s))) return rc;
 
-    CooLoader<Rec> in{keys, others, reinterpret_cast<const uint32_t *>(w), E, V};
-    auto part = csx_partition<Rec, CooLoader<Rec>>;
-    const size_t part_lds = tile_lds_bytes(p.nbuckets, sizeof(Rec));
-    allow_lds(part, part_lds);
-    hipLaunchKernelGGL(part, dim3(nb), dim3(kPartThreads), part_lds, s, in, p.shift, 0x7fffffff, p.nbuckets, bbits,
-                       table, nblk, recs, tile_stage_records(p.nbuckets, sizeof(Rec)));
-
-    hipLaunchKernelGGL(csx_plan_subblocks, dim3(1), dim3(1024), 0, s, table, nblk, p.nbuckets, p.max_sub, sub_bucket,
-                       sub_first);
-    hipLaunchKernelGGL(csx_sub_count<Rec>, dim3((unsigned)p.max_sub), dim3(kPartThreads), 0, s, recs, table, nblk,
-                       sub_bucket, sub_first, p.shift, cnt2);
-    hipLaunchKernelGGL(csx_bucket_offsets, dim3((unsigned)p.nbuckets), dim3(kPartThreads), 0, s, table, nblk,
-                       p.nbuckets, sub_first, p.shift, V, cnt2, out_off);
+    const uint32_t *wbits = reinterpret_cast<const uint32_t *>(w);
     const int nkeys = 1 << p.shift;
-    auto scat = csx_sub_scatter<Rec, PERM>;
-    const size_t scat_lds = tile_lds_bytes(nkeys, sizeof(Rec));
-    allow_lds(scat, scat_lds);
-    hipLaunchKernelGGL(scat, dim3((unsigned)p.max_sub), dim3(kPartThreads), scat_lds, s, recs, table, nblk,
-                       sub_bucket, sub_first, cnt2, p.shift, out_idx, reinterpret_cast<uint32_t *>(out_w), out_perm,
-                       tile_stage_records(nkeys, sizeof(Rec)));
+    int kbits = 0;
+    while (((int64_t)1 << kbits) < (int64_t)V) kbits++;
+    // Packed records need a node id and the low key bits in one word.  Where they do not fit
+    // (V above 2^21 with 2048 keys to a bucket) the records stay unpacked: a seventh of the
+    // endpoints would otherwise be fetched again one by one.
+    const bool packed_ok = kbits + p.shift <= 32;
+    auto level2 = [&](auto *records, auto view) {
+        using R = typename std::remove_pointer<decltype(records)>::type;
+        hipLaunchKernelGGL(csx_plan_subblocks, dim3(1), dim3(1024), 0, s, table, nblk, p.nbuckets, p.max_sub, sub_bucket,
+                           sub_first);
+        hipLaunchKernelGGL((csx_sub_count<R, decltype(view)>), dim3((unsigned)p.max_sub), dim3(kPartThreads), 0, s,
+                           records, table, nblk, sub_bucket, sub_first, view, p.shift, cnt2);
+        hipLaunchKernelGGL(csx_bucket_offsets, dim3((unsigned)p.nbuckets), dim3(kPartThreads), 0, s, table, nblk,
+                           p.nbuckets, sub_first, p.shift, V, cnt2, out_off);
+        auto scat = csx_sub_scatter<R, PERM, decltype(view)>;
+        const size_t scat_lds = tile_lds_bytes(nkeys, sizeof(R));
+        allow_lds(scat, scat_lds);
+        hipLaunchKernelGGL(scat, dim3((unsigned)p.max_sub), dim3(kPartThreads), scat_lds, s, records, table, nblk,
+                           sub_bucket, sub_first, cnt2, view, p.shift, others, wbits, out_idx,
+                           reinterpret_cast<uint32_t *>(out_w), out_perm, tile_stage_records(nkeys, sizeof(R)));
+    };
+    const size_t part_lds = tile_lds_bytes(p.nbuckets, sizeof(Rec));
+    if (packed_ok) {
+        using Packed = typename PackOf<PERM>::type;
+        Packed *packed = reinterpret_cast<Packed *>(recs);
+        PackRule rule;
+        rule.shift = p.shift;
+        rule.obits = 32 - p.shift;
+        rule.omask = p.shift ? (((uint32_t)1 << rule.obits) - 1u) : 0xffffffffu;
+        CooLoader<Rec> in{keys, others, wbits, E, V, rule.omask};
+        auto part = csx_partition_pack<Rec, Packed>;
+        allow_lds(part, part_lds);
+        hipLaunchKernelGGL(part, dim3(nb), dim3(kPartThreads), part_lds, s, in, rule, p.nbuckets, bbits, table, nblk, packed,
+                           tile_stage_records(p.nbuckets, sizeof(Rec)));
+        level2(packed, PackedView{rule});
+    } else {
+        CooLoader<Rec> in{keys, others, wbits, E, V, 0u};
+        auto part = csx_partition<Rec, CooLoader<Rec>>;
+        allow_lds(part, part_lds);
+        hipLaunchKernelGGL(part, dim3(nb), dim3(kPartThreads), part_lds, s, in, p.shift, 0x7fffffff, p.nbuckets, bbits,
+                           table, nblk, recs, tile_stage_records(p.nbuckets, sizeof(Rec)));
+        level2(recs, PlainView{nkeys - 1});
+    }
     zero_tail(out_off, V, E, out_idx, out_w, out_perm, s);
     return launch_status("coo_to_csx");
 }

@@ -75,6 +75,25 @@ def test_all_edges_one_row_and_sorted_and_reversed_inputs():
     check_exact(ei[:, order[::-1]].copy(), w[order[::-1]].copy(), V)
 
 
+def test_endpoints_of_any_size_come_through_unchanged():
+    """The endpoint that is not the key is copied, never interpreted: negative values and values
+    far above V (which do not fit the packed form the records take between the two passes, and
+    are looked up again from the input) must arrive bit for bit, among ordinary ones."""
+    rng = np.random.default_rng(77)
+    for V in (700, 5000, 300_000, 2_000_000):
+        E = 200_000
+        ei, w = rand_graph(rng, V, E, hubs=2)
+        odd = rng.random(E) < 0.3
+        ei[1, odd] = rng.choice(np.array([-1, -2, -2 ** 31, 2 ** 31 - 1, 2 ** 30, 2 ** 22, 2 ** 21, 2 ** 21 - 1, V, V + 1],
+                                         np.int64), odd.sum()).astype(np.int32)
+        from jittorgeometric_amd.ops import cootocsr
+        csr = cootocsr(to_gpu(ei), to_gpu(w), V)          # keyed on row 0: the odd values are the other endpoint
+        col, roff, rw = oracle.cootocsr(ei, w, V)
+        assert np.array_equal(csr.row_offset.cpu().numpy(), roff)
+        assert np.array_equal(csr.column_indices.cpu().numpy(), col)
+        assert np.array_equal(csr.edge_weight.cpu().numpy().view(np.int32), rw.view(np.int32))
+
+
 def test_weights_are_copied_bitwise_including_nan_inf_and_negative_zero():
     rng = np.random.default_rng(21)
     V, E = 500, 4000
