@@ -268,6 +268,46 @@ int32_t jgamd_sample_neighbors(const int32_t *dst, const int32_t *layer_off, con
                                void *stream);
 
 /* ------------------------------------------------------------------------
+ * List lengths and offsets of a layer's destinations.
+ *
+ * jgamd_layer_column_counts: counts[0] = 0, counts[i+1] = min(size of column
+ * dst[i] of the global CSC offsets g_off, cap) for i < n_dst; counts holds
+ * n_dst + 1 int32.  Replaces gpuinitco_op.gpuinitco(dst_size, fanout, dst,
+ * column_offset, global_column_offset) (ops/gpuinitco.py:30-36; the kernel
+ * of ops/cpp/gpuinitco_op.cc:38-52, whose caller turns the counts into
+ * offsets afterwards).  A destination outside [0, g_nodes) counts 0.
+ *
+ * jgamd_layer_column_offsets: offsets[i] = sum of those lengths over the
+ * destinations before i, offsets[n_dst] = their total (n_dst + 1 int32):
+ * the slicing loops of ops/saparse_ops.py:9-71 (from_nodes / to_nodes) size
+ * their result this way, one node at a time.
+ */
+int32_t jgamd_layer_column_counts(const int32_t *dst, const int32_t *g_off, int32_t n_dst,
+                                  int32_t g_nodes, int32_t cap, int32_t *counts, void *stream);
+int32_t jgamd_layer_column_offsets_workspace(int32_t n_dst, size_t *bytes);
+int32_t jgamd_layer_column_offsets(const int32_t *dst, const int32_t *g_off, int32_t n_dst,
+                                   int32_t g_nodes, int32_t cap, int32_t *offsets, void *ws,
+                                   size_t ws_bytes, void *stream);
+
+/* ------------------------------------------------------------------------
+ * Symmetric-normalisation weights of a layer's CSC arrays: with
+ * ins[dst[i]] += size of column i and outs[row[j]] += 1 over the entries
+ * below off[n_dst], w[j] = 1 / (sqrtf(outs[row[j]]) * sqrtf(ins[dst[i]]))
+ * for entry j of column i.  Replaces getweight_op.getweight(vtx_size, dst,
+ * src, column_offset, row_indices, edge_weight) (ops/getweight.py:29-37,
+ * ops/cpp/getweight_op.cc:49-81, same float operations in the same order).
+ * The degrees are integer counts, so their order of accumulation does not
+ * matter.  Entries from off[n_dst] to E get weight 0.  An id outside
+ * [0, vtx_size), which the reference would use as an index out of bounds,
+ * is skipped wherever it would be one: its entries get weight 0 and it adds
+ * to no degree.
+ */
+int32_t jgamd_getweight_workspace(int32_t vtx_size, size_t *bytes);
+int32_t jgamd_getweight(const int32_t *dst, const int32_t *off, const int32_t *row, int32_t n_dst,
+                        int32_t vtx_size, int64_t E, float *w, void *ws, size_t ws_bytes,
+                        void *stream);
+
+/* ------------------------------------------------------------------------
  * Graph preprocessing in front of the conversion.
  *
  * jgamd_add_remaining_self_loops: utils/loop.py:98-136 — the input's

@@ -22,6 +22,11 @@ SIGNATURES = {
     "jgamd_degree_power": [_P, _I32, _c.c_float, _P, _P],
     "jgamd_scale_edge_weights": [_P, _P, _P, _P, _I64, _I32, _P, _P],
     "jgamd_sample_neighbors": [_P, _P, _P, _P, _I32, _I32, _I32, _I64, _c.c_uint64, _P, _P],
+    "jgamd_layer_column_counts": [_P, _P, _I32, _I32, _I32, _P, _P],
+    "jgamd_layer_column_offsets_workspace": [_I32, _SZP],
+    "jgamd_layer_column_offsets": [_P, _P, _I32, _I32, _I32, _P, _P, _c.c_size_t, _P],
+    "jgamd_getweight_workspace": [_I32, _SZP],
+    "jgamd_getweight": [_P, _P, _P, _I32, _I32, _I64, _P, _P, _c.c_size_t, _P],
     "jgamd_spmm_csx_workspace": [_I32, _I64, _I32, _SZP],
     "jgamd_spmm_csx": [_P, _P, _P, _P, _P, _I32, _I32, _I64, _I32, _P, _c.c_size_t, _P],
     "jgamd_spmm_csx_noalloc": [_P, _P, _P, _P, _P, _I32, _I32, _I64, _I32, _P],

@@ -1,7 +1,8 @@
 """Symmetric-normalisation weights of a layer's CSC arrays.  Same call as
 jittor_geometric.ops.getweight (ops/getweight.py:29-37); arithmetic of
 ops/cpp/getweight_op.cc:36-82: in-degree of dst[i] += size of column i, out-degree of
-every row index += 1, weight = 1 / (sqrtf(out[src]) * sqrtf(in[dst]))."""
+every row index += 1, weight = 1 / (sqrtf(out[src]) * sqrtf(in[dst])).  The kernels are in
+csrc/sample.hip; csc_layer_src is accepted and, as in the reference's loop, not read."""
 import torch
 
 from .. import _lib
@@ -9,15 +10,20 @@ from ._common import as_i32
 
 
 def getweight(vtx_size, csc_layer_dst, csc_layer_src, csc_layer_column_offset, csc_layer_row_indices):
+    lib = _lib.load()
     dev = _lib.require_gpu(csc_layer_dst, csc_layer_column_offset, csc_layer_row_indices)
-    dst = as_i32(csc_layer_dst, "csc_layer_dst").to(torch.int64)
-    off = as_i32(csc_layer_column_offset, "csc_layer_column_offset").to(torch.int64)
+    dst = as_i32(csc_layer_dst, "csc_layer_dst")
+    off = as_i32(csc_layer_column_offset, "csc_layer_column_offset")
+    row = as_i32(csc_layer_row_indices, "csc_layer_row_indices")
     n = dst.shape[0]
+    if off.shape[0] < n + 1:
+        raise _lib.JgamdError("getweight: %d offsets for %d destinations" % (off.shape[0], n))
     E = int(off[-1].item()) if off.numel() else 0       # the reference sizes the result the same way (:32)
-    row = as_i32(csc_layer_row_indices, "csc_layer_row_indices").to(torch.int64)[:E]
-    sizes = off[1:n + 1] - off[:n]
-    ins = torch.zeros(vtx_size, dtype=torch.int64, device=dev).index_add_(0, dst, sizes)
-    outs = torch.bincount(row, minlength=vtx_size)
-    col_of_entry = torch.repeat_interleave(dst, sizes, output_size=E)
-    w = 1.0 / (outs[row].to(torch.float32).sqrt() * ins[col_of_entry].to(torch.float32).sqrt())
+    if E < 0 or E > row.shape[0]:
+        raise _lib.JgamdError("getweight: last offset %d, %d row indices" % (E, row.shape[0]))
+    w = torch.empty(E, dtype=torch.float32, device=dev)
+    nbytes = _lib.query(lib.jgamd_getweight_workspace, int(vtx_size))
+    ws = _lib.workspace(nbytes, dev)
+    _lib.check(lib.jgamd_getweight(_lib.ptr(dst), _lib.ptr(off), _lib.ptr(row), n, int(vtx_size), E, _lib.ptr(w),
+                                   _lib.ptr(ws), nbytes, _lib.stream_ptr(dev)))
     return w

@@ -80,6 +80,57 @@ def test_getweight_layer_with_global_ids():
     assert np.array_equal(got.view(np.int32), oracle.getweight(30, dst, dst, off, row).view(np.int32))
 
 
+def test_getweight_repeated_destinations_and_ids_out_of_range():
+    """A destination listed twice adds both of its columns to its in-degree (getweight_op.cc:56-57);
+    an id outside [0, vtx_size), which the reference would use as an index out of bounds, is
+    skipped wherever it would be one: its entries get weight 0, the other entries are as if the id
+    were a valid one that nothing else names."""
+    from jittorgeometric_amd.ops import getweight
+    off = np.array([0, 3, 5, 9], np.int32)
+    row = np.array([1, 2, 3, 1, 4, 2, 2, 5, 1], np.int32)
+    dst = np.array([6, 7, 6], np.int32)
+    got = getweight(8, to_gpu(dst), to_gpu(dst), to_gpu(off), to_gpu(row)).cpu().numpy()
+    assert np.array_equal(got.view(np.int32), oracle.getweight(8, dst, dst, off, row).view(np.int32))
+    ins6 = np.float32(7)                                  # 3 + 4 entries
+    assert got[0] == np.float32(1) / (np.sqrt(np.float32(3)) * np.sqrt(ins6))     # source 1 appears 3 times
+    bad_row = row.copy()
+    bad_row[4] = 100
+    bad_dst = np.array([6, -1, 6], np.int32)
+    got = getweight(8, to_gpu(bad_dst), to_gpu(bad_dst), to_gpu(off), to_gpu(bad_row)).cpu().numpy()
+    assert got[3] == 0 and got[4] == 0                    # column of destination -1; row index 100
+    keep = np.array([0, 1, 2, 5, 6, 7, 8])
+    stand_in = bad_row.copy()
+    stand_in[4] = 0                                       # ids 0 and 7 appear nowhere else
+    want = oracle.getweight(8, np.array([6, 7, 6], np.int32), None, off, stand_in)
+    assert np.array_equal(got[keep].view(np.int32), want[keep].view(np.int32))
+
+
+def test_getweight_at_the_size_of_the_benchmark_graph():
+    from jittorgeometric_amd import synthetic
+    from jittorgeometric_amd.ops import getweight
+    ei, V = synthetic.make("powerlaw_1m")
+    row, off, _ = oracle.cootocsc(np.ascontiguousarray(ei.astype(np.int32)), np.ones(ei.shape[1], np.float32), V)
+    ids = np.arange(V, dtype=np.int32)
+    got = getweight(V, to_gpu(ids), to_gpu(ids), to_gpu(off), to_gpu(row)).cpu().numpy()
+    indeg = np.diff(off).astype(np.float32)
+    outdeg = np.bincount(row, minlength=V).astype(np.float32)
+    want = np.float32(1) / (np.sqrt(outdeg[row]) * np.sqrt(indeg[np.repeat(ids, np.diff(off))]))
+    assert np.array_equal(got.view(np.int32), want.view(np.int32))
+
+
+def test_gpuinitco_edge_cases():
+    from jittorgeometric_amd.ops import gpuinitco
+    goff = np.array([0, 0, 4, 4, 9, 10], np.int32)
+    dst = np.array([3, 0, 1, 4, 3, 2], np.int32)
+    for fanout in (0, 1, 3, 5, 100):
+        for n in (0, 1, 6):
+            got = gpuinitco(n, fanout, to_gpu(dst), to_gpu(goff)).cpu().numpy()
+            assert np.array_equal(got, oracle.gpuinitco(n, fanout, dst[:n], goff)), (fanout, n)
+    from jittorgeometric_amd import JgamdError
+    with pytest.raises(JgamdError):
+        gpuinitco(7, 3, to_gpu(dst), to_gpu(goff))
+
+
 def test_csctocsr_layer_and_full_graph():
     from jittorgeometric_amd.ops import csctocsr
     g = GOLD["csctocsr_readme_v4"]
@@ -132,5 +183,7 @@ def test_from_nodes_and_to_nodes():
     assert np.array_equal(from_nodes(csc, to_gpu(nodes)).cpu().numpy(), oracle.from_nodes(coff, row, nodes))
     assert np.array_equal(to_nodes(csr, to_gpu(nodes)).cpu().numpy(), oracle.from_nodes(roff, col, nodes))
     assert from_nodes(csc, to_gpu(np.zeros(0, np.int32))).numel() == 0
+    many = rng.integers(0, V, 70000).astype(np.int32)                                    # more than one scan tile
+    assert np.array_equal(from_nodes(csc, to_gpu(many)).cpu().numpy(), oracle.from_nodes(coff, row, many))
     with pytest.raises(ValueError):
         from_nodes(None, to_gpu(nodes))
