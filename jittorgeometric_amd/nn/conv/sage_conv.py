@@ -4,7 +4,8 @@ import torch
 from torch import nn
 
 from ...ops import SpmmCsr, aggregateWithWeight, cootocsc, cootocsr
-from ..dense import add_bias, xw
+from ...ops._common import both_orders, spmm, spmm_axpby
+from ..dense import add_bias, column_sum, xt_g, xw
 from ..inits import glorot, zeros
 from .gcn_conv import _degree_norm, _scale
 
@@ -13,6 +14,45 @@ def sage_norm(edge_index, edge_weight=None, num_nodes=None, improved=False, add_
     """Mean weights w * d^-1[col] (nn/conv/sage_conv.py:16-40)."""
     edge_index, edge_weight, dinv = _degree_norm(edge_index, edge_weight, num_nodes, improved, add_self_loops, -1.0)
     return edge_index, _scale(edge_index, edge_weight, None, dinv, dinv.shape[0])
+
+
+class SageLayerFunc(torch.autograd.Function):
+    """(A x) W1 + x W_root + b as one autograd node (sage_conv.py:172-190 builds it from five:
+    product, two dense products, two additions).  The root term is accumulated by the second
+    dense product (beta = 1) and the bias enters through the first one's epilogue; in the
+    backward pass the root term's input gradient is added in the transposed product's row
+    store, so no pass over a [V,F] array only adds two arrays."""
+
+    @staticmethod
+    def forward(ctx, x, w1, w_root, bias, fwd, bwd):
+        agg = spmm(fwd[0], fwd[1], fwd[2], x, x.shape[0])
+        out = torch.addmm(bias, agg, w1) if bias is not None else agg @ w1
+        if w_root is not None:
+            out.addmm_(x, w_root)
+        ctx.bwd = bwd
+        ctx.save_for_backward(x, agg, w1, w_root)
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        x, agg, w1, w_root = ctx.saved_tensors
+        g = g.contiguous()
+        need_x, need_w1, need_root, need_b = ctx.needs_input_grad[:4]
+        gx = gw1 = groot = gb = None
+        if need_b:
+            gb = column_sum(g) if g.dtype == torch.float32 else g.sum(0)
+        if need_w1:
+            gw1 = xt_g(agg, g)
+        if need_root and w_root is not None:
+            groot = xt_g(x, g)
+        if need_x:
+            off, idx, w = ctx.bwd
+            g_agg = g @ w1.t()
+            if w_root is not None:
+                gx = spmm_axpby(off, idx, w, g_agg, g.shape[0], 1.0, 1.0, g @ w_root.t())
+            else:
+                gx = spmm(off, idx, w, g_agg, g.shape[0])
+        return gx, gw1, groot, gb, None, None
 
 
 class SAGEConv(nn.Module):
@@ -65,6 +105,10 @@ class SAGEConv(nn.Module):
                     self._cached_edge_index = (edge_index, edge_weight, csr, csc)
             else:
                 edge_index, edge_weight, csr, csc = cache
+        if self.weight_proj is None and x.dim() == 2 and x.dtype == torch.float32:
+            # spmm=True only needs the CSR arrays (:183-184); both routes give the same product
+            fwd, bwd = both_orders(None if self.spmm and csr is not None else csc, csr)
+            return SageLayerFunc.apply(x.contiguous(), self.weight1, self.root_weight, self.bias, fwd, bwd)
         xs = (x, x)
         if self.weight_proj is not None:
             xs = (torch.relu(xs[0] @ self.weight_proj + self.bias_proj), xs[1])

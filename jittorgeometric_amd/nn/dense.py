@@ -10,6 +10,21 @@ _SLABS = 256          # partial products; V/_SLABS rows of x each
 _MIN_ROWS = 1 << 16   # below this the plain product is used
 
 
+def xt_g(x, g):
+    """x^T @ g for x [V,Fin], g [V,Fout]: partial products over slabs of nodes, then their sum."""
+    V = x.shape[0]
+    rows = V // _SLABS
+    if V < _MIN_ROWS or rows == 0 or not (x.is_contiguous() and g.is_contiguous()):
+        return x.t() @ g
+    main = rows * _SLABS
+    xs = x[:main].view(_SLABS, rows, x.shape[1])
+    gs = g[:main].view(_SLABS, rows, g.shape[1])
+    gw = torch.bmm(xs.transpose(1, 2), gs).sum(0)
+    if main < V:
+        gw = gw + x[main:].t() @ g[main:]
+    return gw
+
+
 class _XW(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, weight):
@@ -23,17 +38,7 @@ class _XW(torch.autograd.Function):
         if ctx.needs_input_grad[0]:
             gx = g @ weight.t()
         if ctx.needs_input_grad[1]:
-            V = x.shape[0]
-            rows = V // _SLABS
-            if V < _MIN_ROWS or rows == 0:
-                gw = x.t() @ g
-            else:
-                main = rows * _SLABS
-                xs = x[:main].view(_SLABS, rows, x.shape[1])
-                gs = g[:main].view(_SLABS, rows, g.shape[1])
-                gw = torch.bmm(xs.transpose(1, 2), gs).sum(0)
-                if main < V:
-                    gw = gw + x[main:].t() @ g[main:]
+            gw = xt_g(x, g)
         return gx, gw
 
 
