@@ -241,6 +241,43 @@ int32_t jgamd_gat_bwd(const int32_t *off, const int32_t *idx, const int32_t *t_o
                       void *stream);
 
 /* ------------------------------------------------------------------------
+ * Column-blocked product for matrices with long rows (hundreds of entries
+ * per row, x larger than an L2): the same result as jgamd_spmm_csx_axpby,
+ * out = beta * (A x) + alpha * h, with the gathers of x confined to one block
+ * of columns at a time.  Follows the same reference loops as jgamd_spmm_csx
+ * (aggregate_op.cc:107-114, spmmcsr_op.cc:81-127); the reference has no
+ * blocked layout.  Sums differ from the unblocked kernels' in rounding only
+ * (per-block partial sums added in block order; no atomics, run-to-run
+ * identical).
+ *
+ * jgamd_spmm_block_plan: *nb = number of column blocks and *block_cols =
+ * columns per block that pay for this shape, or *nb = 0 when the unblocked
+ * product is the better one (short rows, x that fits, too many blocks).
+ *
+ * jgamd_csx_block_columns: regroups the entries of every row by column block,
+ * keeping their order inside a block: b_off [nb*R+1], b_idx [E], b_w [E]
+ * (w and b_w may both be NULL); row b*R + r of the result holds the entries
+ * of row r whose column lies in [b*block_cols, (b+1)*block_cols), the last
+ * block taking what lies beyond.  Entries from off[R] on are not part of it.
+ * Done once per matrix; nb <= 64.
+ *
+ * jgamd_spmm_csx_blocked: the product over arrays made by that call.
+ */
+int32_t jgamd_spmm_block_plan(int32_t R, int32_t C, int64_t E, int32_t F, int32_t *nb,
+                              int32_t *block_cols);
+int32_t jgamd_csx_block_columns_workspace(int32_t R, int32_t nb, size_t *bytes);
+int32_t jgamd_csx_block_columns(const int32_t *off, const int32_t *idx, const float *w, int32_t R,
+                                int64_t E, int32_t block_cols, int32_t nb, int32_t *b_off,
+                                int32_t *b_idx, float *b_w, void *ws, size_t ws_bytes,
+                                void *stream);
+int32_t jgamd_spmm_csx_blocked_workspace(int32_t R, int64_t E, int32_t F, int32_t nb,
+                                         size_t *bytes);
+int32_t jgamd_spmm_csx_blocked(const int32_t *b_off, const int32_t *b_idx, const float *b_w,
+                               const float *x, float *out, float beta, float alpha,
+                               const float *h, int32_t h_rows, int32_t R, int32_t C, int64_t E,
+                               int32_t F, int32_t nb, void *ws, size_t ws_bytes, void *stream);
+
+/* ------------------------------------------------------------------------
  * Column sums of a row-major [R,F] matrix: out[f] = sum_r x[r,f].  The bias
  * gradient of the conv layers (`out += self.bias`, nn/conv/gcn_conv.py:100-101,
  * nn/conv/sage_conv.py:189-190; Jittor derives the reduction).  Two stages,

@@ -455,10 +455,23 @@ struct SpmmShape {
     int vec, nt, slabs, chunk, nchunks;
 };
 
-static SpmmShape spmm_shape(int32_t R, int64_t E, int32_t F, bool aligned16, bool aligned8)
+// narrow_slabs: one 64-float tile per wavefront and the other tiles in grid.y.  Workgroups are
+// handed out with grid.x running fastest, so the whole matrix is walked for one 256-byte slab of
+// the feature rows before the next slab starts: what the column-blocked product needs to keep
+// the gathered block of x inside an L2.
+static SpmmShape spmm_shape(int32_t R, int64_t E, int32_t F, bool aligned16, bool aligned8, bool narrow_slabs = false)
 {
     SpmmShape s{};
     s.vec = (F % 4 == 0 && aligned16) ? 4 : (F % 2 == 0 && aligned8) ? 2 : 1;
+    if (narrow_slabs && F > kWave) {
+        s.vec = 1;
+        s.nt = 1;
+        s.slabs = (int)ceil_div(F, kWave);
+        const int64_t M = (int64_t)R + E;
+        s.chunk = pick_chunk(M);
+        s.nchunks = (int)ceil_div(M > 0 ? M : 1, s.chunk);
+        return s;
+    }
     // prefer the narrowest vector that still covers F with one tile per lane:
     // more lanes per row keeps every load instruction a full 64-lane access
     while (s.vec > 1 && F <= kWave * (s.vec / 2)) s.vec >>= 1;
@@ -556,7 +569,7 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_workspa
 
 static int32_t spmm_call(const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out,
                          int32_t R, int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, void *stream,
-                         hipEvent_t k0, hipEvent_t k1, const RowFinish *fin = nullptr)
+                         hipEvent_t k0, hipEvent_t k1, const RowFinish *fin = nullptr, bool narrow_slabs = false)
 {
     if (int32_t rc = check_spmm_sizes(R, E, F)) return rc;
     if (C < 0) return fail(JGAMD_ERR_SIZE, "spmm_csx: negative C");
@@ -583,7 +596,7 @@ static int32_t spmm_call(const int32_t *off, const int32_t *idx, const float *w,
 
     // h is read with x's vector width: its alignment counts too
     const uintptr_t bits = (uintptr_t)x | (uintptr_t)out | (uintptr_t)(fin ? fin->h : nullptr);
-    const SpmmShape s = spmm_shape(R, E, F, (bits & 15) == 0, (bits & 7) == 0);
+    const SpmmShape s = spmm_shape(R, E, F, (bits & 15) == 0, (bits & 7) == 0, narrow_slabs);
     Carver carve(ws);
     int32_t *chunk_row = carve.take<int32_t>((size_t)s.nchunks + 1);
     float *partial = carve.take<float>((size_t)s.nchunks * (size_t)F);
@@ -631,6 +644,11 @@ int32_t spmm_enqueue(const int32_t *off, const int32_t *idx, const float *w, con
                      int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, hipStream_t s)
 {
     return spmm_call(off, idx, w, x, out, R, C, E, F, ws, ws_bytes, s, nullptr, nullptr);
+}
+int32_t spmm_enqueue_slabs(const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out,
+                           int32_t R, int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, hipStream_t s)
+{
+    return spmm_call(off, idx, w, x, out, R, C, E, F, ws, ws_bytes, s, nullptr, nullptr, nullptr, true);
 }
 }  // namespace jg
 

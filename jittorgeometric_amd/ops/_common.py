@@ -1,4 +1,6 @@
 """Helpers shared by the operator wrappers."""
+import ctypes as _c
+
 import torch
 
 from .. import _lib
@@ -114,47 +116,78 @@ def _raw_arrays(off, idx, w, R):
     return off, idx, w
 
 
-def spmm(off, idx, w, x, R):
-    """out[r,:] = sum_j w[j] * x[idx[j],:]; idx/w may be None (identity / ones)."""
+def _blocked_arrays(off, idx, w, R, E, nb, cols):
+    """The matrix regrouped by column block (csrc/spmm_blocked.hip), built on first use and
+    kept on the offsets tensor it was built from until one of the three arrays is another
+    tensor or has been written in place."""
+    stamp = (_stamp(off), _stamp(idx), _stamp(w), nb, cols)
+    cached = getattr(off, "_jgamd_blocked", None)
+    if cached is not None and cached[0] == stamp and cached[1] is idx and cached[2] is w:
+        return cached[3]
     lib = _lib.load()
-    dev = _lib.require_gpu(off, x, idx, w)
+    dev = off.device
+    b_off = torch.empty(nb * R + 1, dtype=torch.int32, device=dev)
+    b_idx = torch.empty(E, dtype=torch.int32, device=dev)
+    b_w = torch.empty(E, dtype=torch.float32, device=dev) if w is not None else None
+    nbytes = _lib.query(lib.jgamd_csx_block_columns_workspace, R, nb)
+    ws = _lib.workspace(nbytes, dev)
+    _lib.check(lib.jgamd_csx_block_columns(_lib.ptr(off), _lib.ptr(idx), _lib.ptr(w), R, E, cols, nb, _lib.ptr(b_off),
+                                           _lib.ptr(b_idx), _lib.ptr(b_w), _lib.ptr(ws), nbytes, _lib.stream_ptr(dev)))
+    off._jgamd_blocked = (stamp, idx, w, (b_off, b_idx, b_w))
+    return b_off, b_idx, b_w
+
+
+def _product(off, idx, w, x, R, beta, alpha, h):
+    """beta * (A x) + alpha * h through the plain or the column-blocked kernels."""
+    lib = _lib.load()
+    dev = _lib.require_gpu(off, x, idx, w, h)
     x = as_f32(x, "x")
     off, idx, w = _raw_arrays(off, idx, w, R)
     if x.dim() != 2:
         raise _lib.JgamdError("x must be [rows, F], got %s" % (tuple(x.shape),))
     C, F = x.shape
-    E = int(idx.shape[0]) if idx is not None else C
-    out = torch.empty((R, F), dtype=torch.float32, device=dev)
-    nbytes = _lib.query(lib.jgamd_spmm_csx_workspace, R, E, F)
-    ws = _lib.workspace(nbytes, dev)
-    _lib.check(lib.jgamd_spmm_csx(_lib.ptr(off), _lib.ptr(idx), _lib.ptr(w), _lib.ptr(x), _lib.ptr(out), R, C, E, F,
-                                  _lib.ptr(ws), nbytes, _lib.stream_ptr(dev)))
-    return out
-
-
-def spmm_axpby(off, idx, w, x, R, beta, alpha, h):
-    """out[r,:] = beta * sum_j w[j] * x[idx[j],:] + alpha * h[r,:]; h is [R,F], or [F] / [1,F]
-    for one row added to every output row, or None."""
-    lib = _lib.load()
-    dev = _lib.require_gpu(off, x, idx, w, h)
-    x = as_f32(x, "x")
-    off, idx, w = _raw_arrays(off, idx, w, R)
-    h = as_f32(h, "h") if h is not None else None
-    C, F = x.shape
     h_rows = R
     if h is not None:
+        h = as_f32(h, "h")
         if h.dim() == 1 or (h.dim() == 2 and h.shape[0] == 1 and R != 1):
             h_rows = 1
         if h.numel() != h_rows * F:
             raise ValueError("h must be [%d, %d] or [%d], got %s" % (R, F, F, tuple(h.shape)))
     E = int(idx.shape[0]) if idx is not None else C
     out = torch.empty((R, F), dtype=torch.float32, device=dev)
+    stream = _lib.stream_ptr(dev)
+    nb, cols = _c.c_int32(0), _c.c_int32(0)
+    if idx is not None:
+        _lib.check(lib.jgamd_spmm_block_plan(R, C, E, F, _c.byref(nb), _c.byref(cols)))
+    if nb.value > 0:
+        b_off, b_idx, b_w = _blocked_arrays(off, idx, w, R, E, nb.value, cols.value)
+        nbytes = _lib.query(lib.jgamd_spmm_csx_blocked_workspace, R, E, F, nb.value)
+        ws = _lib.workspace(nbytes, dev)
+        _lib.check(lib.jgamd_spmm_csx_blocked(_lib.ptr(b_off), _lib.ptr(b_idx), _lib.ptr(b_w), _lib.ptr(x), _lib.ptr(out),
+                                              float(beta), float(alpha), _lib.ptr(h), h_rows, R, C, E, F, nb.value,
+                                              _lib.ptr(ws), nbytes, stream))
+        return out
     nbytes = _lib.query(lib.jgamd_spmm_csx_workspace, R, E, F)
     ws = _lib.workspace(nbytes, dev)
-    _lib.check(lib.jgamd_spmm_csx_axpby(_lib.ptr(off), _lib.ptr(idx), _lib.ptr(w), _lib.ptr(x), _lib.ptr(out),
-                                        float(beta), float(alpha), _lib.ptr(h), h_rows, R, C, E, F, _lib.ptr(ws), nbytes,
-                                        _lib.stream_ptr(dev)))
+    if h is None and beta == 1.0:
+        _lib.check(lib.jgamd_spmm_csx(_lib.ptr(off), _lib.ptr(idx), _lib.ptr(w), _lib.ptr(x), _lib.ptr(out), R, C, E, F,
+                                      _lib.ptr(ws), nbytes, stream))
+    else:
+        _lib.check(lib.jgamd_spmm_csx_axpby(_lib.ptr(off), _lib.ptr(idx), _lib.ptr(w), _lib.ptr(x), _lib.ptr(out),
+                                            float(beta), float(alpha), _lib.ptr(h), h_rows, R, C, E, F, _lib.ptr(ws),
+                                            nbytes, stream))
     return out
+
+
+def spmm(off, idx, w, x, R):
+    """out[r,:] = sum_j w[j] * x[idx[j],:]; idx/w may be None (identity / ones)."""
+    return _product(off, idx, w, x, R, 1.0, 0.0, None)
+
+
+def spmm_axpby(off, idx, w, x, R, beta, alpha, h):
+    """out[r,:] = beta * sum_j w[j] * x[idx[j],:] + alpha * h[r,:]; h is [R,F], or [F] / [1,F]
+    for one row added to every output row, or None."""
+    return _product(off, idx, w, x, R, beta, alpha, h)
 
 
 def both_orders(csc, csr):
