@@ -278,6 +278,22 @@ int32_t jgamd_spmm_csx_blocked(const int32_t *b_off, const int32_t *b_idx, const
                                int32_t F, int32_t nb, void *ws, size_t ws_bytes, void *stream);
 
 /* ------------------------------------------------------------------------
+ * Dense feature transform of the conv layers on the matrix cores (fp32 in,
+ * fp32 accumulate): out[V,N] = x1[V,K1] @ w1[K1,N] (+ x2[V,K2] @ w2[K2,N])
+ * (+ bias[N]).  Replaces `x @ self.weight` (nn/conv/gcn_conv.py:95) and
+ * `out @ weight1 + x @ root_weight + bias` (nn/conv/sage_conv.py:186-190),
+ * which Jittor runs as cuBLAS products and element-wise additions.  K1, K2
+ * and N must be multiples of 4 with K1 + K2 <= 256 (jgamd_dense_rows_supported
+ * returns 1 for such a shape, else 0; other shapes stay with the BLAS
+ * library); x1, x2, out and bias 16-byte aligned.  K2 = 0 leaves out the
+ * second product, bias = NULL the added row.  Needs no workspace.
+ */
+int32_t jgamd_dense_rows_supported(int32_t K1, int32_t K2, int32_t N);
+int32_t jgamd_dense_rows(const float *x1, const float *w1, int32_t K1, const float *x2,
+                         const float *w2, int32_t K2, const float *bias, float *out, int32_t V,
+                         int32_t N, void *stream);
+
+/* ------------------------------------------------------------------------
  * Column sums of a row-major [R,F] matrix: out[f] = sum_r x[r,f].  The bias
  * gradient of the conv layers (`out += self.bias`, nn/conv/gcn_conv.py:100-101,
  * nn/conv/sage_conv.py:189-190; Jittor derives the reduction).  Two stages,

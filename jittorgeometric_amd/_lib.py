@@ -44,6 +44,8 @@ SIGNATURES = {
     "jgamd_edge_softmax_fwd": [_P, _P, _P, _I32, _I64, _I32, _P, _c.c_size_t, _P],
     "jgamd_edge_softmax_bwd": [_P, _P, _P, _P, _I32, _I64, _I32, _P, _c.c_size_t, _P],
     "jgamd_scatter_to_edge": [_P, _P, _P, _P, _I32, _I64, _I32, _I32, _P],
+    "jgamd_dense_rows_supported": [_I32, _I32, _I32],
+    "jgamd_dense_rows": [_P, _P, _I32, _P, _P, _I32, _P, _P, _I32, _I32, _P],
     "jgamd_column_sum_workspace": [_I64, _I32, _SZP],
     "jgamd_column_sum": [_P, _P, _I64, _I32, _P, _c.c_size_t, _P],
     "jgamd_gat_fwd_workspace": [_I32, _I64, _I32, _I32, _SZP],

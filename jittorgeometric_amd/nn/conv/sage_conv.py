@@ -5,7 +5,7 @@ from torch import nn
 
 from ...ops import SpmmCsr, aggregateWithWeight, cootocsc, cootocsr
 from ...ops._common import both_orders, spmm, spmm_axpby
-from ..dense import add_bias, column_sum, xt_g, xw
+from ..dense import add_bias, column_sum, rows_times, xt_g, xw
 from ..inits import glorot, zeros
 from .gcn_conv import _degree_norm, _scale
 
@@ -18,17 +18,14 @@ def sage_norm(edge_index, edge_weight=None, num_nodes=None, improved=False, add_
 
 class SageLayerFunc(torch.autograd.Function):
     """(A x) W1 + x W_root + b as one autograd node (sage_conv.py:172-190 builds it from five:
-    product, two dense products, two additions).  The root term is accumulated by the second
-    dense product (beta = 1) and the bias enters through the first one's epilogue; in the
-    backward pass the root term's input gradient is added in the transposed product's row
+    product, two dense products, two additions).  Both dense products and the bias row are
+    one pass of the matrix-core kernel (csrc/dense_rows.hip); in the backward pass the root term's input gradient is added in the transposed product's row
     store, so no pass over a [V,F] array only adds two arrays."""
 
     @staticmethod
     def forward(ctx, x, w1, w_root, bias, fwd, bwd):
         agg = spmm(fwd[0], fwd[1], fwd[2], x, x.shape[0])
-        out = torch.addmm(bias, agg, w1) if bias is not None else agg @ w1
-        if w_root is not None:
-            out.addmm_(x, w_root)
+        out = rows_times(agg, w1, x if w_root is not None else None, w_root, bias)
         ctx.bwd = bwd
         ctx.save_for_backward(x, agg, w1, w_root)
         return out
@@ -47,9 +44,9 @@ class SageLayerFunc(torch.autograd.Function):
             groot = xt_g(x, g)
         if need_x:
             off, idx, w = ctx.bwd
-            g_agg = g @ w1.t()
+            g_agg = rows_times(g, w1.t().contiguous())
             if w_root is not None:
-                gx = spmm_axpby(off, idx, w, g_agg, g.shape[0], 1.0, 1.0, g @ w_root.t())
+                gx = spmm_axpby(off, idx, w, g_agg, g.shape[0], 1.0, 1.0, rows_times(g, w_root.t().contiguous()))
             else:
                 gx = spmm(off, idx, w, g_agg, g.shape[0])
         return gx, gw1, groot, gb, None, None

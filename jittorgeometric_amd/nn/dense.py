@@ -1,13 +1,50 @@
 """Dense feature transform x @ W of the conv layers (gcn_conv.py:95 in the
-reference).  The products run in torch's hipBLASLt (MFMA); only the weight
-gradient is arranged differently: x^T @ g has a tiny [Fin,Fout] output and a
-reduction over every node, for which the library picks a kernel without
-split-K (1.8 ms at V=1M, Fin=Fout=128).  It is computed here as a batched
-product over slabs of nodes followed by a sum over the slabs."""
+reference).  Products of the node features with a weight matrix (forward, and
+the input gradient g @ W^T) run in the library's matrix-core kernel
+(csrc/dense_rows.hip), which also takes a second operand pair and a bias row
+in the same pass; shapes it does not cover go to torch's BLAS.  The weight
+gradient x^T @ g has a tiny [Fin,Fout] output and a reduction over every node,
+for which the BLAS library picks a kernel without split-K (1.8 ms at V=1M,
+Fin=Fout=128): it is computed as a batched product over slabs of nodes
+followed by a sum over the slabs."""
 import torch
 
 _SLABS = 256          # partial products; V/_SLABS rows of x each
 _MIN_ROWS = 1 << 16   # below this the plain product is used
+
+
+def _plain(t):
+    return t.dtype == torch.float32 and t.is_cuda and t.dim() == 2 and t.is_contiguous() and t.data_ptr() % 16 == 0
+
+
+def rows_times(x1, w1, x2=None, w2=None, bias=None):
+    """x1 @ w1 (+ x2 @ w2) (+ bias) in one pass over the rows: the library's matrix-core kernel
+    (csrc/dense_rows.hip) for the shapes it covers, torch's BLAS products otherwise."""
+    from .. import _lib
+    two = x2 is not None
+    K1, N = w1.shape
+    K2 = w2.shape[0] if two else 0
+    ok = x1.is_cuda and _plain(x1) and w1.dtype == torch.float32 and x1.shape[1] == K1 and x1.shape[0] >= 1 << 12
+    if two:
+        ok = ok and _plain(x2) and w2.dtype == torch.float32 and x2.shape == (x1.shape[0], K2) and w2.shape[1] == N
+    if bias is not None:
+        ok = ok and bias.dtype == torch.float32 and bias.numel() == N
+    if ok:
+        lib = _lib.load()
+        ok = bool(lib.jgamd_dense_rows_supported(K1, K2, N))
+    if not ok:
+        out = torch.addmm(bias, x1, w1) if bias is not None else x1 @ w1
+        return out.addmm_(x2, w2) if two else out
+    dev = _lib.require_gpu(x1, w1, x2, w2, bias)
+    w1 = w1.contiguous()
+    w2 = w2.contiguous() if two else None
+    bias = bias.contiguous() if bias is not None else None
+    if bias is not None and bias.data_ptr() % 16:
+        bias = bias.clone()
+    out = torch.empty((x1.shape[0], N), dtype=torch.float32, device=dev)
+    _lib.check(lib.jgamd_dense_rows(_lib.ptr(x1), _lib.ptr(w1), K1, _lib.ptr(x2), _lib.ptr(w2), K2, _lib.ptr(bias),
+                                    _lib.ptr(out), x1.shape[0], N, _lib.stream_ptr(dev)))
+    return out
 
 
 def xt_g(x, g):
@@ -29,14 +66,14 @@ class _XW(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, weight):
         ctx.save_for_backward(x, weight)
-        return x @ weight
+        return rows_times(x, weight)
 
     @staticmethod
     def backward(ctx, g):
         x, weight = ctx.saved_tensors
         gx = gw = None
         if ctx.needs_input_grad[0]:
-            gx = g @ weight.t()
+            gx = rows_times(g.contiguous(), weight.t().contiguous())
         if ctx.needs_input_grad[1]:
             gw = xt_g(x, g)
         return gx, gw
