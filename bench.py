@@ -111,7 +111,7 @@ class Bench:
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / iters * 1e3
 
-    def graph(self, name, norm="gcn"):
+    def graph(self, name, norm="gcn", time_conversions=True):
         """(edge_index, weights, V, CSC, CSR, conversion times) of a configuration after the
         normalisation with self-loops, converted on the device."""
         from jittorgeometric_amd import synthetic
@@ -121,20 +121,35 @@ class Bench:
         ei = self.torch.from_numpy(ei_np).to(self.dev)
         ei, w = (gcn_norm if norm == "gcn" else sage_norm)(ei, None, V)
         ei = ei.contiguous()
-        csr_ms = self.timed(lambda: cootocsr(ei, w, V), 10, 2)
-        csc_ms = self.timed(lambda: cootocsc(ei, w, V), 10, 2)
+        csr_ms = self.timed(lambda: cootocsr(ei, w, V), 10, 2) if time_conversions else 0.0
+        csc_ms = self.timed(lambda: cootocsc(ei, w, V), 10, 2) if time_conversions else 0.0
         return ei, w, V, cootocsc(ei, w, V), cootocsr(ei, w, V), csr_ms, csc_ms
 
     def spmm_kernel_ms(self, off, idx, w, x, R, iters):
         """Mean duration of the gather kernel (spmm_merge) and of the whole call, from HIP events
-        recorded on the launch stream inside the library."""
+        recorded on the launch stream inside the library; through the column-blocked kernels when
+        the library's plan picks them for this shape, as the operators do."""
         torch, _lib, lib = self.torch, self._lib, self.lib
+        from jittorgeometric_amd.ops._common import _blocked_arrays
         C, F = x.shape
         E = idx.shape[0]
         out = torch.empty(R, F, device=self.dev)
+        k_ms, c_ms = ctypes.c_float(), ctypes.c_float()
+        nb, cols = ctypes.c_int32(0), ctypes.c_int32(0)
+        _lib.check(lib.jgamd_spmm_block_plan(R, C, E, F, ctypes.byref(nb), ctypes.byref(cols)))
+        self.blocked = nb.value
+        if nb.value > 0:
+            b_off, b_idx, b_w = _blocked_arrays(off, idx, w, R, E, nb.value, cols.value)
+            nbytes = _lib.query(lib.jgamd_spmm_csx_blocked_workspace, R, E, F, nb.value)
+            ws = _lib.workspace(nbytes, self.dev)
+            torch.cuda.synchronize()
+            _lib.check(lib.jgamd_spmm_csx_blocked_timed(b_off.data_ptr(), b_idx.data_ptr(), b_w.data_ptr(), x.data_ptr(),
+                                                        out.data_ptr(), R, C, E, F, nb.value, ws.data_ptr(), nbytes,
+                                                        _lib.stream_ptr(self.dev), iters, ctypes.byref(k_ms),
+                                                        ctypes.byref(c_ms)))
+            return k_ms.value, c_ms.value
         nbytes = _lib.query(lib.jgamd_spmm_csx_workspace, R, E, F)
         ws = _lib.workspace(nbytes, self.dev)
-        k_ms, c_ms = ctypes.c_float(), ctypes.c_float()
         torch.cuda.synchronize()
         _lib.check(lib.jgamd_spmm_csx_timed(off.data_ptr(), idx.data_ptr(), w.data_ptr(), x.data_ptr(), out.data_ptr(),
                                             R, C, E, F, ws.data_ptr(), nbytes, _lib.stream_ptr(self.dev), iters,
@@ -204,7 +219,7 @@ def base_line(args, metric, value, unit, ms, higher, workload, extra_config):
 # --------------------------------------------------------------------------------- config 2
 def config2(b):
     from jittorgeometric_amd import synthetic
-    from jittorgeometric_amd.nn import GCNConv
+    from jittorgeometric_amd.nn import GCNConv, SAGEConv
     from jittorgeometric_amd.ops import EdgeSoftmax, cootocsc, gat_aggregate
     from jittorgeometric_amd.ops._common import spmm, spmm_axpby
     from jittorgeometric_amd.ops.gat import gat_forward_raw
@@ -218,89 +233,107 @@ def config2(b):
         b.calibrate_copy()
 
     step = lambda: spmm(csc.column_offset, csc.row_indices, csc.edge_weight, x, V)
-    ms_per_step = b.timed(step, args.steps, args.warmup)
     bytes_step = spmm_bytes(V, E, F)
-    value = bytes_step / (ms_per_step * 1e-3) / 1e9
-    bwd_ms = b.timed(lambda: spmm(csr.row_offset, csr.column_indices, csr.edge_weight, x, V), 20, 3)
-    k_ms, c_ms = b.spmm_kernel_ms(csc.column_offset, csc.row_indices, csc.edge_weight, x, V, max(args.steps, 10))
-
-    # one GCN layer forward + backward on the same graph
-    layer = GCNConv(F, F, spmm=False).to(dev)
-    xg = x.clone().requires_grad_(True)
-    g_up = torch.randn(V, F, device=dev)
-
-    def layer_step():
-        layer.zero_grad(set_to_none=True)
-        xg.grad = None
-        layer(xg, csc, csr).backward(g_up)
-    gcn_ms = b.timed(layer_step, 10, 2)
-
-    # fused GAT layer core on the 169k-node configuration
-    gei_np, gV = synthetic.make("gat_169k")
-    gei, _ = add_remaining_self_loops(torch.from_numpy(gei_np).to(dev), None, 1.0, gV)
-    gei = gei.contiguous()
-    gE = gei.shape[1]
-    gcsc = cootocsc(gei, torch.ones(gE, device=dev), gV)
-    H, D = 8, 16
-    gh = torch.randn(gV, H, D, device=dev, requires_grad=True)
-    ga_s = (torch.randn(H, D, device=dev) / 4).requires_grad_(True)
-    ga_d = (torch.randn(H, D, device=dev) / 4).requires_grad_(True)
-    gg = torch.randn(gV, H, D, device=dev)
-    gat_fwd_ms = b.timed(lambda: gat_forward_raw(gh.detach(), gcsc, ga_s.detach(), ga_d.detach(), 0.2), 20, 3)
-
-    def gat_step():
-        gh.grad = ga_s.grad = ga_d.grad = None
-        gat_aggregate(gh, gcsc, ga_s, ga_d, 0.2).backward(gg)
-    gat_fb_ms = b.timed(gat_step, 20, 3)
-    gat_bytes = gE * (4 + 4 * H * D) + gV * (4 + 8 * H + 4 * H * D) + gV * H * D * 4 + 2 * gV * H * 4
-
-    # edge softmax (the reference's [E,1] shape, and 8 heads) and one propagation hop
-    logits = torch.randn(E, 1, device=dev, requires_grad=True)
-    esm_fwd_ms = b.timed(lambda: EdgeSoftmax(logits.detach(), csc), 20, 3)
-    y1 = EdgeSoftmax(logits, csc)
-    g1 = torch.randn(E, 1, device=dev)
-    esm_bwd_ms = b.timed(lambda: torch.autograd.grad(y1, logits, g1, retain_graph=True), 20, 3)
-    del y1, g1, logits
-    logits8 = torch.randn(E, 8, device=dev)
-    esm8_fwd_ms = b.timed(lambda: EdgeSoftmax(logits8, csc), 10, 2)
-    del logits8
-    hop_ms = b.timed(lambda: spmm_axpby(csc.column_offset, csc.row_indices, csc.edge_weight, x, V, 0.9, 0.1, x), 10, 2)
-
-    cpu, err = (None, 0.0)
-    if not args.no_cpu_baseline:
-        cpu, err = b.cpu_spmm_baseline(csc, x, step, bytes_step, (ei, w),
-                                       "the same SpMM workload (V=%d, E=%d, F=%d)" % (V, E, F))
-
-    line = base_line(args, "spmm_f128_algorithmic_bandwidth", round(value, 1), "GB/s", ms_per_step, True,
+    line = base_line(args, "spmm_f128_algorithmic_bandwidth", 0.0, "GB/s", 0.0, True,
                      "config 2: weighted CSC SpMM, V=1,000,000 Chung-Lu power-law (exp 2.1, cap 20000) "
                      "+ self-loops, gcn_norm weights, F=128", {"V": V, "E": E, "F": F, "bytes_per_step": bytes_step})
-    esm_b = lambda h, per: (per * E * h + 4 * (V + 1))
-    line.update({
-        "pct_hbm_peak_algorithmic": round(100 * value / HBM_PEAK_GBPS, 2),
-        "spmm_csr_backward_ms": round(bwd_ms, 4),
-        "coo_to_csr_edges_per_s": round(E / (conv_csr_ms * 1e-3)),
-        "coo_to_csc_edges_per_s": round(E / (conv_csc_ms * 1e-3)),
-        "coo_to_csr_ms": round(conv_csr_ms, 4),
-        "coo_to_csr_algorithmic_gbps": round((24 * E + 8 * (V + 1)) / (conv_csr_ms * 1e-3) / 1e9, 1),
-        "gcn_layer_fwd_bwd_ms": round(gcn_ms, 4),
-        "gcn_layer_shape": "GCNConv(128->128) on the same graph, aggregateWithWeight path: x@W, SpMM, bias; "
-                           "backward SpMM, W.grad, x.grad",
-        "gat_fused_fwd_ms": round(gat_fwd_ms, 4),
-        "gat_fused_fwd_bwd_ms": round(gat_fb_ms, 4),
-        "gat_fused_fwd_algorithmic_gbps": round(gat_bytes / (gat_fwd_ms * 1e-3) / 1e9, 1),
-        "gat_shape": "V=%d, E=%d (power-law exp 2.3 + self-loops), 8 heads x 16" % (gV, gE),
-        "edge_softmax_fwd_ms": round(esm_fwd_ms, 4),
-        "edge_softmax_fwd_algorithmic_gbps": round(esm_b(1, 8) / (esm_fwd_ms * 1e-3) / 1e9, 1),
-        "edge_softmax_bwd_ms": round(esm_bwd_ms, 4),
-        "edge_softmax_bwd_algorithmic_gbps": round(esm_b(1, 12) / (esm_bwd_ms * 1e-3) / 1e9, 1),
-        "edge_softmax_h8_fwd_ms": round(esm8_fwd_ms, 4),
-        "edge_softmax_h8_fwd_algorithmic_gbps": round(esm_b(8, 8) / (esm8_fwd_ms * 1e-3) / 1e9, 1),
-        "appnp_hop_f128_ms": round(hop_ms, 4),
-        "roofline": roofline("spmm_merge_powerlaw_1m_f128.txt", {"V": V, "E": E, "F": F}, "spmm_merge", k_ms,
-                             bytes_step, spmm_compulsory_bytes(V, V, E, F), "hipEvents in this run"),
-        "spmm_call_ms": round(c_ms, 4),
-        "cpu_baseline": cpu,
-    })
+    if args.part != "layers":
+        ms_per_step = b.timed(step, args.steps, args.warmup)
+        value = bytes_step / (ms_per_step * 1e-3) / 1e9
+        k_ms, c_ms = b.spmm_kernel_ms(csc.column_offset, csc.row_indices, csc.edge_weight, x, V, max(args.steps, 10))
+        line.update({
+            "value": round(value, 1), "ms_per_step": round(ms_per_step, 4),
+            "pct_hbm_peak_algorithmic": round(100 * value / HBM_PEAK_GBPS, 2),
+            "coo_to_csr_edges_per_s": round(E / (conv_csr_ms * 1e-3)),
+            "coo_to_csc_edges_per_s": round(E / (conv_csc_ms * 1e-3)),
+            "coo_to_csr_ms": round(conv_csr_ms, 4),
+            "coo_to_csr_algorithmic_gbps": round((24 * E + 8 * (V + 1)) / (conv_csr_ms * 1e-3) / 1e9, 1),
+            "roofline": roofline("spmm_merge_powerlaw_1m_f128.txt", {"V": V, "E": E, "F": F}, "spmm_merge", k_ms,
+                                 bytes_step, spmm_compulsory_bytes(V, V, E, F), "hipEvents in this run"),
+            "spmm_call_ms": round(c_ms, 4),
+        })
+
+    if args.part in ("all", "layers"):
+        # one GCN layer and one GraphSAGE (mean) layer, forward + backward, on the same graph
+        xg = x.clone().requires_grad_(True)
+        g_up = torch.randn(V, F, device=dev)
+
+        def layer_ms(layer, call):
+            def one():
+                layer.zero_grad(set_to_none=True)
+                xg.grad = None
+                call(layer).backward(g_up)
+            return b.timed(one, max(args.steps, 10) if args.part == "layers" else 10, 2)
+        gcn_ms = layer_ms(GCNConv(F, F, spmm=False).to(dev), lambda l: l(xg, csc, csr))
+        ei_s, w_s, _, csc_s, csr_s, _, _ = b.graph("powerlaw_1m", "sage", time_conversions=False)
+        sage_ms = layer_ms(SAGEConv(F, F, spmm=False).to(dev), lambda l: l(xg, None, None, csc_s, csr_s))
+        del ei_s, w_s, csc_s, csr_s
+        line.update({
+            "gcn_layer_fwd_bwd_ms": round(gcn_ms, 4),
+            "gcn_layer_shape": "GCNConv(128->128) on the same graph, aggregateWithWeight path: x@W, SpMM + bias; "
+                               "backward: bias column sum, transposed SpMM, W.grad, x.grad",
+            "sage_layer_fwd_bwd_ms": round(sage_ms, 4),
+            "sage_layer_shape": "SAGEConv(128->128, root weight, bias) on the same graph with mean weights: SpMM, "
+                                "both dense products + bias in one pass; backward: column sum, two W.grad, two "
+                                "input-gradient products, transposed SpMM with the root term added in its row store",
+        })
+        if args.part == "layers":
+            line.update({"metric": "gcn_layer_fwd_bwd_ms", "value": round(gcn_ms, 4), "unit": "ms",
+                         "ms_per_step": round(gcn_ms, 4), "higher_is_better": False})
+
+    if args.part == "all":
+        bwd_ms = b.timed(lambda: spmm(csr.row_offset, csr.column_indices, csr.edge_weight, x, V), 20, 3)
+        # fused GAT layer core on the 169k-node configuration
+        gei_np, gV = synthetic.make("gat_169k")
+        gei, _ = add_remaining_self_loops(torch.from_numpy(gei_np).to(dev), None, 1.0, gV)
+        gei = gei.contiguous()
+        gE = gei.shape[1]
+        gcsc = cootocsc(gei, torch.ones(gE, device=dev), gV)
+        H, D = 8, 16
+        gh = torch.randn(gV, H, D, device=dev, requires_grad=True)
+        ga_s = (torch.randn(H, D, device=dev) / 4).requires_grad_(True)
+        ga_d = (torch.randn(H, D, device=dev) / 4).requires_grad_(True)
+        gg = torch.randn(gV, H, D, device=dev)
+        gat_fwd_ms = b.timed(lambda: gat_forward_raw(gh.detach(), gcsc, ga_s.detach(), ga_d.detach(), 0.2), 20, 3)
+
+        def gat_step():
+            gh.grad = ga_s.grad = ga_d.grad = None
+            gat_aggregate(gh, gcsc, ga_s, ga_d, 0.2).backward(gg)
+        gat_fb_ms = b.timed(gat_step, 20, 3)
+        gat_bytes = gE * (4 + 4 * H * D) + gV * (4 + 8 * H + 4 * H * D) + gV * H * D * 4 + 2 * gV * H * 4
+
+        # edge softmax (the reference's [E,1] shape, and 8 heads) and one propagation hop
+        logits = torch.randn(E, 1, device=dev, requires_grad=True)
+        esm_fwd_ms = b.timed(lambda: EdgeSoftmax(logits.detach(), csc), 20, 3)
+        y1 = EdgeSoftmax(logits, csc)
+        g1 = torch.randn(E, 1, device=dev)
+        esm_bwd_ms = b.timed(lambda: torch.autograd.grad(y1, logits, g1, retain_graph=True), 20, 3)
+        del y1, g1, logits
+        logits8 = torch.randn(E, 8, device=dev)
+        esm8_fwd_ms = b.timed(lambda: EdgeSoftmax(logits8, csc), 10, 2)
+        del logits8
+        hop_ms = b.timed(lambda: spmm_axpby(csc.column_offset, csc.row_indices, csc.edge_weight, x, V, 0.9, 0.1, x), 10, 2)
+        esm_b = lambda h, per: (per * E * h + 4 * (V + 1))
+        line.update({
+            "spmm_csr_backward_ms": round(bwd_ms, 4),
+            "gat_fused_fwd_ms": round(gat_fwd_ms, 4),
+            "gat_fused_fwd_bwd_ms": round(gat_fb_ms, 4),
+            "gat_fused_fwd_algorithmic_gbps": round(gat_bytes / (gat_fwd_ms * 1e-3) / 1e9, 1),
+            "gat_shape": "V=%d, E=%d (power-law exp 2.3 + self-loops), 8 heads x 16" % (gV, gE),
+            "edge_softmax_fwd_ms": round(esm_fwd_ms, 4),
+            "edge_softmax_fwd_algorithmic_gbps": round(esm_b(1, 8) / (esm_fwd_ms * 1e-3) / 1e9, 1),
+            "edge_softmax_bwd_ms": round(esm_bwd_ms, 4),
+            "edge_softmax_bwd_algorithmic_gbps": round(esm_b(1, 12) / (esm_bwd_ms * 1e-3) / 1e9, 1),
+            "edge_softmax_h8_fwd_ms": round(esm8_fwd_ms, 4),
+            "edge_softmax_h8_fwd_algorithmic_gbps": round(esm_b(8, 8) / (esm8_fwd_ms * 1e-3) / 1e9, 1),
+            "appnp_hop_f128_ms": round(hop_ms, 4),
+        })
+
+    cpu, err = (None, 0.0)
+    if not args.no_cpu_baseline and args.part == "all":
+        cpu, err = b.cpu_spmm_baseline(csc, x, step, bytes_step, (ei, w),
+                                       "the same SpMM workload (V=%d, E=%d, F=%d)" % (V, E, F))
+    line["cpu_baseline"] = cpu
     return line, err
 
 
@@ -416,26 +449,39 @@ def config4(b):
     ei, w, V, csc, csr, conv_csr_ms, conv_csc_ms = b.graph("dense_233k")
     E = ei.shape[1]
     res = {}
-    for F in (602, 256, 41):
+    for F in ((602,) if args.part == "main" else (602, 256, 41)):
         x = torch.randn(V, F, device=dev)
         step = lambda: spmm(csc.column_offset, csc.row_indices, csc.edge_weight, x, V)
         ms = b.timed(step, args.steps if F == 602 else 10, args.warmup if F == 602 else 2)
         k_ms, _ = b.spmm_kernel_ms(csc.column_offset, csc.row_indices, csc.edge_weight, x, V, 10)
-        res[F] = (ms, k_ms, x, step)
-    ms, k_ms, x, step = res[602]
+        res[F] = (ms, k_ms, x, step, b.blocked)
+    ms, k_ms, x, step, blocks = res[602]
+
+    def regroup():
+        # the once-per-matrix regrouping by column block, which the timed steps above reuse
+        from jittorgeometric_amd.ops._common import _blocked_arrays
+        nb, cols = ctypes.c_int32(0), ctypes.c_int32(0)
+        b._lib.check(b.lib.jgamd_spmm_block_plan(V, V, E, 602, ctypes.byref(nb), ctypes.byref(cols)))
+        if nb.value:
+            csc.column_offset._jgamd_blocked = None
+            _blocked_arrays(csc.column_offset, csc.row_indices, csc.edge_weight, V, E, nb.value, cols.value)
+    regroup_ms = b.timed(regroup, 3, 1) if blocks else 0.0
     bytes_step = spmm_bytes(V, E, 602)
     cpu, err = (None, 0.0)
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and args.part == "all":
         x41 = res[41][2]
         cpu, err = b.cpu_spmm_baseline(csc, x41, res[41][3], spmm_bytes(V, E, 41), (ei, w),
                                        "the F=41 product of this graph (V=%d, E=%d)" % (V, E))
     line = base_line(args, "spmm_f602_algorithmic_bandwidth", round(bytes_step / (ms * 1e-3) / 1e9, 1), "GB/s", ms, True,
                      "config 4: weighted CSC SpMM, V=232,965, lognormal degrees (mean 492) + self-loops, F=602",
                      {"V": V, "E": E, "F": 602, "bytes_per_step": bytes_step})
-    line.update({"spmm_f256_ms": round(res[256][0], 4),
-                 "spmm_f256_algorithmic_gbps": round(spmm_bytes(V, E, 256) / (res[256][0] * 1e-3) / 1e9, 1),
-                 "spmm_f41_ms": round(res[41][0], 4),
-                 "spmm_f41_algorithmic_gbps": round(spmm_bytes(V, E, 41) / (res[41][0] * 1e-3) / 1e9, 1),
+    if args.part == "all":
+        line.update({"spmm_f256_ms": round(res[256][0], 4),
+                     "spmm_f256_algorithmic_gbps": round(spmm_bytes(V, E, 256) / (res[256][0] * 1e-3) / 1e9, 1),
+                     "spmm_f41_ms": round(res[41][0], 4),
+                     "spmm_f41_algorithmic_gbps": round(spmm_bytes(V, E, 41) / (res[41][0] * 1e-3) / 1e9, 1)})
+    line.update({"column_blocks": blocks,
+                 "regroup_by_column_block_ms_once_per_matrix": round(regroup_ms, 4),
                  "coo_to_csr_ms": round(conv_csr_ms, 4), "coo_to_csr_edges_per_s": round(E / (conv_csr_ms * 1e-3)),
                  "coo_to_csc_edges_per_s": round(E / (conv_csc_ms * 1e-3)),
                  "roofline": roofline("spmm_merge_dense_233k_f602.txt", {"V": V, "E": E, "F": 602}, "spmm_merge", k_ms,
@@ -467,21 +513,26 @@ def config5(b):
                 hcur = torch.relu(hcur)
         torch.nn.functional.cross_entropy(hcur, y).backward()
 
-    gcn = [GCNConv(dims[i], dims[i + 1], spmm=False).to(dev) for i in range(3)]
-    gcn_ms = b.timed(lambda: model_step(gcn, lambda l, t: l(t, csc, csr)), args.steps, args.warmup)
-    from jittorgeometric_amd.nn import sage_norm
-    sei, sw = sage_norm(ei[:, :E - V].contiguous(), None, V)       # same edges, mean weights
-    sei = sei.contiguous()
-    scsc, scsr = cootocsc(sei, sw, V), cootocsr(sei, sw, V)
-    sage = [SAGEConv(dims[i], dims[i + 1], root_weight=False, spmm=False).to(dev) for i in range(3)]
-    sage_ms = b.timed(lambda: model_step(sage, lambda l, t: l(t, None, None, scsc, scsr)), args.steps, args.warmup)
+    main_only = args.part == "main"
+    gcn_ms = sage_ms = 0.0
+    if not main_only:
+        gcn = [GCNConv(dims[i], dims[i + 1], spmm=False).to(dev) for i in range(3)]
+        gcn_ms = b.timed(lambda: model_step(gcn, lambda l, t: l(t, csc, csr)), args.steps, args.warmup)
+        from jittorgeometric_amd.nn import sage_norm
+        sei, sw = sage_norm(ei[:, :E - V].contiguous(), None, V)       # same edges, mean weights
+        sei = sei.contiguous()
+        scsc, scsr = cootocsc(sei, sw, V), cootocsr(sei, sw, V)
+        sage = [SAGEConv(dims[i], dims[i + 1], root_weight=False, spmm=False).to(dev) for i in range(3)]
+        sage_ms = b.timed(lambda: model_step(sage, lambda l, t: l(t, None, None, scsc, scsr)), args.steps, args.warmup)
+        del sei, sw, scsc, scsr, sage, gcn
+    widths = (256,) if main_only else (100, 256, 47)
     prod = {}
-    for F in (100, 256, 47):
+    for F in widths:
         xf = torch.randn(V, F, device=dev)
         prod[F] = (b.timed(lambda: spmm(csc.column_offset, csc.row_indices, csc.edge_weight, xf, V), 10, 2),
                    b.spmm_kernel_ms(csc.column_offset, csc.row_indices, csc.edge_weight, xf, V, 10)[0], xf)
     cpu, err = (None, 0.0)
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and not main_only:
         xf = prod[47][2]
         cpu, err = b.cpu_spmm_baseline(csc, xf, lambda: spmm(csc.column_offset, csc.row_indices, csc.edge_weight, xf, V),
                                        spmm_bytes(V, E, 47), (ei, w),
@@ -492,7 +543,7 @@ def config5(b):
     line.update({"sage3_fullgraph_fwd_bwd_ms": round(sage_ms, 3),
                  "coo_to_csr_ms": round(conv_csr_ms, 4), "coo_to_csr_edges_per_s": round(E / (conv_csr_ms * 1e-3)),
                  "coo_to_csc_edges_per_s": round(E / (conv_csc_ms * 1e-3))})
-    for F in (100, 256, 47):
+    for F in widths:
         line["spmm_f%d_ms" % F] = round(prod[F][0], 4)
         line["spmm_f%d_algorithmic_gbps" % F] = round(spmm_bytes(V, E, F) / (prod[F][0] * 1e-3) / 1e9, 1)
     line["roofline"] = roofline("spmm_merge_powerlaw_2m4_f256.txt", {"V": V, "E": E, "F": 256}, "spmm_merge", prod[256][1],
@@ -509,9 +560,14 @@ def main():
     ap.add_argument("--config", type=int, default=2, choices=[1, 2, 3, 4, 5],
                     help="benchmark configuration; 2 (the headline SpMM workload) is the default")
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the single-thread CPU timing")
+    ap.add_argument("--part", default="all", choices=["all", "main", "layers"],
+                    help="main: only the timed workload of the metric (what the counter profiles under profiles/ "
+                         "are taken from); layers: only the GCN and GraphSAGE layer steps of config 2")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (known traffic, for scaling rocprof counters)")
     args = ap.parse_args()
+    if args.part == "layers" and args.config != 2:
+        sys.exit("bench.py: --part layers belongs to --config 2")
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only; --gpus %d is not supported "
                  "(no collectives or sharding are part of it)" % args.gpus)

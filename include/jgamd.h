@@ -276,6 +276,12 @@ int32_t jgamd_spmm_csx_blocked(const int32_t *b_off, const int32_t *b_idx, const
                                const float *x, float *out, float beta, float alpha,
                                const float *h, int32_t h_rows, int32_t R, int32_t C, int64_t E,
                                int32_t F, int32_t nb, void *ws, size_t ws_bytes, void *stream);
+/* measurement aid, as jgamd_spmm_csx_timed: the plain product (beta 1, alpha 0) `iters` times,
+ * mean milliseconds of the gather kernel and of the whole call from HIP events on `stream` */
+int32_t jgamd_spmm_csx_blocked_timed(const int32_t *b_off, const int32_t *b_idx, const float *b_w,
+                                     const float *x, float *out, int32_t R, int32_t C, int64_t E,
+                                     int32_t F, int32_t nb, void *ws, size_t ws_bytes, void *stream,
+                                     int32_t iters, float *kernel_ms, float *call_ms);
 
 /* ------------------------------------------------------------------------
  * Dense feature transform of the conv layers on the matrix cores (fp32 in,

@@ -38,6 +38,8 @@ SIGNATURES = {
     "jgamd_spmm_csx_blocked_workspace": [_I32, _I64, _I32, _I32, _SZP],
     "jgamd_spmm_csx_blocked": [_P, _P, _P, _P, _P, _F32, _F32, _P, _I32, _I32, _I32, _I64, _I32, _I32, _P,
                                _c.c_size_t, _P],
+    "jgamd_spmm_csx_blocked_timed": [_P, _P, _P, _P, _P, _I32, _I32, _I64, _I32, _I32, _P, _c.c_size_t, _P, _I32,
+                                     _c.POINTER(_c.c_float), _c.POINTER(_c.c_float)],
     "jgamd_spmm_csx_timed": [_P, _P, _P, _P, _P, _I32, _I32, _I64, _I32, _P, _c.c_size_t, _P, _I32,
                              _c.POINTER(_c.c_float), _c.POINTER(_c.c_float)],
     "jgamd_edge_softmax_workspace": [_I32, _I64, _SZP],

@@ -646,9 +646,10 @@ int32_t spmm_enqueue(const int32_t *off, const int32_t *idx, const float *w, con
     return spmm_call(off, idx, w, x, out, R, C, E, F, ws, ws_bytes, s, nullptr, nullptr);
 }
 int32_t spmm_enqueue_slabs(const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out,
-                           int32_t R, int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, hipStream_t s)
+                           int32_t R, int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, hipStream_t s,
+                           hipEvent_t k0, hipEvent_t k1)
 {
-    return spmm_call(off, idx, w, x, out, R, C, E, F, ws, ws_bytes, s, nullptr, nullptr, nullptr, true);
+    return spmm_call(off, idx, w, x, out, R, C, E, F, ws, ws_bytes, s, k0, k1, nullptr, true);
 }
 }  // namespace jg
 

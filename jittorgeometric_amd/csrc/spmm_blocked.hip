@@ -173,7 +173,9 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_block_plan(
     // bytes of x one block may cover.  Measured on V = 233k, 492 entries per row, F = 41 .. 602:
     // 1.5 MB .. 16 MB blocks; fastest between 4.5 and 6 MB (fewer partial rows against more misses)
     static const int kb = env_kb("JGAMD_SPMM_BLOCK_KB", 4608);
-    const int64_t slab_bytes = (int64_t)(F < kWave ? F : kWave) * 4;
+    // one blocking per matrix whatever the width: a block is sized for the 256-byte slabs of wide
+    // rows, and rows narrower than that just fill less of it
+    const int64_t slab_bytes = (int64_t)kWave * 4;
     int64_t cols = ((int64_t)kb * 1024 / slab_bytes) & ~(int64_t)255;
     if (cols < 1024) cols = 1024;
     const int64_t blocks = ceil_div((int64_t)C, cols);
@@ -238,10 +240,9 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_blocked
     return 0;
 }
 
-extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_blocked(
-    const int32_t *b_off, const int32_t *b_idx, const float *b_w, const float *x, float *out, float beta, float alpha,
-    const float *h, int32_t h_rows, int32_t R, int32_t C, int64_t E, int32_t F, int32_t nb, void *ws, size_t ws_bytes,
-    void *stream)
+static int32_t blocked_call(const int32_t *b_off, const int32_t *b_idx, const float *b_w, const float *x, float *out,
+                            float beta, float alpha, const float *h, int32_t h_rows, int32_t R, int32_t C, int64_t E,
+                            int32_t F, int32_t nb, void *ws, size_t ws_bytes, void *stream, hipEvent_t k0, hipEvent_t k1)
 {
     size_t need = 0;
     if (int32_t rc = jgamd_spmm_csx_blocked_workspace(R, E, F, nb, &need)) return rc;
@@ -258,7 +259,7 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_blocked
     Carver carve(ws);
     float *partial = carve.take<float>((size_t)nb * (size_t)R * (size_t)F);
     void *inner = static_cast<char *>(ws) + carve.used;
-    if (int32_t rc = spmm_enqueue_slabs(b_off, b_idx, b_w, x, partial, nb * R, C, E, F, inner, ws_bytes - carve.used, s))
+    if (int32_t rc = spmm_enqueue_slabs(b_off, b_idx, b_w, x, partial, nb * R, C, E, F, inner, ws_bytes - carve.used, s, k0, k1))
         return rc;
     const float *hh = alpha != 0.f ? h : nullptr;
     const int h_stride = h_rows == 1 ? 0 : 1;
@@ -272,4 +273,50 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_blocked
                            alpha, hh, h_stride, out);
     }
     return launch_status("spmm_csx_blocked");
+}
+
+extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_blocked(
+    const int32_t *b_off, const int32_t *b_idx, const float *b_w, const float *x, float *out, float beta, float alpha,
+    const float *h, int32_t h_rows, int32_t R, int32_t C, int64_t E, int32_t F, int32_t nb, void *ws, size_t ws_bytes,
+    void *stream)
+{
+    return blocked_call(b_off, b_idx, b_w, x, out, beta, alpha, h, h_rows, R, C, E, F, nb, ws, ws_bytes, stream, nullptr,
+                        nullptr);
+}
+
+// the same call `iters` times with HIP events on the launch stream: mean duration of the gather
+// kernel over the regrouped rows and of the whole call (gather, fix-up, sum over the blocks)
+extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_blocked_timed(
+    const int32_t *b_off, const int32_t *b_idx, const float *b_w, const float *x, float *out, int32_t R, int32_t C,
+    int64_t E, int32_t F, int32_t nb, void *ws, size_t ws_bytes, void *stream, int32_t iters, float *kernel_ms,
+    float *call_ms)
+{
+    if (iters < 1 || iters > 4096) return fail(JGAMD_ERR_SIZE, "spmm_csx_blocked_timed: iters must be in [1, 4096]");
+    if (!kernel_ms || !call_ms) return fail(JGAMD_ERR_NULL, "spmm_csx_blocked_timed: NULL result pointer");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipEvent_t ev[4];
+    for (auto &e : ev)
+        if (hipEventCreate(&e) != hipSuccess)
+            return fail(JGAMD_ERR_UNSUPPORTED, "spmm_csx_blocked_timed: hipEventCreate failed");
+    double ksum = 0, csum = 0;
+    int32_t rc = 0;
+    for (int i = 0; i < iters && rc == 0; i++) {
+        (void)hipEventRecord(ev[0], st);
+        rc = blocked_call(b_off, b_idx, b_w, x, out, 1.f, 0.f, nullptr, 1, R, C, E, F, nb, ws, ws_bytes, stream, ev[1],
+                          ev[2]);
+        (void)hipEventRecord(ev[3], st);
+        if (hipEventSynchronize(ev[3]) != hipSuccess && rc == 0)
+            rc = fail(JGAMD_ERR_UNSUPPORTED, "spmm_csx_blocked_timed: hipEventSynchronize failed");
+        float k = 0, c = 0;
+        if (rc == 0 && R > 0 && F > 0) {
+            (void)hipEventElapsedTime(&k, ev[1], ev[2]);
+            (void)hipEventElapsedTime(&c, ev[0], ev[3]);
+        }
+        ksum += k;
+        csum += c;
+    }
+    for (auto &e : ev) (void)hipEventDestroy(e);
+    *kernel_ms = (float)(ksum / iters);
+    *call_ms = (float)(csum / iters);
+    return rc;
 }
