@@ -451,7 +451,7 @@ def config4(b):
     res = {}
     for F in ((602,) if args.part == "main" else (602, 256, 41)):
         x = torch.randn(V, F, device=dev)
-        step = lambda: spmm(csc.column_offset, csc.row_indices, csc.edge_weight, x, V)
+        step = lambda x=x: spmm(csc.column_offset, csc.row_indices, csc.edge_weight, x, V)
         ms = b.timed(step, args.steps if F == 602 else 10, args.warmup if F == 602 else 2)
         k_ms, _ = b.spmm_kernel_ms(csc.column_offset, csc.row_indices, csc.edge_weight, x, V, 10)
         res[F] = (ms, k_ms, x, step, b.blocked)
@@ -529,7 +529,7 @@ def config5(b):
     prod = {}
     for F in widths:
         xf = torch.randn(V, F, device=dev)
-        prod[F] = (b.timed(lambda: spmm(csc.column_offset, csc.row_indices, csc.edge_weight, xf, V), 10, 2),
+        prod[F] = (b.timed(lambda xf=xf: spmm(csc.column_offset, csc.row_indices, csc.edge_weight, xf, V), 10, 2),
                    b.spmm_kernel_ms(csc.column_offset, csc.row_indices, csc.edge_weight, xf, V, 10)[0], xf)
     cpu, err = (None, 0.0)
     if not args.no_cpu_baseline and not main_only:
