@@ -193,7 +193,11 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__rest
             for (int v = 0; v < VEC; v++) acc[t][v] = 0.f;
         }
         r++;
-        if constexpr (EPI) fetch_h();
+        if constexpr (EPI) {
+            // one row for every output row (a bias) was fetched before the loop; a load here would
+            // make the flush wait for every gather in flight
+            if (fin.h && fin.h_stride != 0) fetch_h();
+        }
         if (r - rb == kWave) {
             rb = r;
             ends = (rb + lane < R) ? off[rb + 1 + lane] : kNever;

@@ -4,6 +4,7 @@ import torch
 from torch import nn
 
 from ...ops import SpmmCsr, aggregateWithWeight, cootocsc
+from ...ops import spmmcsr as _spmmcsr
 from ...ops.propagate import aggregate_bias
 from ...utils import add_remaining_self_loops
 from ...utils.num_nodes import maybe_num_nodes
@@ -82,7 +83,7 @@ class GCNConv(nn.Module):
 
     def forward(self, x, csc, csr):
         x = xw(x, self.weight)
-        if self.bias is not None and x.dim() == 2:
+        if self.bias is not None and x.dim() == 2 and not (self.spmm and _spmmcsr.REFERENCE_GRAD):
             # product and bias in one kernel; spmm=True only needs the CSR (:96-97)
             return aggregate_bias(x, self.bias, None if self.spmm and csr is not None else csc, csr)
         if self.spmm:

@@ -4,6 +4,7 @@ import torch
 from torch import nn
 
 from ...ops import SpmmCsr, aggregateWithWeight, cootocsc, cootocsr
+from ...ops import spmmcsr as _spmmcsr
 from ...ops._common import both_orders, spmm, spmm_axpby
 from ..dense import add_bias, column_sum, rows_times, xt_g, xw
 from ..inits import glorot, zeros
@@ -102,7 +103,8 @@ class SAGEConv(nn.Module):
                     self._cached_edge_index = (edge_index, edge_weight, csr, csc)
             else:
                 edge_index, edge_weight, csr, csc = cache
-        if self.weight_proj is None and x.dim() == 2 and x.dtype == torch.float32:
+        reference_grad = self.spmm and _spmmcsr.REFERENCE_GRAD      # that switch lives in SpmmCsr: unfused route
+        if self.weight_proj is None and x.dim() == 2 and x.dtype == torch.float32 and not reference_grad:
             # spmm=True only needs the CSR arrays (:183-184); both routes give the same product
             fwd, bwd = both_orders(None if self.spmm and csr is not None else csc, csr)
             return SageLayerFunc.apply(x.contiguous(), self.weight1, self.root_weight, self.bias, fwd, bwd)

@@ -212,3 +212,32 @@ def test_preprocessing_refuses_cpu_tensors():
     for fn in (lambda: gcn_norm(ei, None, 2), lambda: sage_norm(ei, None, 2), lambda: add_remaining_self_loops(ei, None, 1.0, 2)):
         with pytest.raises(_lib.JgamdError):
             fn()
+
+
+def test_layers_honour_the_reference_grad_switch():
+    """With REFERENCE_GRAD set, a layer on its spmm=True route back-propagates through the forward
+    product again, as ops/spmmcsr.py:35-39 does; the fused layer paths step aside for it."""
+    from jittorgeometric_amd.nn import SAGEConv, sage_norm
+    from jittorgeometric_amd.ops import cootocsc, cootocsr, spmmcsr
+    from jittorgeometric_amd import synthetic
+    V = 2000
+    ei = synthetic.chung_lu(V, 30000, 2.1, max_degree=500, seed=4)
+    eit, wt = sage_norm(to_gpu(ei), None, V)
+    oei, ow = oracle.sage_norm(ei, None, V)
+    csc, csr = cootocsc(eit, wt, V), cootocsr(eit, wt, V)
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((V, 32)).astype(np.float32)
+    g = rng.standard_normal((V, 16)).astype(np.float32)
+    torch.manual_seed(1)
+    layer = SAGEConv(32, 16, root_weight=False, bias=False, spmm=True).to(dev())
+    A = dense_adj(oei, ow, V).numpy()
+    gW = g.astype(np.float64) @ layer.weight1.detach().cpu().double().numpy().T
+    try:
+        for flag, want in ((False, A.T @ gW), (True, A @ gW)):
+            spmmcsr.REFERENCE_GRAD = flag
+            xt = to_gpu(x).requires_grad_(True)
+            layer(xt, csc=csc, csr=csr).backward(to_gpu(g))
+            assert_close(xt.grad.cpu().numpy(), want, np.abs(want) + np.abs(want).mean(), rtol=1e-4,
+                         what="REFERENCE_GRAD=%s" % flag)
+    finally:
+        spmmcsr.REFERENCE_GRAD = False
