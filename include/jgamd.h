@@ -261,7 +261,9 @@ int32_t jgamd_gat_bwd(const int32_t *off, const int32_t *idx, const int32_t *t_o
  * block taking what lies beyond.  Entries from off[R] on are not part of it.
  * Done once per matrix; nb <= 64.
  *
- * jgamd_spmm_csx_blocked: the product over arrays made by that call.
+ * jgamd_spmm_csx_blocked: the product over arrays made by that call.  When F
+ * is not a multiple of 32 the rows of x are first copied 128-byte aligned into
+ * the workspace (one pass over x), so that the gathered pieces are whole lines.
  */
 int32_t jgamd_spmm_block_plan(int32_t R, int32_t C, int64_t E, int32_t F, int32_t *nb,
                               int32_t *block_cols);
@@ -270,7 +272,7 @@ int32_t jgamd_csx_block_columns(const int32_t *off, const int32_t *idx, const fl
                                 int64_t E, int32_t block_cols, int32_t nb, int32_t *b_off,
                                 int32_t *b_idx, float *b_w, void *ws, size_t ws_bytes,
                                 void *stream);
-int32_t jgamd_spmm_csx_blocked_workspace(int32_t R, int64_t E, int32_t F, int32_t nb,
+int32_t jgamd_spmm_csx_blocked_workspace(int32_t R, int32_t C, int64_t E, int32_t F, int32_t nb,
                                          size_t *bytes);
 int32_t jgamd_spmm_csx_blocked(const int32_t *b_off, const int32_t *b_idx, const float *b_w,
                                const float *x, float *out, float beta, float alpha,

@@ -35,7 +35,7 @@ SIGNATURES = {
     "jgamd_spmm_block_plan": [_I32, _I32, _I64, _I32, _c.POINTER(_I32), _c.POINTER(_I32)],
     "jgamd_csx_block_columns_workspace": [_I32, _I32, _SZP],
     "jgamd_csx_block_columns": [_P, _P, _P, _I32, _I64, _I32, _I32, _P, _P, _P, _P, _c.c_size_t, _P],
-    "jgamd_spmm_csx_blocked_workspace": [_I32, _I64, _I32, _I32, _SZP],
+    "jgamd_spmm_csx_blocked_workspace": [_I32, _I32, _I64, _I32, _I32, _SZP],
     "jgamd_spmm_csx_blocked": [_P, _P, _P, _P, _P, _F32, _F32, _P, _I32, _I32, _I32, _I64, _I32, _I32, _P,
                                _c.c_size_t, _P],
     "jgamd_spmm_csx_blocked_timed": [_P, _P, _P, _P, _P, _I32, _I32, _I64, _I32, _I32, _P, _c.c_size_t, _P, _I32,

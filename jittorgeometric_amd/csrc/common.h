@@ -45,10 +45,11 @@ size_t spmm_ws_bytes(int32_t R, int64_t E, int32_t F);
 int32_t spmm_enqueue(const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out, int32_t R,
                      int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, hipStream_t s);
 // the same product walked one 64-float slab of the feature rows at a time (spmm_blocked.hip)
-// k0 / k1: optional events recorded on s right before and after the gather kernel
+// k0 / k1: optional events recorded on s right before and after the gather kernel; x_stride:
+// floats between the rows of x when they are padded apart (0 = F)
 int32_t spmm_enqueue_slabs(const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out,
                            int32_t R, int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, hipStream_t s,
-                           hipEvent_t k0 = nullptr, hipEvent_t k1 = nullptr);
+                           hipEvent_t k0 = nullptr, hipEvent_t k1 = nullptr, int x_stride = 0);
 
 // ---- tile-based edge softmax for 1, 2, 4 or 8 heads (entry_tiles.hip) --
 // fwd: a = x, b unused; bwd: a = y, b = g.  Needs V > 0, E > 0, off[V] == E.

@@ -100,6 +100,7 @@ struct RowFinish {
     float beta, alpha;
     const float *h;
     int h_stride;   // floats between the rows of h: F, or 0 when one row serves every output row
+    int x_stride;   // floats between the rows of x when they are padded apart; 0 = F
 };
 
 template <int VEC, int NT, int UNROLL, bool WIDE, bool LDS, bool EPI>
@@ -128,7 +129,8 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__rest
         fo_bytes[t] = (uint32_t)fo[t] * 4u;
     }
     const char *xb = reinterpret_cast<const char *>(x);
-    const uint32_t row_bytes = (uint32_t)F * 4u;
+    const int xs = fin.x_stride ? fin.x_stride : F;      // rows of x may be padded to whole cache lines
+    const uint32_t row_bytes = (uint32_t)xs * 4u;
 
     // rows are clamped so that a malformed off/E pair cannot index outside the arrays
     const int r1 = min(max(uniform(chunk_row[k + 1]), 0), R);
@@ -260,7 +262,7 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__rest
 #pragma unroll
                 for (int t = 0; t < NT; t++) {
                     if (WIDE)
-                        vload<VEC>(xv[u][t], x + (size_t)a * F + fo[t]);
+                        vload<VEC>(xv[u][t], x + (size_t)a * xs + fo[t]);
                     else
                         vload<VEC>(xv[u][t], reinterpret_cast<const float *>(
                                                  xb + (size_t)((uint32_t)a + fo_bytes[t])));
@@ -505,7 +507,7 @@ template <int VEC, int NT>
 static void launch_spmm(const SpmmShape &s, const int32_t *off, const int32_t *idx, const float *w, const float *x,
                         float *out, float *partial, float *group_sum, const int32_t *chunk_row, int R, int C, int E,
                         int F, hipStream_t st, hipEvent_t k0 = nullptr, hipEvent_t k1 = nullptr,
-                        const RowFinish *fin = nullptr)
+                        const RowFinish *fin = nullptr, int x_stride = 0)
 {
     dim3 grid((unsigned)ceil_div(s.nchunks, kSpmmWaves), (unsigned)s.slabs), block(kSpmmThreads);
     // gathers in flight per wavefront: bounded by the registers they land in
@@ -518,11 +520,12 @@ static void launch_spmm(const SpmmShape &s, const int32_t *off, const int32_t *i
         return !e ? 0 : (e[0] == 'l' ? 1 : (e[0] == 'r' ? 2 : 0));
     }();
     const bool lds = stage_env ? stage_env == 1 : F >= kLdsStageMinWidth;
-    const bool narrow = (uint64_t)C * (uint64_t)F * 4u < ((uint64_t)1 << 32);
+    const bool narrow = (uint64_t)C * (uint64_t)(x_stride ? x_stride : F) * 4u < ((uint64_t)1 << 32);
     // the fused row finish exists for 32-bit offsets only; wide shapes finish in a pass of their own
     const bool fused = fin && narrow;
-    const RowFinish none{1.f, 0.f, nullptr, 0};
-    const RowFinish f = fused ? *fin : none;
+    const RowFinish none{1.f, 0.f, nullptr, 0, 0};
+    RowFinish f = fused ? *fin : none;
+    f.x_stride = x_stride;
 #define JG_GO(W, L, P)                                                                                              \
     hipLaunchKernelGGL((spmm_merge<VEC, NT, U, W, L, P>), grid, block, 0, st, off, idx, w, x, out, partial,         \
                        chunk_row, R, C, E, F, s.chunk, s.nchunks, f)
@@ -573,7 +576,8 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_workspa
 
 static int32_t spmm_call(const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out,
                          int32_t R, int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, void *stream,
-                         hipEvent_t k0, hipEvent_t k1, const RowFinish *fin = nullptr, bool narrow_slabs = false)
+                         hipEvent_t k0, hipEvent_t k1, const RowFinish *fin = nullptr, bool narrow_slabs = false,
+                         int x_stride = 0)
 {
     if (int32_t rc = check_spmm_sizes(R, E, F)) return rc;
     if (C < 0) return fail(JGAMD_ERR_SIZE, "spmm_csx: negative C");
@@ -611,7 +615,7 @@ static int32_t spmm_call(const int32_t *off, const int32_t *idx, const float *w,
                        s.chunk, s.nchunks, chunk_row);
 #define JG_CASE(V, N)                                                                                \
     if (s.vec == V && s.nt == N) {                                                                   \
-        launch_spmm<V, N>(s, off, idx, w, x, out, partial, group_sum, chunk_row, R, C, (int)E, F, st, k0, k1, fin); \
+        launch_spmm<V, N>(s, off, idx, w, x, out, partial, group_sum, chunk_row, R, C, (int)E, F, st, k0, k1, fin, x_stride); \
         return launch_status("spmm_csx");                                                            \
     }
 #define JG_CASES(V) JG_CASE(V, 1) JG_CASE(V, 2) JG_CASE(V, 3) JG_CASE(V, 4) JG_CASE(V, 5) JG_CASE(V, 6) JG_CASE(V, 8)
@@ -639,7 +643,7 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_axpby(
     if (h && (((uintptr_t)h & 3) != 0)) return fail(JGAMD_ERR_ALIGN, "spmm_csx_axpby: h not 4-byte aligned");
     if (h && h_rows != 1 && h_rows != R)
         return fail(JGAMD_ERR_SIZE, "spmm_csx_axpby: h has %d rows, expected %d or 1", h_rows, R);
-    const RowFinish fin{beta, alpha, alpha != 0.f ? h : nullptr, h_rows == 1 ? 0 : F};
+    const RowFinish fin{beta, alpha, alpha != 0.f ? h : nullptr, h_rows == 1 ? 0 : F, 0};
     return spmm_call(off, idx, w, x, out, R, C, E, F, ws, ws_bytes, stream, nullptr, nullptr, &fin);
 }
 
@@ -651,9 +655,9 @@ int32_t spmm_enqueue(const int32_t *off, const int32_t *idx, const float *w, con
 }
 int32_t spmm_enqueue_slabs(const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out,
                            int32_t R, int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, hipStream_t s,
-                           hipEvent_t k0, hipEvent_t k1)
+                           hipEvent_t k0, hipEvent_t k1, int x_stride)
 {
-    return spmm_call(off, idx, w, x, out, R, C, E, F, ws, ws_bytes, s, k0, k1, nullptr, true);
+    return spmm_call(off, idx, w, x, out, R, C, E, F, ws, ws_bytes, s, k0, k1, nullptr, true, x_stride);
 }
 }  // namespace jg
 

@@ -143,6 +143,23 @@ __global__ __launch_bounds__(256) void blocked_sum4(const f32x4 *__restrict__ pa
     out[i] = s;
 }
 
+// xp[r * fpad + f] = x[r * F + f]: rows moved apart so that each starts on a 128-byte line
+__global__ __launch_bounds__(256) void blocked_pad_rows(const float *__restrict__ x, int64_t rows, int F, int fpad,
+                                                        float *__restrict__ xp)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= rows * fpad) return;
+    const int64_t r = i / fpad;
+    const int f = (int)(i - r * fpad);
+    if (f < F) xp[i] = x[r * F + f];
+}
+
+// Row width the gathers run at.  Wide rows: a multiple of 32 floats, so that every 256-byte slab of
+// a row is two whole lines (a 2408-byte row's slabs straddle three: F = 602 ran 25.4 -> 20.4 ms).
+// Rows of one slab: a multiple of 16 floats, which already fixes the number of lines a row touches
+// and keeps the block's footprint in L2 smaller than whole-line rows would.
+static int padded_width(int F) { return F <= kWave ? (F + 15) & ~15 : (F + 31) & ~31; }
+
 static int env_kb(const char *name, int dflt)
 {
     const char *s = getenv(name);
@@ -228,15 +245,17 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_csx_block_column
     return launch_status("csx_block_columns");
 }
 
-extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_blocked_workspace(int32_t R, int64_t E,
-                                                                                           int32_t F, int32_t nb,
-                                                                                           size_t *bytes)
+extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_blocked_workspace(int32_t R, int32_t C,
+                                                                                           int64_t E, int32_t F,
+                                                                                           int32_t nb, size_t *bytes)
 {
     if (!bytes) return fail(JGAMD_ERR_NULL, "spmm_csx_blocked_workspace: NULL result");
-    if (R < 0 || E < 0 || F < 0) return fail(JGAMD_ERR_SIZE, "spmm_csx_blocked_workspace: negative size");
+    if (R < 0 || C < 0 || E < 0 || F < 0) return fail(JGAMD_ERR_SIZE, "spmm_csx_blocked_workspace: negative size");
     if (!blocked_sizes_ok(R, E, nb)) return fail(JGAMD_ERR_SIZE, "spmm_csx_blocked_workspace: nb = %d, R = %d", nb, R);
-    *bytes = (R == 0 || F == 0) ? 0
-                                : carve_bytes((size_t)nb * (size_t)R * (size_t)F, 4) + spmm_ws_bytes(nb * R, E, F);
+    const size_t padded = padded_width(F) != F ? carve_bytes((size_t)C * (size_t)padded_width(F), 4) : 0;
+    *bytes = (R == 0 || F == 0)
+                 ? 0
+                 : carve_bytes((size_t)nb * (size_t)R * (size_t)F, 4) + padded + spmm_ws_bytes(nb * R, E, F);
     return 0;
 }
 
@@ -245,8 +264,7 @@ static int32_t blocked_call(const int32_t *b_off, const int32_t *b_idx, const fl
                             int32_t F, int32_t nb, void *ws, size_t ws_bytes, void *stream, hipEvent_t k0, hipEvent_t k1)
 {
     size_t need = 0;
-    if (int32_t rc = jgamd_spmm_csx_blocked_workspace(R, E, F, nb, &need)) return rc;
-    if (C < 0) return fail(JGAMD_ERR_SIZE, "spmm_csx_blocked: negative C");
+    if (int32_t rc = jgamd_spmm_csx_blocked_workspace(R, C, E, F, nb, &need)) return rc;
     if (R == 0 || F == 0) return 0;
     if (!b_off || !out) return fail(JGAMD_ERR_NULL, "spmm_csx_blocked: b_off / out is NULL");
     if (h && h_rows != 1 && h_rows != R)
@@ -258,8 +276,18 @@ static int32_t blocked_call(const int32_t *b_off, const int32_t *b_idx, const fl
     hipStream_t s = static_cast<hipStream_t>(stream);
     Carver carve(ws);
     float *partial = carve.take<float>((size_t)nb * (size_t)R * (size_t)F);
+    const int fpad = padded_width(F);
+    const float *gathered = x;
+    if (fpad != F && C > 0 && E > 0) {
+        float *xp = carve.take<float>((size_t)C * (size_t)fpad);
+        const int64_t n = (int64_t)C * fpad;
+        hipLaunchKernelGGL(blocked_pad_rows, dim3((unsigned)ceil_div(n, (int64_t)256)), dim3(256), 0, s, x, (int64_t)C, F, fpad,
+                           xp);
+        gathered = xp;
+    }
     void *inner = static_cast<char *>(ws) + carve.used;
-    if (int32_t rc = spmm_enqueue_slabs(b_off, b_idx, b_w, x, partial, nb * R, C, E, F, inner, ws_bytes - carve.used, s, k0, k1))
+    if (int32_t rc = spmm_enqueue_slabs(b_off, b_idx, b_w, gathered, partial, nb * R, C, E, F, inner,
+                                        ws_bytes - carve.used, s, k0, k1, gathered == x ? 0 : fpad))
         return rc;
     const float *hh = alpha != 0.f ? h : nullptr;
     const int h_stride = h_rows == 1 ? 0 : 1;

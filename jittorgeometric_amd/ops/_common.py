@@ -161,7 +161,7 @@ def _product(off, idx, w, x, R, beta, alpha, h):
         _lib.check(lib.jgamd_spmm_block_plan(R, C, E, F, _c.byref(nb), _c.byref(cols)))
     if nb.value > 0:
         b_off, b_idx, b_w = _blocked_arrays(off, idx, w, R, E, nb.value, cols.value)
-        nbytes = _lib.query(lib.jgamd_spmm_csx_blocked_workspace, R, E, F, nb.value)
+        nbytes = _lib.query(lib.jgamd_spmm_csx_blocked_workspace, R, C, E, F, nb.value)
         ws = _lib.workspace(nbytes, dev)
         _lib.check(lib.jgamd_spmm_csx_blocked(_lib.ptr(b_off), _lib.ptr(b_idx), _lib.ptr(b_w), _lib.ptr(x), _lib.ptr(out),
                                               float(beta), float(alpha), _lib.ptr(h), h_rows, R, C, E, F, nb.value,

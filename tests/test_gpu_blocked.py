@@ -38,7 +38,7 @@ def blocked_product(b_off, b_idx, b_w, x, R, E, nb, beta=1.0, alpha=0.0, h=None)
     L, l = lib()
     C, F = x.shape
     out = torch.empty((R, F), dtype=torch.float32, device=dev())
-    nbytes = L.query(l.jgamd_spmm_csx_blocked_workspace, R, E, F, nb)
+    nbytes = L.query(l.jgamd_spmm_csx_blocked_workspace, R, C, E, F, nb)
     ws = L.workspace(nbytes, dev())
     h_rows = R if h is None or h.dim() == 2 else 1
     L.check(l.jgamd_spmm_csx_blocked(L.ptr(b_off), L.ptr(b_idx), L.ptr(b_w), L.ptr(x), L.ptr(out), beta, alpha,
@@ -144,4 +144,4 @@ def test_blocked_entry_points_reject_bad_sizes():
     with pytest.raises(JgamdError):
         L.query(l.jgamd_csx_block_columns_workspace, 10, 65)
     with pytest.raises(JgamdError):
-        L.query(l.jgamd_spmm_csx_blocked_workspace, 1 << 26, 10, 4, 64)    # nb * R above 2^31
+        L.query(l.jgamd_spmm_csx_blocked_workspace, 1 << 26, 1 << 26, 10, 4, 64)    # nb * R above 2^31
