@@ -518,10 +518,14 @@ def config5(b):
         torch.nn.functional.cross_entropy(hcur, y).backward()
 
     main_only = args.part == "main"
-    gcn_ms = sage_ms = 0.0
+    gcn_ms = sage_ms = gcn_af_ms = 0.0
     if not main_only:
         gcn = [GCNConv(dims[i], dims[i + 1], spmm=False).to(dev) for i in range(3)]
         gcn_ms = b.timed(lambda: model_step(gcn, lambda l, t: l(t, csc, csr)), args.steps, args.warmup)
+        # the same model with each layer's two products in the cheaper order (an option of this build's GCNConv)
+        gcn_af = [GCNConv(dims[i], dims[i + 1], spmm=False, aggregate_first=dims[i] < dims[i + 1]).to(dev) for i in range(3)]
+        gcn_af_ms = b.timed(lambda: model_step(gcn_af, lambda l, t: l(t, csc, csr)), args.steps, args.warmup)
+        del gcn_af
         from jittorgeometric_amd.nn import sage_norm
         sei, sw = sage_norm(ei[:, :E - V].contiguous(), None, V)       # same edges, mean weights
         sei = sei.contiguous()
@@ -545,6 +549,7 @@ def config5(b):
                      "config 5: 3-layer GCN full-graph forward+backward, V=2,449,029 power-law (exp 2.1, mean 50) "
                      "+ self-loops, 100->256->256->47", {"V": V, "E": E})
     line.update({"sage3_fullgraph_fwd_bwd_ms": round(sage_ms, 3),
+                 "gcn3_aggregate_first_where_narrower_ms": round(gcn_af_ms, 3),
                  "coo_to_csr_ms": round(conv_csr_ms, 4), "coo_to_csr_edges_per_s": round(E / (conv_csr_ms * 1e-3)),
                  "coo_to_csc_edges_per_s": round(E / (conv_csc_ms * 1e-3))})
     for F in widths:

@@ -64,26 +64,30 @@ def xt_g(x, g):
 
 class _XW(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, weight):
+    def forward(ctx, x, weight, bias):
         ctx.save_for_backward(x, weight)
-        return rows_times(x, weight)
+        return rows_times(x, weight, bias=bias)
 
     @staticmethod
     def backward(ctx, g):
         x, weight = ctx.saved_tensors
-        gx = gw = None
+        gx = gw = gb = None
+        g = g.contiguous()
         if ctx.needs_input_grad[0]:
-            gx = rows_times(g.contiguous(), weight.t().contiguous())
+            gx = rows_times(g, weight.t().contiguous())
         if ctx.needs_input_grad[1]:
             gw = xt_g(x, g)
-        return gx, gw
+        if ctx.needs_input_grad[2]:
+            gb = column_sum(g) if g.dtype == torch.float32 and g.dim() == 2 else g.sum(0)
+        return gx, gw, gb
 
 
-def xw(x, weight):
-    """x @ weight with a split weight gradient; x [V,Fin], weight [Fin,Fout]."""
+def xw(x, weight, bias=None):
+    """x @ weight (+ bias) with a split weight gradient; x [V,Fin], weight [Fin,Fout]."""
     if x.dim() != 2 or not x.is_contiguous():
-        return x @ weight
-    return _XW.apply(x, weight)
+        out = x @ weight
+        return out if bias is None else out + bias
+    return _XW.apply(x, weight, bias)
 
 
 def column_sum(x):

@@ -241,3 +241,40 @@ def test_layers_honour_the_reference_grad_switch():
                          what="REFERENCE_GRAD=%s" % flag)
     finally:
         spmmcsr.REFERENCE_GRAD = False
+
+
+@pytest.mark.parametrize("spmm", [False, True])
+def test_gcn_aggregate_first_is_the_same_layer(spmm):
+    """(A x) W + b against A (x W) + b, the reference's order (gcn_conv.py:95-101): same
+    output and gradients up to rounding, checked against a float64 dense model."""
+    from jittorgeometric_amd.nn import GCNConv, gcn_norm
+    from jittorgeometric_amd.ops import cootocsc, cootocsr
+    from jittorgeometric_amd import synthetic
+    V = 5000
+    ei = synthetic.chung_lu(V, 70000, 2.1, max_degree=900, seed=12)
+    eit, wt = gcn_norm(to_gpu(ei), None, V)
+    csc, csr = cootocsc(eit.contiguous(), wt, V), cootocsr(eit.contiguous(), wt, V)
+    oei, ow = oracle.gcn_norm(ei, None, V)
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((V, 100)).astype(np.float32)
+    g = rng.standard_normal((V, 256)).astype(np.float32)
+    torch.manual_seed(2)
+    ref_layer = GCNConv(100, 256, spmm=spmm).to(dev())
+    with torch.no_grad():
+        ref_layer.bias.normal_(0, 0.2)
+    layer = GCNConv(100, 256, spmm=spmm, aggregate_first=True).to(dev())
+    layer.load_state_dict(ref_layer.state_dict())
+    A = dense_adj(oei, ow, V)
+    x64 = torch.from_numpy(x.astype(np.float64)).requires_grad_(True)
+    W = layer.weight.detach().cpu().double().requires_grad_(True)
+    b = layer.bias.detach().cpu().double().requires_grad_(True)
+    (A @ (x64 @ W) + b).backward(torch.from_numpy(g.astype(np.float64)))
+    want_out = (A @ (x64 @ W) + b).detach().numpy()
+    for lay in (ref_layer, layer):
+        xt = to_gpu(x).requires_grad_(True)
+        out = lay(xt, csc, csr)
+        out.backward(to_gpu(g))
+        assert_close(out.detach().cpu().numpy(), want_out, rtol=1e-4, atol=1e-5, what="out")
+        for got, want, name in ((xt.grad, x64.grad, "x"), (lay.weight.grad, W.grad, "W"), (lay.bias.grad, b.grad, "b")):
+            want = want.numpy()
+            assert_close(got.cpu().numpy(), want, np.abs(want) + np.abs(want).mean(), rtol=1e-4, what="grad " + name)
