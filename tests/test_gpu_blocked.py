@@ -145,3 +145,27 @@ def test_blocked_entry_points_reject_bad_sizes():
         L.query(l.jgamd_csx_block_columns_workspace, 10, 65)
     with pytest.raises(JgamdError):
         L.query(l.jgamd_spmm_csx_blocked_workspace, 1 << 26, 1 << 26, 10, 4, 64)    # nb * R above 2^31
+
+
+def test_blocked_product_without_weights_and_with_columns_out_of_range():
+    """w = NULL means weight 1 (ScatterToVertex-style sums); an index outside [0, C) contributes
+    nothing, as in the unblocked kernels, whichever block it was filed under."""
+    rng = np.random.default_rng(23)
+    V, E, nb, cols, F = 800, 50000, 7, 120, 44
+    ei, w = rand_graph(rng, V, E, 1)
+    idx, off, wt = oracle.cootocsc(ei, w, V)
+    bad = idx.copy()
+    where = rng.choice(E, 300, replace=False)
+    bad[where[:150]] = V + 5
+    bad[where[150:]] = -3
+    keep = np.ones(E, bool)
+    keep[where] = False
+    x = rng.standard_normal((V, F)).astype(np.float32)
+    ones = np.ones(E, np.float32)
+    # exact row sums: the hub row has 15,000 same-weight terms, where the oracle's sequential fp32
+    # loop has itself drifted past 1e-5 of the sum of absolute terms
+    want, terms = oracle.aggregate_f64(x, idx, off, np.where(keep, ones, 0).astype(np.float32))
+    b_off, b_idx, b_w = block_columns(to_gpu(off), to_gpu(bad), None, V, nb, cols)
+    assert b_w is None
+    got = blocked_product(b_off, b_idx, None, to_gpu(x), V, E, nb).cpu().numpy()
+    assert_close(got, want, terms, what="unweighted blocked product with dropped indices")
