@@ -10,41 +10,55 @@
 namespace jg {
 
 constexpr int kColThreads = 256;
-constexpr int kColStripe = 2048;   // rows per block
+constexpr int kColStripe = 512;    // rows per block: about 2000 blocks at V = 10^6, eight per CU, to keep enough loads in flight
 
+// W = floats per lane (1, or 4 when F % 4 == 0 and x is 16-byte aligned): a row is then F / W
+// lanes wide and every load moves 16 bytes.
+template <int W>
 __global__ __launch_bounds__(kColThreads) void column_partial_sums(const float *__restrict__ x, int64_t R, int F,
                                                                    float *__restrict__ partial)
 {
-    __shared__ float red[kColThreads];
-    const int cols = F < kColThreads ? F : kColThreads;     // columns handled per slab
+    typedef float vec __attribute__((ext_vector_type(W)));
+    __shared__ float red[kColThreads][W];
+    const int FW = F / W;                                   // lanes per row
+    const int cols = FW < kColThreads ? FW : kColThreads;   // lanes of one row handled per slab
     const int groups = kColThreads / cols;                  // rows read together
     const int c = threadIdx.x % cols, g = threadIdx.x / cols;
     const int64_t r0 = (int64_t)blockIdx.x * kColStripe;
     const int64_t r1 = r0 + kColStripe < R ? r0 + kColStripe : R;
-    for (int slab = 0; slab < F; slab += cols) {
+    for (int slab = 0; slab < FW; slab += cols) {
         const int col = slab + c;
-        float s = 0.f;
-        if (g < groups && col < F) {
+        float s[W];
+#pragma unroll
+        for (int k = 0; k < W; k++) s[k] = 0.f;
+        if (g < groups && col < FW) {
             constexpr int kB = 8;                            // loads in flight per thread
             for (int64_t rb = r0 + g; rb < r1; rb += (int64_t)kB * groups) {
-                float v[kB];
+                vec v[kB];
 #pragma unroll
                 for (int i = 0; i < kB; i++) {
                     const int64_t r = rb + (int64_t)i * groups;
-                    v[i] = x[(r < r1 ? r : r1 - 1) * F + col];
+                    v[i] = __builtin_nontemporal_load(reinterpret_cast<const vec *>(x + (r < r1 ? r : r1 - 1) * F) + col);
                 }
 #pragma unroll
                 for (int i = 0; i < kB; i++)
-                    if (rb + (int64_t)i * groups < r1) s += v[i];
+                    if (rb + (int64_t)i * groups < r1) {
+#pragma unroll
+                        for (int k = 0; k < W; k++) s[k] += v[i][k];
+                    }
             }
         }
         __syncthreads();
-        red[threadIdx.x] = s;
+#pragma unroll
+        for (int k = 0; k < W; k++) red[threadIdx.x][k] = s[k];
         __syncthreads();
-        if (g == 0 && col < F) {
-            float t = 0.f;
-            for (int k = 0; k < groups; k++) t += red[k * cols + c];
-            partial[(size_t)blockIdx.x * F + col] = t;
+        if (g == 0 && col < FW) {
+#pragma unroll
+            for (int k = 0; k < W; k++) {
+                float t = 0.f;
+                for (int q = 0; q < groups; q++) t += red[q * cols + c][k];
+                partial[(size_t)blockIdx.x * F + (size_t)col * W + k] = t;
+            }
         }
     }
 }
@@ -95,8 +109,12 @@ JG_EXPORT int32_t jgamd_column_sum(const float *x, float *out, int64_t R, int32_
     hipStream_t st = static_cast<hipStream_t>(stream);
     float *partial = static_cast<float *>(ws);
     const int nblocks = (int)ceil_div(R > 0 ? R : 1, kColStripe);
-    if (R > 0)
-        hipLaunchKernelGGL(column_partial_sums, dim3((unsigned)nblocks), dim3(kColThreads), 0, st, x, R, F, partial);
+    if (R > 0) {
+        if (F % 4 == 0 && ((uintptr_t)x & 15) == 0)
+            hipLaunchKernelGGL((column_partial_sums<4>), dim3((unsigned)nblocks), dim3(kColThreads), 0, st, x, R, F, partial);
+        else
+            hipLaunchKernelGGL((column_partial_sums<1>), dim3((unsigned)nblocks), dim3(kColThreads), 0, st, x, R, F, partial);
+    }
     hipLaunchKernelGGL(column_final_sums, dim3((unsigned)ceil_div(F, 64)), dim3(1024), 0, st, partial, R > 0 ? nblocks : 0,
                        F, out);
     return launch_status("column_sum");
