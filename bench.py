@@ -518,7 +518,7 @@ def config5(b):
         torch.nn.functional.cross_entropy(hcur, y).backward()
 
     main_only = args.part == "main"
-    gcn_ms = sage_ms = gcn_af_ms = 0.0
+    gcn_ms = sage_ms = gcn_af_ms = sage_tf_ms = 0.0
     if not main_only:
         gcn = [GCNConv(dims[i], dims[i + 1], spmm=False).to(dev) for i in range(3)]
         gcn_ms = b.timed(lambda: model_step(gcn, lambda l, t: l(t, csc, csr)), args.steps, args.warmup)
@@ -532,7 +532,10 @@ def config5(b):
         scsc, scsr = cootocsc(sei, sw, V), cootocsr(sei, sw, V)
         sage = [SAGEConv(dims[i], dims[i + 1], root_weight=False, spmm=False).to(dev) for i in range(3)]
         sage_ms = b.timed(lambda: model_step(sage, lambda l, t: l(t, None, None, scsc, scsr)), args.steps, args.warmup)
-        del sei, sw, scsc, scsr, sage, gcn
+        sage_tf = [SAGEConv(dims[i], dims[i + 1], root_weight=False, spmm=False,
+                            transform_first=dims[i + 1] < dims[i]).to(dev) for i in range(3)]
+        sage_tf_ms = b.timed(lambda: model_step(sage_tf, lambda l, t: l(t, None, None, scsc, scsr)), args.steps, args.warmup)
+        del sei, sw, scsc, scsr, sage, gcn, sage_tf
     widths = (256,) if main_only else (100, 256, 47)
     prod = {}
     for F in widths:
@@ -550,6 +553,7 @@ def config5(b):
                      "+ self-loops, 100->256->256->47", {"V": V, "E": E})
     line.update({"sage3_fullgraph_fwd_bwd_ms": round(sage_ms, 3),
                  "gcn3_aggregate_first_where_narrower_ms": round(gcn_af_ms, 3),
+                 "sage3_transform_first_where_narrower_ms": round(sage_tf_ms, 3),
                  "coo_to_csr_ms": round(conv_csr_ms, 4), "coo_to_csr_edges_per_s": round(E / (conv_csr_ms * 1e-3)),
                  "coo_to_csc_edges_per_s": round(E / (conv_csc_ms * 1e-3))})
     for F in widths:

@@ -278,3 +278,52 @@ def test_gcn_aggregate_first_is_the_same_layer(spmm):
         for got, want, name in ((xt.grad, x64.grad, "x"), (lay.weight.grad, W.grad, "W"), (lay.bias.grad, b.grad, "b")):
             want = want.numpy()
             assert_close(got.cpu().numpy(), want, np.abs(want) + np.abs(want).mean(), rtol=1e-4, what="grad " + name)
+
+
+@pytest.mark.parametrize("root,bias", [(True, True), (False, True), (False, False), (True, False)])
+def test_sage_transform_first_is_the_same_layer(root, bias):
+    """A (x W1) + x W_root + b against the reference's (A x) W1 + x W_root + b
+    (sage_conv.py:172-190): same output and gradients up to rounding, both against a float64
+    dense model; the weights are not symmetric, so this also checks the transposed product."""
+    from jittorgeometric_amd.nn import SAGEConv, sage_norm
+    from jittorgeometric_amd.ops import cootocsc, cootocsr
+    from jittorgeometric_amd import synthetic
+    V = 5000
+    ei = synthetic.chung_lu(V, 70000, 2.1, max_degree=900, seed=13)
+    eit, wt = sage_norm(to_gpu(ei), None, V)
+    csc, csr = cootocsc(eit.contiguous(), wt, V), cootocsr(eit.contiguous(), wt, V)
+    oei, ow = oracle.sage_norm(ei, None, V)
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((V, 256)).astype(np.float32)
+    g = rng.standard_normal((V, 48)).astype(np.float32)
+    torch.manual_seed(3)
+    ref_layer = SAGEConv(256, 48, root_weight=root, bias=bias, spmm=False).to(dev())
+    if bias:
+        with torch.no_grad():
+            ref_layer.bias.normal_(0, 0.2)
+    layer = SAGEConv(256, 48, root_weight=root, bias=bias, spmm=False, transform_first=True).to(dev())
+    layer.load_state_dict(ref_layer.state_dict())
+    A = dense_adj(oei, ow, V)
+    x64 = torch.from_numpy(x.astype(np.float64)).requires_grad_(True)
+    W1 = layer.weight1.detach().cpu().double().requires_grad_(True)
+    Wr = layer.root_weight.detach().cpu().double().requires_grad_(True) if root else None
+    b = layer.bias.detach().cpu().double().requires_grad_(True) if bias else None
+    ref = (A @ x64) @ W1
+    if root:
+        ref = ref + x64 @ Wr
+    if bias:
+        ref = ref + b
+    ref.backward(torch.from_numpy(g.astype(np.float64)))
+    for lay in (ref_layer, layer):
+        xt = to_gpu(x).requires_grad_(True)
+        out = lay(xt, csc=csc, csr=csr)
+        out.backward(to_gpu(g))
+        assert_close(out.detach().cpu().numpy(), ref.detach().numpy(), rtol=1e-4, atol=1e-5, what="out")
+        pairs = [(xt.grad, x64.grad, "x"), (lay.weight1.grad, W1.grad, "W1")]
+        if root:
+            pairs.append((lay.root_weight.grad, Wr.grad, "W_root"))
+        if bias:
+            pairs.append((lay.bias.grad, b.grad, "b"))
+        for got, want, name in pairs:
+            want = want.numpy()
+            assert_close(got.cpu().numpy(), want, np.abs(want) + np.abs(want).mean(), rtol=1e-4, what="grad " + name)
