@@ -199,6 +199,7 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_block_plan(
     // worth it when x does not fit anyway, the partial rows are a small share of the gathers
     // (8 entries or more per blocked row on average) and a lane per block suffices
     if (blocks < 3 || blocks > kMaxBlocks) return 0;
+    if ((int64_t)C * F * 4 <= ((int64_t)8 << 20)) return 0;      // narrow rows: all of x is about an L2's worth
     if (E < 8 * blocks * (int64_t)R) return 0;
     if (!blocked_sizes_ok(R, E, (int32_t)blocks)) return 0;
     *nb = (int32_t)blocks;

@@ -136,6 +136,7 @@ def test_plan_takes_long_rows_only():
     assert plan(2_449_029, 2_449_029, 126_000_000, 100)[0] == 0       # too many blocks
     assert plan(232_965, 232_965, 114_848_857, 8)[0] == 0             # narrow rows take the tile kernels
     assert plan(1000, 1000, 500_000, 64)[0] == 0                      # x fits anyway
+    assert plan(100_000, 100_000, 20_000_000, 16)[0] == 0             # 6.4 MB of narrow rows
 
 
 def test_blocked_entry_points_reject_bad_sizes():
