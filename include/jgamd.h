@@ -312,6 +312,27 @@ int32_t jgamd_column_sum(const float *x, float *out, int64_t R, int32_t F, void 
                          size_t ws_bytes, void *stream);
 
 /* ------------------------------------------------------------------------
+ * Mean cross-entropy of row-major logits [V,C] against integer labels, the
+ * loss of the full-graph training step (nn.cross_entropy_loss(pred, label),
+ * examples/gcn_example.py:113; nn.log_softmax + nn.nll_loss,
+ * examples/sage_example.py:69,83 — both live in the jittor package):
+ *   lse[i] = log sum_c exp(logits[i,c])           (max-subtracted)
+ *   loss   = mean over rows with 0 <= label < C of (lse[i] - logits[i,label[i]])
+ * Rows whose label lies outside [0,C) are left out of the mean and get a zero
+ * gradient.  labels: int32, or int64 when labels_are_i64 != 0.  loss[1],
+ * count[1] (rows counted) and lse[V] are written by fwd and read by bwd:
+ *   grad_logits[i,c] = grad_loss[0] / count * (exp(logits[i,c] - lse[i]) - [c == label[i]])
+ * (grad_loss NULL = 1).  Two fixed-order reduction stages, no atomics.
+ */
+int32_t jgamd_cross_entropy_workspace(int64_t V, int32_t C, size_t *bytes);
+int32_t jgamd_cross_entropy_fwd(const float *logits, const void *labels, int32_t labels_are_i64,
+                                int64_t V, int32_t C, float *loss, int32_t *count, float *lse,
+                                void *ws, size_t ws_bytes, void *stream);
+int32_t jgamd_cross_entropy_bwd(const float *logits, const void *labels, int32_t labels_are_i64,
+                                const float *lse, const int32_t *count, const float *grad_loss,
+                                int64_t V, int32_t C, float *grad_logits, void *stream);
+
+/* ------------------------------------------------------------------------
  * Neighbour sampling for one layer of a sampled subgraph: for destination
  * dst[i] (a column of the global CSC arrays g_off / g_idx with g_nodes
  * columns) write its neighbours to out[layer_off[i] .. layer_off[i+1]): all of

@@ -1,0 +1,236 @@
+// Mean cross-entropy of row-major logits [V,C] against integer labels, and its gradient: the
+// loss at the end of the full-graph training step (nn.cross_entropy_loss(pred, label) in
+// examples/gcn_example.py:113; nn.log_softmax + nn.nll_loss in examples/sage_example.py:69,83).
+//
+//     lse[i]  = max_c x[i,c] + log sum_c exp(x[i,c] - max_c x[i,c])
+//     loss    = mean over the rows with a label in [0,C) of (lse[i] - x[i, label[i]])
+//     grad    = g / count * (exp(x[i,c] - lse[i]) - [c == label[i]])      (0 for the other rows)
+//
+// With millions of rows and a few dozen classes a row is shorter than a wavefront: G lanes
+// (a power of two, about C / 4) share a row, so that consecutive lanes read consecutive floats
+// of consecutive rows, and the row's maximum and sum fold with xor-shuffles inside the group.
+// The mean is reduced in two fixed-order stages (per-block partial sums in double, then one
+// block), so the result does not change from run to run.
+#include <math.h>
+
+#include "common.h"
+
+namespace jg {
+
+constexpr int kCeThreads = 256;
+constexpr int kCeRows = 2048;      // rows per block
+
+__device__ __forceinline__ int64_t label_at(const int32_t *y32, const int64_t *y64, int64_t row)
+{
+    return y64 ? y64[row] : (int64_t)y32[row];
+}
+
+// REG: the row fits four floats per lane (C <= 4 G) and is read once; otherwise it is read twice
+template <int G, bool REG>
+__global__ __launch_bounds__(kCeThreads) void ce_rows(const float *__restrict__ x, const int32_t *__restrict__ y32,
+                                                      const int64_t *__restrict__ y64, int64_t V, int C,
+                                                      float *__restrict__ lse_out, double *__restrict__ block_sum,
+                                                      int32_t *__restrict__ block_cnt)
+{
+    constexpr int RP = kCeThreads / G;      // rows per pass
+    __shared__ double s_sum[RP];
+    __shared__ int s_cnt[RP];
+    const int g = threadIdx.x % G, lr = threadIdx.x / G;
+    const int64_t r0 = (int64_t)blockIdx.x * kCeRows;
+    const int64_t r1 = r0 + kCeRows < V ? r0 + kCeRows : V;
+    double acc = 0.0;
+    int cnt = 0;
+    for (int64_t rb = r0; rb < r1; rb += RP) {
+        const int64_t row = rb + lr;
+        const bool ok = row < r1;
+        const float *p = x + (ok ? row : r1 - 1) * (int64_t)C;
+        float m = -INFINITY, s = 0.f;
+        if (REG) {
+            float v[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int c = g + i * G;
+                v[i] = c < C ? p[c] : -INFINITY;
+                m = fmaxf(m, v[i]);
+            }
+#pragma unroll
+            for (int o = G / 2; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, G));
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (g + i * G < C) s += expf(v[i] - m);
+        } else {
+            for (int c = g; c < C; c += G) m = fmaxf(m, p[c]);
+#pragma unroll
+            for (int o = G / 2; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, G));
+            for (int c = g; c < C; c += G) s += expf(p[c] - m);
+        }
+#pragma unroll
+        for (int o = G / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, G);
+        if (g == 0 && ok) {
+            const float l = m + logf(s);
+            lse_out[row] = l;
+            const int64_t lab = label_at(y32, y64, row);
+            if (lab >= 0 && lab < C) {
+                acc += (double)(l - p[lab]);
+                cnt++;
+            }
+        }
+    }
+    if (g == 0) {
+        s_sum[lr] = acc;
+        s_cnt[lr] = cnt;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double t = 0.0;
+        int n = 0;
+        for (int i = 0; i < RP; i++) {
+            t += s_sum[i];
+            n += s_cnt[i];
+        }
+        block_sum[blockIdx.x] = t;
+        block_cnt[blockIdx.x] = n;
+    }
+}
+
+// loss[0] = sum / count (0 / 0 = NaN when no row has a label in range), count[0] = rows counted
+__global__ __launch_bounds__(kCeThreads) void ce_final(const double *__restrict__ block_sum,
+                                                       const int32_t *__restrict__ block_cnt, int nblocks,
+                                                       float *__restrict__ loss, int32_t *__restrict__ count)
+{
+    __shared__ double s_sum[kCeThreads];
+    __shared__ long long s_cnt[kCeThreads];
+    double t = 0.0;
+    long long n = 0;
+    for (int b = threadIdx.x; b < nblocks; b += kCeThreads) {
+        t += block_sum[b];
+        n += block_cnt[b];
+    }
+    s_sum[threadIdx.x] = t;
+    s_cnt[threadIdx.x] = n;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double tt = 0.0;
+        long long nn = 0;
+        for (int i = 0; i < kCeThreads; i++) {
+            tt += s_sum[i];
+            nn += s_cnt[i];
+        }
+        loss[0] = (float)(tt / (double)nn);
+        count[0] = (int32_t)(nn > 0x7fffffffLL ? 0x7fffffffLL : nn);
+    }
+}
+
+template <int G>
+__global__ __launch_bounds__(kCeThreads) void ce_grad(const float *__restrict__ x, const int32_t *__restrict__ y32,
+                                                      const int64_t *__restrict__ y64, const float *__restrict__ lse,
+                                                      const int32_t *__restrict__ count,
+                                                      const float *__restrict__ grad_loss, int64_t V, int C,
+                                                      float *__restrict__ grad)
+{
+    constexpr int RP = kCeThreads / G;
+    const int g = threadIdx.x % G, lr = threadIdx.x / G;
+    const int n = count[0];
+    const float scale = (grad_loss ? grad_loss[0] : 1.f) / (float)n;      // n == 0: no row is counted below
+    const int64_t r0 = (int64_t)blockIdx.x * kCeRows;
+    const int64_t r1 = r0 + kCeRows < V ? r0 + kCeRows : V;
+    for (int64_t row = r0 + lr; row < r1; row += RP) {
+        const int64_t lab = label_at(y32, y64, row);
+        const bool counted = lab >= 0 && lab < C;
+        const float l = lse[row];
+        const float *p = x + row * (int64_t)C;
+        float *q = grad + row * (int64_t)C;
+        for (int c = g; c < C; c += G)
+            q[c] = counted ? scale * (expf(p[c] - l) - (c == lab ? 1.f : 0.f)) : 0.f;
+    }
+}
+
+static int lanes_per_row(int C)
+{
+    int g = 8;
+    while (g < kWave && 4 * g < C) g <<= 1;
+    return g;
+}
+
+}  // namespace jg
+
+using namespace jg;
+#define JG_EXPORT extern "C" __attribute__((visibility("default")))
+
+static int ce_blocks(int64_t V) { return (int)ceil_div(V > 0 ? V : 1, kCeRows); }
+static size_t ce_ws(int64_t V) { return carve_bytes((size_t)ce_blocks(V), 8) + carve_bytes((size_t)ce_blocks(V), 4); }
+
+static int32_t ce_check(const char *who, int64_t V, int32_t C)
+{
+    if (V < 0 || C < 0) return fail(JGAMD_ERR_SIZE, "%s: negative size (V=%lld, C=%d)", who, (long long)V, C);
+    if (V > ((int64_t)1 << 40)) return fail(JGAMD_ERR_SIZE, "%s: V=%lld too large", who, (long long)V);
+    return 0;
+}
+
+JG_EXPORT int32_t jgamd_cross_entropy_workspace(int64_t V, int32_t C, size_t *bytes)
+{
+    if (!bytes) return fail(JGAMD_ERR_NULL, "cross_entropy_workspace: bytes is NULL");
+    if (int32_t rc = ce_check("cross_entropy_workspace", V, C)) return rc;
+    *bytes = ce_ws(V);
+    return 0;
+}
+
+JG_EXPORT int32_t jgamd_cross_entropy_fwd(const float *logits, const void *labels, int32_t labels_are_i64, int64_t V,
+                                          int32_t C, float *loss, int32_t *count, float *lse, void *ws,
+                                          size_t ws_bytes, void *stream)
+{
+    if (int32_t rc = ce_check("cross_entropy_fwd", V, C)) return rc;
+    if (!loss || !count) return fail(JGAMD_ERR_NULL, "cross_entropy_fwd: loss / count is NULL");
+    if (V > 0 && (!labels || !lse || (C > 0 && !logits)))
+        return fail(JGAMD_ERR_NULL, "cross_entropy_fwd: logits / labels / lse is NULL");
+    const size_t need = ce_ws(V);
+    if (!ws || ws_bytes < need)
+        return fail(JGAMD_ERR_WORKSPACE, "cross_entropy_fwd: workspace %zu < %zu bytes", ws ? ws_bytes : (size_t)0, need);
+    if (((uintptr_t)ws & 255) != 0) return fail(JGAMD_ERR_ALIGN, "cross_entropy_fwd: workspace not 256-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    Carver carve(ws);
+    const int nblocks = ce_blocks(V);
+    double *block_sum = carve.take<double>((size_t)nblocks);
+    int32_t *block_cnt = carve.take<int32_t>((size_t)nblocks);
+    const int32_t *y32 = labels_are_i64 ? nullptr : static_cast<const int32_t *>(labels);
+    const int64_t *y64 = labels_are_i64 ? static_cast<const int64_t *>(labels) : nullptr;
+    if (V > 0) {
+        const int G = lanes_per_row(C);
+        const bool reg = C <= 4 * G;
+#define JG_CE(GG)                                                                                                    \
+    if (G == GG) {                                                                                                   \
+        if (reg)                                                                                                     \
+            hipLaunchKernelGGL((ce_rows<GG, true>), dim3((unsigned)nblocks), dim3(kCeThreads), 0, st, logits, y32,   \
+                               y64, V, C, lse, block_sum, block_cnt);                                                \
+        else                                                                                                         \
+            hipLaunchKernelGGL((ce_rows<GG, false>), dim3((unsigned)nblocks), dim3(kCeThreads), 0, st, logits, y32,  \
+                               y64, V, C, lse, block_sum, block_cnt);                                                \
+    }
+        JG_CE(8) JG_CE(16) JG_CE(32) JG_CE(64)
+#undef JG_CE
+    }
+    hipLaunchKernelGGL(ce_final, dim3(1), dim3(kCeThreads), 0, st, block_sum, block_cnt, V > 0 ? nblocks : 0, loss, count);
+    return launch_status("cross_entropy_fwd");
+}
+
+JG_EXPORT int32_t jgamd_cross_entropy_bwd(const float *logits, const void *labels, int32_t labels_are_i64,
+                                          const float *lse, const int32_t *count, const float *grad_loss, int64_t V,
+                                          int32_t C, float *grad_logits, void *stream)
+{
+    if (int32_t rc = ce_check("cross_entropy_bwd", V, C)) return rc;
+    if (V == 0 || C == 0) return 0;
+    if (!logits || !labels || !lse || !count || !grad_logits)
+        return fail(JGAMD_ERR_NULL, "cross_entropy_bwd: NULL array");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int32_t *y32 = labels_are_i64 ? nullptr : static_cast<const int32_t *>(labels);
+    const int64_t *y64 = labels_are_i64 ? static_cast<const int64_t *>(labels) : nullptr;
+    const int nblocks = ce_blocks(V);
+    const int G = lanes_per_row(C);
+#define JG_CE(GG)                                                                                                  \
+    if (G == GG)                                                                                                   \
+        hipLaunchKernelGGL((ce_grad<GG>), dim3((unsigned)nblocks), dim3(kCeThreads), 0, st, logits, y32, y64, lse, \
+                           count, grad_loss, V, C, grad_logits);
+    JG_CE(8) JG_CE(16) JG_CE(32) JG_CE(64)
+#undef JG_CE
+    return launch_status("cross_entropy_bwd");
+}

@@ -24,6 +24,10 @@ jittor==1.3.9.14).  Pins of the numpy restatements at the end of this file:
                 clock-seeded curand, so no output of it can be reproduced.  Pinned
                 here: the copy branch exactly, and for the sampled branch the
                 invariants (distinct, subset, count, order) and uniformity
+  cross_entropy_loss  jittor.nn.cross_entropy_loss / log_softmax + nll_loss live in the
+                jittor package (jittor==1.3.9.14, absent here); the textbook formula,
+                pinned by scipy's logsumexp, log(C) on equal logits, shift invariance,
+                rows of the gradient summing to zero, finite differences
 """
 import ctypes
 import os
@@ -464,3 +468,26 @@ def from_nodes(offset, indices, nodes):
     off, idx = np.asarray(offset), np.asarray(indices)
     parts = [idx[off[n]:off[n + 1]] for n in np.asarray(nodes).reshape(-1)]
     return np.concatenate(parts).astype(np.int32) if parts else np.zeros(0, np.int32)
+
+
+def cross_entropy_loss(output, target):
+    """nn.cross_entropy_loss(pred, label) as examples/gcn_example.py:113 calls it (and
+    nn.nll_loss(nn.log_softmax(x, dim=1), label), examples/sage_example.py:69,83): the mean over
+    rows of logsumexp(row) - row[label], in float64.  Rows whose label lies outside
+    [0, classes) are left out.  Returns (loss, d loss / d output)."""
+    x = np.asarray(output, dtype=np.float64)
+    y = np.asarray(target).astype(np.int64).reshape(-1)
+    V, C = x.shape
+    m = x.max(axis=1, keepdims=True) if C else np.zeros((V, 1))
+    e = np.exp(x - m)
+    lse = m[:, 0] + np.log(e.sum(axis=1))
+    ok = (y >= 0) & (y < C)
+    n = int(ok.sum())
+    rows = np.nonzero(ok)[0]
+    loss = (lse[rows] - x[rows, y[rows]]).sum() / n if n else float("nan")
+    grad = np.zeros_like(x)
+    if n:
+        p = e[rows] / e[rows].sum(axis=1, keepdims=True)
+        p[np.arange(rows.size), y[rows]] -= 1.0
+        grad[rows] = p / n
+    return loss, grad

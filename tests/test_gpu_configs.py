@@ -168,7 +168,20 @@ def test_config5_three_layer_gcn_step():
             if not results:
                 _layer_rows_check("gcn", h_out, lin, layer.bias, ocsc, rows, "GCN layer %d rows" % (i + 1))
             h = torch.relu(h_out) if i < 2 else h_out
-        loss = torch.nn.functional.cross_entropy(h, y)
+        if spmm:
+            # the library's loss on these logits against torch's in float64: value and gradient
+            from jittorgeometric_amd.nn import cross_entropy_loss
+            mine = h.detach().clone().requires_grad_(True)
+            cross_entropy_loss(mine, y).backward()
+            ref_in = h.detach().double().requires_grad_(True)
+            ref = torch.nn.functional.cross_entropy(ref_in, y)
+            ref.backward()
+            assert abs(cross_entropy_loss(mine, y).item() - ref.item()) <= 1e-5 * abs(ref.item())
+            assert (mine.grad.double() - ref_in.grad).abs().max().item() <= 1e-5 / V
+            del mine, ref_in, ref
+            loss = torch.nn.functional.cross_entropy(h, y)
+        else:
+            loss = cross_entropy_loss(h, y)              # nn.cross_entropy_loss, examples/gcn_example.py:113
         loss.backward()
         torch.cuda.synchronize()
         grads = [p.grad.clone() for layer in layers for p in layer.parameters()]

@@ -473,3 +473,40 @@ def test_sampleprocessing_invariants_and_uniformity():
     assert np.all(np.abs(hits - expect) < 5 * np.sqrt(expect))
     assert len({tuple(oracle.sampleprocessing(4, np.array([0], np.int32), np.array([0, 4], np.int32), goff1, grow1,
                                               seed=s)) for s in range(300)}) > 150
+
+
+def test_cross_entropy_closed_forms():
+    from scipy.special import logsumexp
+    rng = np.random.default_rng(21)
+    V, C = 37, 11
+    x = (rng.standard_normal((V, C)) * 3).astype(np.float32)
+    y = rng.integers(0, C, V)
+    loss, grad = oracle.cross_entropy_loss(x, y)
+    want = np.mean(logsumexp(x.astype(np.float64), axis=1) - x[np.arange(V), y].astype(np.float64))
+    assert abs(loss - want) < 1e-12
+    # equal logits: log(C); adding a constant per row changes nothing
+    assert abs(oracle.cross_entropy_loss(np.zeros((5, C)), np.arange(5))[0] - np.log(C)) < 1e-12
+    shifted, gshift = oracle.cross_entropy_loss(x.astype(np.float64) + rng.standard_normal((V, 1)) * 50, y)
+    assert abs(shifted - loss) < 1e-9 and np.allclose(gshift, grad, atol=1e-12)
+    # the gradient: rows sum to zero, and it matches central differences
+    assert np.allclose(grad.sum(axis=1), 0, atol=1e-15)
+    x64 = x.astype(np.float64)
+    for (i, c) in ((0, 0), (3, y[3]), (36, 10), (17, 4)):
+        h = 1e-6
+        xp, xm = x64.copy(), x64.copy()
+        xp[i, c] += h
+        xm[i, c] -= h
+        fd = (oracle.cross_entropy_loss(xp, y)[0] - oracle.cross_entropy_loss(xm, y)[0]) / (2 * h)
+        assert abs(fd - grad[i, c]) < 1e-8
+    # labels outside [0, C) are left out of the mean and of the gradient
+    y2 = y.copy()
+    y2[[1, 5]] = (-100, C)
+    loss2, grad2 = oracle.cross_entropy_loss(x, y2)
+    keep = np.ones(V, bool)
+    keep[[1, 5]] = False
+    want2 = np.mean(logsumexp(x64[keep], axis=1) - x64[keep, y[keep]])
+    assert abs(loss2 - want2) < 1e-12 and not grad2[[1, 5]].any()
+    assert np.isnan(oracle.cross_entropy_loss(x, np.full(V, -1))[0])
+    # very large logits stay finite
+    big = np.array([[1e4, -1e4, 0.0]])
+    assert abs(oracle.cross_entropy_loss(big, [1])[0] - 2e4) < 1e-6
