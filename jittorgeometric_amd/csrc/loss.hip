@@ -25,14 +25,17 @@ __device__ __forceinline__ int64_t label_at(const int32_t *y32, const int64_t *y
     return y64 ? y64[row] : (int64_t)y32[row];
 }
 
-// REG: the row fits four floats per lane (C <= 4 G) and is read once; otherwise it is read twice
+// REG: the row fits four floats per lane (C <= 4 G); a group of lanes then takes kCeUnroll rows per
+// pass, all loads first, so that enough bytes are in flight.  Otherwise the row is read twice.
+constexpr int kCeUnroll = 4;
+
 template <int G, bool REG>
 __global__ __launch_bounds__(kCeThreads) void ce_rows(const float *__restrict__ x, const int32_t *__restrict__ y32,
                                                       const int64_t *__restrict__ y64, int64_t V, int C,
                                                       float *__restrict__ lse_out, double *__restrict__ block_sum,
                                                       int32_t *__restrict__ block_cnt)
 {
-    constexpr int RP = kCeThreads / G;      // rows per pass
+    constexpr int RP = kCeThreads / G;      // row groups per pass
     __shared__ double s_sum[RP];
     __shared__ int s_cnt[RP];
     const int g = threadIdx.x % G, lr = threadIdx.x / G;
@@ -40,40 +43,59 @@ __global__ __launch_bounds__(kCeThreads) void ce_rows(const float *__restrict__ 
     const int64_t r1 = r0 + kCeRows < V ? r0 + kCeRows : V;
     double acc = 0.0;
     int cnt = 0;
-    for (int64_t rb = r0; rb < r1; rb += RP) {
-        const int64_t row = rb + lr;
-        const bool ok = row < r1;
-        const float *p = x + (ok ? row : r1 - 1) * (int64_t)C;
-        float m = -INFINITY, s = 0.f;
-        if (REG) {
-            float v[4];
+    auto finish = [&](int64_t row, const float *p, float m, float s) {
+        const float l = m + logf(s);
+        lse_out[row] = l;
+        const int64_t lab = label_at(y32, y64, row);
+        if (lab >= 0 && lab < C) {
+            acc += (double)(l - p[lab]);
+            cnt++;
+        }
+    };
+    if (REG) {
+        for (int64_t rb = r0; rb < r1; rb += RP * kCeUnroll) {
+            float v[kCeUnroll][4];
+            const float *p[kCeUnroll];
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int c = g + i * G;
-                v[i] = c < C ? p[c] : -INFINITY;
-                m = fmaxf(m, v[i]);
+            for (int u = 0; u < kCeUnroll; u++) {
+                const int64_t row = rb + u * RP + lr;
+                p[u] = x + (row < r1 ? row : r1 - 1) * (int64_t)C;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int c = g + i * G;
+                    v[u][i] = p[u][c < C ? c : 0];
+                }
             }
 #pragma unroll
-            for (int o = G / 2; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, G));
+            for (int u = 0; u < kCeUnroll; u++) {
+                float m = -INFINITY, s = 0.f;
 #pragma unroll
-            for (int i = 0; i < 4; i++)
-                if (g + i * G < C) s += expf(v[i] - m);
-        } else {
+                for (int i = 0; i < 4; i++)
+                    if (g + i * G < C) m = fmaxf(m, v[u][i]);
+#pragma unroll
+                for (int o = G / 2; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, G));
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    if (g + i * G < C) s += expf(v[u][i] - m);
+#pragma unroll
+                for (int o = G / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, G);
+                const int64_t row = rb + u * RP + lr;
+                if (g == 0 && row < r1) finish(row, p[u], m, s);
+            }
+        }
+    } else {
+        for (int64_t rb = r0; rb < r1; rb += RP) {
+            const int64_t row = rb + lr;
+            const bool ok = row < r1;
+            const float *p = x + (ok ? row : r1 - 1) * (int64_t)C;
+            float m = -INFINITY, s = 0.f;
             for (int c = g; c < C; c += G) m = fmaxf(m, p[c]);
 #pragma unroll
             for (int o = G / 2; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, G));
             for (int c = g; c < C; c += G) s += expf(p[c] - m);
-        }
 #pragma unroll
-        for (int o = G / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, G);
-        if (g == 0 && ok) {
-            const float l = m + logf(s);
-            lse_out[row] = l;
-            const int64_t lab = label_at(y32, y64, row);
-            if (lab >= 0 && lab < C) {
-                acc += (double)(l - p[lab]);
-                cnt++;
-            }
+            for (int o = G / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, G);
+            if (g == 0 && ok) finish(row, p, m, s);
         }
     }
     if (g == 0) {
@@ -142,6 +164,52 @@ __global__ __launch_bounds__(kCeThreads) void ce_grad(const float *__restrict__ 
         float *q = grad + row * (int64_t)C;
         for (int c = g; c < C; c += G)
             q[c] = counted ? scale * (expf(p[c] - l) - (c == lab ? 1.f : 0.f)) : 0.f;
+    }
+}
+
+// The same gradient with the matrix taken as one run of V * C floats: a lane owns four
+// consecutive floats (one 16-byte load and store) and finds their rows by one division.
+// Needs V * C < 2^31, C >= 4 and 16-byte aligned arrays; the last V * C % 4 floats are
+// done one by one by the first lanes of the grid.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(kCeThreads) void ce_grad_flat(const float *__restrict__ x,
+                                                           const int32_t *__restrict__ y32,
+                                                           const int64_t *__restrict__ y64,
+                                                           const float *__restrict__ lse,
+                                                           const int32_t *__restrict__ count,
+                                                           const float *__restrict__ grad_loss, int V, int C,
+                                                           float *__restrict__ grad)
+{
+    const int n = count[0];
+    const float scale = (grad_loss ? grad_loss[0] : 1.f) / (float)n;
+    const uint32_t total = (uint32_t)V * (uint32_t)C;
+    const uint32_t quads = total / 4;
+    const uint32_t t = blockIdx.x * kCeThreads + threadIdx.x;
+    auto one = [&](float xv, int row, int c, int64_t lab, float l) {
+        return lab >= 0 && lab < C ? scale * (expf(xv - l) - (c == lab ? 1.f : 0.f)) : 0.f;
+    };
+    if (t < quads) {
+        const uint32_t i = t * 4;
+        const f32x4 xv = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(x + i));
+        int row = (int)(i / (uint32_t)C);
+        int c = (int)(i - (uint32_t)row * (uint32_t)C);
+        // C >= 4: the four floats lie in this row and at most the next one
+        const int row2 = row + 1 < V ? row + 1 : row;
+        const int64_t lab_a = label_at(y32, y64, row), lab_b = label_at(y32, y64, row2);
+        const float l_a = lse[row], l_b = lse[row2];
+        f32x4 out;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const bool next = c + j >= C;
+            out[j] = one(xv[j], 0, next ? c + j - C : c + j, next ? lab_b : lab_a, next ? l_b : l_a);
+        }
+        __builtin_nontemporal_store(out, reinterpret_cast<f32x4 *>(grad + i));
+    }
+    if (t < total - quads * 4) {
+        const uint32_t i = quads * 4 + t;
+        const int row = (int)(i / (uint32_t)C), c = (int)(i - (uint32_t)row * (uint32_t)C);
+        grad[i] = one(x[i], 0, c, label_at(y32, y64, row), lse[row]);
     }
 }
 
@@ -224,6 +292,12 @@ JG_EXPORT int32_t jgamd_cross_entropy_bwd(const float *logits, const void *label
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int32_t *y32 = labels_are_i64 ? nullptr : static_cast<const int32_t *>(labels);
     const int64_t *y64 = labels_are_i64 ? static_cast<const int64_t *>(labels) : nullptr;
+    if (C >= 4 && V * (int64_t)C < ((int64_t)1 << 31) && (((uintptr_t)logits | (uintptr_t)grad_logits) & 15) == 0) {
+        const int64_t quads = V * (int64_t)C / 4;
+        hipLaunchKernelGGL(ce_grad_flat, dim3((unsigned)ceil_div(quads > 0 ? quads : 1, kCeThreads)), dim3(kCeThreads), 0,
+                           st, logits, y32, y64, lse, count, grad_loss, (int)V, C, grad_logits);
+        return launch_status("cross_entropy_bwd");
+    }
     const int nblocks = ce_blocks(V);
     const int G = lanes_per_row(C);
 #define JG_CE(GG)                                                                                                  \
