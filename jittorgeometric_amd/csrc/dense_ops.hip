@@ -11,12 +11,13 @@ namespace jg {
 
 constexpr int kColThreads = 256;
 constexpr int kColStripe = 512;    // rows per block: about 2000 blocks at V = 10^6, eight per CU, to keep enough loads in flight
+constexpr int kColMaxBlocks = 2048;     // more rows per block beyond that: the second stage reads one partial row per block
 
 // W = floats per lane (1, or 4 when F % 4 == 0 and x is 16-byte aligned): a row is then F / W
 // lanes wide and every load moves 16 bytes.
 template <int W>
 __global__ __launch_bounds__(kColThreads) void column_partial_sums(const float *__restrict__ x, int64_t R, int F,
-                                                                   float *__restrict__ partial)
+                                                                   int stripe, float *__restrict__ partial)
 {
     typedef float vec __attribute__((ext_vector_type(W)));
     __shared__ float red[kColThreads][W];
@@ -24,8 +25,8 @@ __global__ __launch_bounds__(kColThreads) void column_partial_sums(const float *
     const int cols = FW < kColThreads ? FW : kColThreads;   // lanes of one row handled per slab
     const int groups = kColThreads / cols;                  // rows read together
     const int c = threadIdx.x % cols, g = threadIdx.x / cols;
-    const int64_t r0 = (int64_t)blockIdx.x * kColStripe;
-    const int64_t r1 = r0 + kColStripe < R ? r0 + kColStripe : R;
+    const int64_t r0 = (int64_t)blockIdx.x * stripe;
+    const int64_t r1 = r0 + stripe < R ? r0 + stripe : R;
     for (int slab = 0; slab < FW; slab += cols) {
         const int col = slab + c;
         float s[W];
@@ -86,7 +87,13 @@ __global__ void column_final_sums(const float *__restrict__ partial, int nblocks
 using namespace jg;
 #define JG_EXPORT extern "C" __attribute__((visibility("default")))
 
-static size_t colsum_ws(int64_t R, int32_t F) { return carve_bytes((size_t)ceil_div(R > 0 ? R : 1, kColStripe) * F, 4); }
+static int col_stripe(int64_t R)
+{
+    const int64_t s = ceil_div(R > 0 ? R : 1, kColMaxBlocks);
+    return s > kColStripe ? (int)(s < 0x7fffffff ? s : 0x7fffffff) : kColStripe;
+}
+static int col_blocks(int64_t R) { return (int)ceil_div(R > 0 ? R : 1, col_stripe(R)); }
+static size_t colsum_ws(int64_t R, int32_t F) { return carve_bytes((size_t)col_blocks(R) * F, 4); }
 
 JG_EXPORT int32_t jgamd_column_sum_workspace(int64_t R, int32_t F, size_t *bytes)
 {
@@ -108,12 +115,15 @@ JG_EXPORT int32_t jgamd_column_sum(const float *x, float *out, int64_t R, int32_
     if (((uintptr_t)ws & 255) != 0) return fail(JGAMD_ERR_ALIGN, "column_sum: workspace not 256-byte aligned");
     hipStream_t st = static_cast<hipStream_t>(stream);
     float *partial = static_cast<float *>(ws);
-    const int nblocks = (int)ceil_div(R > 0 ? R : 1, kColStripe);
+    const int nblocks = col_blocks(R);
+    const int stripe = col_stripe(R);
     if (R > 0) {
         if (F % 4 == 0 && ((uintptr_t)x & 15) == 0)
-            hipLaunchKernelGGL((column_partial_sums<4>), dim3((unsigned)nblocks), dim3(kColThreads), 0, st, x, R, F, partial);
+            hipLaunchKernelGGL((column_partial_sums<4>), dim3((unsigned)nblocks), dim3(kColThreads), 0, st, x, R, F, stripe,
+                               partial);
         else
-            hipLaunchKernelGGL((column_partial_sums<1>), dim3((unsigned)nblocks), dim3(kColThreads), 0, st, x, R, F, partial);
+            hipLaunchKernelGGL((column_partial_sums<1>), dim3((unsigned)nblocks), dim3(kColThreads), 0, st, x, R, F, stripe,
+                               partial);
     }
     hipLaunchKernelGGL(column_final_sums, dim3((unsigned)ceil_div(F, 64)), dim3(1024), 0, st, partial, R > 0 ? nblocks : 0,
                        F, out);
