@@ -359,6 +359,18 @@ def config1(b):
         out = l2(torch.relu(l1(x, csc, csr)), csc, csr)
         cross_entropy_loss(out, y).backward()
     ms = b.timed(step, args.steps, args.warmup)
+    # the same step recorded into a HIP graph once and replayed: at this size the eager step is
+    # a few dozen launches of a few microseconds each
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    graph_ms = b.timed(graph.replay, args.steps, args.warmup)
     h = torch.randn(V, 256, device=dev)
     k_ms, _ = b.spmm_kernel_ms(csc.column_offset, csc.row_indices, csc.edge_weight, h, V, 50)
     cpu = None
@@ -381,7 +393,7 @@ def config1(b):
     line = base_line(args, "gcn2_fwd_bwd_ms", round(ms, 4), "ms", ms, False,
                      "config 1: 2-layer GCN forward+backward, V=2708, 10556 directed edges + self-loops, 1433->256->7",
                      {"V": V, "E": E})
-    line.update({"coo_to_csr_ms": round(conv_csr_ms, 4),
+    line.update({"coo_to_csr_ms": round(conv_csr_ms, 4), "gcn2_fwd_bwd_graph_replay_ms": round(graph_ms, 4),
                  "roofline": roofline("spmm_merge_cora_like_f256.txt", {"V": V, "E": E, "F": 256}, "spmm_merge", k_ms,
                                       spmm_bytes(V, E, 256), spmm_compulsory_bytes(V, V, E, 256), "hipEvents in this run"),
                  "note": "launch-bound at this size: 13k entries are one launch of a few microseconds",

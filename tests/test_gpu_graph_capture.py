@@ -61,3 +61,55 @@ def test_two_layer_gcn_and_appnp_replay_as_a_graph():
     ha = (oracle.aggregate_with_weight((np.abs(xh) @ np.abs(W1)).astype(np.float32), abs_csc) + np.abs(b1))
     za = (oracle.aggregate_with_weight((ha @ np.abs(W2)).astype(np.float32), abs_csc) + np.abs(b2)).astype(np.float32)
     assert_close(want.cpu().numpy(), ref, scale=oracle.appnp(za, abs_csc, 4, 0.1), rtol=8e-5)
+
+
+def test_training_step_replays_as_a_graph():
+    """Forward, the library's loss and backward of a 2-layer GCN (the step of
+    examples/gcn_example.py:96-115) recorded once and replayed: loss and every gradient of every
+    replay equal the eager step's, with eager steps and synchronisations in between."""
+    from jittorgeometric_amd.nn import GCNConv, cross_entropy_loss
+    from jittorgeometric_amd.ops import cootocsc, cootocsr
+    rng = np.random.default_rng(6)
+    V, F, C = 2708, 96, 7
+    ei, _ = rand_graph(rng, V, 10556, 1)
+    ei = ei[:, ei[0] != ei[1]]
+    ei, w = oracle.gcn_norm(ei, None, V)
+    csc = cootocsc(to_gpu(ei.astype(np.int32)), to_gpu(w), V)
+    csr = cootocsr(to_gpu(ei.astype(np.int32)), to_gpu(w), V)
+    torch.manual_seed(7)
+    l1, l2 = GCNConv(F, 32, spmm=False).to(dev()), GCNConv(32, C, spmm=False).to(dev())
+    params = list(l1.parameters()) + list(l2.parameters())
+    static_x = torch.randn(V, F, device=dev())
+    static_y = torch.randint(0, C, (V,), device=dev())
+
+    def step(x, y):
+        for p in params:
+            p.grad = None
+        loss = cross_entropy_loss(l2(torch.relu(l1(x, csc, csr)), csc, csr), y)
+        loss.backward()
+        return loss
+
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        for _ in range(3):
+            step(static_x, static_y)
+    torch.cuda.current_stream().wait_stream(s)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_loss = step(static_x, static_y)
+    static_grads = [p.grad for p in params]          # written in place by every replay
+    for trial in range(4):
+        x = torch.randn(V, F, device=dev())
+        y = torch.randint(0, C, (V,), device=dev())
+        want_loss = step(x, y).clone()               # eager work between the replays
+        want = [p.grad.clone() for p in params]
+        torch.cuda.synchronize()
+        static_x.copy_(x)
+        static_y.copy_(y)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_loss, want_loss), "loss of replay %d differs from the eager step" % trial
+        for got, ref, p in zip(static_grads, want, params):
+            assert torch.equal(got, ref), "a gradient of shape %s differs in replay %d" % (tuple(p.shape), trial)
+    assert all(torch.isfinite(g).all() for g in static_grads)
