@@ -719,7 +719,9 @@ static ConvPlan make_plan(int64_t E, int32_t V)
         p.max_sub = 1;
         return p;
     }
-    p.shift = bits > 10 ? bits - 10 : 0;
+    // about 512 buckets (swept 128 .. 2048 on V = 1M / E = 17M and V = 233k / E = 115M: 256 .. 512 is
+    // fastest; fewer buckets make the first level's runs longer and the second level's shorter)
+    p.shift = bits > 9 ? bits - 9 : 0;
     if (p.shift > kMaxBinBits) p.shift = kMaxBinBits;
     p.nbuckets = (int)ceil_div(V > 0 ? V : 1, (int64_t)1 << p.shift);
     p.max_sub = (int)(E / kSubRecords) + p.nbuckets;
