@@ -141,6 +141,24 @@ __device__ __forceinline__ void set_id(Rec4 &r, int32_t id) { r.id = id; }
 __device__ __forceinline__ int32_t get_id(const Rec3 &) { return 0; }
 __device__ __forceinline__ int32_t get_id(const Rec4 &r) { return r.id; }
 
+// bins[b] += unit for every lane with b >= 0, one LDS atomic per run of equal b over consecutive
+// lanes of a row of 16.  Keys that arrive sorted (an edge list ordered by source) put whole
+// wavefronts on one counter, and 64 atomics on one LDS address take 64 turns; a run costs one.
+// The neighbour's value comes from a row shift on the vector ALU (runs are cut at rows of 16
+// lanes, which the shift does not cross), so unsorted keys pay a few ALU instructions, no LDS trip.
+__device__ __forceinline__ void count_runs(uint32_t *bins, int b, uint32_t unit)
+{
+    const int lane = lane_id();
+    const int prev = __builtin_amdgcn_update_dpp(b, b, 0x111 /* row_shr:1 */, 0xf, 0xf, false);
+    const bool start = (lane & 15) == 0 || b != prev;
+    const uint64_t starts = __ballot(start);
+    if (start && b >= 0) {
+        const uint64_t later = lane == kWave - 1 ? 0ull : (starts >> (lane + 1));
+        const int len = later ? __ffsll((unsigned long long)later) : kWave - lane;
+        atomicAdd(&bins[b], (uint32_t)len * unit);
+    }
+}
+
 // ---------------------------------------------------------------- step 1 ---
 // keys: the key row of edge_index.  Items with key outside [0,V) are ignored
 // here and in every later step.  table is [nbins][nblocks] (+1 trailing zero).
@@ -148,7 +166,7 @@ __global__ __launch_bounds__(kPartThreads) void csx_bucket_histogram(const int32
                                                                      int32_t V, int shift, int nbins,
                                                                      int32_t *__restrict__ table, int nblocks)
 {
-    __shared__ int bins[kMaxBins];
+    __shared__ uint32_t bins[kMaxBins];
     for (int b = threadIdx.x; b < nbins; b += kPartThreads) bins[b] = 0;
     __syncthreads();
     const int64_t base = (int64_t)blockIdx.x * kTile;
@@ -162,10 +180,10 @@ __global__ __launch_bounds__(kPartThreads) void csx_bucket_histogram(const int32
 #pragma unroll
     for (int i = 0; i < kItems; i++) {
         const int64_t e = base + (int64_t)i * kPartThreads + threadIdx.x;
-        if (e < E && (uint32_t)k[i] < (uint32_t)V) atomicAdd(&bins[k[i] >> shift], 1);
+        count_runs(bins, (e < E && (uint32_t)k[i] < (uint32_t)V) ? (k[i] >> shift) : -1, 1u);
     }
     __syncthreads();
-    for (int b = threadIdx.x; b < nbins; b += kPartThreads) table[(int64_t)b * nblocks + blockIdx.x] = bins[b];
+    for (int b = threadIdx.x; b < nbins; b += kPartThreads) table[(int64_t)b * nblocks + blockIdx.x] = (int32_t)bins[b];
     if (blockIdx.x == 0 && threadIdx.x == 0) table[(int64_t)nbins * nblocks] = 0;
 }
 
@@ -232,8 +250,7 @@ __device__ __forceinline__ int tile_sort(uint32_t *raw, int stage_n, TileLds &L,
     for (int i = 0; i < kMaxK; i++) gb[i] = (i < K && b0 + i < nbins) ? gbase(b0 + i) : 0;
     __syncthreads();
 #pragma unroll
-    for (int r = 0; r < kItems; r++)
-        if (bin[r] >= 0) atomicAdd(&mine[bin[r]], 1u << half);
+    for (int r = 0; r < kItems; r++) count_runs(mine, bin[r], 1u << half);
     __syncthreads();
     uint32_t pk[kMaxK][kPartWaves / 2];
     int tot[kMaxK];
@@ -318,6 +335,17 @@ __device__ __forceinline__ void tile_emit(const TileLds &L, int total, BinOfRec 
     }
 }
 
+// Tile a workgroup of the partition takes.  Workgroup b runs on XCD b % 8; every XCD gets a
+// contiguous range of tiles, so that the runs neighbouring tiles append to a bucket meet in one
+// L2 before they are written back (config 5: 3.54 -> 2.73 ms).  The grid is rounded up to a
+// multiple of 8; workgroups past the last tile return.
+__device__ __forceinline__ int tile_of_workgroup(int nblocks)
+{
+    const int per = (nblocks + 7) / 8;
+    const int t = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
+    return ((int)(blockIdx.x >> 3) < per && t < nblocks) ? t : -1;
+}
+
 // ---------------------------------------------------------------- step 3 ---
 // Loader for the first partition: items come from the COO arrays.
 __device__ __forceinline__ void keep_position(Rec3 &r, int32_t c) { r.w = (uint32_t)c; }
@@ -366,7 +394,7 @@ template <typename Rec, typename Loader>
 __global__ __launch_bounds__(kPartThreads) void csx_digit_histogram(Loader in, int shift, int mask, int nbins,
                                                                     int32_t *__restrict__ table, int nblocks)
 {
-    __shared__ int bins[kMaxBins];
+    __shared__ uint32_t bins[kMaxBins];
     for (int b = threadIdx.x; b < nbins; b += kPartThreads) bins[b] = 0;
     __syncthreads();
     const int64_t base = (int64_t)blockIdx.x * kTile;
@@ -375,10 +403,10 @@ __global__ __launch_bounds__(kPartThreads) void csx_digit_histogram(Loader in, i
     for (int i = 0; i < kItems; i++) in.load(base + (int64_t)i * kPartThreads + threadIdx.x, rec[i]);
 #pragma unroll
     for (int i = 0; i < kItems; i++)
-        if (in.valid(base + (int64_t)i * kPartThreads + threadIdx.x, rec[i]))
-            atomicAdd(&bins[(rec[i].key >> shift) & mask], 1);
+        count_runs(bins, in.valid(base + (int64_t)i * kPartThreads + threadIdx.x, rec[i]) ? ((rec[i].key >> shift) & mask) : -1,
+                   1u);
     __syncthreads();
-    for (int b = threadIdx.x; b < nbins; b += kPartThreads) table[(int64_t)b * nblocks + blockIdx.x] = bins[b];
+    for (int b = threadIdx.x; b < nbins; b += kPartThreads) table[(int64_t)b * nblocks + blockIdx.x] = (int32_t)bins[b];
     if (blockIdx.x == 0 && threadIdx.x == 0) table[(int64_t)nbins * nblocks] = 0;
 }
 
@@ -415,7 +443,9 @@ __global__ __launch_bounds__(kPartThreads) void csx_partition(Loader in, int shi
 {
     extern __shared__ uint32_t lds_raw[];
     const int w = threadIdx.x >> 6;
-    const int64_t base = (int64_t)blockIdx.x * kTile + (int64_t)w * kWaveSpan + lane_id();
+    const int blk = tile_of_workgroup(nblocks);
+    if (blk < 0) return;
+    const int64_t base = (int64_t)blk * kTile + (int64_t)w * kWaveSpan + lane_id();
     Rec rec[kItems];
     int bin[kItems], lp[kItems];
 #pragma unroll
@@ -423,7 +453,7 @@ __global__ __launch_bounds__(kPartThreads) void csx_partition(Loader in, int shi
 #pragma unroll
     for (int r = 0; r < kItems; r++)
         bin[r] = in.valid(base + (int64_t)r * kWave, rec[r]) ? ((rec[r].key >> shift) & mask) : -1;
-    const int blk = blockIdx.x;
+
     TileLds L;
     const int total = tile_sort<Rec>(lds_raw, stage_n, L, nbins, nbits, bin, lp,
                                      [&](int b) { return table[(int64_t)b * nblocks + blk]; });
@@ -439,14 +469,16 @@ __global__ __launch_bounds__(kPartThreads) void csx_partition_pack(CooLoader<Rec
 {
     extern __shared__ uint32_t lds_raw[];
     const int w = threadIdx.x >> 6;
-    const int64_t base = (int64_t)blockIdx.x * kTile + (int64_t)w * kWaveSpan + lane_id();
+    const int blk = tile_of_workgroup(nblocks);
+    if (blk < 0) return;
+    const int64_t base = (int64_t)blk * kTile + (int64_t)w * kWaveSpan + lane_id();
     Rec rec[kItems];
     int bin[kItems], lp[kItems];
 #pragma unroll
     for (int r = 0; r < kItems; r++) in.load(base + (int64_t)r * kWave, rec[r]);
 #pragma unroll
     for (int r = 0; r < kItems; r++) bin[r] = in.valid(base + (int64_t)r * kWave, rec[r]) ? (rec[r].key >> rule.shift) : -1;
-    const int blk = blockIdx.x;
+
     TileLds L;
     const int total = tile_sort<Rec>(lds_raw, stage_n, L, nbins, nbits, bin, lp,
                                      [&](int b) { return table[(int64_t)b * nblocks + blk]; });
@@ -532,23 +564,23 @@ __global__ __launch_bounds__(kPartThreads) void csx_sub_count(const Rec *__restr
                                                               const int32_t *__restrict__ sub_first, View view, int shift,
                                                               int32_t *__restrict__ cnt2)
 {
-    __shared__ int bins[kMaxBins];
+    __shared__ uint32_t bins[kMaxBins];
     const SubRange r = sub_range(table, nblocks, sub_bucket, sub_first, blockIdx.x);
     if (r.bucket < 0) return;
     const int nkeys = 1 << shift;
     for (int k = threadIdx.x; k < nkeys; k += kPartThreads) bins[k] = 0;
     __syncthreads();
     constexpr int kBatch = 8;
-    for (int e0 = r.begin + threadIdx.x; e0 < r.end; e0 += kBatch * kPartThreads) {
+    // every wavefront makes the same number of trips, so that count_runs sees whole wavefronts
+    for (int e0 = r.begin + threadIdx.x; e0 - (int)threadIdx.x < r.end; e0 += kBatch * kPartThreads) {
         int k[kBatch];
 #pragma unroll
-        for (int i = 0; i < kBatch; i++) k[i] = view.key_low(recs[min(e0 + i * kPartThreads, r.end - 1)]);
+        for (int i = 0; i < kBatch; i++) k[i] = view.key_low(recs[max(min(e0 + i * kPartThreads, r.end - 1), r.begin)]);
 #pragma unroll
-        for (int i = 0; i < kBatch; i++)
-            if (e0 + i * kPartThreads < r.end) atomicAdd(&bins[k[i]], 1);
+        for (int i = 0; i < kBatch; i++) count_runs(bins, e0 + i * kPartThreads < r.end ? k[i] : -1, 1u);
     }
     __syncthreads();
-    for (int k = threadIdx.x; k < nkeys; k += kPartThreads) cnt2[(int64_t)blockIdx.x * nkeys + k] = bins[k];
+    for (int k = threadIdx.x; k < nkeys; k += kPartThreads) cnt2[(int64_t)blockIdx.x * nkeys + k] = (int32_t)bins[k];
 }
 
 // ---------------------------------------------------------------- step 6 ---
@@ -620,10 +652,17 @@ __global__ __launch_bounds__(kPartThreads) void csx_sub_scatter(const Rec *__res
                                                                 const uint32_t *__restrict__ w_in,
                                                                 int32_t *__restrict__ out_idx,
                                                                 uint32_t *__restrict__ out_w,
-                                                                int32_t *__restrict__ out_perm, int stage_n)
+                                                                int32_t *__restrict__ out_perm, int stage_n,
+                                                                int nbuckets, int max_sub)
 {
     extern __shared__ uint32_t lds_raw[];
-    const int sub = blockIdx.x;
+    // Workgroup b runs on XCD b % 8.  The sub-blocks of one bucket write interleaved runs into the
+    // bucket's output region (a few hundred KB): handing every XCD a contiguous range of
+    // sub-blocks lets those runs meet in one L2 before they are written back.
+    const int nsub = min(sub_first[nbuckets], max_sub);      // the grid holds 8 * ceil(max_sub / 8) workgroups
+    const int per = (nsub + 7) / 8;
+    const int sub = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
+    if ((int)(blockIdx.x >> 3) >= per || sub >= nsub) return;
     const SubRange sr = sub_range(table, nblocks, sub_bucket, sub_first, sub);
     if (sr.bucket < 0) return;
     const int nkeys = 1 << shift;
@@ -793,7 +832,7 @@ static int32_t convert(const int32_t *keys, const int32_t *others, const float *
                 hipLaunchKernelGGL(csx_save_count, dim3(1), dim3(1), 0, s, table + (table_n - 1), count);
                 auto part = csx_partition<Rec, CooLoader<Rec>>;
                 allow_lds(part, lds);
-                hipLaunchKernelGGL(part, dim3(nb), dim3(kPartThreads), lds, s, in, shift, kMaxBins - 1, kMaxBins,
+                hipLaunchKernelGGL(part, dim3((nb + 7) / 8 * 8), dim3(kPartThreads), lds, s, in, shift, kMaxBins - 1, kMaxBins,
                                    kMaxBinBits, table, nblk, dst, stage_n);
             } else {
                 RecLoader<Rec> in{bufs[(d - 1) & 1], count, E};
@@ -802,7 +841,7 @@ static int32_t convert(const int32_t *keys, const int32_t *others, const float *
                 if ((rc = exclusive_scan_i32(table, table, (int64_t)table_n, sums, s))) return rc;
                 auto part = csx_partition<Rec, RecLoader<Rec>>;
                 allow_lds(part, lds);
-                hipLaunchKernelGGL(part, dim3(nb), dim3(kPartThreads), lds, s, in, shift, kMaxBins - 1, kMaxBins,
+                hipLaunchKernelGGL(part, dim3((nb + 7) / 8 * 8), dim3(kPartThreads), lds, s, in, shift, kMaxBins - 1, kMaxBins,
                                    kMaxBinBits, table, nblk, dst, stage_n);
             }
         }
@@ -838,9 +877,10 @@ static int32_t convert(const int32_t *keys, const int32_t *others, const float *
         auto scat = csx_sub_scatter<R, PERM, decltype(view)>;
         const size_t scat_lds = tile_lds_bytes(nkeys, sizeof(R));
         allow_lds(scat, scat_lds);
-        hipLaunchKernelGGL(scat, dim3((unsigned)p.max_sub), dim3(kPartThreads), scat_lds, s, records, table, nblk,
+        hipLaunchKernelGGL(scat, dim3((unsigned)((p.max_sub + 7) / 8 * 8)), dim3(kPartThreads), scat_lds, s, records, table, nblk,
                            sub_bucket, sub_first, cnt2, view, p.shift, others, wbits, out_idx,
-                           reinterpret_cast<uint32_t *>(out_w), out_perm, tile_stage_records(nkeys, sizeof(R)));
+                           reinterpret_cast<uint32_t *>(out_w), out_perm, tile_stage_records(nkeys, sizeof(R)),
+                           p.nbuckets, p.max_sub);
     };
     const size_t part_lds = tile_lds_bytes(p.nbuckets, sizeof(Rec));
     if (packed_ok) {
@@ -853,14 +893,14 @@ static int32_t convert(const int32_t *keys, const int32_t *others, const float *
         CooLoader<Rec> in{keys, others, wbits, E, V, rule.omask};
         auto part = csx_partition_pack<Rec, Packed>;
         allow_lds(part, part_lds);
-        hipLaunchKernelGGL(part, dim3(nb), dim3(kPartThreads), part_lds, s, in, rule, p.nbuckets, bbits, table, nblk, packed,
+        hipLaunchKernelGGL(part, dim3((nb + 7) / 8 * 8), dim3(kPartThreads), part_lds, s, in, rule, p.nbuckets, bbits, table, nblk, packed,
                            tile_stage_records(p.nbuckets, sizeof(Rec)));
         level2(packed, PackedView{rule});
     } else {
         CooLoader<Rec> in{keys, others, wbits, E, V, 0u};
         auto part = csx_partition<Rec, CooLoader<Rec>>;
         allow_lds(part, part_lds);
-        hipLaunchKernelGGL(part, dim3(nb), dim3(kPartThreads), part_lds, s, in, p.shift, 0x7fffffff, p.nbuckets, bbits,
+        hipLaunchKernelGGL(part, dim3((nb + 7) / 8 * 8), dim3(kPartThreads), part_lds, s, in, p.shift, 0x7fffffff, p.nbuckets, bbits,
                            table, nblk, recs, tile_stage_records(p.nbuckets, sizeof(Rec)));
         level2(recs, PlainView{nkeys - 1});
     }
