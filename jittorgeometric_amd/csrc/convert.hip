@@ -141,6 +141,18 @@ __device__ __forceinline__ void set_id(Rec4 &r, int32_t id) { r.id = id; }
 __device__ __forceinline__ int32_t get_id(const Rec3 &) { return 0; }
 __device__ __forceinline__ int32_t get_id(const Rec4 &r) { return r.id; }
 
+// Tile a workgroup of the histogram and of the partition takes.  Workgroup b runs on XCD b % 8;
+// every XCD gets a contiguous range of tiles, so that what neighbouring tiles write side by side
+// (their counts in the table, the runs they append to a bucket) meets in one L2 before it is
+// written back (V = 2.45M, E = 126M: 3.54 -> 2.73 ms).  The grid is rounded up to a
+// multiple of 8; workgroups past the last tile return.
+__device__ __forceinline__ int tile_of_workgroup(int nblocks)
+{
+    const int per = (nblocks + 7) / 8;
+    const int t = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
+    return ((int)(blockIdx.x >> 3) < per && t < nblocks) ? t : -1;
+}
+
 // bins[b] += unit for every lane with b >= 0, one LDS atomic per run of equal b over consecutive
 // lanes of a row of 16.  Keys that arrive sorted (an edge list ordered by source) put whole
 // wavefronts on one counter, and 64 atomics on one LDS address take 64 turns; a run costs one.
@@ -167,9 +179,11 @@ __global__ __launch_bounds__(kPartThreads) void csx_bucket_histogram(const int32
                                                                      int32_t *__restrict__ table, int nblocks)
 {
     __shared__ uint32_t bins[kMaxBins];
+    const int blk = tile_of_workgroup(nblocks);
+    if (blk < 0) return;
     for (int b = threadIdx.x; b < nbins; b += kPartThreads) bins[b] = 0;
     __syncthreads();
-    const int64_t base = (int64_t)blockIdx.x * kTile;
+    const int64_t base = (int64_t)blk * kTile;
     // all loads first (index clamped instead of predicated), then the counting
     int32_t k[kItems];
 #pragma unroll
@@ -183,8 +197,8 @@ __global__ __launch_bounds__(kPartThreads) void csx_bucket_histogram(const int32
         count_runs(bins, (e < E && (uint32_t)k[i] < (uint32_t)V) ? (k[i] >> shift) : -1, 1u);
     }
     __syncthreads();
-    for (int b = threadIdx.x; b < nbins; b += kPartThreads) table[(int64_t)b * nblocks + blockIdx.x] = (int32_t)bins[b];
-    if (blockIdx.x == 0 && threadIdx.x == 0) table[(int64_t)nbins * nblocks] = 0;
+    for (int b = threadIdx.x; b < nbins; b += kPartThreads) table[(int64_t)b * nblocks + blk] = (int32_t)bins[b];
+    if (blk == 0 && threadIdx.x == 0) table[(int64_t)nbins * nblocks] = 0;
 }
 
 // ------------------------------------------------------- stable tile sort ---
@@ -335,17 +349,6 @@ __device__ __forceinline__ void tile_emit(const TileLds &L, int total, BinOfRec 
     }
 }
 
-// Tile a workgroup of the partition takes.  Workgroup b runs on XCD b % 8; every XCD gets a
-// contiguous range of tiles, so that the runs neighbouring tiles append to a bucket meet in one
-// L2 before they are written back (config 5: 3.54 -> 2.73 ms).  The grid is rounded up to a
-// multiple of 8; workgroups past the last tile return.
-__device__ __forceinline__ int tile_of_workgroup(int nblocks)
-{
-    const int per = (nblocks + 7) / 8;
-    const int t = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
-    return ((int)(blockIdx.x >> 3) < per && t < nblocks) ? t : -1;
-}
-
 // ---------------------------------------------------------------- step 3 ---
 // Loader for the first partition: items come from the COO arrays.
 __device__ __forceinline__ void keep_position(Rec3 &r, int32_t c) { r.w = (uint32_t)c; }
@@ -395,9 +398,11 @@ __global__ __launch_bounds__(kPartThreads) void csx_digit_histogram(Loader in, i
                                                                     int32_t *__restrict__ table, int nblocks)
 {
     __shared__ uint32_t bins[kMaxBins];
+    const int blk = tile_of_workgroup(nblocks);
+    if (blk < 0) return;
     for (int b = threadIdx.x; b < nbins; b += kPartThreads) bins[b] = 0;
     __syncthreads();
-    const int64_t base = (int64_t)blockIdx.x * kTile;
+    const int64_t base = (int64_t)blk * kTile;
     Rec rec[kItems];
 #pragma unroll
     for (int i = 0; i < kItems; i++) in.load(base + (int64_t)i * kPartThreads + threadIdx.x, rec[i]);
@@ -406,8 +411,8 @@ __global__ __launch_bounds__(kPartThreads) void csx_digit_histogram(Loader in, i
         count_runs(bins, in.valid(base + (int64_t)i * kPartThreads + threadIdx.x, rec[i]) ? ((rec[i].key >> shift) & mask) : -1,
                    1u);
     __syncthreads();
-    for (int b = threadIdx.x; b < nbins; b += kPartThreads) table[(int64_t)b * nblocks + blockIdx.x] = (int32_t)bins[b];
-    if (blockIdx.x == 0 && threadIdx.x == 0) table[(int64_t)nbins * nblocks] = 0;
+    for (int b = threadIdx.x; b < nbins; b += kPartThreads) table[(int64_t)b * nblocks + blk] = (int32_t)bins[b];
+    if (blk == 0 && threadIdx.x == 0) table[(int64_t)nbins * nblocks] = 0;
 }
 
 __global__ void csx_save_count(const int32_t *__restrict__ table_end, int32_t *__restrict__ count)
@@ -826,7 +831,7 @@ static int32_t convert(const int32_t *keys, const int32_t *others, const float *
             Rec *dst = bufs[d & 1];
             if (d == 0) {
                 CooLoader<Rec> in{keys, others, reinterpret_cast<const uint32_t *>(w), E, V, 0u};
-                hipLaunchKernelGGL((csx_digit_histogram<Rec, CooLoader<Rec>>), dim3(nb), dim3(kPartThreads), 0, s, in,
+                hipLaunchKernelGGL((csx_digit_histogram<Rec, CooLoader<Rec>>), dim3((nb + 7) / 8 * 8), dim3(kPartThreads), 0, s, in,
                                    shift, kMaxBins - 1, kMaxBins, table, nblk);
                 if ((rc = exclusive_scan_i32(table, table, (int64_t)table_n, sums, s))) return rc;
                 hipLaunchKernelGGL(csx_save_count, dim3(1), dim3(1), 0, s, table + (table_n - 1), count);
@@ -836,7 +841,7 @@ static int32_t convert(const int32_t *keys, const int32_t *others, const float *
                                    kMaxBinBits, table, nblk, dst, stage_n);
             } else {
                 RecLoader<Rec> in{bufs[(d - 1) & 1], count, E};
-                hipLaunchKernelGGL((csx_digit_histogram<Rec, RecLoader<Rec>>), dim3(nb), dim3(kPartThreads), 0, s, in,
+                hipLaunchKernelGGL((csx_digit_histogram<Rec, RecLoader<Rec>>), dim3((nb + 7) / 8 * 8), dim3(kPartThreads), 0, s, in,
                                    shift, kMaxBins - 1, kMaxBins, table, nblk);
                 if ((rc = exclusive_scan_i32(table, table, (int64_t)table_n, sums, s))) return rc;
                 auto part = csx_partition<Rec, RecLoader<Rec>>;
@@ -854,7 +859,7 @@ static int32_t convert(const int32_t *keys, const int32_t *others, const float *
 
     int bbits = 0;
     while ((1 << bbits) < p.nbuckets) bbits++;
-    hipLaunchKernelGGL(csx_bucket_histogram, dim3(nb), dim3(kPartThreads), 0, s, keys, E, V, p.shift, p.nbuckets,
+    hipLaunchKernelGGL(csx_bucket_histogram, dim3((nb + 7) / 8 * 8), dim3(kPartThreads), 0, s, keys, E, V, p.shift, p.nbuckets,
                        table, nblk);
     if ((rc = exclusive_scan_i32(table, table, (int64_t)table_n, sums, s))) return rc;
 
