@@ -607,12 +607,25 @@ __global__ __launch_bounds__(kPartThreads) void csx_bucket_offsets(const int32_t
     const int64_t k0 = (int64_t)b << shift;
     if (threadIdx.x == 0) carry = table[(int64_t)b * nblocks];
     __syncthreads();
+    // a bucket of up to kKeep sub-blocks keeps a key's counts in registers between the two loops
+    // (all loads in flight together, the table read once)
+    constexpr int kKeep = 16;
+    const int ns = s1 - s0;
     for (int kb = 0; kb < nkeys; kb += kPartThreads) {
         const int k = kb + threadIdx.x;
         int total = 0;
+        int kept[kKeep];
         if (k < nkeys) {
+            if (ns <= kKeep) {
+#pragma unroll
+                for (int i = 0; i < kKeep; i++) kept[i] = cnt2[(int64_t)(s0 + min(i, ns - 1)) * nkeys + k];
+#pragma unroll
+                for (int i = 0; i < kKeep; i++)
+                    if (i < ns) total += kept[i];
+            } else {
 #pragma unroll 8
-            for (int s = s0; s < s1; s++) total += cnt2[(int64_t)s * nkeys + k];
+                for (int s = s0; s < s1; s++) total += cnt2[(int64_t)s * nkeys + k];
+            }
         }
         // block-exclusive scan of `total` in key order
         int inc = total;
@@ -630,11 +643,20 @@ __global__ __launch_bounds__(kPartThreads) void csx_bucket_offsets(const int32_t
         if (k < nkeys) {
             if (k0 + k < V) off[k0 + k] = key_base;
             int run = key_base;
+            if (ns <= kKeep) {
+#pragma unroll
+                for (int i = 0; i < kKeep; i++)
+                    if (i < ns) {
+                        cnt2[(int64_t)(s0 + i) * nkeys + k] = run;
+                        run += kept[i];
+                    }
+            } else {
 #pragma unroll 8
-            for (int s = s0; s < s1; s++) {
-                const int c = cnt2[(int64_t)s * nkeys + k];
-                cnt2[(int64_t)s * nkeys + k] = run;
-                run += c;
+                for (int s = s0; s < s1; s++) {
+                    const int c = cnt2[(int64_t)s * nkeys + k];
+                    cnt2[(int64_t)s * nkeys + k] = run;
+                    run += c;
+                }
             }
         }
         __syncthreads();
