@@ -597,7 +597,10 @@ __global__ __launch_bounds__(kPartThreads) void csx_bucket_offsets(const int32_t
                                                                    int nbuckets,
                                                                    const int32_t *__restrict__ sub_first, int shift,
                                                                    int32_t V, int32_t *__restrict__ cnt2,
-                                                                   int32_t *__restrict__ off)
+                                                                   int32_t *__restrict__ off, int64_t E,
+                                                                   int32_t *__restrict__ out_idx,
+                                                                   uint32_t *__restrict__ out_w,
+                                                                   int32_t *__restrict__ out_perm)
 {
     __shared__ int wave_tot[kPartWaves];
     __shared__ int carry;
@@ -663,7 +666,16 @@ __global__ __launch_bounds__(kPartThreads) void csx_bucket_offsets(const int32_t
         if (threadIdx.x == kPartThreads - 1) carry = key_base + total;
         __syncthreads();
     }
-    if (b == nbuckets - 1 && threadIdx.x == 0) off[V] = table[(int64_t)nbuckets * nblocks];
+    const int64_t covered = table[(int64_t)nbuckets * nblocks];
+    if (b == nbuckets - 1 && threadIdx.x == 0) off[V] = (int32_t)covered;
+    // Edges with a key outside [0,V) were dropped, so off[V] may be below E: the slots past off[V]
+    // are zeroed (the reference hands zero-filled arrays to the op, ops/cootocsr.py:30-32).
+    // Nothing to do in the usual case.
+    for (int64_t i = covered + (int64_t)b * kPartThreads + threadIdx.x; i < E; i += (int64_t)gridDim.x * kPartThreads) {
+        out_idx[i] = 0;
+        if (out_w) out_w[i] = 0u;
+        if (out_perm) out_perm[i] = 0;
+    }
 }
 
 // ---------------------------------------------------------------- step 7 ---
@@ -900,7 +912,8 @@ static int32_t convert(const int32_t *keys, const int32_t *others, const float *
         hipLaunchKernelGGL((csx_sub_count<R, decltype(view)>), dim3((unsigned)p.max_sub), dim3(kPartThreads), 0, s,
                            records, table, nblk, sub_bucket, sub_first, view, p.shift, cnt2);
         hipLaunchKernelGGL(csx_bucket_offsets, dim3((unsigned)p.nbuckets), dim3(kPartThreads), 0, s, table, nblk,
-                           p.nbuckets, sub_first, p.shift, V, cnt2, out_off);
+                           p.nbuckets, sub_first, p.shift, V, cnt2, out_off, E, out_idx,
+                           reinterpret_cast<uint32_t *>(out_w), out_perm);
         auto scat = csx_sub_scatter<R, PERM, decltype(view)>;
         const size_t scat_lds = tile_lds_bytes(nkeys, sizeof(R));
         allow_lds(scat, scat_lds);
@@ -931,7 +944,6 @@ static int32_t convert(const int32_t *keys, const int32_t *others, const float *
                            table, nblk, recs, tile_stage_records(p.nbuckets, sizeof(Rec)));
         level2(recs, PlainView{nkeys - 1});
     }
-    zero_tail(out_off, V, E, out_idx, out_w, out_perm, s);
     return launch_status("coo_to_csx");
 }
 
