@@ -80,10 +80,14 @@ __device__ __forceinline__ int covered_entries(const int32_t *__restrict__ off, 
 // One thread per column: it owns the entries [off[c], off[c+1]) and marks the
 // tiles whose first or last entry falls among them.
 __global__ void esm_tile_columns(const int32_t *__restrict__ off, int V, int E, int T, int ntiles,
-                                 int32_t *__restrict__ tile_first, int32_t *__restrict__ tile_last)
+                                 int32_t *__restrict__ tile_first, int32_t *__restrict__ tile_last,
+                                 float *__restrict__ zero_rows = nullptr, int zero_width = 0)
 {
     const int c = blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= V) return;
+    // the gather-sum starts from zeroed rows (empty columns belong to no tile): this thread's row
+    if (zero_rows)
+        for (int h = 0; h < zero_width; h++) zero_rows[(int64_t)c * zero_width + h] = 0.f;
     // entries past off[V] belong to no column (offsets of a conversion that dropped keys):
     // only the tiles that hold covered entries get a first and a last column
     const int covered = covered_entries(off, V, E);
@@ -560,13 +564,8 @@ __global__ __launch_bounds__(kFlatThreads) void esm_bwd_tile(const int32_t *__re
 // wide-row kernel gives a whole wavefront to one entry; with a handful of floats
 // per row that leaves most lanes idle, so here a lane gathers K entries and the
 // per-column totals come from the segmented scan.  Columns inside the tile are
-// written by the tile kernel, crossing ones by esm_merge; out is zeroed first
-// (empty columns belong to no tile).
-__global__ void esm_fill_zero(float *__restrict__ p, int64_t n)
-{
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) p[i] = 0.f;
-}
+// written by the tile kernel, crossing ones by esm_merge; out is zeroed first, by the
+// tile-columns kernel (empty columns belong to no tile).
 
 template <int H>
 __global__ __launch_bounds__(kFlatThreads) void esm_colsum_tile(const int32_t *__restrict__ off,
@@ -817,10 +816,8 @@ static void colsum_launch(const int32_t *off, const int32_t *idx, const float *w
     float *stat = carve.take<float>(cap * 2 * 8);
     int32_t *tile_first = carve.take<int32_t>(cap);
     int32_t *tile_last = carve.take<int32_t>(cap);
-    const int64_t n_out = (int64_t)R * H;
-    hipLaunchKernelGGL(esm_fill_zero, dim3((unsigned)ceil_div(n_out, 256)), dim3(256), 0, s, out, n_out);
     hipLaunchKernelGGL(esm_tile_columns, dim3((unsigned)ceil_div(R, 256)), dim3(256), 0, s, off, R, (int)E, T, ntiles,
-                       tile_first, tile_last);
+                       tile_first, tile_last, out, H);
     hipLaunchKernelGGL(esm_colsum_tile<H>, dim3(ntiles), dim3(kFlatThreads), 0, s, off, idx, w, x, out, tile_first,
                        tile_last, R, C, (int)E, meta, pieces);
     hipLaunchKernelGGL((esm_merge<H, T, false>), dim3((unsigned)ceil_div(ntiles, kFlatWaves)), dim3(kFlatThreads), 0, s,
