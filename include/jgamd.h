@@ -322,12 +322,16 @@ int32_t jgamd_column_sum(const float *x, float *out, int64_t R, int32_t F, void 
  * gradient.  labels: int32, or int64 when labels_are_i64 != 0.  loss[1],
  * count[1] (rows counted) and lse[V] are written by fwd and read by bwd:
  *   grad_logits[i,c] = grad_loss[0] / count * (exp(logits[i,c] - lse[i]) - [c == label[i]])
- * (grad_loss NULL = 1).  Two fixed-order reduction stages, no atomics.
+ * (grad_loss NULL = 1).  log_probs != 0: the rows already are log-probabilities
+ * (nn.nll_loss): loss = mean of -logits[i,label[i]], lse is written as +inf
+ * and bwd then yields -[c == label[i]] * grad_loss[0] / count.  Two
+ * fixed-order reduction stages, no atomics.
  */
 int32_t jgamd_cross_entropy_workspace(int64_t V, int32_t C, size_t *bytes);
 int32_t jgamd_cross_entropy_fwd(const float *logits, const void *labels, int32_t labels_are_i64,
-                                int64_t V, int32_t C, float *loss, int32_t *count, float *lse,
-                                void *ws, size_t ws_bytes, void *stream);
+                                int32_t log_probs, int64_t V, int32_t C, float *loss,
+                                int32_t *count, float *lse, void *ws, size_t ws_bytes,
+                                void *stream);
 int32_t jgamd_cross_entropy_bwd(const float *logits, const void *labels, int32_t labels_are_i64,
                                 const float *lse, const int32_t *count, const float *grad_loss,
                                 int64_t V, int32_t C, float *grad_logits, void *stream);

@@ -51,7 +51,7 @@ SIGNATURES = {
     "jgamd_column_sum_workspace": [_I64, _I32, _SZP],
     "jgamd_column_sum": [_P, _P, _I64, _I32, _P, _c.c_size_t, _P],
     "jgamd_cross_entropy_workspace": [_I64, _I32, _SZP],
-    "jgamd_cross_entropy_fwd": [_P, _P, _I32, _I64, _I32, _P, _P, _P, _P, _c.c_size_t, _P],
+    "jgamd_cross_entropy_fwd": [_P, _P, _I32, _I32, _I64, _I32, _P, _P, _P, _P, _c.c_size_t, _P],
     "jgamd_cross_entropy_bwd": [_P, _P, _I32, _P, _P, _P, _I64, _I32, _P, _P],
     "jgamd_gat_fwd_workspace": [_I32, _I64, _I32, _I32, _SZP],
     "jgamd_gat_fwd": [_P, _P, _P, _P, _P, _F32, _P, _P, _P, _P, _P, _P, _I32, _I64, _I32, _I32, _P,

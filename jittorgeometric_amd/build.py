@@ -41,6 +41,10 @@ def build(verbose=False):
     srcs = sources()
     if not srcs:
         raise RuntimeError("no HIP sources under " + CSRC)
+    # a library from older sources must not survive a failed build: the ctypes signatures follow
+    # the sources, and a call through a stale entry point would pass the wrong arguments
+    if os.path.exists(LIB):
+        os.remove(LIB)
     with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
         results = list(ex.map(_compile, srcs))
     objs = [o for o, _ in results]

@@ -32,8 +32,8 @@ constexpr int kCeUnroll = 4;
 template <int G, bool REG>
 __global__ __launch_bounds__(kCeThreads) void ce_rows(const float *__restrict__ x, const int32_t *__restrict__ y32,
                                                       const int64_t *__restrict__ y64, int64_t V, int C,
-                                                      float *__restrict__ lse_out, double *__restrict__ block_sum,
-                                                      int32_t *__restrict__ block_cnt)
+                                                      int log_probs, float *__restrict__ lse_out,
+                                                      double *__restrict__ block_sum, int32_t *__restrict__ block_cnt)
 {
     constexpr int RP = kCeThreads / G;      // row groups per pass
     __shared__ double s_sum[RP];
@@ -44,8 +44,10 @@ __global__ __launch_bounds__(kCeThreads) void ce_rows(const float *__restrict__ 
     double acc = 0.0;
     int cnt = 0;
     auto finish = [&](int64_t row, const float *p, float m, float s) {
-        const float l = m + logf(s);
-        lse_out[row] = l;
+        // rows of log-probabilities (nll_loss): the loss is -row[label] and the gradient has no
+        // softmax term, which an infinite lse switches off in the backward kernels (exp(-inf) = 0)
+        const float l = log_probs ? 0.f : m + logf(s);
+        lse_out[row] = log_probs ? INFINITY : l;
         const int64_t lab = label_at(y32, y64, row);
         if (lab >= 0 && lab < C) {
             acc += (double)(l - p[lab]);
@@ -243,9 +245,9 @@ JG_EXPORT int32_t jgamd_cross_entropy_workspace(int64_t V, int32_t C, size_t *by
     return 0;
 }
 
-JG_EXPORT int32_t jgamd_cross_entropy_fwd(const float *logits, const void *labels, int32_t labels_are_i64, int64_t V,
-                                          int32_t C, float *loss, int32_t *count, float *lse, void *ws,
-                                          size_t ws_bytes, void *stream)
+JG_EXPORT int32_t jgamd_cross_entropy_fwd(const float *logits, const void *labels, int32_t labels_are_i64,
+                                          int32_t log_probs, int64_t V, int32_t C, float *loss, int32_t *count,
+                                          float *lse, void *ws, size_t ws_bytes, void *stream)
 {
     if (int32_t rc = ce_check("cross_entropy_fwd", V, C)) return rc;
     if (!loss || !count) return fail(JGAMD_ERR_NULL, "cross_entropy_fwd: loss / count is NULL");
@@ -269,10 +271,10 @@ JG_EXPORT int32_t jgamd_cross_entropy_fwd(const float *logits, const void *label
     if (G == GG) {                                                                                                   \
         if (reg)                                                                                                     \
             hipLaunchKernelGGL((ce_rows<GG, true>), dim3((unsigned)nblocks), dim3(kCeThreads), 0, st, logits, y32,   \
-                               y64, V, C, lse, block_sum, block_cnt);                                                \
+                               y64, V, C, log_probs, lse, block_sum, block_cnt);                                                \
         else                                                                                                         \
             hipLaunchKernelGGL((ce_rows<GG, false>), dim3((unsigned)nblocks), dim3(kCeThreads), 0, st, logits, y32,  \
-                               y64, V, C, lse, block_sum, block_cnt);                                                \
+                               y64, V, C, log_probs, lse, block_sum, block_cnt);                                                \
     }
         JG_CE(8) JG_CE(16) JG_CE(32) JG_CE(64)
 #undef JG_CE

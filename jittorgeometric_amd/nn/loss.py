@@ -11,7 +11,7 @@ from .. import _lib
 
 class _CrossEntropy(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, output, target):
+    def forward(ctx, output, target, log_probs):
         lib = _lib.load()
         dev = _lib.require_gpu(output, target)
         if output.dim() != 2:
@@ -30,7 +30,8 @@ class _CrossEntropy(torch.autograd.Function):
         nbytes = _lib.query(lib.jgamd_cross_entropy_workspace, V, C)
         ws = _lib.workspace(nbytes, dev)
         i64 = 1 if target.dtype == torch.int64 else 0
-        _lib.check(lib.jgamd_cross_entropy_fwd(_lib.ptr(x), _lib.ptr(target), i64, V, C, _lib.ptr(loss), _lib.ptr(count),
+        _lib.check(lib.jgamd_cross_entropy_fwd(_lib.ptr(x), _lib.ptr(target), i64, int(bool(log_probs)), V, C,
+                                               _lib.ptr(loss), _lib.ptr(count),
                                                _lib.ptr(lse), _lib.ptr(ws), nbytes, _lib.stream_ptr(dev)))
         ctx.save_for_backward(x, target, lse, count)
         ctx.i64 = i64
@@ -40,7 +41,7 @@ class _CrossEntropy(torch.autograd.Function):
     @staticmethod
     def backward(ctx, g):
         if not ctx.needs_input_grad[0]:
-            return None, None
+            return None, None, None
         x, target, lse, count = ctx.saved_tensors
         lib = _lib.load()
         dev = x.device
@@ -49,17 +50,17 @@ class _CrossEntropy(torch.autograd.Function):
         V, C = x.shape
         _lib.check(lib.jgamd_cross_entropy_bwd(_lib.ptr(x), _lib.ptr(target), ctx.i64, _lib.ptr(lse), _lib.ptr(count),
                                                _lib.ptr(g), V, C, _lib.ptr(grad), _lib.stream_ptr(dev)))
-        return (grad if ctx.in_dtype == torch.float32 else grad.to(ctx.in_dtype)), None
+        return (grad if ctx.in_dtype == torch.float32 else grad.to(ctx.in_dtype)), None, None
 
 
 def cross_entropy_loss(output, target):
     """mean_i (logsumexp(output[i,:]) - output[i, target[i]]) over the rows whose label lies in
     [0, classes); the other rows are left out and get a zero gradient."""
-    return _CrossEntropy.apply(output, target)
+    return _CrossEntropy.apply(output, target, False)
 
 
 def nll_loss(log_probs, target):
     """mean_i -log_probs[i, target[i]] for rows of log-probabilities (the second half of
-    log_softmax + nll_loss, examples/sage_example.py:69,83).  For rows that are log-probabilities
-    logsumexp is zero, so this is the same kernel."""
-    return _CrossEntropy.apply(log_probs, target)
+    log_softmax + nll_loss, examples/sage_example.py:69,83); the gradient is -1 / rows at the
+    labels and zero elsewhere.  Same kernels, with the softmax term switched off."""
+    return _CrossEntropy.apply(log_probs, target, True)

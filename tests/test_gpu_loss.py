@@ -96,9 +96,21 @@ def test_run_to_run_identical_and_other_dtypes():
     view = wide[:, :C]
     assert not view.is_contiguous()
     assert abs(cross_entropy_loss(view, to_gpu(y[:500])).item() - want) <= 1e-5 * abs(want)
-    # rows of log-probabilities: the same number as log_softmax + nll_loss
-    logp = torch.log_softmax(to_gpu(x[:500]), dim=1)
-    assert abs(nll_loss(logp, to_gpu(y[:500])).item() - want) <= 1e-5 * abs(want)
+    # rows of log-probabilities: the same number as log_softmax + nll_loss, a gradient of -1 / rows at
+    # the labels, and through torch's log_softmax the gradient of the fused loss
+    xs = to_gpu(x[:500]).requires_grad_(True)
+    logp = torch.log_softmax(xs, dim=1)
+    logp.retain_grad()
+    got = nll_loss(logp, to_gpu(y[:500]))
+    got.backward()
+    assert abs(got.item() - want) <= 1e-5 * abs(want)
+    onehot = np.zeros((500, C))
+    onehot[np.arange(500), y[:500]] = 1
+    assert np.array_equal(logp.grad.cpu().numpy(), (-onehot / 500).astype(np.float32))
+    assert_close(xs.grad.cpu().numpy(), wgrad, scale=np.full_like(wgrad, 1 / 500), rtol=1e-5, atol=0)
+    # not log-probabilities: still -mean(row[label]), whatever the rows sum to
+    raw = to_gpu(x[:500])
+    assert abs(nll_loss(raw, to_gpu(y[:500])).item() + x[np.arange(500), y[:500]].astype(np.float64).mean()) <= 1e-5
 
 
 def test_bad_arguments_are_refused():
