@@ -8,7 +8,8 @@ from ...ops import spmmcsr as _spmmcsr
 from ...ops.propagate import aggregate_bias
 from ...utils import add_remaining_self_loops
 from ...utils.num_nodes import maybe_num_nodes
-from ..dense import add_bias, xw
+from ...ops._common import both_orders, spmm, spmm_axpby
+from ..dense import add_bias, column_sum, rows_times, xt_g, xw
 from ..inits import glorot, zeros
 
 
@@ -63,6 +64,47 @@ def gcn_norm(edge_index, edge_weight=None, num_nodes=None, improved=False, add_s
     return edge_index, _scale(edge_index, edge_weight, dis, dis, dis.shape[0])
 
 
+class GcnLayerFunc(torch.autograd.Function):
+    """A_hat (x W) + b as one autograd node (gcn_conv.py:94-102 builds it from three: dense
+    product, product over the graph, addition).  Forward: the dense kernel, then the product with
+    the bias added in its row store.  Backward: g_W = x^T (A_hat^T g) and g_x = (A_hat^T g) W^T share
+    one transposed product at the output width.  When x needs no gradient (the first layer of a
+    model) and the layer widens, g_W = (A_hat x)^T g instead: the same sum in another order, with
+    the product over the graph at the narrower input width."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, fwd, bwd):
+        h = rows_times(x, weight)
+        if bias is not None:
+            out = spmm_axpby(fwd[0], fwd[1], fwd[2], h, x.shape[0], 1.0, 1.0, bias)
+        else:
+            out = spmm(fwd[0], fwd[1], fwd[2], h, x.shape[0])
+        ctx.fwd, ctx.bwd = fwd, bwd
+        ctx.save_for_backward(x, weight)
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        x, weight = ctx.saved_tensors
+        g = g.contiguous()
+        need_x, need_w, need_b = ctx.needs_input_grad[:3]
+        gx = gw = gb = None
+        if need_b:
+            gb = column_sum(g) if g.dtype == torch.float32 else g.sum(0)
+        f_in, f_out = weight.shape
+        if need_x or (need_w and f_out <= f_in):
+            off, idx, w = ctx.bwd
+            gh = spmm(off, idx, w, g, g.shape[0])
+            if need_w:
+                gw = xt_g(x, gh)
+            if need_x:
+                gx = rows_times(gh, weight.t().contiguous())
+        elif need_w:
+            off, idx, w = ctx.fwd
+            gw = xt_g(spmm(off, idx, w, x, x.shape[0]), g)
+        return gx, gw, gb, None, None
+
+
 class GCNConv(nn.Module):
     """out = A_hat (x W) + b.  `spmm=True` routes through SpmmCsr(x, csr), as
     the reference does on a GPU (gcn_conv.py:96-97); `spmm=False` through
@@ -92,6 +134,10 @@ class GCNConv(nn.Module):
         if self.aggregate_first and x.dim() == 2:
             agg = self.propagate_spmm(x=x, csr=csr) if self.spmm else self.propagate_msg(x=x, csc=csc, csr=csr)
             return xw(agg, self.weight, self.bias)
+        if x.dim() == 2 and x.dtype == torch.float32 and not (self.spmm and _spmmcsr.REFERENCE_GRAD):
+            # spmm=True only needs the CSR (:96-97); both routes give the same product
+            fwd, bwd = both_orders(None if self.spmm and csr is not None else csc, csr)
+            return GcnLayerFunc.apply(x.contiguous(), self.weight, self.bias, fwd, bwd)
         x = xw(x, self.weight)
         if self.bias is not None and x.dim() == 2 and not (self.spmm and _spmmcsr.REFERENCE_GRAD):
             # product and bias in one kernel; spmm=True only needs the CSR (:96-97)

@@ -45,11 +45,21 @@ class SageLayerFunc(torch.autograd.Function):
             groot = xt_g(x, g)
         if need_x:
             off, idx, w = ctx.bwd
-            g_agg = rows_times(g, w1.t().contiguous())
-            if w_root is not None:
-                gx = spmm_axpby(off, idx, w, g_agg, g.shape[0], 1.0, 1.0, rows_times(g, w_root.t().contiguous()))
+            if w1.shape[1] < w1.shape[0]:
+                # A^T (g W1^T) = (A^T g) W1^T: the layer narrows, so the transposed product runs on g
+                # itself, at the output width, and the two dense products of the input gradient are
+                # one pass.  Same gradient, summed in another order; the forward pass is untouched.
+                t = spmm(off, idx, w, g, g.shape[0])
+                if w_root is not None:
+                    gx = rows_times(t, w1.t().contiguous(), g, w_root.t().contiguous())
+                else:
+                    gx = rows_times(t, w1.t().contiguous())
             else:
-                gx = spmm(off, idx, w, g_agg, g.shape[0])
+                g_agg = rows_times(g, w1.t().contiguous())
+                if w_root is not None:
+                    gx = spmm_axpby(off, idx, w, g_agg, g.shape[0], 1.0, 1.0, rows_times(g, w_root.t().contiguous()))
+                else:
+                    gx = spmm(off, idx, w, g_agg, g.shape[0])
         return gx, gw1, groot, gb, None, None
 
 

@@ -327,3 +327,50 @@ def test_sage_transform_first_is_the_same_layer(root, bias):
         for got, want, name in pairs:
             want = want.numpy()
             assert_close(got.cpu().numpy(), want, np.abs(want) + np.abs(want).mean(), rtol=1e-4, what="grad " + name)
+
+
+@pytest.mark.parametrize("spmm", [False, True])
+@pytest.mark.parametrize("f_in,f_out", [(40, 96), (96, 40), (64, 64)])
+def test_gcn_layer_weight_gradient_with_and_without_input_gradient(spmm, f_in, f_out):
+    """A layer whose input needs no gradient (the first of a model) may take
+    g_W = (A x)^T g instead of x^T (A^T g) when it widens: both against a dense float64
+    model, and against each other, on a directed graph with asymmetric weights."""
+    from jittorgeometric_amd.nn import GCNConv
+    from jittorgeometric_amd.ops import cootocsc, cootocsr
+    from util import rand_graph
+    rng = np.random.default_rng(41)
+    V, E = 6000, 70000                       # above the row count from which the matrix-core kernel is used
+    ei, w = rand_graph(rng, V, E, hubs=3)
+    x = rng.standard_normal((V, f_in)).astype(np.float32)
+    g = rng.standard_normal((V, f_out)).astype(np.float32)
+    csc, csr = cootocsc(to_gpu(ei), to_gpu(w), V), cootocsr(to_gpu(ei), to_gpu(w), V)
+    torch.manual_seed(3)
+    layer = GCNConv(f_in, f_out, spmm=spmm).to(dev())
+    with torch.no_grad():
+        layer.bias.normal_(0, 0.1)
+    grads = []
+    for needs in (True, False):
+        layer.zero_grad(set_to_none=True)
+        xt = to_gpu(x).requires_grad_(needs)
+        out = layer(xt, csc, csr)
+        out.backward(to_gpu(g))
+        grads.append((layer.weight.grad.clone(), layer.bias.grad.clone(), xt.grad))
+    A = dense_adj(ei, w, V)
+    x64 = torch.from_numpy(x.astype(np.float64)).requires_grad_(True)
+    W = layer.weight.detach().cpu().double().requires_grad_(True)
+    b = layer.bias.detach().cpu().double().requires_grad_(True)
+    ref = A @ (x64 @ W) + b
+    ref.backward(torch.from_numpy(g.astype(np.float64)))
+    # sums of absolute terms of the same chain, for the tolerance
+    Aa = A.abs()
+    gw_scale = (x64.detach().abs().t() @ (Aa.t() @ torch.from_numpy(np.abs(g).astype(np.float64)))).numpy()
+    gx_scale = ((Aa.t() @ torch.from_numpy(np.abs(g).astype(np.float64))) @ W.detach().abs().t()).numpy()
+    out_scale = (Aa @ (x64.detach().abs() @ W.detach().abs()) + b.detach().abs()).numpy()
+    assert_close(out.detach().cpu().numpy(), ref.detach().numpy(), out_scale, rtol=2e-5, what="out")
+    for (gw, gb, gx), needs in zip(grads, (True, False)):
+        assert_close(gw.cpu().numpy(), W.grad.numpy(), gw_scale, rtol=2e-5, what="grad W (input gradient %s)" % needs)
+        assert_close(gb.cpu().numpy(), b.grad.numpy(), np.abs(g).sum(0), rtol=2e-5, what="grad b")
+        if needs:
+            assert_close(gx.cpu().numpy(), x64.grad.numpy(), gx_scale, rtol=2e-5, what="grad x")
+        else:
+            assert gx is None
