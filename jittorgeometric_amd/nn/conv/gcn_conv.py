@@ -131,6 +131,8 @@ class GCNConv(nn.Module):
         zeros(self.bias)
 
     def forward(self, x, csc, csr):
+        if x.is_floating_point() and x.dtype != torch.float32:
+            x = x.to(torch.float32)      # the kernels and the parameters are float32; other widths are narrowed
         if self.aggregate_first and x.dim() == 2:
             agg = self.propagate_spmm(x=x, csr=csr) if self.spmm else self.propagate_msg(x=x, csc=csc, csr=csr)
             return xw(agg, self.weight, self.bias)

@@ -147,6 +147,8 @@ class SAGEConv(nn.Module):
         self._cached_edge_index = None
 
     def forward(self, x, edge_index=None, edge_weight=None, csc=None, csr=None):
+        if x.is_floating_point() and x.dtype != torch.float32:
+            x = x.to(torch.float32)      # the kernels and the parameters are float32; other widths are narrowed
         if csc is None or csr is None:
             cache = self._cached_edge_index
             if cache is None:

@@ -374,3 +374,39 @@ def test_gcn_layer_weight_gradient_with_and_without_input_gradient(spmm, f_in, f
             assert_close(gx.cpu().numpy(), x64.grad.numpy(), gx_scale, rtol=2e-5, what="grad x")
         else:
             assert gx is None
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_gcn_layer_without_bias_on_a_small_graph(dtype):
+    """No bias row, fewer rows than the matrix-core kernel takes, and float64 features (narrowed to
+    float32 like every other input): the same layer against a dense float64 model."""
+    from jittorgeometric_amd.nn import GCNConv
+    from jittorgeometric_amd.ops import cootocsc, cootocsr
+    from util import rand_graph
+    rng = np.random.default_rng(43)
+    V, E, f_in, f_out = 500, 4000, 24, 40
+    ei, w = rand_graph(rng, V, E, hubs=2)
+    x = rng.standard_normal((V, f_in)).astype(np.float32)
+    g = rng.standard_normal((V, f_out)).astype(np.float32)
+    csc, csr = cootocsc(to_gpu(ei), to_gpu(w), V), cootocsr(to_gpu(ei), to_gpu(w), V)
+    torch.manual_seed(4)
+    layer = GCNConv(f_in, f_out, bias=False, spmm=False).to(dev())
+    assert layer.bias is None
+    xt = to_gpu(x).to(dtype).requires_grad_(True)
+    out = layer(xt, csc, csr)
+    assert out.dtype == torch.float32
+    out.backward(to_gpu(g))
+    assert xt.grad.dtype == dtype
+    A = dense_adj(ei, w, V)
+    x64 = torch.from_numpy(x.astype(np.float64)).requires_grad_(True)
+    W = layer.weight.detach().cpu().double().requires_grad_(True)
+    ref = A @ (x64 @ W)
+    ref.backward(torch.from_numpy(g.astype(np.float64)))
+    g64 = torch.from_numpy(np.abs(g).astype(np.float64))
+    Aa = A.abs()
+    assert_close(out.detach().cpu().numpy(), ref.detach().numpy(), (Aa @ (x64.detach().abs() @ W.detach().abs())).numpy(),
+                 rtol=2e-5, what="out")
+    assert_close(layer.weight.grad.cpu().numpy(), W.grad.numpy(), (x64.detach().abs().t() @ (Aa.t() @ g64)).numpy(),
+                 rtol=2e-5, what="grad W")
+    assert_close(xt.grad.cpu().numpy(), x64.grad.numpy(), ((Aa.t() @ g64) @ W.detach().abs().t()).numpy(), rtol=2e-5,
+                 what="grad x")
