@@ -602,6 +602,13 @@ static int32_t spmm_call(const int32_t *off, const int32_t *idx, const float *w,
         return launch_status("spmm_csx");
     }
 
+    // Rows of two or more whole 64-float slabs are walked slab by slab as well: an L2 then holds the
+    // hot rows' 256-byte pieces of one slab instead of their whole rows, i.e. more hot rows, and the
+    // (index, weight) arrays read once more per slab are small next to the gathers.  Measured on
+    // V = 1M / E = 17M: F = 128 0.99 -> 0.98 ms, F = 256 2.12 -> 1.87 ms, F = 512 4.49 -> 3.64 ms;
+    // V = 2.45M / E = 126M: F = 256 13.0 -> 12.3 ms.  Slabs of 128 or 256 floats gain less, and a
+    // partial last slab loses (F = 100: 0.98 -> 1.34 ms), so other widths keep whole rows.
+    if (F >= 2 * kWave && F % kWave == 0) narrow_slabs = true;
     // h is read with x's vector width: its alignment counts too
     const uintptr_t bits = (uintptr_t)x | (uintptr_t)out | (uintptr_t)(fin ? fin->h : nullptr);
     const SpmmShape s = spmm_shape(R, E, F, (bits & 15) == 0, (bits & 7) == 0, narrow_slabs);
