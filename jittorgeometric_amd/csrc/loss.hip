@@ -188,7 +188,7 @@ __global__ __launch_bounds__(kCeThreads) void ce_grad_flat(const float *__restri
     const uint32_t total = (uint32_t)V * (uint32_t)C;
     const uint32_t quads = total / 4;
     const uint32_t t = blockIdx.x * kCeThreads + threadIdx.x;
-    auto one = [&](float xv, int row, int c, int64_t lab, float l) {
+    auto one = [&](float xv, int c, int64_t lab, float l) {
         return lab >= 0 && lab < C ? scale * (expf(xv - l) - (c == lab ? 1.f : 0.f)) : 0.f;
     };
     if (t < quads) {
@@ -204,14 +204,14 @@ __global__ __launch_bounds__(kCeThreads) void ce_grad_flat(const float *__restri
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const bool next = c + j >= C;
-            out[j] = one(xv[j], 0, next ? c + j - C : c + j, next ? lab_b : lab_a, next ? l_b : l_a);
+            out[j] = one(xv[j], next ? c + j - C : c + j, next ? lab_b : lab_a, next ? l_b : l_a);
         }
         __builtin_nontemporal_store(out, reinterpret_cast<f32x4 *>(grad + i));
     }
     if (t < total - quads * 4) {
         const uint32_t i = quads * 4 + t;
         const int row = (int)(i / (uint32_t)C), c = (int)(i - (uint32_t)row * (uint32_t)C);
-        grad[i] = one(x[i], 0, c, label_at(y32, y64, row), lse[row]);
+        grad[i] = one(x[i], c, label_at(y32, y64, row), lse[row]);
     }
 }
 
