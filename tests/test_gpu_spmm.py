@@ -72,7 +72,7 @@ def test_spmmcsr_fixture_with_int64_indices():
     assert SpmmCsr(x, csr, trans_A=False).tolist() == g["out_no_trans"]
 
 
-@pytest.mark.parametrize("F", [1, 2, 3, 7, 8, 31, 32, 33, 41, 47, 64, 65, 100, 128, 130, 256, 300, 602, 1030])
+@pytest.mark.parametrize("F", [1, 2, 3, 7, 8, 31, 32, 33, 41, 47, 64, 65, 100, 128, 130, 192, 256, 300, 320, 512, 602, 1024, 1030])
 def test_feature_widths(F):
     rng = np.random.default_rng(100 + F)
     V, E = 700, 9000
