@@ -410,3 +410,42 @@ def test_gcn_layer_without_bias_on_a_small_graph(dtype):
                  rtol=2e-5, what="grad W")
     assert_close(xt.grad.cpu().numpy(), x64.grad.numpy(), ((Aa.t() @ g64) @ W.detach().abs().t()).numpy(), rtol=2e-5,
                  what="grad x")
+
+
+def test_training_loop_follows_a_dense_float64_model():
+    """The training loop of examples/gcn_example.py:48-59,96-115 (two GCN layers, relu, mean
+    cross-entropy, Adam with weight decay) for 25 steps on the small configuration: the loss
+    of every step follows a dense float64 model started from the same parameters.  The graph
+    structures are built once and reused while the optimiser updates the parameters in place."""
+    from jittorgeometric_amd.nn import GCNConv, cross_entropy_loss, gcn_norm
+    from jittorgeometric_amd.ops import cootocsc, cootocsr
+    ei, V, x, y = cora_like()
+    eit, wt = gcn_norm(to_gpu(ei), None, V)
+    oei, ow = oracle.gcn_norm(ei, None, V)
+    csc, csr = cootocsc(eit, wt, V), cootocsr(eit, wt, V)
+    torch.manual_seed(11)
+    l1, l2 = GCNConv(1433, 64).to(dev()), GCNConv(64, 7).to(dev())
+    params = list(l1.parameters()) + list(l2.parameters())
+    ref_params = [p.detach().cpu().double().requires_grad_(True) for p in params]
+    opt = torch.optim.Adam(params, lr=0.01, weight_decay=5e-4)
+    ref_opt = torch.optim.Adam(ref_params, lr=0.01, weight_decay=5e-4)
+    A = dense_adj(oei, ow, V)
+    xt, yt = to_gpu(x), to_gpu(y)
+    x64, y64 = torch.from_numpy(x.astype(np.float64)), torch.from_numpy(y)
+    losses, ref_losses = [], []
+    for _ in range(25):
+        opt.zero_grad(set_to_none=True)
+        loss = cross_entropy_loss(l2(torch.relu(l1(xt, csc, csr)), csc, csr), yt)
+        loss.backward()
+        opt.step()
+        losses.append(loss.item())
+        ref_opt.zero_grad(set_to_none=True)
+        W1, b1, W2, b2 = ref_params
+        ref = torch.nn.functional.cross_entropy(A @ (torch.relu(A @ (x64 @ W1) + b1) @ W2) + b2, y64)
+        ref.backward()
+        ref_opt.step()
+        ref_losses.append(ref.item())
+    assert losses[-1] < losses[0], losses                     # random labels: slowly, but it goes down
+    assert np.allclose(losses, ref_losses, rtol=2e-4, atol=0), (losses, ref_losses)
+    # (single parameters are not compared: Adam divides by the running gradient magnitude, so an
+    # entry whose gradient is rounding noise moves by the learning rate in either model)
