@@ -221,3 +221,59 @@ def test_gat_config3_full_size_forward_and_backward():
                                      torch.from_numpy(dst.astype(np.int64)), V)
     ref.backward(torch.from_numpy(g.astype(np.float64)))
     check_against_fp64(raw["alpha"], out, ht.grad, ast.grad, adt.grad, ref, ref_alpha, h64, as64, ad64, g, row, dst, V)
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_gat_training_loop_follows_a_float64_model(fused):
+    """Two GATConv layers (the model of examples/gat_example.py:95-106: relu(x W), attention,
+    weighted sum; log-softmax + nll loss), 12 plain gradient steps: the loss of every step and the
+    parameters at the end follow a float64 model started from the same parameters, through the
+    fused kernels and through the unfused operator chain."""
+    from jittorgeometric_amd.nn import GATConv, nll_loss
+    from jittorgeometric_amd.ops import cootocsc
+    from jittorgeometric_amd import synthetic
+    V, F_in, C1, C2 = 1500, 48, 16, 5
+    ei = synthetic.chung_lu(V, 12000, 2.3, max_degree=300, seed=21)
+    loops = np.arange(V, dtype=np.int32)
+    ei = np.concatenate([ei[:, ei[0] != ei[1]], np.stack([loops, loops])], axis=1).astype(np.int32)
+    E = ei.shape[1]
+    rng = np.random.default_rng(22)
+    x = rng.standard_normal((V, F_in)).astype(np.float32)
+    y = rng.integers(0, C2, V)
+    csc = cootocsc(to_gpu(ei), torch.ones(E, device=dev()), V)
+    row = csc.row_indices.cpu().numpy().astype(np.int64)
+    dst = np.repeat(np.arange(V), np.diff(csc.column_offset.cpu().numpy())).astype(np.int64)
+    src_t, dst_t = torch.from_numpy(row), torch.from_numpy(dst)
+    torch.manual_seed(23)
+    l1, l2 = GATConv(F_in, C1, fused=fused).to(dev()), GATConv(C1, C2, fused=fused).to(dev())
+    params = list(l1.parameters()) + list(l2.parameters())
+    ref_params = [p.detach().cpu().double().requires_grad_(True) for p in params]
+    opt, ref_opt = torch.optim.SGD(params, lr=0.2), torch.optim.SGD(ref_params, lr=0.2)
+    xt, yt = to_gpu(x), to_gpu(y)
+    x64, y64 = torch.from_numpy(x.astype(np.float64)), torch.from_numpy(y)
+
+    def ref_layer(h_in, W, a):
+        C = W.shape[1]
+        h = torch.relu(h_in @ W).reshape(V, 1, C)
+        out, _ = torch_reference(h, a[:C, 0].reshape(1, C), a[C:, 0].reshape(1, C), src_t, dst_t, V)
+        return out.reshape(V, C)
+
+    losses, ref_losses = [], []
+    for _ in range(12):
+        opt.zero_grad(set_to_none=True)
+        out = l2(l1(xt, csc), csc)
+        loss = nll_loss(torch.log_softmax(out, dim=1), yt)
+        loss.backward()
+        opt.step()
+        losses.append(loss.item())
+        ref_opt.zero_grad(set_to_none=True)
+        W1, a1, W2, a2 = ref_params
+        ref = torch.nn.functional.nll_loss(torch.log_softmax(ref_layer(ref_layer(x64, W1, a1), W2, a2), dim=1), y64)
+        ref.backward()
+        ref_opt.step()
+        ref_losses.append(ref.item())
+    assert losses[-1] < losses[0], losses
+    assert np.allclose(losses, ref_losses, rtol=1e-4, atol=0), (losses, ref_losses)
+    for p, q in zip(params, ref_params):
+        q = q.detach().numpy()
+        assert_close(p.detach().cpu().numpy(), q, np.abs(q) + np.abs(q).mean(), rtol=1e-4, what="parameters after 12 steps")
