@@ -449,3 +449,57 @@ def test_training_loop_follows_a_dense_float64_model():
     assert np.allclose(losses, ref_losses, rtol=2e-4, atol=0), (losses, ref_losses)
     # (single parameters are not compared: Adam divides by the running gradient magnitude, so an
     # entry whose gradient is rounding noise moves by the learning rate in either model)
+
+
+@pytest.mark.parametrize("root", [False, True])
+def test_sage_training_loop_through_the_edge_list_route(root):
+    """The model of examples/sage_example.py:57-69 (two SAGEConv layers called with the edge list,
+    cached=True so that normalisation and conversion happen once, relu between, log-softmax +
+    nll loss), 15 plain gradient steps against a dense float64 model.  Both layers narrow, so
+    their backward passes take the transposed product at the output width."""
+    from jittorgeometric_amd.nn import SAGEConv, nll_loss
+    from jittorgeometric_amd import synthetic
+    V, f_in, hid, C = 6000, 96, 48, 7                  # above the row count from which the matrix-core kernel is used
+    ei = synthetic.chung_lu(V, 60000, 2.1, max_degree=900, seed=31)
+    rng = np.random.default_rng(32)
+    x = rng.standard_normal((V, f_in)).astype(np.float32)
+    y = rng.integers(0, C, V)
+    oei, ow = oracle.sage_norm(ei, None, V)
+    A = dense_adj(oei, ow, V)
+    torch.manual_seed(33)
+    l1 = SAGEConv(f_in, hid, cached=True, root_weight=root).to(dev())
+    l2 = SAGEConv(hid, C, cached=True, root_weight=root).to(dev())
+    params = list(l1.parameters()) + list(l2.parameters())
+    names = [n for n, _ in l1.named_parameters()]
+    ref_params = [p.detach().cpu().double().requires_grad_(True) for p in params]
+    opt, ref_opt = torch.optim.SGD(params, lr=0.3), torch.optim.SGD(ref_params, lr=0.3)
+    xt, yt, eit = to_gpu(x), to_gpu(y), to_gpu(ei)
+    x64, y64 = torch.from_numpy(x.astype(np.float64)), torch.from_numpy(y)
+    n = len(names)
+
+    def ref_layer(h, ps):
+        p = dict(zip(names, ps))
+        out = (A @ h) @ p["weight1"]
+        if root:
+            out = out + h @ p["root_weight"]
+        return out + p["bias"]
+
+    losses, ref_losses = [], []
+    for _ in range(15):
+        opt.zero_grad(set_to_none=True)
+        out = l2(torch.relu(l1(xt, eit)), eit)
+        loss = nll_loss(torch.log_softmax(out, dim=1), yt)
+        loss.backward()
+        opt.step()
+        losses.append(loss.item())
+        ref_opt.zero_grad(set_to_none=True)
+        ref_out = ref_layer(torch.relu(ref_layer(x64, ref_params[:n])), ref_params[n:])
+        ref = torch.nn.functional.nll_loss(torch.log_softmax(ref_out, dim=1), y64)
+        ref.backward()
+        ref_opt.step()
+        ref_losses.append(ref.item())
+    assert l1._cached_edge_index is not None and losses[-1] < losses[0], losses
+    assert np.allclose(losses, ref_losses, rtol=1e-4, atol=0), (losses, ref_losses)
+    for p, q in zip(params, ref_params):
+        q = q.detach().numpy()
+        assert_close(p.detach().cpu().numpy(), q, np.abs(q) + np.abs(q).mean(), rtol=1e-4, what="parameters after 15 steps")
