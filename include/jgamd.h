@@ -137,6 +137,54 @@ int32_t jgamd_spmm_csx_axpby(const int32_t *off, const int32_t *idx, const float
                              const float *h, int32_t h_rows, int32_t R, int32_t C, int64_t E,
                              int32_t F, void *ws, size_t ws_bytes, void *stream);
 
+/* ------------------------------------------------------------------------
+ * Per-graph plans.  The reference's aggregate is one launch per call
+ * (ops/cpp/aggregate_op.cc:93-106); how the merge-path kernels here cut a
+ * matrix into chunks, and which chunks hold pieces of a cut row, depends on the
+ * offsets alone, so it can be computed once per graph, kept by the caller (like
+ * the CSR / CSC objects themselves, data/data.py:42-52) and handed to the
+ * *_planned entry points, which then skip the per-call search and launch the
+ * piece kernels over the listed chunks only.  A plan is an opaque block of
+ * device memory owned by the caller, 256-byte aligned, valid for the offsets
+ * array (contents, R, E) it was built from; results with and without a plan are
+ * bit-identical.
+ *
+ *   kind  JGAMD_PLAN_SPMM   chunks for jgamd_spmm_csx_planned
+ *         JGAMD_PLAN_GAT    chunks for jgamd_gat_fwd / jgamd_gat_bwd (of the
+ *                           CSC offsets / of the transposed offsets)
+ *         JGAMD_PLAN_TILES  tile -> column map for jgamd_edge_softmax_*_planned
+ *                           and for products with rows of 1, 2, 4 or 8 floats
+ *
+ * jgamd_csx_plan_counts copies the lengths of the two chunk lists of a SPMM /
+ * GAT plan to the host (it waits for `stream`: the one synchronising call of
+ * this library besides the *_timed ones).  Passing them as n_fix / n_grp lets a
+ * planned call size or skip its piece kernels: 0 = the list is empty, nothing
+ * is launched for it (a graph without rows longer than half a chunk is then
+ * one launch per product); -1 = unknown, the kernels read the lengths from the
+ * plan.
+ */
+#define JGAMD_PLAN_SPMM 0
+#define JGAMD_PLAN_GAT 1
+#define JGAMD_PLAN_TILES 2
+int32_t jgamd_csx_plan_bytes(int32_t R, int64_t E, int32_t kind, size_t *bytes);
+int32_t jgamd_csx_plan(const int32_t *off, int32_t R, int64_t E, int32_t kind, void *plan,
+                       size_t plan_bytes, void *stream);
+int32_t jgamd_csx_plan_counts(const void *plan, int32_t *n_fix, int32_t *n_grp, void *stream);
+
+/* jgamd_spmm_csx_axpby with the partition taken from a plan of `off`:
+ * plan = a JGAMD_PLAN_SPMM plan, tiles = a JGAMD_PLAN_TILES plan (either may be
+ * NULL, not both; rows of 1, 2, 4 or 8 floats use `tiles` when it is given,
+ * every other width needs `plan`).  beta = 1, alpha = 0 or h = NULL is the
+ * plain product of AggregateOp::jit_run (ops/cpp/aggregate_op.cc:26-71).
+ * The workspace holds row pieces only (jgamd_spmm_csx_planned_workspace).
+ */
+int32_t jgamd_spmm_csx_planned_workspace(int32_t R, int64_t E, int32_t F, size_t *bytes);
+int32_t jgamd_spmm_csx_planned(const void *plan, const void *tiles, int32_t n_fix, int32_t n_grp,
+                               const int32_t *off, const int32_t *idx, const float *w,
+                               const float *x, float *out, float beta, float alpha,
+                               const float *h, int32_t h_rows, int32_t R, int32_t C, int64_t E,
+                               int32_t F, void *ws, size_t ws_bytes, void *stream);
+
 /* jgamd_spmm_csx without a workspace argument.  No counterpart in the
  * reference: it is for callers that cannot allocate device memory or own a
  * workspace (code under HIP graph capture, tight serving loops, harnesses
@@ -186,6 +234,15 @@ int32_t jgamd_edge_softmax_fwd(const int32_t *off, const float *x, float *y, int
 int32_t jgamd_edge_softmax_bwd(const int32_t *off, const float *y, const float *g, float *dx,
                                int32_t V, int64_t E, int32_t H, void *ws, size_t ws_bytes,
                                void *stream);
+/* The same two with the tile -> column map taken from a JGAMD_PLAN_TILES plan
+ * of `off` instead of being computed by a launch of its own per call (1, 2, 4
+ * and 8 heads use it; other head counts ignore it). */
+int32_t jgamd_edge_softmax_fwd_planned(const void *tiles, const int32_t *off, const float *x,
+                                       float *y, int32_t V, int64_t E, int32_t H, void *ws,
+                                       size_t ws_bytes, void *stream);
+int32_t jgamd_edge_softmax_bwd_planned(const void *tiles, const int32_t *off, const float *y,
+                                       const float *g, float *dx, int32_t V, int64_t E,
+                                       int32_t H, void *ws, size_t ws_bytes, void *stream);
 
 /* ------------------------------------------------------------------------
  * Vertex -> edge copy.  Replaces ScattertoedgeOp::jit_run
@@ -213,8 +270,8 @@ int32_t jgamd_scatter_to_edge(const int32_t *off, const int32_t *idx, const floa
  * H = 1, D = C reproduces the reference's single head.
  */
 int32_t jgamd_gat_fwd_workspace(int32_t V, int64_t E, int32_t H, int32_t D, size_t *bytes);
-int32_t jgamd_gat_fwd(const int32_t *off, const int32_t *idx, const float *h,
-                      const float *a_src, const float *a_dst, float slope, float *el,
+int32_t jgamd_gat_fwd(const void *plan, int32_t n_fix, int32_t n_grp, const int32_t *off,
+                      const int32_t *idx, const float *h, const float *a_src, const float *a_dst, float slope, float *el,
                       float *er, float *smax, float *ssum, float *alpha, float *out,
                       int32_t V, int64_t E, int32_t H, int32_t D, void *ws, size_t ws_bytes,
                       void *stream);
@@ -232,7 +289,8 @@ int32_t jgamd_gat_fwd(const int32_t *off, const int32_t *idx, const float *h,
  * edgesoftmaxbackward that Jittor autograd builds for gat_conv.py:61-83.
  */
 int32_t jgamd_gat_bwd_workspace(int32_t V, int64_t E, int32_t H, int32_t D, size_t *bytes);
-int32_t jgamd_gat_bwd(const int32_t *off, const int32_t *idx, const int32_t *t_off,
+int32_t jgamd_gat_bwd(const void *t_plan, int32_t n_fix, int32_t n_grp, const void *tiles,
+                      const int32_t *off, const int32_t *idx, const int32_t *t_off,
                       const int32_t *t_idx, const int32_t *t_inv, const float *h, const float *a_src,
                       const float *a_dst, float slope, const float *el, const float *er,
                       const float *smax, const float *ssum, const float *out,

@@ -40,10 +40,44 @@ size_t scan_ws_ints(int64_t n);
 int32_t exclusive_scan_i32(const int32_t *in, int32_t *out, int64_t n, int32_t *sums_ws,
                            hipStream_t s);
 
+// ---- per-graph partition for the merge-path and tile kernels (plan.hip) ------
+constexpr int kPlanGroup = 32;             // chunks per group of pre-summed row pieces
+constexpr int kTileEntriesWide = 2048;     // entries per tile at 1 or 2 floats per entry
+constexpr int kTileEntriesNarrow = 1024;   // and at 4 or 8
+
+struct ChunkPlanShape {
+    int chunk, nchunks, ngroups;
+    size_t header_bytes, start_bytes, fix_bytes, grp_bytes;
+};
+// start[k] = (row, entry) at which chunk k begins, k <= nchunks.  fix / grp: ascending lists of
+// the chunks whose first row has earlier pieces / of the groups a row continues past, their
+// lengths in counts[0] / counts[1]; all three NULL when only the starts were computed (every
+// chunk and group is then looked at).
+struct ChunkPlan {
+    const int2 *start;
+    const int32_t *fix, *grp, *counts;
+    int chunk, nchunks;
+};
+struct TilePlan {
+    const int32_t *tile_first, *tile_last;
+};
+int spmm_chunk_for(int64_t M);      // items per wavefront of the product (spmm.hip)
+int gat_chunk_for(int64_t M);       // and of the fused attention kernels (gat.hip)
+ChunkPlanShape chunk_plan_shape(int kind, int32_t R, int64_t E);
+size_t chunk_plan_bytes(int kind, int32_t R, int64_t E);
+ChunkPlan chunk_plan_view(int kind, int32_t R, int64_t E, const void *plan);
+void chunk_starts_enqueue(const int32_t *off, int32_t R, int64_t E, int chunk, int nchunks, int2 *start, hipStream_t s);
+size_t tile_plan_bytes(int64_t E);
+TilePlan tile_plan_view(int64_t E, int T, const void *plan);
+void tile_columns_enqueue(const int32_t *off, int32_t V, int64_t E, int T, int32_t *tile_first, int32_t *tile_last,
+                          hipStream_t s);
+
 // ---- row-gather SpMM for use by other kernels' host code (spmm.hip) ---------
 size_t spmm_ws_bytes(int32_t R, int64_t E, int32_t F);
+// tiles: the tile plan of `off` (rows of 1, 2, 4 or 8 floats take the tile kernels), or NULL
 int32_t spmm_enqueue(const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out, int32_t R,
-                     int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, hipStream_t s);
+                     int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, hipStream_t s,
+                     const void *tiles = nullptr);
 // the same product walked one 64-float slab of the feature rows at a time (spmm_blocked.hip)
 // k0 / k1: optional events recorded on s right before and after the gather kernel; x_stride:
 // floats between the rows of x when they are padded apart (0 = F)
@@ -56,13 +90,13 @@ int32_t spmm_enqueue_slabs(const int32_t *off, const int32_t *idx, const float *
 bool edge_softmax_flat_supported(int H);
 size_t entry_tiles_ws_bytes(int64_t E);
 void edge_softmax_flat_enqueue(bool fwd, const int32_t *off, const float *a, const float *b, float *out, int32_t V,
-                               int64_t E, int32_t H, void *ws, hipStream_t s);
+                               int64_t E, int32_t H, void *ws, hipStream_t s, const void *tiles = nullptr);
 
 // ---- gather-sum for rows of 1, 2, 4 or 8 floats (entry_tiles.hip) ----------
 // Same result as the wide-row product; shares entry_tiles_ws_bytes(E) of workspace.
 bool narrow_spmm_supported(int F, const void *x);
 void narrow_spmm_enqueue(const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out, int32_t R,
-                         int32_t C, int64_t E, int32_t F, void *ws, hipStream_t s);
+                         int32_t C, int64_t E, int32_t F, void *ws, hipStream_t s, const void *tiles = nullptr);
 
 #ifdef __HIPCC__
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }

@@ -11,6 +11,7 @@ namespace jg {
 
 constexpr int kColThreads = 256;
 constexpr int kColStripe = 512;    // rows per block: about 2000 blocks at V = 10^6, eight per CU, to keep enough loads in flight
+constexpr int kColMinStripe = 16;
 constexpr int kColMaxBlocks = 2048;     // more rows per block beyond that: the second stage reads one partial row per block
 
 // W = floats per lane (1, or 4 when F % 4 == 0 and x is 16-byte aligned): a row is then F / W
@@ -90,7 +91,12 @@ using namespace jg;
 static int col_stripe(int64_t R)
 {
     const int64_t s = ceil_div(R > 0 ? R : 1, kColMaxBlocks);
-    return s > kColStripe ? (int)(s < 0x7fffffff ? s : 0x7fffffff) : kColStripe;
+    if (s > kColStripe) return (int)(s < 0x7fffffff ? s : 0x7fffffff);
+    // a small matrix: shorter stripes, so that a few thousand rows are still a block or two per
+    // compute unit instead of half a dozen blocks in all
+    int stripe = kColStripe;
+    while (stripe > kColMinStripe && R / stripe < 512) stripe >>= 1;
+    return stripe;
 }
 static int col_blocks(int64_t R) { return (int)ceil_div(R > 0 ? R : 1, col_stripe(R)); }
 static size_t colsum_ws(int64_t R, int32_t F) { return carve_bytes((size_t)col_blocks(R) * F, 4); }

@@ -23,6 +23,8 @@
 // by the 1 GB the rows move, about equally; sharing a read of the rows between two products
 // does not pay at this arithmetic intensity, which is why the weight gradient keeps its own
 // pass.
+#include <mutex>
+
 #include "common.h"
 
 namespace jg {
@@ -154,13 +156,15 @@ __global__ __launch_bounds__(WAVES *kWave) void dense_rows(DenseArgs a)
 
 template <int KQ, int WAVES> static void launch_dense(const DenseArgs &a, hipStream_t s)
 {
-    const size_t lds = (size_t)16 * KQ * kDenseCols * sizeof(float);
-    static bool raised = false;
-    if (!raised && lds > 64 * 1024) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&dense_rows<KQ, WAVES>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        raised = true;
-    }
+    constexpr size_t lds = (size_t)16 * KQ * kDenseCols * sizeof(float);
+    // once per instantiation, whichever thread gets here first (the attribute belongs to the
+    // function, not to the call)
+    static std::once_flag raised;
+    if (lds > 64 * 1024)
+        std::call_once(raised, [] {
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&dense_rows<KQ, WAVES>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        });
     const int tiles = (a.V + kDenseRows - 1) / kDenseRows;
     const int per_cu = (int)((160 * 1024) / lds) > 0 ? (int)((160 * 1024) / lds) : 1;
     int blocks = 256 * (per_cu > 2 ? 2 : per_cu);

@@ -379,8 +379,9 @@ static int list_long_columns(const int32_t *off, int32_t V, int64_t E, void *ws,
     return cap;
 }
 
-JG_EXPORT int32_t jgamd_edge_softmax_fwd(const int32_t *off, const float *x, float *y, int32_t V, int64_t E,
-                                         int32_t H, void *ws, size_t ws_bytes, void *stream)
+// tiles: the tile plan of `off` (jgamd_csx_plan, JGAMD_PLAN_TILES) or NULL
+static int32_t softmax_fwd(const void *tiles, const int32_t *off, const float *x, float *y, int32_t V, int64_t E,
+                           int32_t H, void *ws, size_t ws_bytes, void *stream)
 {
     if (int32_t rc = check_softmax("edge_softmax_fwd", off, x, y, V, E, H)) return rc;
     if (V == 0 || E == 0) return 0;
@@ -392,7 +393,8 @@ JG_EXPORT int32_t jgamd_edge_softmax_fwd(const int32_t *off, const float *x, flo
     }
     if (int32_t rc = check_softmax_ws("edge_softmax_fwd", ws, ws_bytes, V, E)) return rc;
     if (use_flat(H)) {
-        edge_softmax_flat_enqueue(true, off, x, nullptr, y, V, E, H, static_cast<char *>(ws) + group_ws_bytes(V, E), s);
+        edge_softmax_flat_enqueue(true, off, x, nullptr, y, V, E, H, static_cast<char *>(ws) + group_ws_bytes(V, E), s,
+                                  tiles);
         return launch_status("edge_softmax_fwd");
     }
     switch (pick_group(E, V, H)) {
@@ -408,8 +410,29 @@ JG_EXPORT int32_t jgamd_edge_softmax_fwd(const int32_t *off, const float *x, flo
     return launch_status("edge_softmax_fwd");
 }
 
-JG_EXPORT int32_t jgamd_edge_softmax_bwd(const int32_t *off, const float *y, const float *g, float *dx, int32_t V,
-                                         int64_t E, int32_t H, void *ws, size_t ws_bytes, void *stream)
+JG_EXPORT int32_t jgamd_edge_softmax_fwd(const int32_t *off, const float *x, float *y, int32_t V, int64_t E,
+                                         int32_t H, void *ws, size_t ws_bytes, void *stream)
+{
+    return softmax_fwd(nullptr, off, x, y, V, E, H, ws, ws_bytes, stream);
+}
+
+static int32_t check_tiles(const char *who, const void *tiles)
+{
+    if (!tiles) return fail(JGAMD_ERR_NULL, "%s: tiles is NULL", who);
+    if (((uintptr_t)tiles & 255) != 0) return fail(JGAMD_ERR_ALIGN, "%s: tiles not 256-byte aligned", who);
+    return 0;
+}
+
+JG_EXPORT int32_t jgamd_edge_softmax_fwd_planned(const void *tiles, const int32_t *off, const float *x, float *y,
+                                                 int32_t V, int64_t E, int32_t H, void *ws, size_t ws_bytes,
+                                                 void *stream)
+{
+    if (int32_t rc = check_tiles("edge_softmax_fwd_planned", tiles)) return rc;
+    return softmax_fwd(tiles, off, x, y, V, E, H, ws, ws_bytes, stream);
+}
+
+static int32_t softmax_bwd(const void *tiles, const int32_t *off, const float *y, const float *g, float *dx, int32_t V,
+                           int64_t E, int32_t H, void *ws, size_t ws_bytes, void *stream)
 {
     if (int32_t rc = check_softmax("edge_softmax_bwd", off, y, dx, V, E, H)) return rc;
     if (E > 0 && !g) return fail(JGAMD_ERR_NULL, "edge_softmax_bwd: g is NULL");
@@ -422,7 +445,8 @@ JG_EXPORT int32_t jgamd_edge_softmax_bwd(const int32_t *off, const float *y, con
     }
     if (int32_t rc = check_softmax_ws("edge_softmax_bwd", ws, ws_bytes, V, E)) return rc;
     if (use_flat(H)) {
-        edge_softmax_flat_enqueue(false, off, y, g, dx, V, E, H, static_cast<char *>(ws) + group_ws_bytes(V, E), s);
+        edge_softmax_flat_enqueue(false, off, y, g, dx, V, E, H, static_cast<char *>(ws) + group_ws_bytes(V, E), s,
+                                  tiles);
         return launch_status("edge_softmax_bwd");
     }
     switch (pick_group(E, V, H)) {
@@ -437,6 +461,20 @@ JG_EXPORT int32_t jgamd_edge_softmax_bwd(const int32_t *off, const float *y, con
     hipLaunchKernelGGL(edge_softmax_bwd_long, dim3((unsigned)cap), dim3(kLongThreads), 0, s, off, y, g, dx, H, counter,
                        list);
     return launch_status("edge_softmax_bwd");
+}
+
+JG_EXPORT int32_t jgamd_edge_softmax_bwd(const int32_t *off, const float *y, const float *g, float *dx, int32_t V,
+                                         int64_t E, int32_t H, void *ws, size_t ws_bytes, void *stream)
+{
+    return softmax_bwd(nullptr, off, y, g, dx, V, E, H, ws, ws_bytes, stream);
+}
+
+JG_EXPORT int32_t jgamd_edge_softmax_bwd_planned(const void *tiles, const int32_t *off, const float *y, const float *g,
+                                                 float *dx, int32_t V, int64_t E, int32_t H, void *ws,
+                                                 size_t ws_bytes, void *stream)
+{
+    if (int32_t rc = check_tiles("edge_softmax_bwd_planned", tiles)) return rc;
+    return softmax_bwd(tiles, off, y, g, dx, V, E, H, ws, ws_bytes, stream);
 }
 
 JG_EXPORT int32_t jgamd_scatter_to_edge(const int32_t *off, const int32_t *idx, const float *x, float *out, int32_t V,

@@ -7,7 +7,8 @@
 // but a tile of T consecutive entries of the [E,H] array:
 //
 //   0. tile columns : one thread per column records, for every tile, the
-//                     column of its first and of its last entry.
+//                     column of its first and of its last entry (plan.hip;
+//                     once per graph when the caller keeps a tile plan).
 //   1. tile kernel  : a lane holds K consecutive entries (all H heads, loaded
 //                     as vectors).  Each entry's column is found from the
 //                     offsets staged in LDS; per-column totals (max, then sum
@@ -36,6 +37,7 @@ constexpr int kFlatWaves = kFlatThreads / kWave;
 template <int H> struct FlatShape {
     static constexpr int K = H <= 2 ? 8 : 4;        // entries per lane
     static constexpr int T = kFlatThreads * K;      // entries per tile
+    static_assert(T == (H <= 2 ? kTileEntriesWide : kTileEntriesNarrow), "tile sizes of the tile plan");
 };
 
 struct FlatMeta {
@@ -74,29 +76,6 @@ struct OpAdd {
 __device__ __forceinline__ int covered_entries(const int32_t *__restrict__ off, int V, int E)
 {
     return min(max(off[V], 0), E);
-}
-
-// tile_first[i] / tile_last[i] = column of the first / last entry of tile i.
-// One thread per column: it owns the entries [off[c], off[c+1]) and marks the
-// tiles whose first or last entry falls among them.
-__global__ void esm_tile_columns(const int32_t *__restrict__ off, int V, int E, int T, int ntiles,
-                                 int32_t *__restrict__ tile_first, int32_t *__restrict__ tile_last,
-                                 float *__restrict__ zero_rows = nullptr, int zero_width = 0)
-{
-    const int c = blockIdx.x * blockDim.x + threadIdx.x;
-    if (c >= V) return;
-    // the gather-sum starts from zeroed rows (empty columns belong to no tile): this thread's row
-    if (zero_rows)
-        for (int h = 0; h < zero_width; h++) zero_rows[(int64_t)c * zero_width + h] = 0.f;
-    // entries past off[V] belong to no column (offsets of a conversion that dropped keys):
-    // only the tiles that hold covered entries get a first and a last column
-    const int covered = covered_entries(off, V, E);
-    const int s = off[c], e = min(off[c + 1], covered);
-    if (e <= s) return;
-    ntiles = (covered + T - 1) / T;
-    for (int i = (s + T - 1) / T; i < ntiles && (int64_t)i * T < e; i++) tile_first[i] = c;
-    for (int i = s / T + 1; i <= ntiles && (int64_t)i * T <= e; i++) tile_last[i - 1] = c;   // last entry i*T - 1
-    if (e == covered) tile_last[ntiles - 1] = c;
 }
 
 // A tile that holds no covered entry: no column is open in it, and (zero_out) its slots of the
@@ -564,8 +543,10 @@ __global__ __launch_bounds__(kFlatThreads) void esm_bwd_tile(const int32_t *__re
 // wide-row kernel gives a whole wavefront to one entry; with a handful of floats
 // per row that leaves most lanes idle, so here a lane gathers K entries and the
 // per-column totals come from the segmented scan.  Columns inside the tile are
-// written by the tile kernel, crossing ones by esm_merge; out is zeroed first, by the
-// tile-columns kernel (empty columns belong to no tile).
+// written by the tile kernel, crossing ones by esm_merge.  Empty columns hold no
+// entry of any tile: a tile answers for the empty ones between the previous
+// tile's last column and its own last column (the last covered tile for those
+// after it as well) and writes their zeros.
 
 template <int H>
 __global__ __launch_bounds__(kFlatThreads) void esm_colsum_tile(const int32_t *__restrict__ off,
@@ -582,6 +563,8 @@ __global__ __launch_bounds__(kFlatThreads) void esm_colsum_tile(const int32_t *_
     const int tile = blockIdx.x;
     const int t0 = tile * T;
     const int covered = covered_entries(off, V, E);
+    if (covered == 0 && tile == 0)          // no entry at all: every column is empty
+        for (int64_t p = threadIdx.x; p < (int64_t)V * H; p += kFlatThreads) out[p] = 0.f;
     if (skip_uncovered_tile<H, T>(t0, covered, E, meta + tile, nullptr)) return;
     const int c_lo = min(max(tile_first[tile], 0), V - 1);
     const int c_hi = min(max(tile_last[tile], c_lo), V - 1);
@@ -618,15 +601,23 @@ __global__ __launch_bounds__(kFlatThreads) void esm_colsum_tile(const int32_t *_
         piece<H>(pieces, tile, 0)[threadIdx.x] = L.tot[threadIdx.x];
         piece<H>(pieces, tile, 1)[threadIdx.x] = L.tot[cols.tail_slot * H + threadIdx.x];
     }
-    // the columns that lie inside the tile: one thread each
-    for (int c = c_lo + (int)threadIdx.x; c <= c_hi; c += kFlatThreads) {
-        const int cs = cols.staged ? L.off[c - c_lo] : off[c];
-        const int ce = cols.staged ? L.off[c - c_lo + 1] : off[c + 1];
-        if (ce > cs && cs >= t0 && ce <= t0 + n) {
-            float t[H];
-            read_totals<H>(L.tot, cs - t0, t);
+    // the columns that lie inside the tile, and the empty ones this tile answers for: one thread each
+    const int c_from = tile == 0 ? 0 : min(max(tile_last[tile - 1] + 1, 0), c_lo);
+    const int c_to = t0 + T >= covered ? V - 1 : c_hi;
+    for (int c = c_from + (int)threadIdx.x; c <= c_to; c += kFlatThreads) {
+        const bool inside = c >= c_lo && c <= c_hi;
+        const int cs = !inside ? 0 : cols.staged ? L.off[c - c_lo] : off[c];
+        const int ce = !inside ? 0 : cols.staged ? L.off[c - c_lo + 1] : off[c + 1];
+        if (ce > cs) {
+            if (cs >= t0 && ce <= t0 + n) {
+                float t[H];
+                read_totals<H>(L.tot, cs - t0, t);
 #pragma unroll
-            for (int h = 0; h < H; h++) out[(int64_t)c * H + h] = t[h];
+                for (int h = 0; h < H; h++) out[(int64_t)c * H + h] = t[h];
+            }
+        } else {
+#pragma unroll
+            for (int h = 0; h < H; h++) out[(int64_t)c * H + h] = 0.f;
         }
     }
 }
@@ -767,9 +758,18 @@ size_t entry_tiles_ws_bytes(int64_t E)
            2 * carve_bytes(tiles, 4);
 }
 
+// (first, last) column per tile: from the caller's tile plan, or computed into the workspace now
+static TilePlan tile_columns(const void *tiles, const int32_t *off, int32_t V, int64_t E, int T, int32_t *tile_first,
+                             int32_t *tile_last, hipStream_t s)
+{
+    if (tiles) return tile_plan_view(E, T, tiles);
+    tile_columns_enqueue(off, V, E, T, tile_first, tile_last, s);
+    return TilePlan{tile_first, tile_last};
+}
+
 template <int H>
 static void flat_launch(bool fwd, const int32_t *off, const float *a, const float *b, float *out, int32_t V, int64_t E,
-                        void *ws, hipStream_t s)
+                        void *ws, hipStream_t s, const void *tiles)
 {
     constexpr int T = FlatShape<H>::T;
     const int ntiles = flat_tiles(E, H);
@@ -778,14 +778,12 @@ static void flat_launch(bool fwd, const int32_t *off, const float *a, const floa
     FlatMeta *meta = carve.take<FlatMeta>(cap);
     float *pieces = carve.take<float>(cap * 4 * 8);
     float *stat = carve.take<float>(cap * 2 * 8);
-    int32_t *tile_first = carve.take<int32_t>(cap);
-    int32_t *tile_last = carve.take<int32_t>(cap);
+    const TilePlan tp = tile_columns(tiles, off, V, E, T, carve.take<int32_t>(cap), carve.take<int32_t>(cap), s);
+    const int32_t *tile_first = tp.tile_first, *tile_last = tp.tile_last;
     // Through LDS pays once a lane's K*H floats span 64 bytes or more (measured:
     // 1 head 42 vs 44 us direct, 8 heads 390 vs 319 us); JGAMD_SOFTMAX_STAGE=0/1 overrides.
     const char *env = getenv("JGAMD_SOFTMAX_STAGE");
     const int staged = env ? atoi(env) : (H >= 2 ? 1 : 0);
-    hipLaunchKernelGGL(esm_tile_columns, dim3((unsigned)ceil_div(V, 256)), dim3(256), 0, s, off, V, (int)E, T, ntiles,
-                       tile_first, tile_last);
     if (fwd) {
         hipLaunchKernelGGL(esm_fwd_tile<H>, dim3(ntiles), dim3(kFlatThreads), 0, s, off, a, out, tile_first, tile_last,
                            V, (int)E, meta, pieces, staged);
@@ -805,7 +803,7 @@ static void flat_launch(bool fwd, const int32_t *off, const float *a, const floa
 
 template <int H>
 static void colsum_launch(const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out, int32_t R,
-                          int32_t C, int64_t E, void *ws, hipStream_t s)
+                          int32_t C, int64_t E, void *ws, hipStream_t s, const void *tiles)
 {
     constexpr int T = FlatShape<H>::T;
     const int ntiles = flat_tiles(E, H);
@@ -814,10 +812,8 @@ static void colsum_launch(const int32_t *off, const int32_t *idx, const float *w
     FlatMeta *meta = carve.take<FlatMeta>(cap);
     float *pieces = carve.take<float>(cap * 4 * 8);
     float *stat = carve.take<float>(cap * 2 * 8);
-    int32_t *tile_first = carve.take<int32_t>(cap);
-    int32_t *tile_last = carve.take<int32_t>(cap);
-    hipLaunchKernelGGL(esm_tile_columns, dim3((unsigned)ceil_div(R, 256)), dim3(256), 0, s, off, R, (int)E, T, ntiles,
-                       tile_first, tile_last, out, H);
+    const TilePlan tp = tile_columns(tiles, off, R, E, T, carve.take<int32_t>(cap), carve.take<int32_t>(cap), s);
+    const int32_t *tile_first = tp.tile_first, *tile_last = tp.tile_last;
     hipLaunchKernelGGL(esm_colsum_tile<H>, dim3(ntiles), dim3(kFlatThreads), 0, s, off, idx, w, x, out, tile_first,
                        tile_last, R, C, (int)E, meta, pieces);
     hipLaunchKernelGGL((esm_merge<H, T, false>), dim3((unsigned)ceil_div(ntiles, kFlatWaves)), dim3(kFlatThreads), 0, s,
@@ -833,25 +829,25 @@ bool narrow_spmm_supported(int F, const void *x)
 }
 
 void narrow_spmm_enqueue(const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out, int32_t R,
-                         int32_t C, int64_t E, int32_t F, void *ws, hipStream_t s)
+                         int32_t C, int64_t E, int32_t F, void *ws, hipStream_t s, const void *tiles)
 {
     switch (F) {
-    case 1: colsum_launch<1>(off, idx, w, x, out, R, C, E, ws, s); break;
-    case 2: colsum_launch<2>(off, idx, w, x, out, R, C, E, ws, s); break;
-    case 4: colsum_launch<4>(off, idx, w, x, out, R, C, E, ws, s); break;
-    default: colsum_launch<8>(off, idx, w, x, out, R, C, E, ws, s); break;
+    case 1: colsum_launch<1>(off, idx, w, x, out, R, C, E, ws, s, tiles); break;
+    case 2: colsum_launch<2>(off, idx, w, x, out, R, C, E, ws, s, tiles); break;
+    case 4: colsum_launch<4>(off, idx, w, x, out, R, C, E, ws, s, tiles); break;
+    default: colsum_launch<8>(off, idx, w, x, out, R, C, E, ws, s, tiles); break;
     }
 }
 
 // fwd: a = x, b unused; bwd: a = y, b = g.  V > 0, E > 0, off[V] == E.
 void edge_softmax_flat_enqueue(bool fwd, const int32_t *off, const float *a, const float *b, float *out, int32_t V,
-                               int64_t E, int32_t H, void *ws, hipStream_t s)
+                               int64_t E, int32_t H, void *ws, hipStream_t s, const void *tiles)
 {
     switch (H) {
-    case 1: flat_launch<1>(fwd, off, a, b, out, V, E, ws, s); break;
-    case 2: flat_launch<2>(fwd, off, a, b, out, V, E, ws, s); break;
-    case 4: flat_launch<4>(fwd, off, a, b, out, V, E, ws, s); break;
-    default: flat_launch<8>(fwd, off, a, b, out, V, E, ws, s); break;
+    case 1: flat_launch<1>(fwd, off, a, b, out, V, E, ws, s, tiles); break;
+    case 2: flat_launch<2>(fwd, off, a, b, out, V, E, ws, s, tiles); break;
+    case 4: flat_launch<4>(fwd, off, a, b, out, V, E, ws, s, tiles); break;
+    default: flat_launch<8>(fwd, off, a, b, out, V, E, ws, s, tiles); break;
     }
 }
 

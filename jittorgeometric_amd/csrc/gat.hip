@@ -59,26 +59,6 @@ __device__ __forceinline__ float lrelu(float z, float slope) { return z > 0.f ? 
 // library expf costs ~20 VALU instructions per call and made these kernels VALU-bound.
 __device__ __forceinline__ float fast_exp(float x) { return __expf(x); }
 
-// chunk_row[k] = the row owning merged position k*chunk (row r owns positions
-// off[r]+r .. off[r+1]+r, an increasing function of r): binary search per chunk.
-__global__ void gat_chunk_rows(const int32_t *__restrict__ off, int R, int chunk, int nchunks,
-                               int32_t *__restrict__ chunk_row)
-{
-    const int k = blockIdx.x * blockDim.x + threadIdx.x;
-    if (k > nchunks) return;
-    if (k == nchunks) {
-        chunk_row[k] = R;
-        return;
-    }
-    const int64_t p = (int64_t)k * chunk;
-    int lo = 0, hi = R;                      // largest r in [0,R) with off[r] + r <= p
-    while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if ((int64_t)off[mid] + mid <= p) lo = mid; else hi = mid;
-    }
-    chunk_row[k] = lo;
-}
-
 // el[v,k] = a_src[k,:].h[v,k,:], er[v,k] = a_dst[k,:].h[v,k,:]
 // Generic form: one thread per (node, head) walks the head's D values.
 __global__ void gat_node_scores(const float *__restrict__ h, const float *__restrict__ a_src,
@@ -153,8 +133,7 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_merge(
     const int32_t *__restrict__ off, const int32_t *__restrict__ idx, const float *__restrict__ h,
     const float *__restrict__ el, const float *__restrict__ er, float slope, float *__restrict__ out,
     float *__restrict__ smax, float *__restrict__ ssum, float *__restrict__ partial, float *__restrict__ pmax,
-    float *__restrict__ psum, const int32_t *__restrict__ chunk_row, int R, int E, int H, int D, int chunk,
-    int nchunks)
+    float *__restrict__ psum, const int2 *__restrict__ start, int R, int E, int H, int D, int nchunks)
 {
     constexpr int kGatUnroll = gat_unroll(VEC * NT);
     const int k = blockIdx.x * kGatWaves + wave_in_block();
@@ -172,14 +151,14 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_merge(
         lead[t] = act[t] && (f % D == 0);
         fo[t] = act[t] ? f : 0;
     }
-    const int r1 = min(max(uniform(chunk_row[k + 1]), 0), R);
-    int r = min(max(uniform(chunk_row[k]), 0), r1);
-    const int p0 = k * chunk;
-    const int p1 = min(p0 + chunk, R + E);
-    const int j0 = max(p0 - r, 0);
-    const int j1 = min(p1 - r1, E);
+    // the chunk runs from (row, entry) = start[k] to start[k + 1], clamped against malformed offsets
+    const int2 s0 = start[k], s1 = start[k + 1];
+    const int r1 = min(max(uniform(s1.x), 0), R);
+    int r = min(max(uniform(s0.x), 0), r1);
+    const int j0 = min(max(uniform(s0.y), 0), E);
+    const int j1 = min(uniform(s1.y), E);
     // the first row of the chunk began in an earlier chunk: its piece stays unnormalised
-    bool continued = (r < R) && (uniform(off[r]) + r < p0);
+    bool continued = (r < R) && (uniform(off[r]) < j0);
 
     int rb = r;
     int ends = (rb + lane < R) ? off[rb + 1 + lane] : 0x7fffffff;
@@ -284,7 +263,7 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_merge(
         }
     }
     while (r < r1) flush_row();
-    if (r1 < R) {
+    if (r1 < R && j1 > uniform(off[r1])) {     // the leading piece of a row that goes on in the next chunk
         float *dst = partial + (size_t)k * F + f0;
 #pragma unroll
         for (int t = 0; t < NT; t++)
@@ -357,8 +336,9 @@ template <int VEC, int NT> struct SoftState {
 // Pieces of a long row are pre-merged in groups of kGatGroup consecutive
 // chunks (see spmm_group_sums): group g's wavefront merges the pieces of the
 // row that continues past the end of the group.
-constexpr int kGatGroup = 32;
+constexpr int kGatGroup = kPlanGroup;
 
+// `list` (ascending, count[0] entries) names the groups to look at; without one every group is.
 template <int VEC, int NT>
 __global__ __launch_bounds__(kGatThreads) void gat_fwd_group(const int32_t *__restrict__ off,
                                                              const float *__restrict__ partial,
@@ -366,30 +346,36 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_group(const int32_t *__re
                                                              const float *__restrict__ psum,
                                                              float *__restrict__ gvec, float *__restrict__ gmax,
                                                              float *__restrict__ gsum,
-                                                             const int32_t *__restrict__ chunk_row, int R, int H,
+                                                             const int2 *__restrict__ start,
+                                                             const int32_t *__restrict__ list,
+                                                             const int32_t *__restrict__ count, int R, int H,
                                                              int D, int chunk, int nchunks)
 {
-    const int g = blockIdx.x * kGatWaves + wave_in_block();
-    const int kend = (g + 1) * kGatGroup;
-    if (kend >= nchunks) return;
-    const int r = uniform(chunk_row[kend]);
-    if (r >= R) return;
-    const int lo = uniform(off[r]) + r;
-    if (lo >= kend * chunk) return;
-    const int a = max(max(lo, 0) / chunk, g * kGatGroup);
-    const int F = H * D;
-    const int f0 = lane_id() * VEC;
-    SoftState<VEC, NT> st;
-    st.clear();
-    st.merge(partial, pmax, psum, a, kend, F, H, D, f0);
+    const int n = list ? uniform(count[0]) : (nchunks + kGatGroup - 1) / kGatGroup;
+    const int stride = gridDim.x * kGatWaves;
+    for (int i = blockIdx.x * kGatWaves + wave_in_block(); i < n; i += stride) {
+        const int g = list ? uniform(list[i]) : i;
+        const int kend = (g + 1) * kGatGroup;
+        if (kend >= nchunks) continue;
+        const int r = uniform(start[kend].x);
+        if (r < 0 || r >= R) continue;
+        const int s = uniform(off[r]);
+        if (uniform(start[kend].y) <= s) continue;
+        const int a = max((int)(((int64_t)max(s, 0) + r) / chunk), g * kGatGroup);
+        const int F = H * D;
+        const int f0 = lane_id() * VEC;
+        SoftState<VEC, NT> st;
+        st.clear();
+        st.merge(partial, pmax, psum, a, kend, F, H, D, f0);
 #pragma unroll
-    for (int t = 0; t < NT; t++) {
-        const int f = f0 + t * kWave * VEC;
-        if (f < F) {
-            gstore<VEC>(gvec + (size_t)g * F + f, st.acc[t]);
-            if (f % D == 0) {
-                gmax[(size_t)g * H + f / D] = st.M[t];
-                gsum[(size_t)g * H + f / D] = st.L[t];
+        for (int t = 0; t < NT; t++) {
+            const int f = f0 + t * kWave * VEC;
+            if (f < F) {
+                gstore<VEC>(gvec + (size_t)g * F + f, st.acc[t]);
+                if (f % D == 0) {
+                    gmax[(size_t)g * H + f / D] = st.M[t];
+                    gsum[(size_t)g * H + f / D] = st.L[t];
+                }
             }
         }
     }
@@ -402,48 +388,53 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_fixup(
     const int32_t *__restrict__ off, float *__restrict__ out, float *__restrict__ smax, float *__restrict__ ssum,
     const float *__restrict__ partial, const float *__restrict__ pmax, const float *__restrict__ psum,
     const float *__restrict__ gvec, const float *__restrict__ gmax, const float *__restrict__ gsum,
-    const int32_t *__restrict__ chunk_row, int H, int D, int chunk, int nchunks)
+    const int2 *__restrict__ start, const int32_t *__restrict__ list, const int32_t *__restrict__ count, int R, int H,
+    int D, int chunk, int nchunks)
 {
-    const int k = blockIdx.x * kGatWaves + wave_in_block();
-    if (k >= nchunks) return;
-    const int r0 = uniform(chunk_row[k]);
-    const int r1 = uniform(chunk_row[k + 1]);
-    if (r1 <= r0) return;
-    const int lo = uniform(off[r0]) + r0;
-    if (lo >= k * chunk) return;
-    const int a = max(lo, 0) / chunk;
-    const int F = H * D;
-    const int f0 = lane_id() * VEC;
-    SoftState<VEC, NT> st;
-    st.clear();
-    const int ga = a / kGatGroup, gb = k / kGatGroup;
-    if (ga == gb) {
-        st.merge(partial, pmax, psum, a, k, F, H, D, f0);
-    } else {
-        st.merge(gvec, gmax, gsum, ga, gb, F, H, D, f0);
-        st.merge(partial, pmax, psum, gb * kGatGroup, k, F, H, D, f0);
-    }
-    st.merge(out, smax, ssum, r0, r0 + 1, F, H, D, f0);
-#pragma unroll
-    for (int t = 0; t < NT; t++) {
-        const int f = f0 + t * kWave * VEC;
-        if (f < F) {
-            float o[VEC];
-            const float inv = st.L[t] > 0.f ? 1.f / st.L[t] : 0.f;
-#pragma unroll
-            for (int v = 0; v < VEC; v++) o[v] = st.acc[t][v] * inv;
-            gstore<VEC>(out + (size_t)r0 * F + f, o);
+    const int n = list ? min(uniform(count[0]), nchunks) : nchunks;
+    const int stride = gridDim.x * kGatWaves;
+    for (int i = blockIdx.x * kGatWaves + wave_in_block(); i < n; i += stride) {
+        const int k = list ? uniform(list[i]) : i;
+        if (k < 0 || k >= nchunks) continue;
+        const int r0 = uniform(start[k].x);
+        const int r1 = uniform(start[k + 1].x);
+        if (r0 < 0 || r0 >= R || r1 <= r0) continue;
+        const int s = uniform(off[r0]);
+        if (uniform(start[k].y) <= s) continue;
+        const int a = min((int)(((int64_t)max(s, 0) + r0) / chunk), k);
+        const int F = H * D;
+        const int f0 = lane_id() * VEC;
+        SoftState<VEC, NT> st;
+        st.clear();
+        const int ga = a / kGatGroup, gb = k / kGatGroup;
+        if (ga == gb) {
+            st.merge(partial, pmax, psum, a, k, F, H, D, f0);
+        } else {
+            st.merge(gvec, gmax, gsum, ga, gb, F, H, D, f0);
+            st.merge(partial, pmax, psum, gb * kGatGroup, k, F, H, D, f0);
         }
-    }
-    // every lane of a head holds the same (M, L); the head's first lane stores them.  The
-    // loads of the old values above are complete before these stores issue (their
-    // results feed the stored values, same wavefront).
+        st.merge(out, smax, ssum, r0, r0 + 1, F, H, D, f0);
 #pragma unroll
-    for (int t = 0; t < NT; t++) {
-        const int f = f0 + t * kWave * VEC;
-        if (f < F && f % D == 0) {
-            smax[(size_t)r0 * H + f / D] = st.M[t];
-            ssum[(size_t)r0 * H + f / D] = st.L[t];
+        for (int t = 0; t < NT; t++) {
+            const int f = f0 + t * kWave * VEC;
+            if (f < F) {
+                float o[VEC];
+                const float inv = st.L[t] > 0.f ? 1.f / st.L[t] : 0.f;
+#pragma unroll
+                for (int v = 0; v < VEC; v++) o[v] = st.acc[t][v] * inv;
+                gstore<VEC>(out + (size_t)r0 * F + f, o);
+            }
+        }
+        // every lane of a head holds the same (M, L); the head's first lane stores them.  The
+        // loads of the old values above are complete before these stores issue (their
+        // results feed the stored values, same wavefront).
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const int f = f0 + t * kWave * VEC;
+            if (f < F && f % D == 0) {
+                smax[(size_t)r0 * H + f / D] = st.M[t];
+                ssum[(size_t)r0 * H + f / D] = st.L[t];
+            }
         }
     }
 }
@@ -523,7 +514,7 @@ __global__ __launch_bounds__(kGatThreads) void gat_bwd_merge(
     const float *__restrict__ h, const float *__restrict__ el, const float4 *__restrict__ stat,
     const float *__restrict__ g_out, float slope, float *__restrict__ g_h, float *__restrict__ g_el,
     float *__restrict__ gz_t, float *__restrict__ partial, float *__restrict__ pel,
-    const int32_t *__restrict__ chunk_row, int R, int E, int H, int D, int lph, int chunk, int nchunks)
+    const int2 *__restrict__ start, int R, int E, int H, int D, int lph, int nchunks)
 {
     constexpr int kGatUnroll = gat_unroll(VEC * NT);
     // The logit gradients of a group of 64 entries wait in LDS and leave as one contiguous
@@ -548,12 +539,11 @@ __global__ __launch_bounds__(kGatThreads) void gat_bwd_merge(
         lead[t] = act[t] && (f % D == 0);
         fo[t] = act[t] ? f : 0;
     }
-    const int r1 = min(max(uniform(chunk_row[k + 1]), 0), R);
-    int r = min(max(uniform(chunk_row[k]), 0), r1);
-    const int p0 = k * chunk;
-    const int p1 = min(p0 + chunk, R + E);
-    const int j0 = max(p0 - r, 0);
-    const int j1 = min(p1 - r1, E);
+    const int2 s0 = start[k], s1 = start[k + 1];
+    const int r1 = min(max(uniform(s1.x), 0), R);
+    int r = min(max(uniform(s0.x), 0), r1);
+    const int j0 = min(max(uniform(s0.y), 0), E);
+    const int j1 = min(uniform(s1.y), E);
 
     int rb = r;
     int ends = (rb + lane < R) ? t_off[rb + 1 + lane] : 0x7fffffff;
@@ -684,7 +674,7 @@ __global__ __launch_bounds__(kGatThreads) void gat_bwd_merge(
         }
     }
     while (r < r1) flush_row();
-    if (r1 < R) store_piece(partial + (size_t)k * F, pel + (size_t)k * H);
+    if (r1 < R && j1 > uniform(t_off[r1])) store_piece(partial + (size_t)k * F, pel + (size_t)k * H);
 }
 
 // Plain sums of backward pieces: vec [.,F] and per-head scalars elp [.,H].
@@ -751,23 +741,29 @@ __global__ __launch_bounds__(kGatThreads) void gat_bwd_group(const int32_t *__re
                                                              const float *__restrict__ partial,
                                                              const float *__restrict__ pel, float *__restrict__ gvec,
                                                              float *__restrict__ gel,
-                                                             const int32_t *__restrict__ chunk_row, int R, int H,
+                                                             const int2 *__restrict__ start,
+                                                             const int32_t *__restrict__ list,
+                                                             const int32_t *__restrict__ count, int R, int H,
                                                              int D, int chunk, int nchunks)
 {
-    const int g = blockIdx.x * kGatWaves + wave_in_block();
-    const int kend = (g + 1) * kGatGroup;
-    if (kend >= nchunks) return;
-    const int r = uniform(chunk_row[kend]);
-    if (r >= R) return;
-    const int lo = uniform(t_off[r]) + r;
-    if (lo >= kend * chunk) return;
-    const int a = max(max(lo, 0) / chunk, g * kGatGroup);
-    const int F = H * D;
-    const int f0 = lane_id() * VEC;
-    SumState<VEC, NT> st;
-    st.clear();
-    st.add(partial, pel, a, kend, F, H, D, f0);
-    st.store(gvec + (size_t)g * F, gel + (size_t)g * H, F, D, f0);
+    const int n = list ? uniform(count[0]) : (nchunks + kGatGroup - 1) / kGatGroup;
+    const int stride = gridDim.x * kGatWaves;
+    for (int i = blockIdx.x * kGatWaves + wave_in_block(); i < n; i += stride) {
+        const int g = list ? uniform(list[i]) : i;
+        const int kend = (g + 1) * kGatGroup;
+        if (kend >= nchunks) continue;
+        const int r = uniform(start[kend].x);
+        if (r < 0 || r >= R) continue;
+        const int s = uniform(t_off[r]);
+        if (uniform(start[kend].y) <= s) continue;
+        const int a = max((int)(((int64_t)max(s, 0) + r) / chunk), g * kGatGroup);
+        const int F = H * D;
+        const int f0 = lane_id() * VEC;
+        SumState<VEC, NT> st;
+        st.clear();
+        st.add(partial, pel, a, kend, F, H, D, f0);
+        st.store(gvec + (size_t)g * F, gel + (size_t)g * H, F, D, f0);
+    }
 }
 
 template <int VEC, int NT>
@@ -777,30 +773,36 @@ __global__ __launch_bounds__(kGatThreads) void gat_bwd_fixup(const int32_t *__re
                                                              const float *__restrict__ pel,
                                                              const float *__restrict__ gvec,
                                                              const float *__restrict__ gel,
-                                                             const int32_t *__restrict__ chunk_row, int H, int D,
+                                                             const int2 *__restrict__ start,
+                                                             const int32_t *__restrict__ list,
+                                                             const int32_t *__restrict__ count, int R, int H, int D,
                                                              int chunk, int nchunks)
 {
-    const int k = blockIdx.x * kGatWaves + wave_in_block();
-    if (k >= nchunks) return;
-    const int r0 = uniform(chunk_row[k]);
-    const int r1 = uniform(chunk_row[k + 1]);
-    if (r1 <= r0) return;
-    const int lo = uniform(t_off[r0]) + r0;
-    if (lo >= k * chunk) return;
-    const int a = max(lo, 0) / chunk;
-    const int F = H * D;
-    const int f0 = lane_id() * VEC;
-    SumState<VEC, NT> st;
-    st.clear();
-    const int ga = a / kGatGroup, gb = k / kGatGroup;
-    if (ga == gb) {
-        st.add(partial, pel, a, k, F, H, D, f0);
-    } else {
-        st.add(gvec, gel, ga, gb, F, H, D, f0);
-        st.add(partial, pel, gb * kGatGroup, k, F, H, D, f0);
+    const int n = list ? min(uniform(count[0]), nchunks) : nchunks;
+    const int stride = gridDim.x * kGatWaves;
+    for (int i = blockIdx.x * kGatWaves + wave_in_block(); i < n; i += stride) {
+        const int k = list ? uniform(list[i]) : i;
+        if (k < 0 || k >= nchunks) continue;
+        const int r0 = uniform(start[k].x);
+        const int r1 = uniform(start[k + 1].x);
+        if (r0 < 0 || r0 >= R || r1 <= r0) continue;
+        const int s = uniform(t_off[r0]);
+        if (uniform(start[k].y) <= s) continue;
+        const int a = min((int)(((int64_t)max(s, 0) + r0) / chunk), k);
+        const int F = H * D;
+        const int f0 = lane_id() * VEC;
+        SumState<VEC, NT> st;
+        st.clear();
+        const int ga = a / kGatGroup, gb = k / kGatGroup;
+        if (ga == gb) {
+            st.add(partial, pel, a, k, F, H, D, f0);
+        } else {
+            st.add(gvec, gel, ga, gb, F, H, D, f0);
+            st.add(partial, pel, gb * kGatGroup, k, F, H, D, f0);
+        }
+        st.add(g_h, g_el, r0, r0 + 1, F, H, D, f0);
+        st.store(g_h + (size_t)r0 * F, g_el + (size_t)r0 * H, F, D, f0);
     }
-    st.add(g_h, g_el, r0, r0 + 1, F, H, D, f0);
-    st.store(g_h + (size_t)r0 * F, g_el + (size_t)r0 * H, F, D, f0);
 }
 
 // g_h[v,f] += g_el[v,k] a_src[f] + g_er[v,k] a_dst[f]; per-block partial sums of
@@ -884,6 +886,21 @@ struct GatShape {
     bool bwd_ok;
 };
 
+// items per wavefront: the start-up chain of a chunk (row lookup, offsets, indices, first
+// gathers) is a few microseconds, so chunks stay at 64 items or more
+int gat_chunk_for(int64_t M)
+{
+    int chunk = 128;
+    while (chunk > 64 && M / chunk < 16384) chunk >>= 1;
+    return chunk;
+}
+
+static unsigned gat_list_grid(int hint, int upper)
+{
+    const int64_t n = hint >= 0 ? (hint < upper ? hint : upper) : (upper < 8192 ? upper : 8192);
+    return (unsigned)ceil_div(n > 0 ? n : 1, kGatWaves);
+}
+
 static GatShape gat_shape(int32_t V, int64_t E, int32_t H, int32_t D)
 {
     GatShape s{};
@@ -892,10 +909,7 @@ static GatShape gat_shape(int32_t V, int64_t E, int32_t H, int32_t D)
     while (s.vec > 1 && F <= kWave * (s.vec / 2)) s.vec >>= 1;
     s.nt = (int)ceil_div(F, kWave * s.vec);
     const int64_t M = (int64_t)V + E;
-    // items per wavefront: the start-up chain of a chunk (row lookup, offsets, indices, first
-    // gathers) is a few microseconds, so chunks stay at 64 items or more
-    s.chunk = 128;
-    while (s.chunk > 64 && M / s.chunk < 16384) s.chunk >>= 1;
+    s.chunk = gat_chunk_for(M);
     s.nchunks = (int)ceil_div(M > 0 ? M : 1, s.chunk);
     s.lph = D / s.vec;
     s.bwd_ok = H == 1 || (s.lph >= 1 && s.lph <= kWave && (s.lph & (s.lph - 1)) == 0);
@@ -923,7 +937,7 @@ static size_t gat_fwd_ws(int32_t V, int64_t E, int32_t H, int32_t D)
 {
     GatShape s = gat_shape(V, E, H, D);
     const size_t ng = (size_t)ceil_div(s.nchunks, kGatGroup);
-    return carve_bytes((size_t)s.nchunks + 1, 4) + carve_bytes((size_t)s.nchunks * H * D, 4) +
+    return carve_bytes((size_t)s.nchunks + 1, sizeof(int2)) + carve_bytes((size_t)s.nchunks * H * D, 4) +
            2 * carve_bytes((size_t)s.nchunks * H, 4) + carve_bytes(ng * H * D, 4) + 2 * carve_bytes(ng * H, 4);
 }
 
@@ -932,7 +946,7 @@ static size_t gat_bwd_ws(int32_t V, int64_t E, int32_t H, int32_t D)
     GatShape s = gat_shape(V, E, H, D);
     const size_t nred = (size_t)ceil_div(V > 0 ? V : 1, kRedRows);
     const size_t ng = (size_t)ceil_div(s.nchunks, kGatGroup);
-    return carve_bytes(ng * H * D, 4) + carve_bytes(ng * H, 4) + carve_bytes((size_t)s.nchunks + 1, 4) + carve_bytes((size_t)s.nchunks * H * D, 4) +
+    return carve_bytes(ng * H * D, 4) + carve_bytes(ng * H, 4) + carve_bytes((size_t)s.nchunks + 1, sizeof(int2)) + carve_bytes((size_t)s.nchunks * H * D, 4) +
            carve_bytes((size_t)s.nchunks * H, 4) + carve_bytes((size_t)V * H, 16) + carve_bytes((size_t)E * H, 4) +
            2 * carve_bytes((size_t)V * H, 4) + carve_bytes(nred * 2 * H * D, 4) +
            align_up(spmm_ws_bytes(V, E, H), 256);
@@ -959,10 +973,10 @@ JG_EXPORT int32_t jgamd_gat_fwd_workspace(int32_t V, int64_t E, int32_t H, int32
     return 0;
 }
 
-JG_EXPORT int32_t jgamd_gat_fwd(const int32_t *off, const int32_t *idx, const float *h, const float *a_src,
-                                const float *a_dst, float slope, float *el, float *er, float *smax, float *ssum,
-                                float *alpha, float *out, int32_t V, int64_t E, int32_t H, int32_t D, void *ws,
-                                size_t ws_bytes, void *stream)
+JG_EXPORT int32_t jgamd_gat_fwd(const void *plan, int32_t n_fix, int32_t n_grp, const int32_t *off,
+                                const int32_t *idx, const float *h, const float *a_src, const float *a_dst,
+                                float slope, float *el, float *er, float *smax, float *ssum, float *alpha, float *out,
+                                int32_t V, int64_t E, int32_t H, int32_t D, void *ws, size_t ws_bytes, void *stream)
 {
     if (int32_t rc = check_gat("gat_fwd", V, E, H, D)) return rc;
     if (V == 0) return 0;
@@ -973,9 +987,19 @@ JG_EXPORT int32_t jgamd_gat_fwd(const int32_t *off, const int32_t *idx, const fl
     const size_t need = gat_fwd_ws(V, E, H, D);
     if (!ws || ws_bytes < need) return fail(JGAMD_ERR_WORKSPACE, "gat_fwd: workspace %zu < %zu bytes", ws ? ws_bytes : (size_t)0, need);
     if (((uintptr_t)ws & 255) != 0) return fail(JGAMD_ERR_ALIGN, "gat_fwd: workspace not 256-byte aligned");
+    if (((uintptr_t)plan & 255) != 0) return fail(JGAMD_ERR_ALIGN, "gat_fwd: plan not 256-byte aligned");
     const GatShape s = gat_shape(V, E, H, D);
+    hipStream_t st = static_cast<hipStream_t>(stream);
     Carver carve(ws);
-    int32_t *chunk_row = carve.take<int32_t>((size_t)s.nchunks + 1);
+    int2 *own_start = carve.take<int2>((size_t)s.nchunks + 1);
+    ChunkPlan pv{};
+    if (plan) {
+        pv = chunk_plan_view(JGAMD_PLAN_GAT, V, E, plan);
+    } else {
+        chunk_starts_enqueue(off, V, E, s.chunk, s.nchunks, own_start, st);
+        pv.start = own_start;
+        n_fix = n_grp = -1;
+    }
     float *partial = carve.take<float>((size_t)s.nchunks * H * D);
     float *pmax = carve.take<float>((size_t)s.nchunks * H);
     float *psum = carve.take<float>((size_t)s.nchunks * H);
@@ -983,7 +1007,6 @@ JG_EXPORT int32_t jgamd_gat_fwd(const int32_t *off, const int32_t *idx, const fl
     float *gvec = carve.take<float>((size_t)ngroups * H * D);
     float *gmax = carve.take<float>((size_t)ngroups * H);
     float *gsum = carve.take<float>((size_t)ngroups * H);
-    hipStream_t st = static_cast<hipStream_t>(stream);
     const int64_t VH = (int64_t)V * H;
     if (vec_nodes_ok(D) && (((uintptr_t)a_src | (uintptr_t)a_dst) & 15) == 0)
         hipLaunchKernelGGL(gat_node_scores_vec, dim3((unsigned)ceil_div(VH * (D / 4), 256)), dim3(256), 0, st,
@@ -992,19 +1015,22 @@ JG_EXPORT int32_t jgamd_gat_fwd(const int32_t *off, const int32_t *idx, const fl
     else
         hipLaunchKernelGGL(gat_node_scores, dim3((unsigned)ceil_div(VH, 256)), dim3(256), 0, st, h, a_src, a_dst, el,
                            er, VH, H, D);
-    hipLaunchKernelGGL(gat_chunk_rows, dim3((unsigned)ceil_div(s.nchunks + 1, 256)), dim3(256), 0, st, off, V, s.chunk,
-                       s.nchunks, chunk_row);
     dim3 grid((unsigned)ceil_div(s.nchunks, kGatWaves)), block(kGatThreads);
+    // pieces of rows cut across chunks: over the plan's lists, or over every chunk and group
+    const bool listed = pv.fix != nullptr;
+    const dim3 ggrid(listed ? gat_list_grid(n_grp, ngroups) : (unsigned)ceil_div(ngroups, kGatWaves));
+    const dim3 fgrid(listed ? gat_list_grid(n_fix, s.nchunks) : grid.x);
 #define JG_FWD(VV, NN)                                                                                           \
     case VV * 16 + NN:                                                                                           \
         hipLaunchKernelGGL((gat_fwd_merge<VV, NN>), grid, block, 0, st, off, idx, h, el, er, slope, out, smax,   \
-                           ssum, partial, pmax, psum, chunk_row, V, (int)E, H, D, s.chunk, s.nchunks);           \
-        if (ngroups > 1)                                                                                         \
-            hipLaunchKernelGGL((gat_fwd_group<VV, NN>), dim3((unsigned)ceil_div(ngroups, kGatWaves)), block, 0,  \
-                               st, off, partial, pmax, psum, gvec, gmax, gsum, chunk_row, V, H, D, s.chunk,      \
+                           ssum, partial, pmax, psum, pv.start, V, (int)E, H, D, s.nchunks);                     \
+        if (ngroups > 1 && n_grp != 0 && n_fix != 0)                                                             \
+            hipLaunchKernelGGL((gat_fwd_group<VV, NN>), ggrid, block, 0, st, off, partial, pmax, psum, gvec,     \
+                               gmax, gsum, pv.start, pv.grp, pv.counts + 1, V, H, D, s.chunk, s.nchunks);        \
+        if (n_fix != 0)                                                                                          \
+            hipLaunchKernelGGL((gat_fwd_fixup<VV, NN>), fgrid, block, 0, st, off, out, smax, ssum, partial,      \
+                               pmax, psum, gvec, gmax, gsum, pv.start, pv.fix, pv.counts, V, H, D, s.chunk,      \
                                s.nchunks);                                                                       \
-        hipLaunchKernelGGL((gat_fwd_fixup<VV, NN>), grid, block, 0, st, off, out, smax, ssum, partial, pmax,     \
-                           psum, gvec, gmax, gsum, chunk_row, H, D, s.chunk, s.nchunks);                         \
         break;
     JG_GAT_DISPATCH(JG_FWD)
 #undef JG_FWD
@@ -1025,7 +1051,8 @@ JG_EXPORT int32_t jgamd_gat_bwd_workspace(int32_t V, int64_t E, int32_t H, int32
     return 0;
 }
 
-JG_EXPORT int32_t jgamd_gat_bwd(const int32_t *off, const int32_t *idx, const int32_t *t_off, const int32_t *t_idx,
+JG_EXPORT int32_t jgamd_gat_bwd(const void *t_plan, int32_t n_fix, int32_t n_grp, const void *tiles,
+                                const int32_t *off, const int32_t *idx, const int32_t *t_off, const int32_t *t_idx,
                                 const int32_t *t_inv, const float *h, const float *a_src, const float *a_dst,
                                 float slope, const float *el, const float *er, const float *smax, const float *ssum,
                                 const float *out, const float *g_out, float *g_h, float *g_a_src, float *g_a_dst,
@@ -1053,11 +1080,21 @@ JG_EXPORT int32_t jgamd_gat_bwd(const int32_t *off, const int32_t *idx, const in
     const size_t need = gat_bwd_ws(V, E, H, D);
     if (!ws || ws_bytes < need) return fail(JGAMD_ERR_WORKSPACE, "gat_bwd: workspace %zu < %zu bytes", ws ? ws_bytes : (size_t)0, need);
     if (((uintptr_t)ws & 255) != 0) return fail(JGAMD_ERR_ALIGN, "gat_bwd: workspace not 256-byte aligned");
+    if ((((uintptr_t)t_plan | (uintptr_t)tiles) & 255) != 0)
+        return fail(JGAMD_ERR_ALIGN, "gat_bwd: plan not 256-byte aligned");
     Carver carve(ws);
     const int ngroups = (int)ceil_div(s.nchunks, kGatGroup);
     float *gvec = carve.take<float>((size_t)ngroups * F);
     float *ggel = carve.take<float>((size_t)ngroups * H);
-    int32_t *chunk_row = carve.take<int32_t>((size_t)s.nchunks + 1);
+    int2 *own_start = carve.take<int2>((size_t)s.nchunks + 1);
+    ChunkPlan pv{};
+    if (t_plan) {
+        pv = chunk_plan_view(JGAMD_PLAN_GAT, V, E, t_plan);
+    } else {
+        chunk_starts_enqueue(t_off, V, E, s.chunk, s.nchunks, own_start, st);
+        pv.start = own_start;
+        n_fix = n_grp = -1;
+    }
     float *partial = carve.take<float>((size_t)s.nchunks * F);
     float *pel = carve.take<float>((size_t)s.nchunks * H);
     float4 *stat = carve.take<float4>((size_t)V * H);
@@ -1076,26 +1113,27 @@ JG_EXPORT int32_t jgamd_gat_bwd(const int32_t *off, const int32_t *idx, const in
     else
         hipLaunchKernelGGL(gat_bwd_node_stats, dim3((unsigned)ceil_div(VH, 256)), dim3(256), 0, st, er, smax, ssum,
                            g_out, out, stat, VH, D);
-    hipLaunchKernelGGL(gat_chunk_rows, dim3((unsigned)ceil_div(s.nchunks + 1, 256)), dim3(256), 0, st, t_off, V, s.chunk,
-                       s.nchunks, chunk_row);
     dim3 grid((unsigned)ceil_div(s.nchunks, kGatWaves)), block(kGatThreads);
+    const bool listed = pv.fix != nullptr;
+    const dim3 ggrid(listed ? gat_list_grid(n_grp, ngroups) : (unsigned)ceil_div(ngroups, kGatWaves));
+    const dim3 fgrid(listed ? gat_list_grid(n_fix, s.nchunks) : grid.x);
 #define JG_BWD(VV, NN)                                                                                             \
     case VV * 16 + NN:                                                                                             \
         hipLaunchKernelGGL((gat_bwd_merge<VV, NN>), grid, block, 0, st, t_off, t_idx, h, el, stat, g_out,          \
-                           slope, g_h, g_el, gz, partial, pel, chunk_row, V, (int)E, H, D, s.lph, s.chunk,         \
-                           s.nchunks);                                                                             \
-        if (ngroups > 1)                                                                                           \
-            hipLaunchKernelGGL((gat_bwd_group<VV, NN>), dim3((unsigned)ceil_div(ngroups, kGatWaves)), block, 0,    \
-                               st, t_off, partial, pel, gvec, ggel, chunk_row, V, H, D, s.chunk, s.nchunks);       \
-        hipLaunchKernelGGL((gat_bwd_fixup<VV, NN>), grid, block, 0, st, t_off, g_h, g_el, partial, pel, gvec,      \
-                           ggel, chunk_row, H, D, s.chunk, s.nchunks);                                             \
+                           slope, g_h, g_el, gz, partial, pel, pv.start, V, (int)E, H, D, s.lph, s.nchunks);       \
+        if (ngroups > 1 && n_grp != 0 && n_fix != 0)                                                               \
+            hipLaunchKernelGGL((gat_bwd_group<VV, NN>), ggrid, block, 0, st, t_off, partial, pel, gvec, ggel,      \
+                               pv.start, pv.grp, pv.counts + 1, V, H, D, s.chunk, s.nchunks);                      \
+        if (n_fix != 0)                                                                                            \
+            hipLaunchKernelGGL((gat_bwd_fixup<VV, NN>), fgrid, block, 0, st, t_off, g_h, g_el, partial, pel,       \
+                               gvec, ggel, pv.start, pv.fix, pv.counts, V, H, D, s.chunk, s.nchunks);              \
         break;
     JG_GAT_DISPATCH(JG_BWD)
 #undef JG_BWD
     // g_er[c,k] = sum of gz over the CSC slots of column c: the row-gather SpMM with unit
     // weights; slot j's row of the [E,H] array sits at its transposed position t_inv[j]
     if (int32_t rc = spmm_enqueue(off, t_inv, nullptr, gz, g_er, V, (int32_t)E, E, H, spmm_ws,
-                                  spmm_ws_bytes(V, E, H), st))
+                                  spmm_ws_bytes(V, E, H), st, tiles))
         return rc;
     hipLaunchKernelGGL(gat_bwd_finish, dim3((unsigned)nred), dim3(256), 0, st, h, a_src, a_dst, g_el, g_er, g_h, red,
                        V, H, D);

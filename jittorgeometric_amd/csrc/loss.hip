@@ -18,7 +18,18 @@
 namespace jg {
 
 constexpr int kCeThreads = 256;
-constexpr int kCeRows = 2048;      // rows per block
+constexpr int kCeRows = 2048;      // rows per block, at most
+constexpr int kCeMinRows = 32;     // and at least (one pass of the narrowest lane group)
+
+// Rows per block: as many as keep the per-block partial sums few, but never so many that a small
+// matrix leaves most of the 256 compute units without a block (2,708 rows of 7 classes at 2048
+// rows per block were two blocks and 56 us; at 32 rows per block 85 blocks and a few us).
+static int ce_rows_per_block(int64_t V)
+{
+    int rows = kCeRows;
+    while (rows > kCeMinRows && V / rows < 1024) rows >>= 1;
+    return rows;
+}
 
 __device__ __forceinline__ int64_t label_at(const int32_t *y32, const int64_t *y64, int64_t row)
 {
@@ -32,15 +43,16 @@ constexpr int kCeUnroll = 4;
 template <int G, bool REG>
 __global__ __launch_bounds__(kCeThreads) void ce_rows(const float *__restrict__ x, const int32_t *__restrict__ y32,
                                                       const int64_t *__restrict__ y64, int64_t V, int C,
-                                                      int log_probs, float *__restrict__ lse_out,
+                                                      int rows_per_block, int log_probs,
+                                                      float *__restrict__ lse_out,
                                                       double *__restrict__ block_sum, int32_t *__restrict__ block_cnt)
 {
     constexpr int RP = kCeThreads / G;      // row groups per pass
     __shared__ double s_sum[RP];
     __shared__ int s_cnt[RP];
     const int g = threadIdx.x % G, lr = threadIdx.x / G;
-    const int64_t r0 = (int64_t)blockIdx.x * kCeRows;
-    const int64_t r1 = r0 + kCeRows < V ? r0 + kCeRows : V;
+    const int64_t r0 = (int64_t)blockIdx.x * rows_per_block;
+    const int64_t r1 = r0 + rows_per_block < V ? r0 + rows_per_block : V;
     double acc = 0.0;
     int cnt = 0;
     auto finish = [&](int64_t row, const float *p, float m, float s) {
@@ -150,14 +162,14 @@ __global__ __launch_bounds__(kCeThreads) void ce_grad(const float *__restrict__ 
                                                       const int64_t *__restrict__ y64, const float *__restrict__ lse,
                                                       const int32_t *__restrict__ count,
                                                       const float *__restrict__ grad_loss, int64_t V, int C,
-                                                      float *__restrict__ grad)
+                                                      int rows_per_block, float *__restrict__ grad)
 {
     constexpr int RP = kCeThreads / G;
     const int g = threadIdx.x % G, lr = threadIdx.x / G;
     const int n = count[0];
     const float scale = (grad_loss ? grad_loss[0] : 1.f) / (float)n;      // n == 0: no row is counted below
-    const int64_t r0 = (int64_t)blockIdx.x * kCeRows;
-    const int64_t r1 = r0 + kCeRows < V ? r0 + kCeRows : V;
+    const int64_t r0 = (int64_t)blockIdx.x * rows_per_block;
+    const int64_t r1 = r0 + rows_per_block < V ? r0 + rows_per_block : V;
     for (int64_t row = r0 + lr; row < r1; row += RP) {
         const int64_t lab = label_at(y32, y64, row);
         const bool counted = lab >= 0 && lab < C;
@@ -227,7 +239,7 @@ static int lanes_per_row(int C)
 using namespace jg;
 #define JG_EXPORT extern "C" __attribute__((visibility("default")))
 
-static int ce_blocks(int64_t V) { return (int)ceil_div(V > 0 ? V : 1, kCeRows); }
+static int ce_blocks(int64_t V) { return (int)ceil_div(V > 0 ? V : 1, ce_rows_per_block(V)); }
 static size_t ce_ws(int64_t V) { return carve_bytes((size_t)ce_blocks(V), 8) + carve_bytes((size_t)ce_blocks(V), 4); }
 
 static int32_t ce_check(const char *who, int64_t V, int32_t C)
@@ -251,7 +263,9 @@ JG_EXPORT int32_t jgamd_cross_entropy_fwd(const float *logits, const void *label
 {
     if (int32_t rc = ce_check("cross_entropy_fwd", V, C)) return rc;
     if (!loss || !count) return fail(JGAMD_ERR_NULL, "cross_entropy_fwd: loss / count is NULL");
-    if (V > 0 && (!labels || !lse || (C > 0 && !logits)))
+    // rows without classes have no logsumexp (and a [V,0] array has no address to read)
+    if (V > 0 && C == 0) return fail(JGAMD_ERR_SIZE, "cross_entropy_fwd: V=%lld rows of C=0 classes", (long long)V);
+    if (V > 0 && (!labels || !lse || !logits))
         return fail(JGAMD_ERR_NULL, "cross_entropy_fwd: logits / labels / lse is NULL");
     const size_t need = ce_ws(V);
     if (!ws || ws_bytes < need)
@@ -260,6 +274,7 @@ JG_EXPORT int32_t jgamd_cross_entropy_fwd(const float *logits, const void *label
     hipStream_t st = static_cast<hipStream_t>(stream);
     Carver carve(ws);
     const int nblocks = ce_blocks(V);
+    const int rows = ce_rows_per_block(V);
     double *block_sum = carve.take<double>((size_t)nblocks);
     int32_t *block_cnt = carve.take<int32_t>((size_t)nblocks);
     const int32_t *y32 = labels_are_i64 ? nullptr : static_cast<const int32_t *>(labels);
@@ -271,10 +286,10 @@ JG_EXPORT int32_t jgamd_cross_entropy_fwd(const float *logits, const void *label
     if (G == GG) {                                                                                                   \
         if (reg)                                                                                                     \
             hipLaunchKernelGGL((ce_rows<GG, true>), dim3((unsigned)nblocks), dim3(kCeThreads), 0, st, logits, y32,   \
-                               y64, V, C, log_probs, lse, block_sum, block_cnt);                                                \
+                               y64, V, C, rows, log_probs, lse, block_sum, block_cnt);                                                \
         else                                                                                                         \
             hipLaunchKernelGGL((ce_rows<GG, false>), dim3((unsigned)nblocks), dim3(kCeThreads), 0, st, logits, y32,  \
-                               y64, V, C, log_probs, lse, block_sum, block_cnt);                                                \
+                               y64, V, C, rows, log_probs, lse, block_sum, block_cnt);                                                \
     }
         JG_CE(8) JG_CE(16) JG_CE(32) JG_CE(64)
 #undef JG_CE
@@ -305,7 +320,7 @@ JG_EXPORT int32_t jgamd_cross_entropy_bwd(const float *logits, const void *label
 #define JG_CE(GG)                                                                                                  \
     if (G == GG)                                                                                                   \
         hipLaunchKernelGGL((ce_grad<GG>), dim3((unsigned)nblocks), dim3(kCeThreads), 0, st, logits, y32, y64, lse, \
-                           count, grad_loss, V, C, grad_logits);
+                           count, grad_loss, V, C, ce_rows_per_block(V), grad_logits);
     JG_CE(8) JG_CE(16) JG_CE(32) JG_CE(64)
 #undef JG_CE
     return launch_status("cross_entropy_bwd");

@@ -66,28 +66,6 @@ template <int VEC> __device__ __forceinline__ void vstore_stream(float *p, const
 }
 template <typename T> __device__ __forceinline__ T load_stream(const T *p) { return __builtin_nontemporal_load(p); }
 
-// chunk_row[k] = the row that owns merged position k*chunk, k < nchunks;
-// chunk_row[nchunks] = R.  Row r owns positions off[r]+r .. off[r+1]+r, an
-// increasing function of r, so each chunk finds its row by binary search
-// (a hub row spans thousands of chunks; per-chunk search keeps the work even).
-__global__ void spmm_chunk_rows(const int32_t *__restrict__ off, int R, int chunk, int nchunks,
-                                int32_t *__restrict__ chunk_row)
-{
-    const int k = blockIdx.x * blockDim.x + threadIdx.x;
-    if (k > nchunks) return;
-    if (k == nchunks) {
-        chunk_row[k] = R;
-        return;
-    }
-    const int64_t p = (int64_t)k * chunk;
-    int lo = 0, hi = R;                      // largest r in [0,R) with off[r] + r <= p
-    while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if ((int64_t)off[mid] + mid <= p) lo = mid; else hi = mid;
-    }
-    chunk_row[k] = lo;
-}
-
 // WIDE = false: every row of x starts less than 4 GiB from x, so a gathered
 // row is addressed as (scalar base) + (32-bit byte offset): one readlane and
 // one vector add per entry.  WIDE = true keeps 64-bit row arithmetic.
@@ -109,8 +87,8 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__rest
                                                            const float *__restrict__ w,
                                                            const float *__restrict__ x, float *__restrict__ out,
                                                            float *__restrict__ partial,
-                                                           const int32_t *__restrict__ chunk_row, int R, int C,
-                                                           int E, int F, int chunk, int nchunks, RowFinish fin)
+                                                           const int2 *__restrict__ start, int R, int C, int E,
+                                                           int F, int nchunks, RowFinish fin)
 {
     static_assert(kWave % UNROLL == 0, "groups tile a 64-entry batch");
     __shared__ int2 staged_all[LDS ? kSpmmThreads : 1];
@@ -132,15 +110,13 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__rest
     const int xs = fin.x_stride ? fin.x_stride : F;      // rows of x may be padded to whole cache lines
     const uint32_t row_bytes = (uint32_t)xs * 4u;
 
-    // rows are clamped so that a malformed off/E pair cannot index outside the arrays
-    const int r1 = min(max(uniform(chunk_row[k + 1]), 0), R);
-    int r = min(max(uniform(chunk_row[k]), 0), r1);
-    const int M = R + E;
-    const int p0 = k * chunk;
-    const int p1 = min(p0 + chunk, M);
-    int j0 = p0 - r;
-    int j1 = min(p1 - r1, E);
-    j0 = max(j0, 0);
+    // the chunk runs from (row, entry) = start[k] to start[k + 1]; both are clamped so that a
+    // malformed off/E pair cannot index outside the arrays
+    const int2 s0 = start[k], s1 = start[k + 1];
+    const int r1 = min(max(uniform(s1.x), 0), R);
+    int r = min(max(uniform(s0.x), 0), r1);
+    const int j0 = min(max(uniform(s0.y), 0), E);
+    const int j1 = min(uniform(s1.y), E);
 
     // window of 64 row ends starting at row rb: lane l holds off[rb + 1 + l].
     // row_end = entry index at which row r ends; "never" once r has reached r1
@@ -174,7 +150,7 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__rest
         }
     };
     if constexpr (EPI) {
-        if (r < r1 && uniform(off[r]) + r < p0) raw_row = r;
+        if (r < r1 && uniform(off[r]) < j0) raw_row = r;
         fetch_h();
     }
 
@@ -294,7 +270,8 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__rest
         }
     }
     while (r < r1) flush_row();   // rows whose end marker lies in this chunk after its last entry
-    if (r1 < R) {
+    // the leading piece of a row that goes on in the next chunk (most chunks end where a row ends)
+    if (r1 < R && j1 > uniform(off[r1])) {
         float *dst = partial + (size_t)k * F + f0;
 #pragma unroll
         for (int t = 0; t < NT; t++)
@@ -340,91 +317,104 @@ __device__ __forceinline__ void add_pieces(float (&acc)[NT][VEC], const float *_
 // therefore pre-summed in groups of kGroup consecutive chunks: group g's
 // wavefront adds, in order, the pieces of the row that continues past the end
 // of the group (a suffix of the group's chunks) into group_sum[g].
-constexpr int kGroup = 32;
+constexpr int kGroup = kPlanGroup;
 
+// `list` (ascending, *count entries) names the groups to look at; without one every group is.
 template <int VEC, int NT>
 __global__ __launch_bounds__(kSpmmThreads) void spmm_group_sums(const int32_t *__restrict__ off,
                                                                 const float *__restrict__ partial,
                                                                 float *__restrict__ group_sum,
-                                                                const int32_t *__restrict__ chunk_row, int R, int F,
+                                                                const int2 *__restrict__ start,
+                                                                const int32_t *__restrict__ list,
+                                                                const int32_t *__restrict__ count, int R, int F,
                                                                 int chunk, int nchunks)
 {
-    const int g = blockIdx.x * kSpmmWaves + wave_in_block();
-    const int kend = (g + 1) * kGroup;            // first chunk after the group
-    if (kend >= nchunks) return;                  // the last group has no row continuing past it
-    const int r = uniform(chunk_row[kend]);       // row that owns the first item after the group
-    if (r >= R) return;
-    const int lo = uniform(off[r]) + r;           // merged position of the row's first item
-    if (lo >= kend * chunk) return;               // it starts after the group: nothing continues
-    const int a = max(max(lo, 0) / chunk, g * kGroup);
-    const int f0 = blockIdx.y * (kWave * VEC * NT) + lane_id() * VEC;
-    float acc[NT][VEC];
+    const int n = list ? uniform(count[0]) : (nchunks + kGroup - 1) / kGroup;
+    const int stride = gridDim.x * kSpmmWaves;
+    for (int i = blockIdx.x * kSpmmWaves + wave_in_block(); i < n; i += stride) {
+        const int g = list ? uniform(list[i]) : i;
+        const int kend = (g + 1) * kGroup;            // first chunk after the group
+        if (kend >= nchunks) continue;                // the last group has no row continuing past it
+        const int r = uniform(start[kend].x);         // row that owns the first item after the group
+        if (r < 0 || r >= R) continue;
+        const int s = uniform(off[r]);
+        if (uniform(start[kend].y) <= s) continue;    // that chunk begins with the row: nothing continues
+        const int a = max((int)(((int64_t)max(s, 0) + r) / chunk), g * kGroup);
+        const int f0 = blockIdx.y * (kWave * VEC * NT) + lane_id() * VEC;
+        float acc[NT][VEC];
 #pragma unroll
-    for (int t = 0; t < NT; t++)
+        for (int t = 0; t < NT; t++)
 #pragma unroll
-        for (int v = 0; v < VEC; v++) acc[t][v] = 0.f;
-    add_pieces<VEC, NT>(acc, partial, a, kend, F, f0);
-    float *dst = group_sum + (size_t)g * F + f0;
+            for (int v = 0; v < VEC; v++) acc[t][v] = 0.f;
+        add_pieces<VEC, NT>(acc, partial, a, kend, F, f0);
+        float *dst = group_sum + (size_t)g * F + f0;
 #pragma unroll
-    for (int t = 0; t < NT; t++)
-        if (f0 + t * kWave * VEC < F) vstore<VEC>(dst + t * kWave * VEC, acc[t]);
+        for (int t = 0; t < NT; t++)
+            if (f0 + t * kWave * VEC < F) vstore<VEC>(dst + t * kWave * VEC, acc[t]);
+    }
 }
 
-// One wavefront per chunk b: if the first row of b started in an earlier
-// chunk a and ends in b, out[row] = (pieces a .. b-1, in order) + out[row];
-// whole groups between a and b come from group_sum.
+// One wavefront per chunk b of `list` (or per chunk): if the first row of b started in an
+// earlier chunk a and ends in b, out[row] = (pieces a .. b-1, in order) + out[row]; whole groups
+// between a and b come from group_sum.
 template <int VEC, int NT, bool EPI>
 __global__ __launch_bounds__(kSpmmThreads) void spmm_fixup(const int32_t *__restrict__ off, float *__restrict__ out,
                                                            const float *__restrict__ partial,
                                                            const float *__restrict__ group_sum,
-                                                           const int32_t *__restrict__ chunk_row, int F, int chunk,
+                                                           const int2 *__restrict__ start,
+                                                           const int32_t *__restrict__ list,
+                                                           const int32_t *__restrict__ count, int R, int F, int chunk,
                                                            int nchunks, RowFinish fin)
 {
-    const int k = blockIdx.x * kSpmmWaves + wave_in_block();
-    if (k >= nchunks) return;
-    const int r0 = uniform(chunk_row[k]);
-    const int r1 = uniform(chunk_row[k + 1]);
-    if (r1 <= r0) return;
-    const int lo = uniform(off[r0]) + r0;
-    if (lo >= k * chunk) return;
-    const int a = max(lo, 0) / chunk;
-    const int lane = lane_id();
-    const int f0 = blockIdx.y * (kWave * VEC * NT) + lane * VEC;
-    float acc[NT][VEC];
-#pragma unroll
-    for (int t = 0; t < NT; t++)
-#pragma unroll
-        for (int v = 0; v < VEC; v++) acc[t][v] = 0.f;
-    const int ga = a / kGroup, gb = k / kGroup;
-    if (ga == gb) {
-        add_pieces<VEC, NT>(acc, partial, a, k, F, f0);
-    } else {
-        // group ga's sum starts at piece a (the row continues past that group),
-        // groups ga+1 .. gb-1 belong to the row entirely, the rest of gb is added piecewise
-        add_pieces<VEC, NT>(acc, group_sum, ga, gb, F, f0);
-        add_pieces<VEC, NT>(acc, partial, gb * kGroup, k, F, f0);
-    }
-    float *dst = out + (size_t)r0 * F;
-    add_pieces<VEC, NT>(acc, dst, 0, 1, F, f0);
-    if constexpr (EPI) {
+    const int n = list ? min(uniform(count[0]), nchunks) : nchunks;
+    const int stride = gridDim.x * kSpmmWaves;
+    for (int i = blockIdx.x * kSpmmWaves + wave_in_block(); i < n; i += stride) {
+        const int k = list ? uniform(list[i]) : i;
+        if (k < 0 || k >= nchunks) continue;
+        const int r0 = uniform(start[k].x);
+        const int r1 = uniform(start[k + 1].x);
+        if (r0 < 0 || r0 >= R || r1 <= r0) continue;
+        const int s = uniform(off[r0]);
+        if (uniform(start[k].y) <= s) continue;       // the chunk begins with the row
+        const int a = min((int)(((int64_t)max(s, 0) + r0) / chunk), k);
+        const int lane = lane_id();
+        const int f0 = blockIdx.y * (kWave * VEC * NT) + lane * VEC;
+        float acc[NT][VEC];
 #pragma unroll
         for (int t = 0; t < NT; t++)
 #pragma unroll
-            for (int v = 0; v < VEC; v++) acc[t][v] *= fin.beta;
-        if (fin.h) {
-            float hv[NT][VEC];
+            for (int v = 0; v < VEC; v++) acc[t][v] = 0.f;
+        const int ga = a / kGroup, gb = k / kGroup;
+        if (ga == gb) {
+            add_pieces<VEC, NT>(acc, partial, a, k, F, f0);
+        } else {
+            // group ga's sum starts at piece a (the row continues past that group),
+            // groups ga+1 .. gb-1 belong to the row entirely, the rest of gb is added piecewise
+            add_pieces<VEC, NT>(acc, group_sum, ga, gb, F, f0);
+            add_pieces<VEC, NT>(acc, partial, gb * kGroup, k, F, f0);
+        }
+        float *dst = out + (size_t)r0 * F;
+        add_pieces<VEC, NT>(acc, dst, 0, 1, F, f0);
+        if constexpr (EPI) {
 #pragma unroll
-            for (int t = 0; t < NT; t++) {
-                const int f = f0 + t * kWave * VEC;
-                vload<VEC>(hv[t], fin.h + (size_t)r0 * fin.h_stride + (f < F ? f : 0));
+            for (int t = 0; t < NT; t++)
 #pragma unroll
-                for (int v = 0; v < VEC; v++) acc[t][v] = fmaf(fin.alpha, hv[t][v], acc[t][v]);
+                for (int v = 0; v < VEC; v++) acc[t][v] *= fin.beta;
+            if (fin.h) {
+                float hv[NT][VEC];
+#pragma unroll
+                for (int t = 0; t < NT; t++) {
+                    const int f = f0 + t * kWave * VEC;
+                    vload<VEC>(hv[t], fin.h + (size_t)r0 * fin.h_stride + (f < F ? f : 0));
+#pragma unroll
+                    for (int v = 0; v < VEC; v++) acc[t][v] = fmaf(fin.alpha, hv[t][v], acc[t][v]);
+                }
             }
         }
-    }
 #pragma unroll
-    for (int t = 0; t < NT; t++)
-        if (f0 + t * kWave * VEC < F) vstore<VEC>(dst + f0 + t * kWave * VEC, acc[t]);
+        for (int t = 0; t < NT; t++)
+            if (f0 + t * kWave * VEC < F) vstore<VEC>(dst + f0 + t * kWave * VEC, acc[t]);
+    }
 }
 
 // out = beta * out + alpha * h, element-wise (the finish as a pass of its own, for the
@@ -447,7 +437,7 @@ static int env_int(const char *name, int dflt)
 
 // Items per wavefront: enough chunks to fill the 256 CUs many times over,
 // few enough that the per-chunk partial row stays a small share of the work.
-static int pick_chunk(int64_t M)
+int spmm_chunk_for(int64_t M)
 {
     // benchmark override, read once per process (the workspace query and the launch agree)
     static const int forced = env_int("JGAMD_SPMM_CHUNK", 0);
@@ -468,14 +458,14 @@ struct SpmmShape {
 static SpmmShape spmm_shape(int32_t R, int64_t E, int32_t F, bool aligned16, bool aligned8, bool narrow_slabs = false)
 {
     SpmmShape s{};
+    const int64_t M = (int64_t)R + E;
+    s.chunk = spmm_chunk_for(M);
+    s.nchunks = (int)ceil_div(M > 0 ? M : 1, s.chunk);
     s.vec = (F % 4 == 0 && aligned16) ? 4 : (F % 2 == 0 && aligned8) ? 2 : 1;
     if (narrow_slabs && F > kWave) {
         s.vec = 1;
         s.nt = 1;
         s.slabs = (int)ceil_div(F, kWave);
-        const int64_t M = (int64_t)R + E;
-        s.chunk = pick_chunk(M);
-        s.nchunks = (int)ceil_div(M > 0 ? M : 1, s.chunk);
         return s;
     }
     // prefer the narrowest vector that still covers F with one tile per lane:
@@ -486,27 +476,40 @@ static SpmmShape spmm_shape(int32_t R, int64_t E, int32_t F, bool aligned16, boo
     s.nt = tiles <= 8 ? tiles : 8;
     if (s.nt == 7) s.nt = 8;
     s.slabs = (int)ceil_div(F, per_tile * s.nt);
-    const int64_t M = (int64_t)R + E;
-    s.chunk = pick_chunk(M);
-    s.nchunks = (int)ceil_div(M > 0 ? M : 1, s.chunk);
     return s;
 }
 
 static bool narrow_width(int32_t F) { return F == 1 || F == 2 || F == 4 || F == 8; }
 
-size_t spmm_ws_bytes(int32_t R, int64_t E, int32_t F)
+// Row pieces and group sums; `with_starts` adds the chunk starts of a call that brings no plan.
+static size_t spmm_scratch_bytes(int32_t R, int64_t E, int32_t F, bool with_starts)
 {
     SpmmShape s = spmm_shape(R, E, F, true, true);
-    const size_t wide = carve_bytes((size_t)s.nchunks + 1, 4) + carve_bytes((size_t)s.nchunks * (size_t)F, 4) +
+    const size_t wide = (with_starts ? carve_bytes((size_t)s.nchunks + 1, sizeof(int2)) : 0) +
+                        carve_bytes((size_t)s.nchunks * (size_t)F, 4) +
                         carve_bytes((size_t)ceil_div(s.nchunks, kGroup) * (size_t)F, 4);
     const size_t narrow = narrow_width(F) ? entry_tiles_ws_bytes(E) : 0;
     return wide > narrow ? wide : narrow;
 }
 
+size_t spmm_ws_bytes(int32_t R, int64_t E, int32_t F) { return spmm_scratch_bytes(R, E, F, true); }
+
+// What the host knows about the lists of a plan: -1 = nothing (the kernels read the lengths from
+// the plan and loop over a grid of fixed size), 0 = empty (no launch), n > 0 = at most n entries.
+struct PlanHints {
+    int n_fix = -1, n_grp = -1;
+};
+
+static unsigned list_grid(int hint, int upper)
+{
+    const int64_t n = hint >= 0 ? (hint < upper ? hint : upper) : (upper < 8192 ? upper : 8192);
+    return (unsigned)ceil_div(n > 0 ? n : 1, kSpmmWaves);
+}
+
 template <int VEC, int NT>
 static void launch_spmm(const SpmmShape &s, const int32_t *off, const int32_t *idx, const float *w, const float *x,
-                        float *out, float *partial, float *group_sum, const int32_t *chunk_row, int R, int C, int E,
-                        int F, hipStream_t st, hipEvent_t k0 = nullptr, hipEvent_t k1 = nullptr,
+                        float *out, float *partial, float *group_sum, const ChunkPlan &plan, const PlanHints &hints,
+                        int R, int C, int E, int F, hipStream_t st, hipEvent_t k0 = nullptr, hipEvent_t k1 = nullptr,
                         const RowFinish *fin = nullptr, int x_stride = 0)
 {
     dim3 grid((unsigned)ceil_div(s.nchunks, kSpmmWaves), (unsigned)s.slabs), block(kSpmmThreads);
@@ -528,7 +531,7 @@ static void launch_spmm(const SpmmShape &s, const int32_t *off, const int32_t *i
     f.x_stride = x_stride;
 #define JG_GO(W, L, P)                                                                                              \
     hipLaunchKernelGGL((spmm_merge<VEC, NT, U, W, L, P>), grid, block, 0, st, off, idx, w, x, out, partial,         \
-                       chunk_row, R, C, E, F, s.chunk, s.nchunks, f)
+                       plan.start, R, C, E, F, s.nchunks, f)
     if (fused && lds) JG_GO(false, true, true);
     else if (fused) JG_GO(false, false, true);
     else if (narrow && lds) JG_GO(false, true, false);
@@ -537,16 +540,25 @@ static void launch_spmm(const SpmmShape &s, const int32_t *off, const int32_t *i
     else JG_GO(true, false, false);
 #undef JG_GO
     if (k1) (void)hipEventRecord(k1, st);
+    // pieces of rows cut across chunks: only rows longer than half a chunk ever are
     const int ngroups = (int)ceil_div(s.nchunks, kGroup);
-    if (ngroups > 1)
-        hipLaunchKernelGGL((spmm_group_sums<VEC, NT>), dim3((unsigned)ceil_div(ngroups, kSpmmWaves), (unsigned)s.slabs),
-                           block, 0, st, off, partial, group_sum, chunk_row, R, F, s.chunk, s.nchunks);
-    if (fused)
-        hipLaunchKernelGGL((spmm_fixup<VEC, NT, true>), grid, block, 0, st, off, out, partial, group_sum, chunk_row, F,
-                           s.chunk, s.nchunks, f);
-    else
-        hipLaunchKernelGGL((spmm_fixup<VEC, NT, false>), grid, block, 0, st, off, out, partial, group_sum, chunk_row, F,
-                           s.chunk, s.nchunks, f);
+    const bool listed = plan.fix != nullptr;
+    const int n_grp = listed ? hints.n_grp : -1, n_fix = listed ? hints.n_fix : -1;
+    if (ngroups > 1 && n_grp != 0 && n_fix != 0)
+        hipLaunchKernelGGL((spmm_group_sums<VEC, NT>),
+                           dim3(listed ? list_grid(n_grp, ngroups) : (unsigned)ceil_div(ngroups, kSpmmWaves),
+                                (unsigned)s.slabs),
+                           block, 0, st, off, partial, group_sum, plan.start, plan.grp, plan.counts + 1, R, F, s.chunk,
+                           s.nchunks);
+    if (n_fix != 0) {
+        const dim3 fgrid(listed ? list_grid(n_fix, s.nchunks) : grid.x, (unsigned)s.slabs);
+        if (fused)
+            hipLaunchKernelGGL((spmm_fixup<VEC, NT, true>), fgrid, block, 0, st, off, out, partial, group_sum,
+                               plan.start, plan.fix, plan.counts, R, F, s.chunk, s.nchunks, f);
+        else
+            hipLaunchKernelGGL((spmm_fixup<VEC, NT, false>), fgrid, block, 0, st, off, out, partial, group_sum,
+                               plan.start, plan.fix, plan.counts, R, F, s.chunk, s.nchunks, f);
+    }
     if (fin && !fused) {
         const int64_t n = (int64_t)R * F;
         hipLaunchKernelGGL(spmm_finish_rows, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, st, out, fin->h, n, F,
@@ -574,10 +586,13 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_workspa
     return 0;
 }
 
+// plan == nullptr: the chunk starts are computed into the workspace first (one more launch) and
+// every chunk and group is looked at by the fix-up kernels.
 static int32_t spmm_call(const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out,
                          int32_t R, int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, void *stream,
                          hipEvent_t k0, hipEvent_t k1, const RowFinish *fin = nullptr, bool narrow_slabs = false,
-                         int x_stride = 0)
+                         int x_stride = 0, const void *plan = nullptr, const void *tiles = nullptr,
+                         PlanHints hints = PlanHints())
 {
     if (int32_t rc = check_spmm_sizes(R, E, F)) return rc;
     if (C < 0) return fail(JGAMD_ERR_SIZE, "spmm_csx: negative C");
@@ -586,19 +601,21 @@ static int32_t spmm_call(const int32_t *off, const int32_t *idx, const float *w,
     if (E > 0 && !x) return fail(JGAMD_ERR_NULL, "spmm_csx: x is NULL with E > 0");
     if (E > 0 && C == 0) return fail(JGAMD_ERR_SIZE, "spmm_csx: E > 0 entries but x has no rows");
     if ((((uintptr_t)x | (uintptr_t)out) & 3) != 0) return fail(JGAMD_ERR_ALIGN, "spmm_csx: x/out not 4-byte aligned");
-    const size_t need = spmm_ws_bytes(R, E, F);
-    if (!ws || ws_bytes < need)
-        return fail(JGAMD_ERR_WORKSPACE, "spmm_csx: workspace %zu < %zu bytes", ws ? ws_bytes : (size_t)0, need);
-    if (((uintptr_t)ws & 255) != 0) return fail(JGAMD_ERR_ALIGN, "spmm_csx: workspace not 256-byte aligned");
-
     // Rows of 1, 2, 4 or 8 floats: a lane per entry and a segmented scan instead of a wavefront
     // per entry (JGAMD_SPMM_NARROW=merge keeps the wide-row kernels).  Entries must tile [0, E).
     static const bool narrow_off = [] {
         const char *e = getenv("JGAMD_SPMM_NARROW");
         return e && e[0] == 'm';
     }();
-    if (!fin && !k0 && !narrow_off && E > 0 && narrow_width(F) && narrow_spmm_supported(F, x)) {
-        narrow_spmm_enqueue(off, idx, w, x, out, R, C, E, F, ws, static_cast<hipStream_t>(stream));
+    const bool narrow_route = !fin && !k0 && !narrow_off && x_stride == 0 && E > 0 && narrow_width(F) &&
+                              narrow_spmm_supported(F, x) && (tiles || !plan);
+    const size_t need = narrow_route ? entry_tiles_ws_bytes(E) : spmm_scratch_bytes(R, E, F, plan == nullptr);
+    if (!ws || ws_bytes < need)
+        return fail(JGAMD_ERR_WORKSPACE, "spmm_csx: workspace %zu < %zu bytes", ws ? ws_bytes : (size_t)0, need);
+    if (((uintptr_t)ws & 255) != 0) return fail(JGAMD_ERR_ALIGN, "spmm_csx: workspace not 256-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (narrow_route) {
+        narrow_spmm_enqueue(off, idx, w, x, out, R, C, E, F, ws, st, tiles);
         return launch_status("spmm_csx");
     }
 
@@ -613,16 +630,22 @@ static int32_t spmm_call(const int32_t *off, const int32_t *idx, const float *w,
     const uintptr_t bits = (uintptr_t)x | (uintptr_t)out | (uintptr_t)(fin ? fin->h : nullptr);
     const SpmmShape s = spmm_shape(R, E, F, (bits & 15) == 0, (bits & 7) == 0, narrow_slabs);
     Carver carve(ws);
-    int32_t *chunk_row = carve.take<int32_t>((size_t)s.nchunks + 1);
+    ChunkPlan pv{};
+    if (plan) {
+        pv = chunk_plan_view(JGAMD_PLAN_SPMM, R, E, plan);
+    } else {
+        int2 *start = carve.take<int2>((size_t)s.nchunks + 1);
+        chunk_starts_enqueue(off, R, E, s.chunk, s.nchunks, start, st);
+        pv.start = start;
+        pv.chunk = s.chunk;
+        pv.nchunks = s.nchunks;
+    }
     float *partial = carve.take<float>((size_t)s.nchunks * (size_t)F);
     float *group_sum = carve.take<float>((size_t)ceil_div(s.nchunks, kGroup) * (size_t)F);
-    hipStream_t st = static_cast<hipStream_t>(stream);
 
-    hipLaunchKernelGGL(spmm_chunk_rows, dim3((unsigned)ceil_div(s.nchunks + 1, 256)), dim3(256), 0, st, off, R,
-                       s.chunk, s.nchunks, chunk_row);
 #define JG_CASE(V, N)                                                                                \
     if (s.vec == V && s.nt == N) {                                                                   \
-        launch_spmm<V, N>(s, off, idx, w, x, out, partial, group_sum, chunk_row, R, C, (int)E, F, st, k0, k1, fin, x_stride); \
+        launch_spmm<V, N>(s, off, idx, w, x, out, partial, group_sum, pv, hints, R, C, (int)E, F, st, k0, k1, fin, x_stride); \
         return launch_status("spmm_csx");                                                            \
     }
 #define JG_CASES(V) JG_CASE(V, 1) JG_CASE(V, 2) JG_CASE(V, 3) JG_CASE(V, 4) JG_CASE(V, 5) JG_CASE(V, 6) JG_CASE(V, 8)
@@ -654,11 +677,45 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_axpby(
     return spmm_call(off, idx, w, x, out, R, C, E, F, ws, ws_bytes, stream, nullptr, nullptr, &fin);
 }
 
+// The product with the partition of a plan (jgamd_csx_plan): no per-call search of the chunk
+// starts, and the piece kernels run over the plan's lists only.
+extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_planned(
+    const void *plan, const void *tiles, int32_t n_fix, int32_t n_grp, const int32_t *off, const int32_t *idx,
+    const float *w, const float *x, float *out, float beta, float alpha, const float *h, int32_t h_rows, int32_t R,
+    int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, void *stream)
+{
+    if (!plan && !tiles) return fail(JGAMD_ERR_NULL, "spmm_csx_planned: plan and tiles are both NULL");
+    if (!plan && !narrow_width(F))
+        return fail(JGAMD_ERR_NULL, "spmm_csx_planned: rows of %d floats need the chunk plan, not the tile plan", F);
+    if ((((uintptr_t)plan | (uintptr_t)tiles) & 255) != 0)
+        return fail(JGAMD_ERR_ALIGN, "spmm_csx_planned: plan not 256-byte aligned");
+    if (h && (((uintptr_t)h & 3) != 0)) return fail(JGAMD_ERR_ALIGN, "spmm_csx_planned: h not 4-byte aligned");
+    if (h && h_rows != 1 && h_rows != R)
+        return fail(JGAMD_ERR_SIZE, "spmm_csx_planned: h has %d rows, expected %d or 1", h_rows, R);
+    PlanHints hints;
+    hints.n_fix = n_fix < 0 ? -1 : n_fix;
+    hints.n_grp = n_grp < 0 ? -1 : n_grp;
+    const bool plain = beta == 1.f && (alpha == 0.f || !h);
+    const RowFinish fin{beta, alpha, alpha != 0.f ? h : nullptr, h_rows == 1 ? 0 : F, 0};
+    return spmm_call(off, idx, w, x, out, R, C, E, F, ws, ws_bytes, stream, nullptr, nullptr, plain ? nullptr : &fin,
+                     false, 0, plan, tiles, hints);
+}
+
+extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_planned_workspace(int32_t R, int64_t E,
+                                                                                           int32_t F, size_t *bytes)
+{
+    if (!bytes) return fail(JGAMD_ERR_NULL, "spmm_csx_planned_workspace: bytes is NULL");
+    if (int32_t rc = check_spmm_sizes(R, E, F)) return rc;
+    *bytes = (R == 0 || F == 0) ? 0 : spmm_scratch_bytes(R, E, F, false);
+    return 0;
+}
+
 namespace jg {
 int32_t spmm_enqueue(const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out, int32_t R,
-                     int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, hipStream_t s)
+                     int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, hipStream_t s, const void *tiles)
 {
-    return spmm_call(off, idx, w, x, out, R, C, E, F, ws, ws_bytes, s, nullptr, nullptr);
+    return spmm_call(off, idx, w, x, out, R, C, E, F, ws, ws_bytes, s, nullptr, nullptr, nullptr, false, 0, nullptr,
+                     tiles);
 }
 int32_t spmm_enqueue_slabs(const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out,
                            int32_t R, int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, hipStream_t s,

@@ -158,7 +158,13 @@ __global__ __launch_bounds__(256) void blocked_pad_rows(const float *__restrict_
 // a row is two whole lines (a 2408-byte row's slabs straddle three: F = 602 ran 25.4 -> 20.4 ms).
 // Rows of one slab: a multiple of 16 floats, which already fixes the number of lines a row touches
 // and keeps the block's footprint in L2 smaller than whole-line rows would.
-static int padded_width(int F) { return F <= kWave ? (F + 15) & ~15 : (F + 31) & ~31; }
+// Rows of 1, 2, 4 or 8 floats stay as they are: they never straddle a line they need not, and
+// the product's kernels for those widths read rows F floats apart.
+static int padded_width(int F)
+{
+    if (F == 1 || F == 2 || F == 4 || F == 8) return F;
+    return F <= kWave ? (F + 15) & ~15 : (F + 31) & ~31;
+}
 
 static int env_kb(const char *name, int dflt)
 {

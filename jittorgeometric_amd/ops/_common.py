@@ -26,6 +26,17 @@ def _stamp(t):
     return None if t is None else (id(t), t._version)
 
 
+def _same_storage(a, b):
+    """a and b are the same array: one object, or two views of the same memory with the same
+    shape and strides (x.reshape(-1) of a flat tensor makes a new object every call)."""
+    if a is b:
+        return True
+    if a is None or b is None:
+        return False
+    return (a.data_ptr() == b.data_ptr() and a.shape == b.shape and a.stride() == b.stride()
+            and a.dtype == b.dtype and a._version == b._version)
+
+
 def _holder_arrays(holder, names, what):
     """(off, idx, w) of a CSC / CSR object as contiguous int32 / int32 / float32
     device arrays.  Holders built by hand carry whatever torch.tensor([...]) gave
@@ -103,6 +114,40 @@ def transposed_inverse(holder, perm):
     return inv
 
 
+PLAN_SPMM, PLAN_GAT, PLAN_TILES = 0, 1, 2
+
+
+def csx_plan(off, R, E, kind):
+    """(plan, n_fix, n_grp) for the offsets `off` of R rows and E entries: the partition the
+    merge-path kernels (PLAN_SPMM, PLAN_GAT) or the tile kernels (PLAN_TILES) work from, built
+    on first use and kept on the offsets tensor until it is written in place (a rebound
+    attribute is another tensor and gets its own).  The two counts are the lengths of the
+    plan's lists of cut rows, read back once when the plan is built; 0 lets a call skip the
+    kernels that add up row pieces.  Returns (None, -1, -1) while a HIP graph is being captured
+    and no plan exists yet: building one would allocate from the graph's pool and read back."""
+    cache = getattr(off, "_jgamd_plans", None)
+    if cache is None:
+        cache = {}
+        off._jgamd_plans = cache
+    stamp = (off._version, R, E)
+    hit = cache.get(kind)
+    if hit is not None and hit[0] == stamp:
+        return hit[1], hit[2], hit[3]
+    if torch.cuda.is_current_stream_capturing():
+        return None, -1, -1
+    lib = _lib.load()
+    dev = off.device
+    nbytes = _lib.query(lib.jgamd_csx_plan_bytes, R, E, kind)
+    plan = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=dev)
+    stream = _lib.stream_ptr(dev)
+    _lib.check(lib.jgamd_csx_plan(_lib.ptr(off), R, E, kind, _lib.ptr(plan), nbytes, stream))
+    n_fix, n_grp = _c.c_int32(-1), _c.c_int32(-1)
+    if kind != PLAN_TILES and R > 0:
+        _lib.check(lib.jgamd_csx_plan_counts(_lib.ptr(plan), _c.byref(n_fix), _c.byref(n_grp), stream))
+    cache[kind] = (stamp, plan, n_fix.value, n_grp.value)
+    return plan, n_fix.value, n_grp.value
+
+
 def _raw_arrays(off, idx, w, R):
     """Last line of defence in front of the pointer hand-over: dtype, layout and the
     length of the offsets (no copy when the arrays already are what the kernels read)."""
@@ -120,9 +165,11 @@ def _blocked_arrays(off, idx, w, R, E, nb, cols):
     """The matrix regrouped by column block (csrc/spmm_blocked.hip), built on first use and
     kept on the offsets tensor it was built from until one of the three arrays is another
     tensor or has been written in place."""
-    stamp = (_stamp(off), _stamp(idx), _stamp(w), nb, cols)
+    # the weights are matched by memory and version, not by object: an explicit edge_weight
+    # arrives as a fresh view (reshape(-1)) on every call
+    stamp = (_stamp(off), _stamp(idx), None if w is None else w._version, nb, cols)
     cached = getattr(off, "_jgamd_blocked", None)
-    if cached is not None and cached[0] == stamp and cached[1] is idx and cached[2] is w:
+    if cached is not None and cached[0] == stamp and cached[1] is idx and _same_storage(cached[2], w):
         return cached[3]
     lib = _lib.load()
     dev = off.device
@@ -166,6 +213,18 @@ def _product(off, idx, w, x, R, beta, alpha, h):
         _lib.check(lib.jgamd_spmm_csx_blocked(_lib.ptr(b_off), _lib.ptr(b_idx), _lib.ptr(b_w), _lib.ptr(x), _lib.ptr(out),
                                               float(beta), float(alpha), _lib.ptr(h), h_rows, R, C, E, F, nb.value,
                                               _lib.ptr(ws), nbytes, stream))
+        return out
+    # the partition of the rows is kept with the offsets: the chunk plan, or the tile plan for
+    # rows of 1, 2, 4 or 8 floats
+    narrow = F in (1, 2, 4, 8) and E > 0
+    plan, n_fix, n_grp = csx_plan(off, R, E, PLAN_TILES if narrow else PLAN_SPMM) if R > 0 else (None, -1, -1)
+    if plan is not None:
+        nbytes = _lib.query(lib.jgamd_spmm_csx_planned_workspace, R, E, F)
+        ws = _lib.workspace(nbytes, dev)
+        _lib.check(lib.jgamd_spmm_csx_planned(None if narrow else _lib.ptr(plan), _lib.ptr(plan) if narrow else None,
+                                              n_fix, n_grp, _lib.ptr(off), _lib.ptr(idx), _lib.ptr(w), _lib.ptr(x),
+                                              _lib.ptr(out), float(beta), float(alpha), _lib.ptr(h), h_rows, R, C, E,
+                                              F, _lib.ptr(ws), nbytes, stream))
         return out
     nbytes = _lib.query(lib.jgamd_spmm_csx_workspace, R, E, F)
     ws = _lib.workspace(nbytes, dev)

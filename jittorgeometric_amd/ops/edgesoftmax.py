@@ -6,7 +6,7 @@ independent heads."""
 import torch
 
 from .. import _lib
-from ._common import as_f32, csc_arrays
+from ._common import PLAN_TILES, as_f32, csc_arrays, csx_plan
 
 
 def _heads(x):
@@ -26,8 +26,13 @@ class EdgeSoftmaxFunc(torch.autograd.Function):
         y = torch.empty(x.shape, dtype=torch.float32, device=dev)
         nbytes = _lib.query(lib.jgamd_edge_softmax_workspace, V, E)
         ws = _lib.workspace(nbytes, dev)
-        _lib.check(lib.jgamd_edge_softmax_fwd(_lib.ptr(off), _lib.ptr(x), _lib.ptr(y), V, E, H, _lib.ptr(ws), nbytes,
-                                              _lib.stream_ptr(dev)))
+        tiles = csx_plan(off, V, E, PLAN_TILES)[0] if H in (1, 2, 4, 8) and V > 0 and E > 0 else None
+        if tiles is not None:
+            _lib.check(lib.jgamd_edge_softmax_fwd_planned(_lib.ptr(tiles), _lib.ptr(off), _lib.ptr(x), _lib.ptr(y), V, E,
+                                                          H, _lib.ptr(ws), nbytes, _lib.stream_ptr(dev)))
+        else:
+            _lib.check(lib.jgamd_edge_softmax_fwd(_lib.ptr(off), _lib.ptr(x), _lib.ptr(y), V, E, H, _lib.ptr(ws),
+                                                  nbytes, _lib.stream_ptr(dev)))
         ctx.save_for_backward(y)
         ctx.csc = csc
         return y
@@ -43,8 +48,14 @@ class EdgeSoftmaxFunc(torch.autograd.Function):
         dx = torch.empty(y.shape, dtype=torch.float32, device=dev)
         nbytes = _lib.query(lib.jgamd_edge_softmax_workspace, V, E)
         ws = _lib.workspace(nbytes, dev)
-        _lib.check(lib.jgamd_edge_softmax_bwd(_lib.ptr(off), _lib.ptr(y), _lib.ptr(g), _lib.ptr(dx), V, E, H,
-                                              _lib.ptr(ws), nbytes, _lib.stream_ptr(dev)))
+        tiles = csx_plan(off, V, E, PLAN_TILES)[0] if H in (1, 2, 4, 8) and V > 0 and E > 0 else None
+        if tiles is not None:
+            _lib.check(lib.jgamd_edge_softmax_bwd_planned(_lib.ptr(tiles), _lib.ptr(off), _lib.ptr(y), _lib.ptr(g),
+                                                          _lib.ptr(dx), V, E, H, _lib.ptr(ws), nbytes,
+                                                          _lib.stream_ptr(dev)))
+        else:
+            _lib.check(lib.jgamd_edge_softmax_bwd(_lib.ptr(off), _lib.ptr(y), _lib.ptr(g), _lib.ptr(dx), V, E, H,
+                                                  _lib.ptr(ws), nbytes, _lib.stream_ptr(dev)))
         return dx, None
 
 

@@ -6,7 +6,7 @@ EdgeSoftmax -> multiply -> ScatterToVertex of GATConv.propagate
 import torch
 
 from .. import _lib
-from ._common import as_f32, csc_arrays, transposed, transposed_inverse
+from ._common import PLAN_GAT, PLAN_TILES, as_f32, csc_arrays, csx_plan, transposed, transposed_inverse
 
 
 def fused_supported(H, D, backward=True):
@@ -41,7 +41,8 @@ def gat_forward_raw(h, csc, a_src, a_dst, slope=0.2, want_alpha=False):
     alpha = mk(E, H) if want_alpha else None
     nbytes = _lib.query(lib.jgamd_gat_fwd_workspace, V, E, H, D)
     ws = _lib.workspace(nbytes, dev)
-    _lib.check(lib.jgamd_gat_fwd(_lib.ptr(off), _lib.ptr(idx), _lib.ptr(h),
+    plan, n_fix, n_grp = csx_plan(off, V, E, PLAN_GAT) if V > 0 else (None, -1, -1)
+    _lib.check(lib.jgamd_gat_fwd(_lib.ptr(plan), n_fix, n_grp, _lib.ptr(off), _lib.ptr(idx), _lib.ptr(h),
                                  _lib.ptr(a_src), _lib.ptr(a_dst), float(slope), _lib.ptr(el), _lib.ptr(er),
                                  _lib.ptr(smax), _lib.ptr(ssum), _lib.ptr(alpha), _lib.ptr(out), V, E, H, D,
                                  _lib.ptr(ws), nbytes, _lib.stream_ptr(dev)))
@@ -76,7 +77,10 @@ class GatFusedFunc(torch.autograd.Function):
         g_ad = torch.empty((H, D), dtype=torch.float32, device=dev)
         nbytes = _lib.query(lib.jgamd_gat_bwd_workspace, V, E, H, D)
         ws = _lib.workspace(nbytes, dev)
-        _lib.check(lib.jgamd_gat_bwd(_lib.ptr(off), _lib.ptr(idx), _lib.ptr(off_t),
+        plan, n_fix, n_grp = csx_plan(off_t, V, E, PLAN_GAT) if V > 0 else (None, -1, -1)
+        tiles = csx_plan(off, V, E, PLAN_TILES)[0] if V > 0 and E > 0 else None
+        _lib.check(lib.jgamd_gat_bwd(_lib.ptr(plan), n_fix, n_grp, _lib.ptr(tiles), _lib.ptr(off), _lib.ptr(idx),
+                                     _lib.ptr(off_t),
                                      _lib.ptr(idx_t), _lib.ptr(inv), _lib.ptr(h), _lib.ptr(a_src), _lib.ptr(a_dst),
                                      float(ctx.slope), _lib.ptr(el), _lib.ptr(er), _lib.ptr(smax), _lib.ptr(ssum),
                                      _lib.ptr(out), _lib.ptr(g_out), _lib.ptr(g_h), _lib.ptr(g_as), _lib.ptr(g_ad),

@@ -78,6 +78,9 @@ def test_argument_errors_are_reported_not_launched(lib):
     assert lib.jgamd_gat_fwd_workspace(10, 10, 4, 1024, ctypes.byref(n)) == -4
     assert lib.jgamd_gat_bwd_workspace(10, 10, 3, 7, ctypes.byref(n)) == -4
     assert lib.jgamd_gat_bwd_workspace(10, 10, 1, 7, ctypes.byref(n)) == 0
+    # rows without classes: refused on the host, nothing is launched on a [V,0] array's NULL address
+    assert lib.jgamd_cross_entropy_fwd(None, bad, 0, 0, 5, 0, bad, bad, bad, bad, 1 << 20, None) == -2
+    assert b"C=0" in lib.jgamd_last_error()
 
 
 def test_operators_refuse_cpu_tensors():

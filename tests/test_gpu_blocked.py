@@ -88,7 +88,7 @@ def test_regrouping_without_weights_and_with_entries_past_the_last_offset():
     assert (b_idx.cpu().numpy()[covered:] == -7).all()      # slots past the covered entries are left alone
 
 
-@pytest.mark.parametrize("F", [9, 41, 64, 100, 130, 256])
+@pytest.mark.parametrize("F", [1, 3, 4, 8, 9, 41, 64, 100, 130, 256])
 @pytest.mark.parametrize("V,E,nb,cols", [(600, 90000, 8, 80), (3000, 40000, 5, 700)])
 def test_blocked_product_matches_oracle_and_unblocked(V, E, nb, cols, F):
     from jittorgeometric_amd.ops._common import spmm

@@ -63,4 +63,5 @@ def test_shape_beyond_the_fixed_array_is_rejected_without_a_launch():
     assert lib.jgamd_spmm_csx_workspace(V, E, F, ctypes.byref(n)) == 0 and n.value > 64 << 20
     bad = ctypes.c_void_p(256)     # never dereferenced
     rc = lib.jgamd_spmm_csx_noalloc(bad, bad, bad, bad, bad, V, V, E, F, None)
-    assert rc == -2 and b"64" in lib.jgamd_last_error() or b"67108864" in lib.jgamd_last_error()
+    assert rc == -2
+    assert b"67108864" in lib.jgamd_last_error()
