@@ -265,38 +265,45 @@ int32_t jgamd_scatter_to_edge(const int32_t *off, const int32_t *idx, const floa
  *   el,er  [V,H]  outputs: a_src.h and a_dst.h per node and head
  *   smax, ssum [V,H] outputs: per destination and head, the max logit and
  *          the sum of exp(logit - max) (what backward needs to rebuild alpha)
+ *   pos [V,H,D], spos [V,H]  optional outputs (both or neither): the share of
+ *          out / of the attention that lies on edges with a positive logit,
+ *          pos[v,k,:] = sum_{e: z_e > 0} alpha[e,k] h[idx[e],k,:],
+ *          spos[v,k] = sum_{e: z_e > 0} alpha[e,k].  jgamd_gat_bwd takes them:
+ *          with LeakyReLU' in {1, slope} they give the gradient with respect
+ *          to er per node, without a second pass over the edges.
  *   alpha  optional [E,H] output (NULL to skip): attention per CSC slot
  *   out    [V,H,D]:  out[v,k,:] = sum_e alpha[e,k] * h[idx[e],k,:]
+ *   plan   a JGAMD_PLAN_GAT plan of `off` with its list lengths n_fix / n_grp
+ *          (see jgamd_csx_plan), or NULL (n_fix, n_grp ignored)
  * H = 1, D = C reproduces the reference's single head.
  */
 int32_t jgamd_gat_fwd_workspace(int32_t V, int64_t E, int32_t H, int32_t D, size_t *bytes);
 int32_t jgamd_gat_fwd(const void *plan, int32_t n_fix, int32_t n_grp, const int32_t *off,
-                      const int32_t *idx, const float *h, const float *a_src, const float *a_dst, float slope, float *el,
-                      float *er, float *smax, float *ssum, float *alpha, float *out,
-                      int32_t V, int64_t E, int32_t H, int32_t D, void *ws, size_t ws_bytes,
-                      void *stream);
+                      const int32_t *idx, const float *h, const float *a_src,
+                      const float *a_dst, float slope, float *el, float *er, float *smax,
+                      float *ssum, float *pos, float *spos, float *alpha, float *out, int32_t V,
+                      int64_t E, int32_t H, int32_t D, void *ws, size_t ws_bytes, void *stream);
 
-/* Backward of jgamd_gat_fwd.  Needs both orders of the graph: (off, idx) are
- * the CSC arrays used forward, (t_off, t_idx) their transpose as produced by
- * jgamd_csx_transpose, and t_inv[j] = transposed slot of CSC slot j, i.e. the
- * inverse of that call's out_perm (jgamd_invert_permutation).
+/* Backward of jgamd_gat_fwd, one pass over the transposed arrays (t_off, t_idx)
+ * of the graph as produced by jgamd_csx_transpose (rows = sources); t_plan is a
+ * JGAMD_PLAN_GAT plan of t_off, or NULL.
  * With H > 1 the head width D must span a power-of-two number of lanes
  * (D in {1,2,4,...,256}); other shapes return JGAMD_ERR_UNSUPPORTED and are
  * served by the unfused operator chain.
- *   g_out [V,H,D] upstream gradient, out [V,H,D] forward result
+ *   el, er, smax, ssum, spos, out, pos: what jgamd_gat_fwd wrote
+ *   g_out [V,H,D] upstream gradient
  *   g_h   [V,H,D], g_a_src [H,D], g_a_dst [H,D] outputs
  * Replaces the grad chain edgetovertex <-> scattertoedge <->
  * edgesoftmaxbackward that Jittor autograd builds for gat_conv.py:61-83.
  */
 int32_t jgamd_gat_bwd_workspace(int32_t V, int64_t E, int32_t H, int32_t D, size_t *bytes);
-int32_t jgamd_gat_bwd(const void *t_plan, int32_t n_fix, int32_t n_grp, const void *tiles,
-                      const int32_t *off, const int32_t *idx, const int32_t *t_off,
-                      const int32_t *t_idx, const int32_t *t_inv, const float *h, const float *a_src,
+int32_t jgamd_gat_bwd(const void *t_plan, int32_t n_fix, int32_t n_grp, const int32_t *t_off,
+                      const int32_t *t_idx, const float *h, const float *a_src,
                       const float *a_dst, float slope, const float *el, const float *er,
-                      const float *smax, const float *ssum, const float *out,
-                      const float *g_out, float *g_h, float *g_a_src, float *g_a_dst,
-                      int32_t V, int64_t E, int32_t H, int32_t D, void *ws, size_t ws_bytes,
-                      void *stream);
+                      const float *smax, const float *ssum, const float *spos, const float *out,
+                      const float *pos, const float *g_out, float *g_h, float *g_a_src,
+                      float *g_a_dst, int32_t V, int64_t E, int32_t H, int32_t D, void *ws,
+                      size_t ws_bytes, void *stream);
 
 /* ------------------------------------------------------------------------
  * Column-blocked product for matrices with long rows (hundreds of entries

@@ -62,11 +62,11 @@ SIGNATURES = {
     "jgamd_cross_entropy_fwd": [_P, _P, _I32, _I32, _I64, _I32, _P, _P, _P, _P, _c.c_size_t, _P],
     "jgamd_cross_entropy_bwd": [_P, _P, _I32, _P, _P, _P, _I64, _I32, _P, _P],
     "jgamd_gat_fwd_workspace": [_I32, _I64, _I32, _I32, _SZP],
-    "jgamd_gat_fwd": [_P, _I32, _I32, _P, _P, _P, _P, _P, _F32, _P, _P, _P, _P, _P, _P, _I32, _I64, _I32, _I32, _P,
-                      _c.c_size_t, _P],
+    "jgamd_gat_fwd": [_P, _I32, _I32, _P, _P, _P, _P, _P, _F32, _P, _P, _P, _P, _P, _P, _P, _P, _I32, _I64, _I32,
+                      _I32, _P, _c.c_size_t, _P],
     "jgamd_gat_bwd_workspace": [_I32, _I64, _I32, _I32, _SZP],
-    "jgamd_gat_bwd": [_P, _I32, _I32, _P, _P, _P, _P, _P, _P, _P, _P, _P, _F32, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I32, _I64,
-                      _I32, _I32, _P, _c.c_size_t, _P],
+    "jgamd_gat_bwd": [_P, _I32, _I32, _P, _P, _P, _P, _P, _F32, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I32,
+                      _I64, _I32, _I32, _P, _c.c_size_t, _P],
 }
 
 _lib = None

@@ -16,7 +16,25 @@
 // accumulator when the max grows; a row cut by a chunk boundary leaves its
 // unnormalised (acc, max, sum) piece in scratch and a second kernel merges
 // the pieces in order.  No float atomics anywhere.
+//
+// Backward.  With z_e = el[src] + er[dst], alpha the softmax of lrelu(z) over a
+// destination's in-edges and out[c] = sum_e alpha_e h[src_e]:
+//   dz_e    = lrelu'(z_e) alpha_e (g[c].h[src_e] - g[c].out[c])
+//   g_h[r]  = sum_{e out of r} alpha_e g[dst_e] + a_src g_el[r] + a_dst g_er[r]
+//   g_el[r] = sum_{e out of r} dz_e          g_er[c] = sum_{e into c} dz_e
+// One pass over the transposed arrays (rows = sources) gives the first two sums.
+// The destination-side sum needs no pass over the edges at all: with lrelu' in
+// {1, slope} and the alpha of a destination adding up to one,
+//   g_er[c] = (1 - slope) (g[c].pos[c] - (g[c].out[c]) spos[c]),
+//   pos[c] = sum_{e into c, z_e > 0} alpha_e h[src_e],  spos[c] = sum_{z_e > 0} alpha_e,
+// two more accumulators of the forward pass, which gathers those rows anyway.
+// g_er is therefore known per node before the pass over the sources starts, and
+// that pass writes g_h complete; the gradients of a_src and a_dst are sums over
+// the nodes of g_el[r] h[r] and g_er[r] h[r], accumulated by the same pass (the
+// h row of the current source is in registers) per workgroup and added up in a
+// fixed order by two small kernels.
 #include <math.h>
+#include <stdlib.h>
 
 #include "common.h"
 
@@ -24,7 +42,6 @@ namespace jg {
 
 constexpr int kGatThreads = 256;
 constexpr int kGatWaves = kGatThreads / kWave;
-constexpr int kGzHeads = 16;   // heads whose logit gradients are staged in LDS by the backward pass
 // gathers in flight per wavefront, bounded by the registers they land in
 constexpr int gat_unroll(int regs) { return regs >= 16 ? 2 : regs >= 8 ? 4 : 8; }
 
@@ -128,14 +145,23 @@ __device__ __forceinline__ float lane_group_sum(float v, int lanes)
 }
 
 // ----------------------------------------------------------------- forward ---
-template <int VEC, int NT>
+// POS: also accumulate, per destination, the share of the softmax that lies on positive
+// logits -- pos[r,:] = sum_{z_e > 0} alpha_e h[src_e], spos[r,k] = sum_{z_e > 0} alpha_e --
+// which is what the backward pass needs for the destination-side logit gradient.  The two
+// accumulators ride along with (acc, l): same rescaling, same pieces, same fix-up.
+struct GatPieces {
+    float *vec, *mx, *sum;     // [n, F], [n, H], [n, H]
+    float *pvec, *psum;        // the positive-logit share, POS only
+};
+
+template <int VEC, int NT, bool POS>
 __global__ __launch_bounds__(kGatThreads) void gat_fwd_merge(
     const int32_t *__restrict__ off, const int32_t *__restrict__ idx, const float *__restrict__ h,
     const float *__restrict__ el, const float *__restrict__ er, float slope, float *__restrict__ out,
-    float *__restrict__ smax, float *__restrict__ ssum, float *__restrict__ partial, float *__restrict__ pmax,
-    float *__restrict__ psum, const int2 *__restrict__ start, int R, int E, int H, int D, int nchunks)
+    float *__restrict__ smax, float *__restrict__ ssum, float *__restrict__ pos, float *__restrict__ spos,
+    GatPieces piece, const int2 *__restrict__ start, int R, int E, int H, int D, int nchunks)
 {
-    constexpr int kGatUnroll = gat_unroll(VEC * NT);
+    constexpr int kGatUnroll = gat_unroll(VEC * NT * (POS ? 2 : 1));
     const int k = blockIdx.x * kGatWaves + wave_in_block();
     if (k >= nchunks) return;
     const int lane = lane_id();
@@ -167,11 +193,13 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_merge(
     // er of the current row and, already on its way, of the next one: a row end must not
     // wait for a fresh load (rows are a handful of entries long)
     float m[NT], l[NT], acc[NT][VEC], er_r[NT], er_next[NT];
-    auto fetch_next = [&]() {
-        const size_t rn = (size_t)min(r + 1, R - 1);
+    float lp[POS ? NT : 1], pacc[POS ? NT : 1][POS ? VEC : 1];
+    auto fetch_row = [&](int row) {
+        const size_t rn = (size_t)min(row, R - 1);
 #pragma unroll
         for (int t = 0; t < NT; t++) er_next[t] = er[rn * H + head[t]];
     };
+    auto fetch_next = [&]() { fetch_row(r + 1); };
     auto reset = [&]() {
 #pragma unroll
         for (int t = 0; t < NT; t++) {
@@ -179,19 +207,20 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_merge(
             l[t] = 0.f;
 #pragma unroll
             for (int v = 0; v < VEC; v++) acc[t][v] = 0.f;
+            if constexpr (POS) {
+                lp[t] = 0.f;
+#pragma unroll
+                for (int v = 0; v < VEC; v++) pacc[t][v] = 0.f;
+            }
             er_r[t] = er_next[t];
         }
         fetch_next();
     };
-    {
-        const size_t rc = (size_t)min(r, R - 1);
-#pragma unroll
-        for (int t = 0; t < NT; t++) er_next[t] = er[rc * H + head[t]];
-    }
+    fetch_row(r);
     reset();
 
     auto flush_row = [&]() {
-        float *dst = out + (size_t)r * F + f0;
+        const size_t base = (size_t)r * F + f0;
 #pragma unroll
         for (int t = 0; t < NT; t++) {
             if (act[t]) {
@@ -199,10 +228,16 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_merge(
                 const float inv = continued ? 1.f : (l[t] > 0.f ? 1.f / l[t] : 0.f);
 #pragma unroll
                 for (int v = 0; v < VEC; v++) o[v] = acc[t][v] * inv;
-                gstore<VEC>(dst + t * kWave * VEC, o);
+                gstore<VEC>(out + base + t * kWave * VEC, o);
+                if constexpr (POS) {
+#pragma unroll
+                    for (int v = 0; v < VEC; v++) o[v] = pacc[t][v] * inv;
+                    gstore<VEC>(pos + base + t * kWave * VEC, o);
+                }
                 if (lead[t]) {
                     smax[(size_t)r * H + head[t]] = m[t];
                     ssum[(size_t)r * H + head[t]] = l[t];
+                    if constexpr (POS) spos[(size_t)r * H + head[t]] = lp[t] * inv;
                 }
             }
         }
@@ -248,13 +283,20 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_merge(
 #pragma unroll
                         for (int t = 0; t < NT; t++)
                             if (act[t]) {
-                                const float s = lrelu(sv[u][t] + er_r[t], slope);
+                                const float z = sv[u][t] + er_r[t];
+                                const float s = lrelu(z, slope);
                                 const float mn = fmaxf(m[t], s);
                                 const float sc = fast_exp(m[t] - mn);   // 0 on the first entry (m = -inf)
                                 const float p = fast_exp(s - mn);
                                 l[t] = fmaf(l[t], sc, p);
 #pragma unroll
                                 for (int v = 0; v < VEC; v++) acc[t][v] = fmaf(acc[t][v], sc, p * xv[u][t][v]);
+                                if constexpr (POS) {
+                                    const float pp = z > 0.f ? p : 0.f;
+                                    lp[t] = fmaf(lp[t], sc, pp);
+#pragma unroll
+                                    for (int v = 0; v < VEC; v++) pacc[t][v] = fmaf(pacc[t][v], sc, pp * xv[u][t][v]);
+                                }
                                 m[t] = mn;
                             }
                     }
@@ -264,22 +306,26 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_merge(
     }
     while (r < r1) flush_row();
     if (r1 < R && j1 > uniform(off[r1])) {     // the leading piece of a row that goes on in the next chunk
-        float *dst = partial + (size_t)k * F + f0;
+        const size_t base = (size_t)k * F + f0;
 #pragma unroll
         for (int t = 0; t < NT; t++)
             if (act[t]) {
-                gstore<VEC>(dst + t * kWave * VEC, acc[t]);
+                gstore<VEC>(piece.vec + base + t * kWave * VEC, acc[t]);
+                if constexpr (POS) gstore<VEC>(piece.pvec + base + t * kWave * VEC, pacc[t]);
                 if (lead[t]) {
-                    pmax[(size_t)k * H + head[t]] = m[t];
-                    psum[(size_t)k * H + head[t]] = l[t];
+                    piece.mx[(size_t)k * H + head[t]] = m[t];
+                    piece.sum[(size_t)k * H + head[t]] = l[t];
+                    if constexpr (POS) piece.psum[(size_t)k * H + head[t]] = lp[t];
                 }
             }
     }
 }
 
-// Running softmax state of one row piece per lane: acc (unnormalised), max, sum.
-template <int VEC, int NT> struct SoftState {
+// Running softmax state of one row piece per lane: acc (unnormalised), max, sum, and with POS
+// the positive-logit share of both.
+template <int VEC, int NT, bool POS> struct SoftState {
     float M[NT], L[NT], acc[NT][VEC];
+    float LP[POS ? NT : 1], pacc[POS ? NT : 1][POS ? VEC : 1];
     __device__ __forceinline__ void clear()
     {
 #pragma unroll
@@ -288,17 +334,23 @@ template <int VEC, int NT> struct SoftState {
             L[t] = 0.f;
 #pragma unroll
             for (int v = 0; v < VEC; v++) acc[t][v] = 0.f;
+            if constexpr (POS) {
+                LP[t] = 0.f;
+#pragma unroll
+                for (int v = 0; v < VEC; v++) pacc[t][v] = 0.f;
+            }
         }
     }
-    // Merges pieces first..last-1 of (vec [.,F], pmax [.,H], psum [.,H]) in order;
-    // a few pieces are fetched at a time so that their loads overlap.
-    __device__ __forceinline__ void merge(const float *__restrict__ vec, const float *__restrict__ pmax,
-                                          const float *__restrict__ psum, int first, int last, int F, int H, int D,
-                                          int f0)
+    // Merges pieces first..last-1 of p in order; a few pieces are fetched at a time so that
+    // their loads overlap.
+    __device__ __forceinline__ void merge(const GatPieces &p, int first, int last, int F, int H, int D, int f0)
     {
-        constexpr int kBatch = VEC * NT >= 16 ? 2 : (VEC * NT >= 8 ? 4 : 8);
+        // pieces in flight: a long row's merge is a chain of such batches, one memory latency each
+        constexpr int kRegs = VEC * NT * (POS ? 2 : 1);
+        constexpr int kBatch = kRegs >= 16 ? 2 : (kRegs >= 8 ? 4 : (kRegs >= 4 ? 8 : 16));
         for (int kb = first; kb < last; kb += kBatch) {
             float x[kBatch][NT][VEC], pm[kBatch][NT], pl[kBatch][NT];
+            float px[POS ? kBatch : 1][POS ? NT : 1][POS ? VEC : 1], pp[POS ? kBatch : 1][POS ? NT : 1];
             // issue phase without branches: slots past `last` re-read the last piece and
             // lanes past F read offset 0; both are ignored below
 #pragma unroll
@@ -308,9 +360,13 @@ template <int VEC, int NT> struct SoftState {
                 for (int t = 0; t < NT; t++) {
                     const int f = f0 + t * kWave * VEC;
                     const int fc = f < F ? f : 0;
-                    gload<VEC>(x[b][t], vec + pc * F + fc);
-                    pm[b][t] = pmax[pc * H + fc / D];
-                    pl[b][t] = psum[pc * H + fc / D];
+                    gload<VEC>(x[b][t], p.vec + pc * F + fc);
+                    pm[b][t] = p.mx[pc * H + fc / D];
+                    pl[b][t] = p.sum[pc * H + fc / D];
+                    if constexpr (POS) {
+                        gload<VEC>(px[b][t], p.pvec + pc * F + fc);
+                        pp[b][t] = p.psum[pc * H + fc / D];
+                    }
                 }
             }
 #pragma unroll
@@ -325,6 +381,11 @@ template <int VEC, int NT> struct SoftState {
                             L[t] = L[t] * so + pl[b][t] * si;
 #pragma unroll
                             for (int v = 0; v < VEC; v++) acc[t][v] = acc[t][v] * so + x[b][t][v] * si;
+                            if constexpr (POS) {
+                                LP[t] = LP[t] * so + pp[b][t] * si;
+#pragma unroll
+                                for (int v = 0; v < VEC; v++) pacc[t][v] = pacc[t][v] * so + px[b][t][v] * si;
+                            }
                             M[t] = mn;
                         }
                     }
@@ -339,14 +400,9 @@ template <int VEC, int NT> struct SoftState {
 constexpr int kGatGroup = kPlanGroup;
 
 // `list` (ascending, count[0] entries) names the groups to look at; without one every group is.
-template <int VEC, int NT>
-__global__ __launch_bounds__(kGatThreads) void gat_fwd_group(const int32_t *__restrict__ off,
-                                                             const float *__restrict__ partial,
-                                                             const float *__restrict__ pmax,
-                                                             const float *__restrict__ psum,
-                                                             float *__restrict__ gvec, float *__restrict__ gmax,
-                                                             float *__restrict__ gsum,
-                                                             const int2 *__restrict__ start,
+template <int VEC, int NT, bool POS>
+__global__ __launch_bounds__(kGatThreads) void gat_fwd_group(const int32_t *__restrict__ off, GatPieces piece,
+                                                             GatPieces group, const int2 *__restrict__ start,
                                                              const int32_t *__restrict__ list,
                                                              const int32_t *__restrict__ count, int R, int H,
                                                              int D, int chunk, int nchunks)
@@ -356,7 +412,7 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_group(const int32_t *__re
     for (int i = blockIdx.x * kGatWaves + wave_in_block(); i < n; i += stride) {
         const int g = list ? uniform(list[i]) : i;
         const int kend = (g + 1) * kGatGroup;
-        if (kend >= nchunks) continue;
+        if (g < 0 || kend >= nchunks) continue;
         const int r = uniform(start[kend].x);
         if (r < 0 || r >= R) continue;
         const int s = uniform(off[r]);
@@ -364,17 +420,19 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_group(const int32_t *__re
         const int a = max((int)(((int64_t)max(s, 0) + r) / chunk), g * kGatGroup);
         const int F = H * D;
         const int f0 = lane_id() * VEC;
-        SoftState<VEC, NT> st;
+        SoftState<VEC, NT, POS> st;
         st.clear();
-        st.merge(partial, pmax, psum, a, kend, F, H, D, f0);
+        st.merge(piece, a, kend, F, H, D, f0);
 #pragma unroll
         for (int t = 0; t < NT; t++) {
             const int f = f0 + t * kWave * VEC;
             if (f < F) {
-                gstore<VEC>(gvec + (size_t)g * F + f, st.acc[t]);
+                gstore<VEC>(group.vec + (size_t)g * F + f, st.acc[t]);
+                if constexpr (POS) gstore<VEC>(group.pvec + (size_t)g * F + f, st.pacc[t]);
                 if (f % D == 0) {
-                    gmax[(size_t)g * H + f / D] = st.M[t];
-                    gsum[(size_t)g * H + f / D] = st.L[t];
+                    group.mx[(size_t)g * H + f / D] = st.M[t];
+                    group.sum[(size_t)g * H + f / D] = st.L[t];
+                    if constexpr (POS) group.psum[(size_t)g * H + f / D] = st.LP[t];
                 }
             }
         }
@@ -383,11 +441,10 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_group(const int32_t *__re
 
 // Merges, in chunk order, the pieces of a row that started in an earlier
 // chunk and ends in chunk k (its last piece sits unnormalised in out/smax/ssum).
-template <int VEC, int NT>
+template <int VEC, int NT, bool POS>
 __global__ __launch_bounds__(kGatThreads) void gat_fwd_fixup(
     const int32_t *__restrict__ off, float *__restrict__ out, float *__restrict__ smax, float *__restrict__ ssum,
-    const float *__restrict__ partial, const float *__restrict__ pmax, const float *__restrict__ psum,
-    const float *__restrict__ gvec, const float *__restrict__ gmax, const float *__restrict__ gsum,
+    float *__restrict__ pos, float *__restrict__ spos, GatPieces piece, GatPieces group,
     const int2 *__restrict__ start, const int32_t *__restrict__ list, const int32_t *__restrict__ count, int R, int H,
     int D, int chunk, int nchunks)
 {
@@ -404,16 +461,18 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_fixup(
         const int a = min((int)(((int64_t)max(s, 0) + r0) / chunk), k);
         const int F = H * D;
         const int f0 = lane_id() * VEC;
-        SoftState<VEC, NT> st;
+        SoftState<VEC, NT, POS> st;
         st.clear();
         const int ga = a / kGatGroup, gb = k / kGatGroup;
         if (ga == gb) {
-            st.merge(partial, pmax, psum, a, k, F, H, D, f0);
+            st.merge(piece, a, k, F, H, D, f0);
         } else {
-            st.merge(gvec, gmax, gsum, ga, gb, F, H, D, f0);
-            st.merge(partial, pmax, psum, gb * kGatGroup, k, F, H, D, f0);
+            st.merge(group, ga, gb, F, H, D, f0);
+            st.merge(piece, gb * kGatGroup, k, F, H, D, f0);
         }
-        st.merge(out, smax, ssum, r0, r0 + 1, F, H, D, f0);
+        // the row's last piece, as the chunk's wavefront left it in the output arrays
+        const GatPieces last{out, smax, ssum, pos, spos};
+        st.merge(last, r0, r0 + 1, F, H, D, f0);
 #pragma unroll
         for (int t = 0; t < NT; t++) {
             const int f = f0 + t * kWave * VEC;
@@ -423,6 +482,11 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_fixup(
 #pragma unroll
                 for (int v = 0; v < VEC; v++) o[v] = st.acc[t][v] * inv;
                 gstore<VEC>(out + (size_t)r0 * F + f, o);
+                if constexpr (POS) {
+#pragma unroll
+                    for (int v = 0; v < VEC; v++) o[v] = st.pacc[t][v] * inv;
+                    gstore<VEC>(pos + (size_t)r0 * F + f, o);
+                }
             }
         }
         // every lane of a head holds the same (M, L); the head's first lane stores them.  The
@@ -432,8 +496,10 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_fixup(
         for (int t = 0; t < NT; t++) {
             const int f = f0 + t * kWave * VEC;
             if (f < F && f % D == 0) {
+                const float inv = st.L[t] > 0.f ? 1.f / st.L[t] : 0.f;
                 smax[(size_t)r0 * H + f / D] = st.M[t];
                 ssum[(size_t)r0 * H + f / D] = st.L[t];
+                if constexpr (POS) spos[(size_t)r0 * H + f / D] = st.LP[t] * inv;
             }
         }
     }
@@ -464,71 +530,98 @@ __global__ void gat_alpha(const int32_t *__restrict__ off, const int32_t *__rest
 }
 
 // ---------------------------------------------------------------- backward ---
-// stat[v,k] = (er, smax, 1/ssum, g_out[v,k,:].out[v,k,:])
+// Per node and head: stat[v,k] = (er, smax + log ssum, g[v,k,:].out[v,k,:], -) for the pass over
+// the sources (alpha = exp(lrelu(z) - smax) / ssum = exp(lrelu(z) - (smax + log ssum)): one
+// value to gather instead of two), and the destination-side logit gradient
+//   g_er[v,k] = (1 - slope) (g[v,k,:].pos[v,k,:] - (g[v,k,:].out[v,k,:]) spos[v,k]).
+__device__ __forceinline__ float log_denominator(float smax, float ssum)
+{
+    return ssum > 0.f ? smax + logf(ssum) : INFINITY;      // no in-edges: alpha = exp(-inf) = 0
+}
 __global__ void gat_bwd_node_stats(const float *__restrict__ er, const float *__restrict__ smax,
-                                   const float *__restrict__ ssum, const float *__restrict__ g_out,
-                                   const float *__restrict__ out, float4 *__restrict__ stat, int64_t VH, int D)
+                                   const float *__restrict__ ssum, const float *__restrict__ spos,
+                                   const float *__restrict__ g_out, const float *__restrict__ out,
+                                   const float *__restrict__ pos, float slope, float4 *__restrict__ stat,
+                                   float *__restrict__ g_er, int64_t VH, int D)
 {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= VH) return;
-    const float *g = g_out + i * D, *o = out + i * D;
-    float dot = 0.f;
-    for (int j = 0; j < D; j++) dot = fmaf(g[j], o[j], dot);
-    const float l = ssum[i];
-    stat[i] = make_float4(er[i], smax[i], l > 0.f ? 1.f / l : 0.f, dot);
+    const float *g = g_out + i * D, *o = out + i * D, *p = pos + i * D;
+    float dot = 0.f, dp = 0.f;
+    for (int j = 0; j < D; j++) {
+        dot = fmaf(g[j], o[j], dot);
+        dp = fmaf(g[j], p[j], dp);
+    }
+    stat[i] = make_float4(er[i], log_denominator(smax[i], ssum[i]), dot, 0.f);
+    g_er[i] = (1.f - slope) * (dp - dot * spos[i]);
 }
 
 // Coalesced form (D = 4*lph, lph a power of two <= 64), as gat_node_scores_vec.
 __global__ __launch_bounds__(256) void gat_bwd_node_stats_vec(const float *__restrict__ er,
                                                               const float *__restrict__ smax,
                                                               const float *__restrict__ ssum,
+                                                              const float *__restrict__ spos,
                                                               const float4 *__restrict__ g_out,
                                                               const float4 *__restrict__ out,
-                                                              float4 *__restrict__ stat, int64_t n4, int lph)
+                                                              const float4 *__restrict__ pos, float slope,
+                                                              float4 *__restrict__ stat, float *__restrict__ g_er,
+                                                              int64_t n4, int lph)
 {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    float dot = 0.f;
+    float dot = 0.f, dp = 0.f;
     if (i < n4) {
-        const float4 g = g_out[i], o = out[i];
+        const float4 g = g_out[i], o = out[i], p = pos[i];
         dot = g.x * o.x + g.y * o.y + g.z * o.z + g.w * o.w;
+        dp = g.x * p.x + g.y * p.y + g.z * p.z + g.w * p.w;
     }
-    for (int o = 1; o < lph; o <<= 1) dot += __shfl_xor(dot, o, kWave);
+    for (int o = 1; o < lph; o <<= 1) {
+        dot += __shfl_xor(dot, o, kWave);
+        dp += __shfl_xor(dp, o, kWave);
+    }
     if (i < n4 && i % lph == 0) {
         const int64_t vh = i / lph;
-        const float l = ssum[vh];
-        stat[vh] = make_float4(er[vh], smax[vh], l > 0.f ? 1.f / l : 0.f, dot);
+        stat[vh] = make_float4(er[vh], log_denominator(smax[vh], ssum[vh]), dot, 0.f);
+        g_er[vh] = (1.f - slope) * (dp - dot * spos[vh]);
     }
 }
 
 // Pass over the transposed arrays: row r = source, entries = destinations c.
-//   alpha  = exp(lrelu(el[r]+er[c]) - smax[c]) / ssum[c]
+//   alpha  = exp(lrelu(el[r]+er[c]) - smax[c]) / ssum[c]  (as one exp, see gat_bwd_node_stats)
 //   galpha = g_out[c,k,:].h[r,k,:]                     (reduced over the head's lanes)
-//   gz     = alpha (galpha - g_out[c,k,:].out[c,k,:]) * lrelu'(z)
-//   g_h[r,:] += alpha g_out[c,:];  g_el[r,k] += gz;  gz_t[j,k] = gz  (transposed order: consecutive
-//   entries store consecutive addresses; the destination-side sum gathers them through t_inv)
+//   dz     = alpha (galpha - g_out[c,k,:].out[c,k,:]) * lrelu'(z)
+//   acc   += alpha g_out[c,:];  g_el += dz
+// and at the end of the row  g_h[r,:] = acc + g_el a_src + g_er[r] a_dst.  The row of h and the
+// two scalars of the current source are in registers, so the gradients of a_src and a_dst
+// (sums over the nodes of g_el[r] h[r,:] and g_er[r] h[r,:]) are accumulated on the way: every
+// piece of a row adds its share of g_el, the piece that ends the row adds the g_er term, and
+// the wavefront leaves one partial row of each in red[chunk][2][F].
+// A row cut across chunks: the leading pieces (acc, g_el) go to `partial` / `pel`; the piece that
+// ends the row is stored as it is in g_h / g_el_row, and gat_bwd_fixup adds everything up.
 // lph = lanes per head (power of two) when H > 1; for H == 1 the whole
 // wavefront (all tiles) reduces into the single head.
 template <int VEC, int NT>
 __global__ __launch_bounds__(kGatThreads) void gat_bwd_merge(
     const int32_t *__restrict__ t_off, const int32_t *__restrict__ t_idx,
     const float *__restrict__ h, const float *__restrict__ el, const float4 *__restrict__ stat,
-    const float *__restrict__ g_out, float slope, float *__restrict__ g_h, float *__restrict__ g_el,
-    float *__restrict__ gz_t, float *__restrict__ partial, float *__restrict__ pel,
+    const float *__restrict__ g_er, const float *__restrict__ g_out, const float *__restrict__ a_src,
+    const float *__restrict__ a_dst, float slope, float *__restrict__ g_h, float *__restrict__ g_el_row,
+    float *__restrict__ partial, float *__restrict__ pel, float *__restrict__ red,
     const int2 *__restrict__ start, int R, int E, int H, int D, int lph, int nchunks)
 {
     constexpr int kGatUnroll = gat_unroll(VEC * NT);
-    // The logit gradients of a group of 64 entries wait in LDS and leave as one contiguous
-    // block when the group is done: a global store inside the gather loop makes every wait
-    // for a gathered row wait for the stores in flight as well (loads and stores share one
-    // counter and do not complete in order with each other).
-    __shared__ float gz_stage[kGatWaves][kWave * kGzHeads];
+    // a_src and a_dst wait in LDS for the row ends (a read there costs no vector-memory wait,
+    // and the registers are needed for the gathers in flight)
+    __shared__ float a_lds[2][NT * VEC * kWave];
     const int k = blockIdx.x * kGatWaves + wave_in_block();
-    if (k >= nchunks) return;
-    float *gzbuf = gz_stage[wave_in_block()];
-    const bool staged = H <= kGzHeads;
     const int lane = lane_id();
     const int F = H * D;
     const int f0 = lane * VEC;
+    for (int f = threadIdx.x; f < NT * VEC * kWave; f += kGatThreads) {
+        a_lds[0][f] = f < F ? a_src[f] : 0.f;
+        a_lds[1][f] = f < F ? a_dst[f] : 0.f;
+    }
+    __syncthreads();
+    if (k >= nchunks) return;
     bool act[NT], lead[NT];
     int head[NT], fo[NT];
 #pragma unroll
@@ -539,142 +632,176 @@ __global__ __launch_bounds__(kGatThreads) void gat_bwd_merge(
         lead[t] = act[t] && (f % D == 0);
         fo[t] = act[t] ? f : 0;
     }
-    const int2 s0 = start[k], s1 = start[k + 1];
-    const int r1 = min(max(uniform(s1.x), 0), R);
-    int r = min(max(uniform(s0.x), 0), r1);
-    const int j0 = min(max(uniform(s0.y), 0), E);
-    const int j1 = min(uniform(s1.y), E);
+    // this wavefront's share of the gradients of a_src and a_dst
+    float pas[NT][VEC], pad[NT][VEC];
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int v = 0; v < VEC; v++) pas[t][v] = pad[t][v] = 0.f;
 
-    int rb = r;
-    int ends = (rb + lane < R) ? t_off[rb + 1 + lane] : 0x7fffffff;
-    int row_end = bcast_i(ends, 0);
+    {
+        const int2 s0 = start[k], s1 = start[k + 1];
+        const int r1 = min(max(uniform(s1.x), 0), R);
+        int r = min(max(uniform(s0.x), 0), r1);
+        const int j0 = min(max(uniform(s0.y), 0), E);
+        const int j1 = min(uniform(s1.y), E);
+        // the chunk's first row began in an earlier chunk: its sums are one piece of several
+        const int raw_row = (r < r1 && uniform(t_off[r]) < j0) ? r : -1;
 
-    // h row and el of the current source row and, already on their way, of the next one: a
-    // row end must not wait for fresh loads (lanes past F read offset 0 and are ignored)
-    float acc[NT][VEC], gel[NT], hr[NT][VEC], el_r[NT], hr_next[NT][VEC], el_next[NT];
-    auto fetch_row = [&](int row) {
-        const size_t rc = (size_t)min(row, R - 1);
+        int rb = r;
+        int ends = (rb + lane < R) ? t_off[rb + 1 + lane] : 0x7fffffff;
+        int row_end = bcast_i(ends, 0);
+
+        // h row, el and g_er of the current source row and, already on their way, of the next one:
+        // a row end must not wait for fresh loads (lanes past F read offset 0 and are ignored)
+        float acc[NT][VEC], gel[NT], hr[NT][VEC], el_r[NT], ger_r[NT];
+        float hr_next[NT][VEC], el_next[NT], ger_next[NT];
+        auto fetch_row = [&](int row) {
+            const size_t rc = (size_t)min(row, R - 1);
 #pragma unroll
-        for (int t = 0; t < NT; t++) {
-            gload<VEC>(hr_next[t], h + rc * F + fo[t]);
-            el_next[t] = el[rc * H + head[t]];
-        }
-    };
-    auto reset = [&]() {
-#pragma unroll
-        for (int t = 0; t < NT; t++) {
-            gel[t] = 0.f;
-            el_r[t] = el_next[t];
-#pragma unroll
-            for (int v = 0; v < VEC; v++) {
-                acc[t][v] = 0.f;
-                hr[t][v] = hr_next[t][v];
+            for (int t = 0; t < NT; t++) {
+                gload<VEC>(hr_next[t], h + rc * F + fo[t]);
+                el_next[t] = el[rc * H + head[t]];
+                ger_next[t] = g_er[rc * H + head[t]];
             }
-        }
-        fetch_row(r + 1);
-    };
-    fetch_row(r);
-    reset();
-    auto store_piece = [&](float *vec, float *elp) {
+        };
+        auto reset = [&]() {
 #pragma unroll
-        for (int t = 0; t < NT; t++)
-            if (act[t]) {
-                gstore<VEC>(vec + f0 + t * kWave * VEC, acc[t]);
-                if (lead[t]) elp[head[t]] = gel[t];
-            }
-    };
-    auto flush_row = [&]() {
-        store_piece(g_h + (size_t)r * F, g_el + (size_t)r * H);
-        r++;
-        if (r - rb == kWave) {
-            rb = r;
-            ends = (rb + lane < R) ? t_off[rb + 1 + lane] : 0x7fffffff;
-        }
-        row_end = bcast_i(ends, r - rb);
-        reset();
-    };
-
-    for (int jb = j0; jb < j1; jb += kWave) {
-        const int n = min(kWave, j1 - jb);
-        int my_c = -1;
-        if (lane < n) {
-            my_c = t_idx[jb + lane];
-            if ((unsigned)my_c >= (unsigned)R) my_c = -1;
-        }
-        for (int i0 = 0; i0 < n; i0 += kGatUnroll) {
-            float gv[kGatUnroll][NT][VEC];
-            float4 st[kGatUnroll][NT];
+            for (int t = 0; t < NT; t++) {
+                gel[t] = 0.f;
+                el_r[t] = el_next[t];
+                ger_r[t] = ger_next[t];
 #pragma unroll
-            for (int u = 0; u < kGatUnroll; u++) {
-                const int c = max(bcast_i(my_c, (i0 + u) & (kWave - 1)), 0);
-                const float *src = g_out + (size_t)c * F;
-                const float4 *ss = stat + (size_t)c * H;
-#pragma unroll
-                for (int t = 0; t < NT; t++) {
-                    gload<VEC>(gv[u][t], src + fo[t]);
-                    st[u][t] = ss[head[t]];
+                for (int v = 0; v < VEC; v++) {
+                    acc[t][v] = 0.f;
+                    hr[t][v] = hr_next[t][v];
                 }
             }
+            fetch_row(r + 1);
+        };
+        fetch_row(r);
+        reset();
+        // this piece's share of sum_r g_el[r] h[r,:]
+        auto add_el_share = [&]() {
 #pragma unroll
-            for (int u = 0; u < kGatUnroll; u++) {
-                if (i0 + u < n) {
-                    const int jj = jb + i0 + u;
-                    while (jj == row_end && r < r1) flush_row();
-                    const int c = bcast_i(my_c, i0 + u);
-                    if (c >= 0) {
-                        float dot[NT];
+            for (int t = 0; t < NT; t++)
 #pragma unroll
-                        for (int t = 0; t < NT; t++) {
-                            dot[t] = 0.f;
-                            if (act[t]) {
+                for (int v = 0; v < VEC; v++) pas[t][v] = fmaf(gel[t], hr[t][v], pas[t][v]);
+        };
+        auto store_piece = [&](float *vec, float *elp) {
 #pragma unroll
-                                for (int v = 0; v < VEC; v++) dot[t] = fmaf(gv[u][t][v], hr[t][v], dot[t]);
-                            }
-                        }
-                        if (H == 1) {
-                            float s = 0.f;
+            for (int t = 0; t < NT; t++)
+                if (act[t]) {
+                    gstore<VEC>(vec + f0 + t * kWave * VEC, acc[t]);
+                    if (lead[t]) elp[head[t]] = gel[t];
+                }
+        };
+        auto flush_row = [&]() {
+            add_el_share();
 #pragma unroll
-                            for (int t = 0; t < NT; t++) s += dot[t];
-                            s = lane_group_sum(s, kWave);
+            for (int t = 0; t < NT; t++)
 #pragma unroll
-                            for (int t = 0; t < NT; t++) dot[t] = s;
-                        } else {
+                for (int v = 0; v < VEC; v++) pad[t][v] = fmaf(ger_r[t], hr[t][v], pad[t][v]);
+            if (r == raw_row) {
+                store_piece(g_h + (size_t)r * F, g_el_row + (size_t)r * H);
+            } else {
 #pragma unroll
-                            for (int t = 0; t < NT; t++) dot[t] = lane_group_sum(dot[t], lph);
-                        }
+                for (int t = 0; t < NT; t++)
+                    if (act[t]) {
+                        float o[VEC];
 #pragma unroll
-                        for (int t = 0; t < NT; t++)
-                            if (act[t]) {
-                                const float z = el_r[t] + st[u][t].x;
-                                const float alpha = fast_exp(lrelu(z, slope) - st[u][t].y) * st[u][t].z;
-                                const float gz = alpha * (dot[t] - st[u][t].w) * (z > 0.f ? 1.f : slope);
-                                gel[t] += gz;
+                        for (int v = 0; v < VEC; v++)
+                            o[v] = acc[t][v] + gel[t] * a_lds[0][fo[t] + v] + ger_r[t] * a_lds[1][fo[t] + v];
+                        gstore<VEC>(g_h + (size_t)r * F + f0 + t * kWave * VEC, o);
+                    }
+            }
+            r++;
+            if (r - rb == kWave) {
+                rb = r;
+                ends = (rb + lane < R) ? t_off[rb + 1 + lane] : 0x7fffffff;
+            }
+            row_end = bcast_i(ends, r - rb);
+            reset();
+        };
+
+        for (int jb = j0; jb < j1; jb += kWave) {
+            const int n = min(kWave, j1 - jb);
+            int my_c = -1;
+            if (lane < n) {
+                my_c = t_idx[jb + lane];
+                if ((unsigned)my_c >= (unsigned)R) my_c = -1;
+            }
+            for (int i0 = 0; i0 < n; i0 += kGatUnroll) {
+                float gv[kGatUnroll][NT][VEC];
+                float3 st[kGatUnroll][NT];          // (er, smax + log ssum, g.out) of the destination
 #pragma unroll
-                                for (int v = 0; v < VEC; v++) acc[t][v] = fmaf(alpha, gv[u][t][v], acc[t][v]);
-                                if (lead[t]) {
-                                    if (staged) gzbuf[(i0 + u) * H + head[t]] = gz;
-                                    else gz_t[(uint32_t)jj * (uint32_t)H + (uint32_t)head[t]] = gz;
+                for (int u = 0; u < kGatUnroll; u++) {
+                    const int c = max(bcast_i(my_c, (i0 + u) & (kWave - 1)), 0);
+                    const float *src = g_out + (size_t)c * F;
+                    const float4 *ss = stat + (size_t)c * H;
+#pragma unroll
+                    for (int t = 0; t < NT; t++) {
+                        gload<VEC>(gv[u][t], src + fo[t]);
+                        st[u][t] = *reinterpret_cast<const float3 *>(ss + head[t]);
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < kGatUnroll; u++) {
+                    if (i0 + u < n) {
+                        const int jj = jb + i0 + u;
+                        while (jj == row_end && r < r1) flush_row();
+                        const int c = bcast_i(my_c, i0 + u);
+                        if (c >= 0) {        // a destination out of range counts for nothing on either side
+                            float dot[NT];
+#pragma unroll
+                            for (int t = 0; t < NT; t++) {
+                                dot[t] = 0.f;
+                                if (act[t]) {
+#pragma unroll
+                                    for (int v = 0; v < VEC; v++) dot[t] = fmaf(gv[u][t][v], hr[t][v], dot[t]);
                                 }
                             }
-                    } else {
-                        // destination out of range: the edge counts for nothing on either side
+                            if (H == 1) {
+                                float s = 0.f;
 #pragma unroll
-                        for (int t = 0; t < NT; t++)
-                            if (act[t] && lead[t]) {
-                                if (staged) gzbuf[(i0 + u) * H + head[t]] = 0.f;
-                                else gz_t[(uint32_t)jj * (uint32_t)H + (uint32_t)head[t]] = 0.f;
+                                for (int t = 0; t < NT; t++) s += dot[t];
+                                s = lane_group_sum(s, kWave);
+#pragma unroll
+                                for (int t = 0; t < NT; t++) dot[t] = s;
+                            } else {
+#pragma unroll
+                                for (int t = 0; t < NT; t++) dot[t] = lane_group_sum(dot[t], lph);
                             }
+#pragma unroll
+                            for (int t = 0; t < NT; t++)
+                                if (act[t]) {
+                                    const float z = el_r[t] + st[u][t].x;
+                                    const float alpha = fast_exp(lrelu(z, slope) - st[u][t].y);
+                                    const float gz = alpha * (dot[t] - st[u][t].z) * (z > 0.f ? 1.f : slope);
+                                    gel[t] += gz;
+#pragma unroll
+                                    for (int v = 0; v < VEC; v++) acc[t][v] = fmaf(alpha, gv[u][t][v], acc[t][v]);
+                                }
+                        }
                     }
                 }
             }
         }
-        if (staged) {
-            float *dst = gz_t + (size_t)jb * H;
-            for (int i = lane; i < n * H; i += kWave) dst[i] = gzbuf[i];
+        while (r < r1) flush_row();
+        if (r1 < R && j1 > uniform(t_off[r1])) {
+            add_el_share();
+            store_piece(partial + (size_t)k * F, pel + (size_t)k * H);
         }
     }
-    while (r < r1) flush_row();
-    if (r1 < R && j1 > uniform(t_off[r1])) store_piece(partial + (size_t)k * F, pel + (size_t)k * H);
+
+    // this chunk's partial rows of the two parameter gradients
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+        if (act[t]) {
+            float *dst = red + (size_t)k * 2 * F + f0 + t * kWave * VEC;
+            gstore<VEC>(dst, pas[t]);
+            gstore<VEC>(dst + F, pad[t]);
+        }
 }
 
 // Plain sums of backward pieces: vec [.,F] and per-head scalars elp [.,H].
@@ -692,7 +819,7 @@ template <int VEC, int NT> struct SumState {
     __device__ __forceinline__ void add(const float *__restrict__ vec, const float *__restrict__ elp, int first,
                                         int last, int F, int H, int D, int f0)
     {
-        constexpr int kBatch = VEC * NT >= 16 ? 2 : (VEC * NT >= 8 ? 4 : 8);
+        constexpr int kBatch = VEC * NT >= 16 ? 2 : (VEC * NT >= 8 ? 4 : (VEC * NT >= 4 ? 8 : 16));
         for (int kb = first; kb < last; kb += kBatch) {
             float x[kBatch][NT][VEC], pe[kBatch][NT];
 #pragma unroll
@@ -751,7 +878,7 @@ __global__ __launch_bounds__(kGatThreads) void gat_bwd_group(const int32_t *__re
     for (int i = blockIdx.x * kGatWaves + wave_in_block(); i < n; i += stride) {
         const int g = list ? uniform(list[i]) : i;
         const int kend = (g + 1) * kGatGroup;
-        if (kend >= nchunks) continue;
+        if (g < 0 || kend >= nchunks) continue;
         const int r = uniform(start[kend].x);
         if (r < 0 || r >= R) continue;
         const int s = uniform(t_off[r]);
@@ -766,9 +893,16 @@ __global__ __launch_bounds__(kGatThreads) void gat_bwd_group(const int32_t *__re
     }
 }
 
+// A row cut across chunks and ending in chunk k: adds its pieces in chunk order to the last
+// piece (left in g_h / g_el_row by that chunk's wavefront) and finishes the row,
+// g_h[r,:] = acc + g_el a_src + g_er[r] a_dst.
 template <int VEC, int NT>
 __global__ __launch_bounds__(kGatThreads) void gat_bwd_fixup(const int32_t *__restrict__ t_off,
-                                                             float *__restrict__ g_h, float *__restrict__ g_el,
+                                                             float *__restrict__ g_h,
+                                                             const float *__restrict__ g_el_row,
+                                                             const float *__restrict__ g_er,
+                                                             const float *__restrict__ a_src,
+                                                             const float *__restrict__ a_dst,
                                                              const float *__restrict__ partial,
                                                              const float *__restrict__ pel,
                                                              const float *__restrict__ gvec,
@@ -800,83 +934,59 @@ __global__ __launch_bounds__(kGatThreads) void gat_bwd_fixup(const int32_t *__re
             st.add(gvec, gel, ga, gb, F, H, D, f0);
             st.add(partial, pel, gb * kGatGroup, k, F, H, D, f0);
         }
-        st.add(g_h, g_el, r0, r0 + 1, F, H, D, f0);
-        st.store(g_h + (size_t)r0 * F, g_el + (size_t)r0 * H, F, D, f0);
-    }
-}
-
-// g_h[v,f] += g_el[v,k] a_src[f] + g_er[v,k] a_dst[f]; per-block partial sums of
-// g_el*h and g_er*h over the block's rows go to red[block][2][F].
-constexpr int kRedRows = 128;
-__global__ __launch_bounds__(256) void gat_bwd_finish(const float *__restrict__ h, const float *__restrict__ a_src,
-                                                      const float *__restrict__ a_dst,
-                                                      const float *__restrict__ g_el, const float *__restrict__ g_er,
-                                                      float *__restrict__ g_h, float *__restrict__ red, int V, int H,
-                                                      int D)
-{
-    const int F = H * D;
-    const int v0 = blockIdx.x * kRedRows;
-    const int v1 = min(V, v0 + kRedRows);
-    constexpr int kB = 8;                     // rows fetched together
-    for (int f = threadIdx.x; f < F; f += blockDim.x) {
-        const int k = f / D;
-        const float as = a_src[f], ad = a_dst[f];
-        float ss = 0.f, sd = 0.f;
-        for (int vb = v0; vb < v1; vb += kB) {
-            float gl[kB], gr[kB], hv[kB], gh[kB];
+        st.add(g_h, g_el_row, r0, r0 + 1, F, H, D, f0);
 #pragma unroll
-            for (int i = 0; i < kB; i++) {
-                const size_t v = (size_t)min(vb + i, v1 - 1);
-                gl[i] = g_el[v * H + k];
-                gr[i] = g_er[v * H + k];
-                hv[i] = h[v * F + f];
-                gh[i] = g_h[v * F + f];
+        for (int t = 0; t < NT; t++) {
+            const int f = f0 + t * kWave * VEC;
+            if (f < F) {
+                float as[VEC], ad[VEC], o[VEC];
+                gload<VEC>(as, a_src + f);
+                gload<VEC>(ad, a_dst + f);
+                const float ger = g_er[(size_t)r0 * H + f / D];
+#pragma unroll
+                for (int v = 0; v < VEC; v++) o[v] = st.acc[t][v] + st.gel[t] * as[v] + ger * ad[v];
+                gstore<VEC>(g_h + (size_t)r0 * F + f, o);
             }
-#pragma unroll
-            for (int i = 0; i < kB; i++)
-                if (vb + i < v1) {
-                    g_h[(size_t)(vb + i) * F + f] = gh[i] + gl[i] * as + gr[i] * ad;
-                    ss = fmaf(gl[i], hv[i], ss);
-                    sd = fmaf(gr[i], hv[i], sd);
-                }
         }
-        red[((size_t)blockIdx.x * 2 + 0) * F + f] = ss;
-        red[((size_t)blockIdx.x * 2 + 1) * F + f] = sd;
     }
 }
 
-// Sums red[0..nblocks) per (which, f): 64 features per block, 16 strided
-// groups of partials added in a fixed order, then the 16 group sums in order.
-__global__ __launch_bounds__(1024) void gat_bwd_reduce(const float *__restrict__ red, int nblocks, int F,
-                                                       float *__restrict__ g_a_src, float *__restrict__ g_a_dst)
+// Sums of the per-chunk partial rows red[0..nrows)[2][F], in two fixed-order stages:
+// kRedSlices slices of the rows into mid[slice][2F], then the slices.  64 columns per block,
+// 16 strided groups of rows added in a fixed order, then the 16 group sums in order.
+constexpr int kRedSlices = 32;
+__global__ __launch_bounds__(1024) void gat_bwd_reduce(const float *__restrict__ red, int nrows, int per_slice, int W,
+                                                       float *__restrict__ out_rows, float *__restrict__ g_a_src,
+                                                       float *__restrict__ g_a_dst, int F)
 {
     __shared__ float part[16][64];
     const int col = blockIdx.x * 64 + (threadIdx.x & 63);   // index into [2][F]
     const int grp = threadIdx.x >> 6;
+    const int b_lo = blockIdx.y * per_slice, b_hi = min(nrows, b_lo + per_slice);
     float s = 0.f;
-    if (col < 2 * F) {
-        const int which = col / F, f = col % F;
+    if (col < W) {
         // eight partials fetched together, added in the same order as one by one
         constexpr int kB = 8;
-        for (int b0 = grp; b0 < nblocks; b0 += 16 * kB) {
+        for (int b0 = b_lo + grp; b0 < b_hi; b0 += 16 * kB) {
             float v[kB];
 #pragma unroll
             for (int i = 0; i < kB; i++) {
-                const int b = min(b0 + 16 * i, nblocks - 1);
-                v[i] = red[((size_t)b * 2 + which) * F + f];
+                const int b = min(b0 + 16 * i, b_hi - 1);
+                v[i] = red[(size_t)b * W + col];
             }
 #pragma unroll
             for (int i = 0; i < kB; i++)
-                if (b0 + 16 * i < nblocks) s += v[i];
+                if (b0 + 16 * i < b_hi) s += v[i];
         }
     }
     part[grp][threadIdx.x & 63] = s;
     __syncthreads();
-    if (grp == 0 && col < 2 * F) {
+    if (grp == 0 && col < W) {
         float t = 0.f;
 #pragma unroll
         for (int g = 0; g < 16; g++) t += part[g][threadIdx.x];
-        (col / F ? g_a_dst : g_a_src)[col % F] = t;
+        if (out_rows) out_rows[(size_t)blockIdx.y * W + col] = t;
+        else (col / F ? g_a_dst : g_a_src)[col % F] = t;
     }
 }
 
@@ -890,6 +1000,13 @@ struct GatShape {
 // gathers) is a few microseconds, so chunks stay at 64 items or more
 int gat_chunk_for(int64_t M)
 {
+    // tuning aid, read once per process
+    static const int forced = [] {
+        const char *e = getenv("JGAMD_GAT_CHUNK");
+        const int v = e ? atoi(e) : 0;
+        return v < 16 ? 0 : (v > 4096 ? 4096 : v);
+    }();
+    if (forced) return forced;
     int chunk = 128;
     while (chunk > 64 && M / chunk < 16384) chunk >>= 1;
     return chunk;
@@ -933,23 +1050,38 @@ static int32_t check_gat(const char *who, int32_t V, int64_t E, int32_t H, int32
     return 0;
 }
 
+static size_t pieces_bytes(size_t n, int H, int D)
+{
+    return 2 * carve_bytes(n * H * D, 4) + 3 * carve_bytes(n * H, 4);
+}
+static GatPieces carve_pieces(Carver &carve, size_t n, int H, int D)
+{
+    GatPieces p;
+    p.vec = carve.take<float>(n * H * D);
+    p.pvec = carve.take<float>(n * H * D);
+    p.mx = carve.take<float>(n * H);
+    p.sum = carve.take<float>(n * H);
+    p.psum = carve.take<float>(n * H);
+    return p;
+}
+
 static size_t gat_fwd_ws(int32_t V, int64_t E, int32_t H, int32_t D)
 {
     GatShape s = gat_shape(V, E, H, D);
     const size_t ng = (size_t)ceil_div(s.nchunks, kGatGroup);
-    return carve_bytes((size_t)s.nchunks + 1, sizeof(int2)) + carve_bytes((size_t)s.nchunks * H * D, 4) +
-           2 * carve_bytes((size_t)s.nchunks * H, 4) + carve_bytes(ng * H * D, 4) + 2 * carve_bytes(ng * H, 4);
+    return carve_bytes((size_t)s.nchunks + 1, sizeof(int2)) + pieces_bytes((size_t)s.nchunks, H, D) +
+           pieces_bytes(ng, H, D);
 }
 
 static size_t gat_bwd_ws(int32_t V, int64_t E, int32_t H, int32_t D)
 {
     GatShape s = gat_shape(V, E, H, D);
-    const size_t nred = (size_t)ceil_div(V > 0 ? V : 1, kRedRows);
     const size_t ng = (size_t)ceil_div(s.nchunks, kGatGroup);
-    return carve_bytes(ng * H * D, 4) + carve_bytes(ng * H, 4) + carve_bytes((size_t)s.nchunks + 1, sizeof(int2)) + carve_bytes((size_t)s.nchunks * H * D, 4) +
-           carve_bytes((size_t)s.nchunks * H, 4) + carve_bytes((size_t)V * H, 16) + carve_bytes((size_t)E * H, 4) +
-           2 * carve_bytes((size_t)V * H, 4) + carve_bytes(nred * 2 * H * D, 4) +
-           align_up(spmm_ws_bytes(V, E, H), 256);
+    const size_t F = (size_t)H * D;
+    return carve_bytes(ng * F, 4) + carve_bytes(ng * H, 4) + carve_bytes((size_t)s.nchunks + 1, sizeof(int2)) +
+           carve_bytes((size_t)s.nchunks * F, 4) + carve_bytes((size_t)s.nchunks * H, 4) +
+           carve_bytes((size_t)V * H, 16) + 2 * carve_bytes((size_t)V * H, 4) +
+           carve_bytes((size_t)s.nchunks * 2 * F, 4) + carve_bytes((size_t)kRedSlices * 2 * F, 4);
 }
 
 #define JG_GAT_DISPATCH(CALL)                         \
@@ -975,15 +1107,18 @@ JG_EXPORT int32_t jgamd_gat_fwd_workspace(int32_t V, int64_t E, int32_t H, int32
 
 JG_EXPORT int32_t jgamd_gat_fwd(const void *plan, int32_t n_fix, int32_t n_grp, const int32_t *off,
                                 const int32_t *idx, const float *h, const float *a_src, const float *a_dst,
-                                float slope, float *el, float *er, float *smax, float *ssum, float *alpha, float *out,
-                                int32_t V, int64_t E, int32_t H, int32_t D, void *ws, size_t ws_bytes, void *stream)
+                                float slope, float *el, float *er, float *smax, float *ssum, float *pos, float *spos,
+                                float *alpha, float *out, int32_t V, int64_t E, int32_t H, int32_t D, void *ws,
+                                size_t ws_bytes, void *stream)
 {
     if (int32_t rc = check_gat("gat_fwd", V, E, H, D)) return rc;
     if (V == 0) return 0;
     if (!off || !h || !a_src || !a_dst || !el || !er || !smax || !ssum || !out)
         return fail(JGAMD_ERR_NULL, "gat_fwd: NULL array");
+    if ((pos == nullptr) != (spos == nullptr)) return fail(JGAMD_ERR_NULL, "gat_fwd: pos and spos go together");
     if (E > 0 && !idx) return fail(JGAMD_ERR_NULL, "gat_fwd: idx is NULL with E > 0");
-    if ((((uintptr_t)h | (uintptr_t)out) & 15) != 0) return fail(JGAMD_ERR_ALIGN, "gat_fwd: h/out not 16-byte aligned");
+    if ((((uintptr_t)h | (uintptr_t)out | (uintptr_t)pos) & 15) != 0)
+        return fail(JGAMD_ERR_ALIGN, "gat_fwd: h/out/pos not 16-byte aligned");
     const size_t need = gat_fwd_ws(V, E, H, D);
     if (!ws || ws_bytes < need) return fail(JGAMD_ERR_WORKSPACE, "gat_fwd: workspace %zu < %zu bytes", ws ? ws_bytes : (size_t)0, need);
     if (((uintptr_t)ws & 255) != 0) return fail(JGAMD_ERR_ALIGN, "gat_fwd: workspace not 256-byte aligned");
@@ -1000,14 +1135,11 @@ JG_EXPORT int32_t jgamd_gat_fwd(const void *plan, int32_t n_fix, int32_t n_grp, 
         pv.start = own_start;
         n_fix = n_grp = -1;
     }
-    float *partial = carve.take<float>((size_t)s.nchunks * H * D);
-    float *pmax = carve.take<float>((size_t)s.nchunks * H);
-    float *psum = carve.take<float>((size_t)s.nchunks * H);
     const int ngroups = (int)ceil_div(s.nchunks, kGatGroup);
-    float *gvec = carve.take<float>((size_t)ngroups * H * D);
-    float *gmax = carve.take<float>((size_t)ngroups * H);
-    float *gsum = carve.take<float>((size_t)ngroups * H);
+    const GatPieces piece = carve_pieces(carve, (size_t)s.nchunks, H, D);
+    const GatPieces group = carve_pieces(carve, (size_t)ngroups, H, D);
     const int64_t VH = (int64_t)V * H;
+    if (pos && !s.bwd_ok) return fail(JGAMD_ERR_UNSUPPORTED, "gat_fwd: pos / spos need a shape jgamd_gat_bwd takes");
     if (vec_nodes_ok(D) && (((uintptr_t)a_src | (uintptr_t)a_dst) & 15) == 0)
         hipLaunchKernelGGL(gat_node_scores_vec, dim3((unsigned)ceil_div(VH * (D / 4), 256)), dim3(256), 0, st,
                            reinterpret_cast<const float4 *>(h), reinterpret_cast<const float4 *>(a_src),
@@ -1020,68 +1152,77 @@ JG_EXPORT int32_t jgamd_gat_fwd(const void *plan, int32_t n_fix, int32_t n_grp, 
     const bool listed = pv.fix != nullptr;
     const dim3 ggrid(listed ? gat_list_grid(n_grp, ngroups) : (unsigned)ceil_div(ngroups, kGatWaves));
     const dim3 fgrid(listed ? gat_list_grid(n_fix, s.nchunks) : grid.x);
-#define JG_FWD(VV, NN)                                                                                           \
-    case VV * 16 + NN:                                                                                           \
-        hipLaunchKernelGGL((gat_fwd_merge<VV, NN>), grid, block, 0, st, off, idx, h, el, er, slope, out, smax,   \
-                           ssum, partial, pmax, psum, pv.start, V, (int)E, H, D, s.nchunks);                     \
-        if (ngroups > 1 && n_grp != 0 && n_fix != 0)                                                             \
-            hipLaunchKernelGGL((gat_fwd_group<VV, NN>), ggrid, block, 0, st, off, partial, pmax, psum, gvec,     \
-                               gmax, gsum, pv.start, pv.grp, pv.counts + 1, V, H, D, s.chunk, s.nchunks);        \
+    const bool with_group = ngroups > 1 && n_grp != 0 && n_fix != 0;
+#define JG_FWD_P(VV, NN, PP)                                                                                     \
+    {                                                                                                            \
+        hipLaunchKernelGGL((gat_fwd_merge<VV, NN, PP>), grid, block, 0, st, off, idx, h, el, er, slope, out,     \
+                           smax, ssum, pos, spos, piece, pv.start, V, (int)E, H, D, s.nchunks);                  \
+        if (with_group)                                                                                          \
+            hipLaunchKernelGGL((gat_fwd_group<VV, NN, PP>), ggrid, block, 0, st, off, piece, group, pv.start,    \
+                               pv.grp, pv.counts + 1, V, H, D, s.chunk, s.nchunks);                              \
         if (n_fix != 0)                                                                                          \
-            hipLaunchKernelGGL((gat_fwd_fixup<VV, NN>), fgrid, block, 0, st, off, out, smax, ssum, partial,      \
-                               pmax, psum, gvec, gmax, gsum, pv.start, pv.fix, pv.counts, V, H, D, s.chunk,      \
-                               s.nchunks);                                                                       \
+            hipLaunchKernelGGL((gat_fwd_fixup<VV, NN, PP>), fgrid, block, 0, st, off, out, smax, ssum, pos,      \
+                               spos, piece, group, pv.start, pv.fix, pv.counts, V, H, D, s.chunk, s.nchunks);    \
+    }
+#define JG_FWD(VV, NN)                  \
+    case VV * 16 + NN:                  \
+        if (pos) JG_FWD_P(VV, NN, true) \
+        else JG_FWD_P(VV, NN, false)    \
         break;
     JG_GAT_DISPATCH(JG_FWD)
 #undef JG_FWD
+#undef JG_FWD_P
     if (alpha && E > 0)
         hipLaunchKernelGGL(gat_alpha, dim3((unsigned)ceil_div(E * H, 256)), dim3(256), 0, st, off, idx, el, er, smax,
                            ssum, slope, alpha, V, E, H);
     return launch_status("gat_fwd");
 }
 
-JG_EXPORT int32_t jgamd_gat_bwd_workspace(int32_t V, int64_t E, int32_t H, int32_t D, size_t *bytes)
+static int32_t check_gat_bwd(int32_t V, int64_t E, int32_t H, int32_t D)
 {
-    if (!bytes) return fail(JGAMD_ERR_NULL, "gat_bwd_workspace: bytes is NULL");
     if (int32_t rc = check_gat("gat_bwd", V, E, H, D)) return rc;
     if (!gat_shape(V, E, H, D).bwd_ok)
         return fail(JGAMD_ERR_UNSUPPORTED, "gat_bwd: with H > 1 the head width D=%d must give a power-of-two lane count", D);
-    if ((int64_t)E * H >= ((int64_t)1 << 32)) return fail(JGAMD_ERR_UNSUPPORTED, "gat_bwd: E*H does not fit 32 bits");
+    return 0;
+}
+
+JG_EXPORT int32_t jgamd_gat_bwd_workspace(int32_t V, int64_t E, int32_t H, int32_t D, size_t *bytes)
+{
+    if (!bytes) return fail(JGAMD_ERR_NULL, "gat_bwd_workspace: bytes is NULL");
+    if (int32_t rc = check_gat_bwd(V, E, H, D)) return rc;
     *bytes = V == 0 ? 0 : gat_bwd_ws(V, E, H, D);
     return 0;
 }
 
-JG_EXPORT int32_t jgamd_gat_bwd(const void *t_plan, int32_t n_fix, int32_t n_grp, const void *tiles,
-                                const int32_t *off, const int32_t *idx, const int32_t *t_off, const int32_t *t_idx,
-                                const int32_t *t_inv, const float *h, const float *a_src, const float *a_dst,
+JG_EXPORT int32_t jgamd_gat_bwd(const void *t_plan, int32_t n_fix, int32_t n_grp, const int32_t *t_off,
+                                const int32_t *t_idx, const float *h, const float *a_src, const float *a_dst,
                                 float slope, const float *el, const float *er, const float *smax, const float *ssum,
-                                const float *out, const float *g_out, float *g_h, float *g_a_src, float *g_a_dst,
-                                int32_t V, int64_t E, int32_t H, int32_t D, void *ws, size_t ws_bytes, void *stream)
+                                const float *spos, const float *out, const float *pos, const float *g_out,
+                                float *g_h, float *g_a_src, float *g_a_dst, int32_t V, int64_t E, int32_t H, int32_t D,
+                                void *ws, size_t ws_bytes, void *stream)
 {
-    (void)idx;
-    if (int32_t rc = check_gat("gat_bwd", V, E, H, D)) return rc;
+    if (int32_t rc = check_gat_bwd(V, E, H, D)) return rc;
     const GatShape s = gat_shape(V, E, H, D);
-    if (!s.bwd_ok)
-        return fail(JGAMD_ERR_UNSUPPORTED, "gat_bwd: with H > 1 the head width D=%d must give a power-of-two lane count", D);
-    if ((int64_t)E * H >= ((int64_t)1 << 32)) return fail(JGAMD_ERR_UNSUPPORTED, "gat_bwd: E*H does not fit 32 bits");
     if (!g_a_src || !g_a_dst) return fail(JGAMD_ERR_NULL, "gat_bwd: NULL gradient output");
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int F = H * D;
+    const unsigned col_blocks = (unsigned)ceil_div(2 * F, 64);
     if (V == 0) {
-        hipLaunchKernelGGL(gat_bwd_reduce, dim3((unsigned)ceil_div(2 * F, 64)), dim3(1024), 0, st, nullptr, 0, F,
-                           g_a_src, g_a_dst);
+        hipLaunchKernelGGL(gat_bwd_reduce, dim3(col_blocks), dim3(1024), 0, st, nullptr, 0, 1, 2 * F, nullptr, g_a_src,
+                           g_a_dst, F);
         return launch_status("gat_bwd");
     }
-    if (!off || !t_off || !h || !a_src || !a_dst || !el || !er || !smax || !ssum || !out || !g_out || !g_h)
+    if (!t_off || !h || !a_src || !a_dst || !el || !er || !smax || !ssum || !spos || !out || !pos || !g_out || !g_h)
         return fail(JGAMD_ERR_NULL, "gat_bwd: NULL array");
-    if (E > 0 && (!t_idx || !t_inv)) return fail(JGAMD_ERR_NULL, "gat_bwd: transposed arrays are NULL with E > 0");
-    if ((((uintptr_t)h | (uintptr_t)g_out | (uintptr_t)g_h) & 15) != 0)
-        return fail(JGAMD_ERR_ALIGN, "gat_bwd: h/g_out/g_h not 16-byte aligned");
+    if (E > 0 && !t_idx) return fail(JGAMD_ERR_NULL, "gat_bwd: t_idx is NULL with E > 0");
+    if ((((uintptr_t)h | (uintptr_t)g_out | (uintptr_t)g_h | (uintptr_t)out | (uintptr_t)pos) & 15) != 0)
+        return fail(JGAMD_ERR_ALIGN, "gat_bwd: h/g_out/g_h/out/pos not 16-byte aligned");
+    if ((((uintptr_t)a_src | (uintptr_t)a_dst) & (uintptr_t)(4 * s.vec - 1)) != 0)
+        return fail(JGAMD_ERR_ALIGN, "gat_bwd: a_src/a_dst not %d-byte aligned", 4 * s.vec);
     const size_t need = gat_bwd_ws(V, E, H, D);
     if (!ws || ws_bytes < need) return fail(JGAMD_ERR_WORKSPACE, "gat_bwd: workspace %zu < %zu bytes", ws ? ws_bytes : (size_t)0, need);
     if (((uintptr_t)ws & 255) != 0) return fail(JGAMD_ERR_ALIGN, "gat_bwd: workspace not 256-byte aligned");
-    if ((((uintptr_t)t_plan | (uintptr_t)tiles) & 255) != 0)
-        return fail(JGAMD_ERR_ALIGN, "gat_bwd: plan not 256-byte aligned");
+    if (((uintptr_t)t_plan & 255) != 0) return fail(JGAMD_ERR_ALIGN, "gat_bwd: plan not 256-byte aligned");
     Carver carve(ws);
     const int ngroups = (int)ceil_div(s.nchunks, kGatGroup);
     float *gvec = carve.take<float>((size_t)ngroups * F);
@@ -1098,46 +1239,51 @@ JG_EXPORT int32_t jgamd_gat_bwd(const void *t_plan, int32_t n_fix, int32_t n_grp
     float *partial = carve.take<float>((size_t)s.nchunks * F);
     float *pel = carve.take<float>((size_t)s.nchunks * H);
     float4 *stat = carve.take<float4>((size_t)V * H);
-    float *gz = carve.take<float>((size_t)E * H);
-    float *g_el = carve.take<float>((size_t)V * H);
     float *g_er = carve.take<float>((size_t)V * H);
-    const int nred = (int)ceil_div(V, kRedRows);
+    float *g_el_row = carve.take<float>((size_t)V * H);
+    const int nblocks = (int)ceil_div(s.nchunks, kGatWaves);
+    const int nred = s.nchunks;                                     // one partial row per chunk
     float *red = carve.take<float>((size_t)nred * 2 * F);
+    float *mid = carve.take<float>((size_t)kRedSlices * 2 * F);
     const int64_t VH = (int64_t)V * H;
 
-    void *spmm_ws = carve.base + carve.used;
-    if (vec_nodes_ok(D) && (((uintptr_t)out) & 15) == 0)
+    if (vec_nodes_ok(D))
         hipLaunchKernelGGL(gat_bwd_node_stats_vec, dim3((unsigned)ceil_div(VH * (D / 4), 256)), dim3(256), 0, st, er,
-                           smax, ssum, reinterpret_cast<const float4 *>(g_out), reinterpret_cast<const float4 *>(out),
-                           stat, VH * (D / 4), D / 4);
+                           smax, ssum, spos, reinterpret_cast<const float4 *>(g_out),
+                           reinterpret_cast<const float4 *>(out), reinterpret_cast<const float4 *>(pos), slope, stat,
+                           g_er, VH * (D / 4), D / 4);
     else
         hipLaunchKernelGGL(gat_bwd_node_stats, dim3((unsigned)ceil_div(VH, 256)), dim3(256), 0, st, er, smax, ssum,
-                           g_out, out, stat, VH, D);
-    dim3 grid((unsigned)ceil_div(s.nchunks, kGatWaves)), block(kGatThreads);
+                           spos, g_out, out, pos, slope, stat, g_er, VH, D);
+    dim3 grid((unsigned)nblocks), block(kGatThreads);
     const bool listed = pv.fix != nullptr;
     const dim3 ggrid(listed ? gat_list_grid(n_grp, ngroups) : (unsigned)ceil_div(ngroups, kGatWaves));
     const dim3 fgrid(listed ? gat_list_grid(n_fix, s.nchunks) : grid.x);
 #define JG_BWD(VV, NN)                                                                                             \
     case VV * 16 + NN:                                                                                             \
-        hipLaunchKernelGGL((gat_bwd_merge<VV, NN>), grid, block, 0, st, t_off, t_idx, h, el, stat, g_out,          \
-                           slope, g_h, g_el, gz, partial, pel, pv.start, V, (int)E, H, D, s.lph, s.nchunks);       \
+        hipLaunchKernelGGL((gat_bwd_merge<VV, NN>), grid, block, 0, st, t_off, t_idx, h, el, stat, g_er, g_out,    \
+                           a_src, a_dst, slope, g_h, g_el_row, partial, pel, red, pv.start, V, (int)E, H, D,       \
+                           s.lph, s.nchunks);                                                                      \
         if (ngroups > 1 && n_grp != 0 && n_fix != 0)                                                               \
             hipLaunchKernelGGL((gat_bwd_group<VV, NN>), ggrid, block, 0, st, t_off, partial, pel, gvec, ggel,      \
                                pv.start, pv.grp, pv.counts + 1, V, H, D, s.chunk, s.nchunks);                      \
         if (n_fix != 0)                                                                                            \
-            hipLaunchKernelGGL((gat_bwd_fixup<VV, NN>), fgrid, block, 0, st, t_off, g_h, g_el, partial, pel,       \
-                               gvec, ggel, pv.start, pv.fix, pv.counts, V, H, D, s.chunk, s.nchunks);              \
+            hipLaunchKernelGGL((gat_bwd_fixup<VV, NN>), fgrid, block, 0, st, t_off, g_h, g_el_row, g_er, a_src,    \
+                               a_dst, partial, pel, gvec, ggel, pv.start, pv.fix, pv.counts, V, H, D, s.chunk,     \
+                               s.nchunks);                                                                         \
         break;
     JG_GAT_DISPATCH(JG_BWD)
 #undef JG_BWD
-    // g_er[c,k] = sum of gz over the CSC slots of column c: the row-gather SpMM with unit
-    // weights; slot j's row of the [E,H] array sits at its transposed position t_inv[j]
-    if (int32_t rc = spmm_enqueue(off, t_inv, nullptr, gz, g_er, V, (int32_t)E, E, H, spmm_ws,
-                                  spmm_ws_bytes(V, E, H), st, tiles))
-        return rc;
-    hipLaunchKernelGGL(gat_bwd_finish, dim3((unsigned)nred), dim3(256), 0, st, h, a_src, a_dst, g_el, g_er, g_h, red,
-                       V, H, D);
-    hipLaunchKernelGGL(gat_bwd_reduce, dim3((unsigned)ceil_div(2 * F, 64)), dim3(1024), 0, st, red, nred, F, g_a_src,
-                       g_a_dst);
+    // the parameter gradients: the workgroups' partial rows, summed in a fixed order
+    if (nred > 4 * kRedSlices) {
+        const int per_slice = (int)ceil_div(nred, kRedSlices);
+        hipLaunchKernelGGL(gat_bwd_reduce, dim3(col_blocks, kRedSlices), dim3(1024), 0, st, red, nred, per_slice,
+                           2 * F, mid, nullptr, nullptr, F);
+        hipLaunchKernelGGL(gat_bwd_reduce, dim3(col_blocks), dim3(1024), 0, st, mid, kRedSlices, kRedSlices, 2 * F,
+                           nullptr, g_a_src, g_a_dst, F);
+    } else {
+        hipLaunchKernelGGL(gat_bwd_reduce, dim3(col_blocks), dim3(1024), 0, st, red, nred, nred, 2 * F, nullptr,
+                           g_a_src, g_a_dst, F);
+    }
     return launch_status("gat_bwd");
 }

@@ -19,6 +19,8 @@
 // in this one (its pieces have to be added up); grp[] = the groups of kPlanGroup
 // chunks past whose end a row continues (their pieces are pre-summed).  Both
 // ascending; their lengths sit at the start of the plan.
+#include <stdlib.h>
+
 #include "common.h"
 
 namespace jg {
@@ -158,8 +160,14 @@ ChunkPlan chunk_plan_view(int kind, int32_t R, int64_t E, const void *plan)
 
 void chunk_starts_enqueue(const int32_t *off, int32_t R, int64_t E, int chunk, int nchunks, int2 *start, hipStream_t s)
 {
+    // tuning aid, read once per process: the longest row kept whole, in percent of a chunk (below 100)
+    static const int pct = [] {
+        const char *e = getenv("JGAMD_PLAN_SNAP");
+        const int v = e ? atoi(e) : 50;
+        return v < 0 ? 0 : (v > 99 ? 99 : v);
+    }();
     hipLaunchKernelGGL(plan_chunk_starts, dim3((unsigned)ceil_div(nchunks + 1, 256)), dim3(256), 0, s, off, R, (int)E,
-                       chunk, nchunks, chunk / 2, start);
+                       chunk, nchunks, chunk * pct / 100, start);
 }
 
 size_t tile_plan_bytes(int64_t E)

@@ -6,7 +6,7 @@ EdgeSoftmax -> multiply -> ScatterToVertex of GATConv.propagate
 import torch
 
 from .. import _lib
-from ._common import PLAN_GAT, PLAN_TILES, as_f32, csc_arrays, csx_plan, transposed, transposed_inverse
+from ._common import PLAN_GAT, as_f32, csc_arrays, csx_plan, transposed
 
 
 def fused_supported(H, D, backward=True):
@@ -23,8 +23,10 @@ def fused_supported(H, D, backward=True):
     return True
 
 
-def gat_forward_raw(h, csc, a_src, a_dst, slope=0.2, want_alpha=False):
-    """h [V,H,D], a_src/a_dst [H,D] -> dict(out, el, er, smax, ssum, alpha)."""
+def gat_forward_raw(h, csc, a_src, a_dst, slope=0.2, want_alpha=False, for_backward=False):
+    """h [V,H,D], a_src/a_dst [H,D] -> dict(out, el, er, smax, ssum, alpha, pos, spos); pos / spos
+    (the positive-logit share of out and of the attention, which the backward kernels read) are
+    only computed with for_backward."""
     lib = _lib.load()
     dev = _lib.require_gpu(h, csc.row_indices, csc.column_offset, a_src, a_dst)
     h, a_src, a_dst = as_f32(h, "h"), as_f32(a_src, "a_src"), as_f32(a_dst, "a_dst")
@@ -39,14 +41,15 @@ def gat_forward_raw(h, csc, a_src, a_dst, slope=0.2, want_alpha=False):
     mk = lambda *s: torch.empty(s, dtype=torch.float32, device=dev)
     out, el, er, smax, ssum = mk(V, H, D), mk(V, H), mk(V, H), mk(V, H), mk(V, H)
     alpha = mk(E, H) if want_alpha else None
+    pos, spos = (mk(V, H, D), mk(V, H)) if for_backward else (None, None)
     nbytes = _lib.query(lib.jgamd_gat_fwd_workspace, V, E, H, D)
     ws = _lib.workspace(nbytes, dev)
     plan, n_fix, n_grp = csx_plan(off, V, E, PLAN_GAT) if V > 0 else (None, -1, -1)
     _lib.check(lib.jgamd_gat_fwd(_lib.ptr(plan), n_fix, n_grp, _lib.ptr(off), _lib.ptr(idx), _lib.ptr(h),
                                  _lib.ptr(a_src), _lib.ptr(a_dst), float(slope), _lib.ptr(el), _lib.ptr(er),
-                                 _lib.ptr(smax), _lib.ptr(ssum), _lib.ptr(alpha), _lib.ptr(out), V, E, H, D,
-                                 _lib.ptr(ws), nbytes, _lib.stream_ptr(dev)))
-    return dict(out=out, el=el, er=er, smax=smax, ssum=ssum, alpha=alpha)
+                                 _lib.ptr(smax), _lib.ptr(ssum), _lib.ptr(pos), _lib.ptr(spos), _lib.ptr(alpha),
+                                 _lib.ptr(out), V, E, H, D, _lib.ptr(ws), nbytes, _lib.stream_ptr(dev)))
+    return dict(out=out, el=el, er=er, smax=smax, ssum=ssum, alpha=alpha, pos=pos, spos=spos)
 
 
 class GatFusedFunc(torch.autograd.Function):
@@ -54,8 +57,11 @@ class GatFusedFunc(torch.autograd.Function):
     def forward(ctx, h, a_src, a_dst, csc, slope):
         # what backward reads must be what forward read: dense fp32 copies, not the caller's views
         h, a_src, a_dst = as_f32(h, "h"), as_f32(a_src, "a_src"), as_f32(a_dst, "a_dst")
-        r = gat_forward_raw(h, csc, a_src, a_dst, slope)
-        ctx.save_for_backward(h, a_src, a_dst, r["el"], r["er"], r["smax"], r["ssum"], r["out"])
+        needs_grad = any(ctx.needs_input_grad[:3])
+        r = gat_forward_raw(h, csc, a_src, a_dst, slope, for_backward=needs_grad)
+        if needs_grad:
+            ctx.save_for_backward(h, a_src, a_dst, r["el"], r["er"], r["smax"], r["ssum"], r["out"], r["pos"],
+                                  r["spos"])
         ctx.csc = csc
         ctx.slope = slope
         return r["out"]
@@ -63,28 +69,25 @@ class GatFusedFunc(torch.autograd.Function):
     @staticmethod
     def backward(ctx, g_out):
         lib = _lib.load()
-        h, a_src, a_dst, el, er, smax, ssum, out = ctx.saved_tensors
+        h, a_src, a_dst, el, er, smax, ssum, out, pos, spos = ctx.saved_tensors
         csc = ctx.csc
         g_out = as_f32(g_out, "g_out")
         dev = _lib.require_gpu(g_out, h)
         V, H, D = h.shape
         off, idx, w = csc_arrays(csc)
         E = idx.shape[0]
-        off_t, idx_t, _, perm = transposed(csc, off, idx, w, V, V)
-        inv = transposed_inverse(csc, perm)
+        off_t, idx_t, _, _ = transposed(csc, off, idx, w, V, V)
         g_h = torch.empty((V, H, D), dtype=torch.float32, device=dev)
         g_as = torch.empty((H, D), dtype=torch.float32, device=dev)
         g_ad = torch.empty((H, D), dtype=torch.float32, device=dev)
         nbytes = _lib.query(lib.jgamd_gat_bwd_workspace, V, E, H, D)
         ws = _lib.workspace(nbytes, dev)
         plan, n_fix, n_grp = csx_plan(off_t, V, E, PLAN_GAT) if V > 0 else (None, -1, -1)
-        tiles = csx_plan(off, V, E, PLAN_TILES)[0] if V > 0 and E > 0 else None
-        _lib.check(lib.jgamd_gat_bwd(_lib.ptr(plan), n_fix, n_grp, _lib.ptr(tiles), _lib.ptr(off), _lib.ptr(idx),
-                                     _lib.ptr(off_t),
-                                     _lib.ptr(idx_t), _lib.ptr(inv), _lib.ptr(h), _lib.ptr(a_src), _lib.ptr(a_dst),
-                                     float(ctx.slope), _lib.ptr(el), _lib.ptr(er), _lib.ptr(smax), _lib.ptr(ssum),
-                                     _lib.ptr(out), _lib.ptr(g_out), _lib.ptr(g_h), _lib.ptr(g_as), _lib.ptr(g_ad),
-                                     V, E, H, D, _lib.ptr(ws), nbytes, _lib.stream_ptr(dev)))
+        _lib.check(lib.jgamd_gat_bwd(_lib.ptr(plan), n_fix, n_grp, _lib.ptr(off_t), _lib.ptr(idx_t), _lib.ptr(h),
+                                     _lib.ptr(a_src), _lib.ptr(a_dst), float(ctx.slope), _lib.ptr(el), _lib.ptr(er),
+                                     _lib.ptr(smax), _lib.ptr(ssum), _lib.ptr(spos), _lib.ptr(out), _lib.ptr(pos),
+                                     _lib.ptr(g_out), _lib.ptr(g_h), _lib.ptr(g_as), _lib.ptr(g_ad), V, E, H, D,
+                                     _lib.ptr(ws), nbytes, _lib.stream_ptr(dev)))
         return g_h, g_as, g_ad, None, None
 
 
