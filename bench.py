@@ -27,6 +27,14 @@ entry, the output) or the step time for the time-like configurations.
                     is an upper bound of the HBM share; `compulsory_frac` (every array once) is
                     the lower bound
   effective         algorithmic bytes / kernel time (can exceed the peak: it counts rows L2 serves)
+  copy_gbps         what a plain 1 GiB device-to-device copy moves per second on this GPU in this
+                    run (bytes read + bytes written, HIP events); frac_of_copy = achieved / copy_gbps
+  hbm_frac_range    [compulsory_frac, frac]: the share of the HBM peak lies between every array
+                    moved once and everything that missed L2
+
+Times: `ms_per_step` and `value` are the wall-clock mean over exactly --steps steps between two
+device synchronisations; `ms_per_step_event_median` is the median of per-step HIP-event times of a
+second loop of the same length.
 """
 import argparse
 import ctypes
@@ -68,11 +76,12 @@ def read_profile(name, expect):
     return vals
 
 
-def roofline(profile_name, expect, kernel, kernel_ms, algorithmic, compulsory, timing):
+def roofline(profile_name, expect, kernel, kernel_ms, algorithmic, compulsory, timing, copy_gbps=None,
+             bound="hbm"):
     prof = read_profile(profile_name, expect)
     traffic = float(prof["traffic_bytes"]) if prof and "traffic_bytes" in prof else None
     rate = lambda b: round(b / (kernel_ms * 1e-3) / 1e9, 1)
-    out = {"bound": "hbm", "peak": HBM_PEAK_GBPS, "unit": "GB/s", "kernel": kernel, "kernel_ms": round(kernel_ms, 4),
+    out = {"bound": bound, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "kernel": kernel, "kernel_ms": round(kernel_ms, 4),
            "kernel_ms_source": timing, "traffic": traffic,
            "traffic_source": ("profiles/" + profile_name) if traffic else None,
            "algorithmic_bytes": algorithmic, "compulsory_bytes": compulsory,
@@ -82,11 +91,20 @@ def roofline(profile_name, expect, kernel, kernel_ms, algorithmic, compulsory, t
     else:
         out["achieved"], out["achieved_basis"] = rate(algorithmic), "algorithmic bytes / kernel time (no counter summary)"
     out["frac"] = round(out["achieved"] / HBM_PEAK_GBPS, 4)
+    out["hbm_frac_range"] = [out["compulsory_frac"], out["frac"]]
+    if copy_gbps:
+        out["copy_gbps"] = round(copy_gbps, 1)
+        out["frac_of_copy"] = round(out["achieved"] / copy_gbps, 4)
     if prof:
         for k in ("l2_hit_rate", "profile_kernel_us"):
             if k in prof:
                 out[k] = float(prof[k])
     return out
+
+
+class Ms(float):
+    """A mean time in ms that also carries the event-timed median of the same call."""
+    median = None
 
 
 class Bench:
@@ -101,6 +119,8 @@ class Bench:
         torch.manual_seed(0)
 
     def timed(self, fn, iters, warm):
+        """Wall-clock mean per call over `iters` calls between two synchronisations (the returned
+        number) and, as its .median, the median of per-call HIP-event times of a second loop."""
         torch = self.torch
         for _ in range(warm):
             fn()
@@ -109,7 +129,25 @@ class Bench:
         for _ in range(iters):
             fn()
         torch.cuda.synchronize()
-        return (time.perf_counter() - t0) / iters * 1e3
+        mean = Ms((time.perf_counter() - t0) / iters * 1e3)
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+        for a, b in ev:
+            a.record()
+            fn()
+            b.record()
+        torch.cuda.synchronize()
+        times = sorted(a.elapsed_time(b) for a, b in ev)
+        mean.median = times[len(times) // 2] if len(times) % 2 else 0.5 * (times[len(times) // 2 - 1] + times[len(times) // 2])
+        return mean
+
+    def copy_rate_gbps(self):
+        """Bytes read + written per second by a plain 1 GiB device copy, median of 7 (HIP events)."""
+        torch = self.torch
+        a = torch.empty(1 << 28, dtype=torch.float32, device=self.dev).fill_(1.0)
+        b = torch.empty_like(a)
+        ms = self.timed(lambda: b.copy_(a), 7, 2).median
+        del a, b
+        return 2 * (1 << 30) / (ms * 1e-3) / 1e9
 
     def graph(self, name, norm="gcn", time_conversions=True):
         """(edge_index, weights, V, CSC, CSR, conversion times) of a configuration after the
@@ -148,12 +186,14 @@ class Bench:
                                                         _lib.stream_ptr(self.dev), iters, ctypes.byref(k_ms),
                                                         ctypes.byref(c_ms)))
             return k_ms.value, c_ms.value
-        nbytes = _lib.query(lib.jgamd_spmm_csx_workspace, R, E, F)
+        from jittorgeometric_amd.ops._common import PLAN_SPMM, csx_plan
+        plan, n_fix, n_grp = csx_plan(off, R, E, PLAN_SPMM)       # the partition the operators keep with the offsets
+        nbytes = _lib.query(lib.jgamd_spmm_csx_planned_workspace, R, E, F)
         ws = _lib.workspace(nbytes, self.dev)
         torch.cuda.synchronize()
-        _lib.check(lib.jgamd_spmm_csx_timed(off.data_ptr(), idx.data_ptr(), w.data_ptr(), x.data_ptr(), out.data_ptr(),
-                                            R, C, E, F, ws.data_ptr(), nbytes, _lib.stream_ptr(self.dev), iters,
-                                            ctypes.byref(k_ms), ctypes.byref(c_ms)))
+        _lib.check(lib.jgamd_spmm_csx_timed(plan.data_ptr(), n_fix, n_grp, off.data_ptr(), idx.data_ptr(), w.data_ptr(),
+                                            x.data_ptr(), out.data_ptr(), R, C, E, F, ws.data_ptr(), nbytes,
+                                            _lib.stream_ptr(self.dev), iters, ctypes.byref(k_ms), ctypes.byref(c_ms)))
         return k_ms.value, c_ms.value
 
     def calibrate_copy(self):
@@ -198,6 +238,44 @@ class Bench:
                 "gpu_vs_cpu_max_scaled_err": round(err_loop, 4)}, err
 
 
+def cpu_spmm_rows_baseline(csc, x, step, what, seconds=12.0):
+    """The reference's loop (oracle port, one thread) on a random sample of the rows of a product
+    too large for a full pass within the time the benchmark may take: a 0.5 % sample is timed
+    first, then a sample sized for about `seconds` of work.  The rate is the sample's own
+    algorithmic bytes over its time; the GPU's rows of the same sample are held against the
+    exact (float64) sums and against the loop."""
+    import numpy as np
+    import oracle
+    col, off, wv = (t.cpu().numpy() for t in (csc.row_indices, csc.column_offset, csc.edge_weight))
+    xh = x.cpu().numpy()
+    V, F = xh.shape
+    rng = np.random.default_rng(0)
+
+    def run(nrows):
+        rows = np.sort(rng.choice(V, size=nrows, replace=False))
+        t0 = time.perf_counter()
+        ref = oracle.aggregate_rows(xh, col, off, wv, rows)
+        return rows, ref, time.perf_counter() - t0
+    rows, ref, dt = run(max(V // 200, 1))
+    entries = int((off[rows + 1] - off[rows]).sum())
+    want = int(min(V, max(len(rows), len(rows) * seconds / max(dt, 1e-3))))
+    if want > 2 * len(rows):
+        rows, ref, dt = run(want)
+        entries = int((off[rows + 1] - off[rows]).sum())
+    nbytes = 4 * (len(rows) + 1) + 8 * entries + 4 * entries * F + 4 * len(rows) * F
+    exact, terms = oracle.aggregate_rows_f64(xh, col, off, wv, rows)
+    deg = (off[rows + 1] - off[rows]).astype(np.float64)[:, None]
+    got = step().cpu().numpy()[rows].astype(np.float64)
+    err_exact = float(np.max(np.abs(got - exact) / (1e-6 + 1e-5 * terms)))
+    err_loop = float(np.max(np.abs(got - ref) / (1e-6 + (1e-5 + deg * 2.0 ** -24) * terms)))
+    return {"value": round(nbytes / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": "%d of %d rows (%d of %d entries) of %s, chosen at random, one pass of %.1f s; a full pass "
+                      "would take about %.0f s" % (len(rows), V, entries, int(off[-1]), what, dt, dt * int(off[-1]) / max(entries, 1)),
+            "cpu_model": cpu_model(), "host_cores_available": os.cpu_count(),
+            "gpu_vs_exact_max_scaled_err": round(err_exact, 4),
+            "gpu_vs_cpu_max_scaled_err": round(err_loop, 4)}, max(err_exact, err_loop)
+
+
 def cpu_model():
     try:
         for line in open("/proc/cpuinfo"):
@@ -211,9 +289,12 @@ def cpu_model():
 def base_line(args, metric, value, unit, ms, higher, workload, extra_config):
     cfg = {"workload": workload}
     cfg.update(extra_config)
-    return {"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+    line = {"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
             "ms_per_step": round(ms, 4), "higher_is_better": higher, "scaling": "weak", "vs_baseline": None,
             "dtype": "f32", "data": "synthetic", "config": cfg}
+    if getattr(ms, "median", None) is not None:
+        line["ms_per_step_event_median"] = round(ms.median, 4)
+    return line
 
 
 # --------------------------------------------------------------------------------- config 2
@@ -243,13 +324,15 @@ def config2(b):
         k_ms, c_ms = b.spmm_kernel_ms(csc.column_offset, csc.row_indices, csc.edge_weight, x, V, max(args.steps, 10))
         line.update({
             "value": round(value, 1), "ms_per_step": round(ms_per_step, 4),
+            "ms_per_step_event_median": round(ms_per_step.median, 4),
             "pct_hbm_peak_algorithmic": round(100 * value / HBM_PEAK_GBPS, 2),
             "coo_to_csr_edges_per_s": round(E / (conv_csr_ms * 1e-3)),
             "coo_to_csc_edges_per_s": round(E / (conv_csc_ms * 1e-3)),
             "coo_to_csr_ms": round(conv_csr_ms, 4),
             "coo_to_csr_algorithmic_gbps": round((24 * E + 8 * (V + 1)) / (conv_csr_ms * 1e-3) / 1e9, 1),
             "roofline": roofline("spmm_merge_powerlaw_1m_f128.txt", {"V": V, "E": E, "F": F}, "spmm_merge", k_ms,
-                                 bytes_step, spmm_compulsory_bytes(V, V, E, F), "hipEvents in this run"),
+                                 bytes_step, spmm_compulsory_bytes(V, V, E, F), "hipEvents in this run",
+                                 b.copy_rate_gbps()),
             "spmm_call_ms": round(c_ms, 4),
         })
 
@@ -394,8 +477,10 @@ def config1(b):
                      "config 1: 2-layer GCN forward+backward, V=2708, 10556 directed edges + self-loops, 1433->256->7",
                      {"V": V, "E": E})
     line.update({"coo_to_csr_ms": round(conv_csr_ms, 4), "gcn2_fwd_bwd_graph_replay_ms": round(graph_ms, 4),
+                 "gcn2_fwd_bwd_graph_replay_event_median_ms": round(graph_ms.median, 4),
                  "roofline": roofline("spmm_merge_cora_like_f256.txt", {"V": V, "E": E, "F": 256}, "spmm_merge", k_ms,
-                                      spmm_bytes(V, E, 256), spmm_compulsory_bytes(V, V, E, 256), "hipEvents in this run"),
+                                      spmm_bytes(V, E, 256), spmm_compulsory_bytes(V, V, E, 256), "hipEvents in this run",
+                                      b.copy_rate_gbps(), bound="launch latency (13k entries; every array fits L2)"),
                  "note": "launch-bound at this size: 13k entries are one launch of a few microseconds",
                  "cpu_baseline": cpu})
     return line, 0.0
@@ -432,12 +517,19 @@ def config3(b):
         import oracle
         row, off = csc.row_indices.cpu().numpy(), csc.column_offset.cpu().numpy()
         hh, s, d = h.detach().cpu().numpy(), a_s.detach().cpu().numpy(), a_d.detach().cpu().numpy()
-        n, t0 = 0, time.perf_counter()
-        while n < 1 or time.perf_counter() - t0 < 5.0:
+        gh = g.cpu().numpy()
+        n, t0, fwd_s = 0, time.perf_counter(), 0.0
+        while n < 1 or time.perf_counter() - t0 < 10.0:
+            t1 = time.perf_counter()
             oracle.gat_forward_heads(hh, (row, off, None), s, d, 0.2)
+            fwd_s += time.perf_counter() - t1
+            oracle.gat_backward_heads(hh, (row, off, None), s, d, gh, 0.2)
             n += 1
-        cpu = {"value": round((time.perf_counter() - t0) / n * 1e3, 2), "unit": "ms (forward only)", "cores": 1,
-               "kind": "port", "sample": "%d forward passes of the reference's operator chain (oracle loops), all heads" % n,
+        cpu = {"value": round((time.perf_counter() - t0) / n * 1e3, 2), "unit": "ms", "cores": 1, "kind": "port",
+               "forward_only_ms": round(fwd_s / n * 1e3, 2),
+               "sample": "%d passes of the same step, forward + backward, all heads: the reference's operator chain and "
+                         "the chain of its operators' grad functions (oracle loops; the backward recomputes the "
+                         "forward's per-edge tensors as autograd would have kept them)" % n,
                "cpu_model": cpu_model()}
     prof = read_profile("gat_merge_gat_169k_h8x16.txt", {"V": V, "E": E, "F": H * D})
     k_ms = float(prof["profile_kernel_us"]) / 1e3 if prof and "profile_kernel_us" in prof else fwd_ms
@@ -446,9 +538,13 @@ def config3(b):
                      {"V": V, "E": E, "H": H, "D": D})
     line.update({"gat_fused_fwd_ms": round(fwd_ms, 4),
                  "gat_fused_fwd_algorithmic_gbps": round(fwd_bytes / (fwd_ms * 1e-3) / 1e9, 1),
+                 "gat_fused_fwd_event_median_ms": round(fwd_ms.median, 4),
                  "roofline": roofline("gat_merge_gat_169k_h8x16.txt", {"V": V, "E": E, "F": H * D}, "gat_fwd_merge", k_ms,
                                       fwd_bytes, compulsory,
-                                      "rocprofv3 summary" if prof else "whole forward call in this run (4 launches)"),
+                                      "rocprofv3 summary" if prof else "whole forward call in this run (4 launches)",
+                                      b.copy_rate_gbps(),
+                                      bound="fabric (L2-miss traffic; the 87 MB feature table fits the 256 MB "
+                                            "Infinity Cache, so most of it is not HBM traffic)"),
                  "cpu_baseline": cpu})
     return line, 0.0
 
@@ -481,9 +577,7 @@ def config4(b):
     bytes_step = spmm_bytes(V, E, 602)
     cpu, err = (None, 0.0)
     if not args.no_cpu_baseline and args.part == "all":
-        x41 = res[41][2]
-        cpu, err = b.cpu_spmm_baseline(csc, x41, res[41][3], spmm_bytes(V, E, 41), (ei, w),
-                                       "the F=41 product of this graph (V=%d, E=%d)" % (V, E))
+        cpu, err = cpu_spmm_rows_baseline(csc, x, step, "the F=602 product of this graph (V=%d, E=%d)" % (V, E))
     line = base_line(args, "spmm_f602_algorithmic_bandwidth", round(bytes_step / (ms * 1e-3) / 1e9, 1), "GB/s", ms, True,
                      "config 4: weighted CSC SpMM, V=232,965, lognormal degrees (mean 492) + self-loops, F=602",
                      {"V": V, "E": E, "F": 602, "bytes_per_step": bytes_step})
@@ -501,7 +595,10 @@ def config4(b):
                  "coo_to_csr_ms": round(conv_csr_ms, 4), "coo_to_csr_edges_per_s": round(E / (conv_csr_ms * 1e-3)),
                  "coo_to_csc_edges_per_s": round(E / (conv_csc_ms * 1e-3)),
                  "roofline": roofline("spmm_merge_dense_233k_f602.txt", {"V": V, "E": E, "F": 602}, "spmm_merge", k_ms,
-                                      bytes_step, spmm_compulsory_bytes(V, V, E, 602), "hipEvents in this run"),
+                                      bytes_step, spmm_compulsory_bytes(V, V, E, 602), "hipEvents in this run",
+                                      b.copy_rate_gbps(),
+                                      bound="L2 delivery (column-blocked gathers; hbm_frac_range is what reaches the fabric)"
+                                      if blocks else "hbm"),
                  "cpu_baseline": cpu})
     return line, err
 
@@ -559,10 +656,9 @@ def config5(b):
                    b.spmm_kernel_ms(csc.column_offset, csc.row_indices, csc.edge_weight, xf, V, 10)[0], xf)
     cpu, err = (None, 0.0)
     if not args.no_cpu_baseline and not main_only:
-        xf = prod[47][2]
-        cpu, err = b.cpu_spmm_baseline(csc, xf, lambda: spmm(csc.column_offset, csc.row_indices, csc.edge_weight, xf, V),
-                                       spmm_bytes(V, E, 47), (ei, w),
-                                       "the F=47 product of this graph (V=%d, E=%d)" % (V, E))
+        xf = prod[256][2]
+        cpu, err = cpu_spmm_rows_baseline(csc, xf, lambda: spmm(csc.column_offset, csc.row_indices, csc.edge_weight, xf, V),
+                                          "the F=256 product of this graph (V=%d, E=%d)" % (V, E))
     line = base_line(args, "gcn3_fullgraph_fwd_bwd_ms", round(gcn_ms, 3), "ms", gcn_ms, False,
                      "config 5: 3-layer GCN full-graph forward+backward, V=2,449,029 power-law (exp 2.1, mean 50) "
                      "+ self-loops, 100->256->256->47", {"V": V, "E": E})
@@ -577,7 +673,8 @@ def config5(b):
         line["spmm_f%d_ms" % F] = round(prod[F][0], 4)
         line["spmm_f%d_algorithmic_gbps" % F] = round(spmm_bytes(V, E, F) / (prod[F][0] * 1e-3) / 1e9, 1)
     line["roofline"] = roofline("spmm_merge_powerlaw_2m4_f256.txt", {"V": V, "E": E, "F": 256}, "spmm_merge", prod[256][1],
-                                spmm_bytes(V, E, 256), spmm_compulsory_bytes(V, V, E, 256), "hipEvents in this run")
+                                spmm_bytes(V, E, 256), spmm_compulsory_bytes(V, V, E, 256), "hipEvents in this run",
+                                b.copy_rate_gbps())
     line["cpu_baseline"] = cpu
     if main_only:
         # only the F=256 product ran (the part the counter summaries are taken from): that is the line's metric

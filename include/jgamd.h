@@ -204,14 +204,16 @@ int32_t jgamd_spmm_csx_noalloc(const int32_t *off, const int32_t *idx, const flo
                                const float *x, float *out, int32_t R, int32_t C, int64_t E,
                                int32_t F, void *stream);
 
-/* Benchmark support; no counterpart in the reference.  Runs jgamd_spmm_csx
- * `iters` times on `stream`, with one hipEvent pair around each launch of the
- * gather kernel (spmm_merge) and one around each whole call (three launches),
+/* Benchmark support; no counterpart in the reference.  Runs the product
+ * `iters` times on `stream` (jgamd_spmm_csx_planned with `plan`, n_fix, n_grp,
+ * or jgamd_spmm_csx when plan is NULL), with one hipEvent pair around each
+ * launch of the gather kernel (spmm_merge) and one around each whole call,
  * WAITS for the stream after every call, and returns the two mean durations
  * in milliseconds.  Unlike every other entry point it synchronises and
  * creates/destroys events. */
-int32_t jgamd_spmm_csx_timed(const int32_t *off, const int32_t *idx, const float *w, const float *x,
-                             float *out, int32_t R, int32_t C, int64_t E, int32_t F, void *ws,
+int32_t jgamd_spmm_csx_timed(const void *plan, int32_t n_fix, int32_t n_grp, const int32_t *off,
+                             const int32_t *idx, const float *w, const float *x, float *out,
+                             int32_t R, int32_t C, int64_t E, int32_t F, void *ws,
                              size_t ws_bytes, void *stream, int32_t iters, float *kernel_ms,
                              float *call_ms);
 

@@ -46,7 +46,7 @@ SIGNATURES = {
                                _c.c_size_t, _P],
     "jgamd_spmm_csx_blocked_timed": [_P, _P, _P, _P, _P, _I32, _I32, _I64, _I32, _I32, _P, _c.c_size_t, _P, _I32,
                                      _c.POINTER(_c.c_float), _c.POINTER(_c.c_float)],
-    "jgamd_spmm_csx_timed": [_P, _P, _P, _P, _P, _I32, _I32, _I64, _I32, _P, _c.c_size_t, _P, _I32,
+    "jgamd_spmm_csx_timed": [_P, _I32, _I32, _P, _P, _P, _P, _P, _I32, _I32, _I64, _I32, _P, _c.c_size_t, _P, _I32,
                              _c.POINTER(_c.c_float), _c.POINTER(_c.c_float)],
     "jgamd_edge_softmax_workspace": [_I32, _I64, _SZP],
     "jgamd_edge_softmax_fwd": [_P, _P, _P, _I32, _I64, _I32, _P, _c.c_size_t, _P],

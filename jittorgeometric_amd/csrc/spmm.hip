@@ -726,9 +726,14 @@ int32_t spmm_enqueue_slabs(const int32_t *off, const int32_t *idx, const float *
 }  // namespace jg
 
 extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_timed(
-    const int32_t *off, const int32_t *idx, const float *w, const float *x, float *out, int32_t R, int32_t C,
-    int64_t E, int32_t F, void *ws, size_t ws_bytes, void *stream, int32_t iters, float *kernel_ms, float *call_ms)
+    const void *plan, int32_t n_fix, int32_t n_grp, const int32_t *off, const int32_t *idx, const float *w,
+    const float *x, float *out, int32_t R, int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, void *stream,
+    int32_t iters, float *kernel_ms, float *call_ms)
 {
+    if (((uintptr_t)plan & 255) != 0) return fail(JGAMD_ERR_ALIGN, "spmm_csx_timed: plan not 256-byte aligned");
+    PlanHints hints;
+    hints.n_fix = n_fix < 0 ? -1 : n_fix;
+    hints.n_grp = n_grp < 0 ? -1 : n_grp;
     if (iters < 1 || iters > 4096) return fail(JGAMD_ERR_SIZE, "spmm_csx_timed: iters must be in [1, 4096]");
     if (!kernel_ms || !call_ms) return fail(JGAMD_ERR_NULL, "spmm_csx_timed: NULL result pointer");
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -739,7 +744,8 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_timed(
     int32_t rc = 0;
     for (int i = 0; i < iters && rc == 0; i++) {
         (void)hipEventRecord(ev[0], st);
-        rc = spmm_call(off, idx, w, x, out, R, C, E, F, ws, ws_bytes, stream, ev[1], ev[2]);
+        rc = spmm_call(off, idx, w, x, out, R, C, E, F, ws, ws_bytes, stream, ev[1], ev[2], nullptr, false, 0, plan,
+                       nullptr, hints);
         (void)hipEventRecord(ev[3], st);
         if (hipEventSynchronize(ev[3]) != hipSuccess && rc == 0)
             rc = fail(JGAMD_ERR_UNSUPPORTED, "spmm_csx_timed: hipEventSynchronize failed");

@@ -10,6 +10,8 @@ Functions with no independent pin (see oracle.c header for the pins of the
 rest): none of the arithmetic.  The cuSPARSE-internal summation order behind
 the reference's SpmmCsr and SpmmCoo is "parity unpinned" (third-party,
 jittor==1.3.9.14).  Pins of the numpy restatements at the end of this file:
+  gat_backward  float64 autograd of the same layer on a small graph, a directional
+                finite difference of gat_forward
   spmmcoo       hand-derived fixture of tests/test_spmmcoo.py, dense fp64 product
   toundirected  hand-derived fixture of tests/test_undirected.py, brute force over
                 Python sets; which of several equal (row, col) pairs survives is
@@ -334,6 +336,49 @@ def gat_forward_heads(h, csc, a_src, a_dst, slope=0.2):
         outs.append(o)
         alphas.append(al[:, 0])
     return np.stack(outs, axis=1), np.stack(alphas, axis=1)
+
+
+def gat_backward(h, csc, a, g_out, slope=0.2):
+    """Gradients of gat_forward with respect to h and a for the upstream gradient g_out [V,C]:
+    the chain Jittor's autograd runs through the reference operators' own grad functions
+    (nn/conv/gat_conv.py:61-83 backwards): ScatterToVertex.grad = scattertoedge with flag 1
+    (ops/scatterToVertex.py:43-47), the product with alpha, EdgeSoftmax.grad
+    (ops/edgesoftmax.py:71-74 -> edgesoftmaxbackward_op.cc:27-54), leaky_relu', the [E,2C]x[2C,1]
+    product, ScatterToEdge.grad = edgetovertex with the flag of the forward call
+    (ops/scatterToEdge.py:42-46).  Returns (g_h [V,C], g_a [2C])."""
+    row, off = _i32(csc[0]), _i32(csc[1])
+    h, g_out = _f32(h), _f32(g_out)
+    V, C = h.shape
+    slope = np.float32(slope)
+    a = _f32(a).reshape(2 * C, 1)
+    e_src = scattertoedge(h, row, off, 0)
+    e_dst = scattertoedge(h, row, off, 1)
+    e = np.concatenate([e_src, e_dst], axis=1)
+    z = (e @ a).astype(np.float32)
+    m = np.where(z > 0, z, slope * z).astype(np.float32)
+    alpha = edgesoftmax(m, off)
+    g_msg = scattertoedge(g_out, row, off, 1)                       # grad of ScatterToVertex
+    g_alpha = (g_msg * e_src).sum(axis=1, keepdims=True).astype(np.float32)
+    g_m = edgesoftmax_backward(g_alpha, alpha, off)
+    g_z = (g_m * np.where(z > 0, np.float32(1), slope)).astype(np.float32)
+    g_a = (e.T @ g_z).astype(np.float32)[:, 0]
+    g_e = (g_z @ a.T).astype(np.float32)
+    g_e_src = (g_msg * alpha + g_e[:, :C]).astype(np.float32)
+    g_h = edgetovertex(g_e_src, row, off, 0, out_rows=V) + edgetovertex(np.ascontiguousarray(g_e[:, C:]), row, off, 1)
+    return g_h.astype(np.float32), g_a
+
+
+def gat_backward_heads(h, csc, a_src, a_dst, g_out, slope=0.2):
+    """Head k is gat_backward on h[:,k,:]; returns (g_h [V,H,D], g_a_src [H,D], g_a_dst [H,D])."""
+    V, H, D = h.shape
+    gh, gs, gd = [], [], []
+    for k in range(H):
+        a = np.concatenate([a_src[k], a_dst[k]]).astype(np.float32)
+        g, ga = gat_backward(np.ascontiguousarray(h[:, k, :]), csc, a, np.ascontiguousarray(g_out[:, k, :]), slope)
+        gh.append(g)
+        gs.append(ga[:D])
+        gd.append(ga[D:])
+    return np.stack(gh, axis=1), np.stack(gs), np.stack(gd)
 
 
 def spmmcoo(x, edge_index, edge_weight, trans_A=True):
