@@ -27,9 +27,7 @@ def _product(x, csr, trans_A):
 
 class SpmmCsrFunc(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, csr, trans_A, trans_B):
-        if trans_B:
-            raise _lib.JgamdError("SpmmCsr: trans_B=True is not supported")
+    def forward(ctx, x, csr, trans_A):
         ctx.csr = csr
         ctx.trans_A = trans_A
         return _product(x, csr, trans_A)
@@ -37,8 +35,17 @@ class SpmmCsrFunc(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output):
         trans = ctx.trans_A if REFERENCE_GRAD else not ctx.trans_A
-        return _product(grad_output, ctx.csr, trans), None, None, None
+        return _product(grad_output, ctx.csr, trans), None, None
 
 
 def SpmmCsr(x, csr, trans_A=True, trans_B=False):
-    return SpmmCsrFunc.apply(x, csr, trans_A, trans_B)
+    """op(A) x, or op(A) x^T with trans_B=True (x is then [F, V], the dense operand stored
+    transposed, as the flag tells cuSPARSE: ops/spmmcsr.py:31 hands it on unread).  No caller
+    in the reference sets trans_B and its output allocation (v_num rows, size(x, 1) columns,
+    ops/spmmcsr.py:24-28) only fits a square x; what cuSPARSE does with the flag is the
+    documented op(B) = B^T, "parity unpinned" like the rest of that third-party product."""
+    if trans_B:
+        if x.dim() != 2:
+            raise _lib.JgamdError("SpmmCsr: x must be two-dimensional, got %s" % (tuple(x.shape),))
+        x = x.t().contiguous()          # differentiable: the gradient comes back transposed
+    return SpmmCsrFunc.apply(x, csr, trans_A)
