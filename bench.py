@@ -315,6 +315,19 @@ def config2(b):
 
     step = lambda: spmm(csc.column_offset, csc.row_indices, csc.edge_weight, x, V)
     bytes_step = spmm_bytes(V, E, F)
+    setup_ms = None
+    if args.part == "all":
+        # the graph set-up of examples/gcn_example.py:48-59 as one sequence: normalisation with
+        # self-loops, then both conversions of the normalised edge list
+        from jittorgeometric_amd.nn import gcn_norm
+        from jittorgeometric_amd.ops import cootocsr
+        raw = torch.from_numpy(synthetic.make("powerlaw_1m")[0]).to(dev)
+
+        def setup():
+            e2, w2 = gcn_norm(raw, None, V)
+            return cootocsc(e2, w2, V), cootocsr(e2, w2, V)
+        setup_ms = b.timed(setup, 10, 2)
+        del raw
     line = base_line(args, "spmm_f128_algorithmic_bandwidth", 0.0, "GB/s", 0.0, True,
                      "config 2: weighted CSC SpMM, V=1,000,000 Chung-Lu power-law (exp 2.1, cap 20000) "
                      "+ self-loops, gcn_norm weights, F=128", {"V": V, "E": E, "F": F, "bytes_per_step": bytes_step})
@@ -335,6 +348,8 @@ def config2(b):
                                  b.copy_rate_gbps()),
             "spmm_call_ms": round(c_ms, 4),
         })
+        if setup_ms is not None:
+            line["graph_setup_gcn_norm_csc_csr_ms"] = round(setup_ms, 4)
 
     if args.part in ("all", "layers"):
         # one GCN layer and one GraphSAGE (mean) layer, forward + backward, on the same graph

@@ -475,6 +475,15 @@ int32_t jgamd_getweight(const int32_t *dst, const int32_t *off, const int32_t *r
  * (nn/conv/gcn_conv.py:35-36).  jgamd_scale_edge_weights:
  * out[e] = by_row[row[e]] * w[e] * by_col[col[e]] (either factor array may be
  * NULL) — gcn_conv.py:37, sage_conv.py:40.
+ *
+ * jgamd_scale_csx_weights: the same product for weights already in compressed
+ * order, out[j] = by_idx[idx[j]] * w[j] * by_seg[c] for every slot j of segment
+ * c of (off, idx) — term for term what jgamd_scale_edge_weights gives for the
+ * edge in that slot, so a caller that has sorted an edge list once (to sum the
+ * degrees) gets the normalised weights of the compressed arrays without
+ * converting the edge list again (examples/gcn_example.py:48-59 calls gcn_norm,
+ * then cootocsc on its result).  N bounds the factor arrays; slots past off[V]
+ * are set to zero.
  */
 int32_t jgamd_add_remaining_self_loops_workspace(int64_t E, int32_t N, size_t *bytes);
 int32_t jgamd_add_remaining_self_loops(const int32_t *edge_index, const float *edge_weight,
@@ -482,6 +491,10 @@ int32_t jgamd_add_remaining_self_loops(const int32_t *edge_index, const float *e
                                        float *out_weight, int32_t *out_kept, void *ws,
                                        size_t ws_bytes, void *stream);
 int32_t jgamd_degree_power(const float *deg, int32_t N, float power, float *out, void *stream);
+int32_t jgamd_scale_csx_weights_workspace(int64_t E, size_t *bytes);
+int32_t jgamd_scale_csx_weights(const int32_t *off, const int32_t *idx, const float *w,
+                                const float *by_idx, const float *by_seg, int32_t V, int64_t E,
+                                int32_t N, float *out, void *ws, size_t ws_bytes, void *stream);
 int32_t jgamd_scale_edge_weights(const int32_t *edge_index, const float *edge_weight,
                                  const float *by_row, const float *by_col, int64_t E, int32_t N,
                                  float *out, void *stream);

@@ -17,6 +17,8 @@ SIGNATURES = {
     "jgamd_csx_transpose_workspace": [_I64, _I32, _I32, _SZP],
     "jgamd_csx_transpose": [_P, _P, _P, _I32, _I32, _I64, _P, _P, _P, _P, _P, _c.c_size_t, _P],
     "jgamd_invert_permutation": [_P, _I64, _P, _P],
+    "jgamd_scale_csx_weights_workspace": [_I64, _SZP],
+    "jgamd_scale_csx_weights": [_P, _P, _P, _P, _P, _I32, _I64, _I32, _P, _P, _c.c_size_t, _P],
     "jgamd_add_remaining_self_loops_workspace": [_I64, _I32, _SZP],
     "jgamd_add_remaining_self_loops": [_P, _P, _I64, _I32, _c.c_float, _P, _P, _P, _P, _c.c_size_t, _P],
     "jgamd_degree_power": [_P, _I32, _c.c_float, _P, _P],

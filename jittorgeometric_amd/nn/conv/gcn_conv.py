@@ -18,11 +18,21 @@ def _degree_by_col(edge_index, edge_weight, num_nodes):
     (jt.scatter(..., reduce='add') by col in gcn_conv.py:33-34): the column sum
     of the CSC arrays, i.e. conversion + gather-sum, in a fixed order and
     without the same-address atomics a hub destination causes."""
+    return _degree_and_order(edge_index, edge_weight, num_nodes)[0]
+
+
+def _degree_and_order(edge_index, edge_weight, num_nodes):
+    """(deg, order): the degrees as above and, for a contiguous int32 edge list, what the sort by
+    destination produced (row indices, offsets, weights in slot order), so that the conversion
+    the caller runs next on the same edges with the normalised weights need not sort again."""
     from ...ops._common import spmm
+    from ...ops.cootocsr import _convert
     if edge_index.shape[1] == 0:
-        return torch.zeros((num_nodes,), dtype=torch.float32, device=edge_weight.device)
-    csc = cootocsc(edge_index.contiguous(), edge_weight, num_nodes)
-    return spmm(csc.column_offset, None, None, csc.edge_weight.view(-1, 1), num_nodes).view(-1)
+        return torch.zeros((num_nodes,), dtype=torch.float32, device=edge_weight.device), None
+    keep = edge_index.dtype == torch.int32 and edge_index.is_contiguous()
+    idx, off, w, _ = _convert(edge_index, edge_weight, num_nodes, 1)
+    deg = spmm(off, None, None, w.view(-1, 1), num_nodes).view(-1)
+    return deg, ((idx, off, w) if keep else None)
 
 
 def _scale(edge_index, edge_weight, by_row, by_col, num_nodes):
@@ -51,17 +61,27 @@ def _degree_norm(edge_index, edge_weight, num_nodes, improved, add_self_loops, p
         edge_weight = edge_weight.to(torch.float32)
     if add_self_loops:
         edge_index, edge_weight = add_remaining_self_loops(edge_index, edge_weight, fill_value, num_nodes)
-    deg = _degree_by_col(edge_index, edge_weight, num_nodes)
+    deg, order = _degree_and_order(edge_index, edge_weight, num_nodes)
     dinv = torch.empty_like(deg)
     _lib.check(lib.jgamd_degree_power(_lib.ptr(deg), num_nodes, float(power), _lib.ptr(dinv), _lib.stream_ptr(dev)))
-    return edge_index, edge_weight, dinv
+    return edge_index, edge_weight, dinv, order
+
+
+def _normalised(edge_index, edge_weight, by_row, by_col, num_nodes, order):
+    """(edge_index, by_row[row] * w * by_col[col]); the sort by destination that the degree sum
+    needed is handed on to the conversion that follows."""
+    weights = _scale(edge_index, edge_weight, by_row, by_col, num_nodes)
+    if order is not None:
+        from ...ops.cootocsr import remember_order
+        remember_order(edge_index, weights, num_nodes, 1, order[0], order[1], order[2], by_row, by_col)
+    return edge_index, weights
 
 
 def gcn_norm(edge_index, edge_weight=None, num_nodes=None, improved=False, add_self_loops=True, dtype=None):
     """Symmetric normalisation w = d^-1/2[row] * w * d^-1/2[col] with the
     degree summed by column (nn/conv/gcn_conv.py:18-37)."""
-    edge_index, edge_weight, dis = _degree_norm(edge_index, edge_weight, num_nodes, improved, add_self_loops, -0.5)
-    return edge_index, _scale(edge_index, edge_weight, dis, dis, dis.shape[0])
+    edge_index, edge_weight, dis, order = _degree_norm(edge_index, edge_weight, num_nodes, improved, add_self_loops, -0.5)
+    return _normalised(edge_index, edge_weight, dis, dis, dis.shape[0], order)
 
 
 class GcnLayerFunc(torch.autograd.Function):

@@ -8,13 +8,13 @@ from ...ops import spmmcsr as _spmmcsr
 from ...ops._common import both_orders, spmm, spmm_axpby
 from ..dense import add_bias, column_sum, rows_times, xt_g, xw
 from ..inits import glorot, zeros
-from .gcn_conv import _degree_norm, _scale
+from .gcn_conv import _degree_norm, _normalised, _scale
 
 
 def sage_norm(edge_index, edge_weight=None, num_nodes=None, improved=False, add_self_loops=True, dtype=None):
     """Mean weights w * d^-1[col] (nn/conv/sage_conv.py:16-40)."""
-    edge_index, edge_weight, dinv = _degree_norm(edge_index, edge_weight, num_nodes, improved, add_self_loops, -1.0)
-    return edge_index, _scale(edge_index, edge_weight, None, dinv, dinv.shape[0])
+    edge_index, edge_weight, dinv, order = _degree_norm(edge_index, edge_weight, num_nodes, improved, add_self_loops, -1.0)
+    return _normalised(edge_index, edge_weight, None, dinv, dinv.shape[0], order)
 
 
 class SageLayerFunc(torch.autograd.Function):

@@ -186,3 +186,73 @@ def test_one_hub_with_millions_of_edges_bit_exact():
     ei[0, rng.random(E) < 0.38] = 31337
     ei[1, rng.random(E) < 0.38] = 4242
     check_exact(ei, w, V)
+
+
+@pytest.mark.parametrize("norm", ["gcn", "sage"])
+def test_conversion_after_a_normalisation_reuses_its_sort_and_stays_bit_exact(norm):
+    """gcn_norm / sage_norm sort the edge list by destination to sum the degrees; the cootocsc the
+    caller runs next on the same edges (examples/gcn_example.py:48-59) takes that order instead of
+    sorting again.  Result: the oracle's arrays bit for bit, whichever way it was produced."""
+    from jittorgeometric_amd.nn import gcn_norm, sage_norm
+    from jittorgeometric_amd.ops import cootocsc, cootocsr
+    rng = np.random.default_rng(31)
+    V, E = 5000, 90000
+    ei, _ = rand_graph(rng, V, E, 2)
+    ei_g, w_g = (gcn_norm if norm == "gcn" else sage_norm)(to_gpu(ei), None, V)
+    assert getattr(w_g, "_jgamd_order", None) is not None
+    ei_h, w_h = ei_g.cpu().numpy(), w_g.cpu().numpy()
+    want_c, want_r = oracle.cootocsc(ei_h, w_h, V), oracle.cootocsr(ei_h, w_h, V)
+
+    def same(holder, names, want):
+        for n, a in zip(names, want):
+            got = getattr(holder, n).cpu().numpy()
+            assert np.array_equal(got.view(np.int32), a.view(np.int32)), n
+    csc = cootocsc(ei_g, w_g, V)                      # takes the remembered order
+    assert getattr(w_g, "_jgamd_order", None) is None      # handed out once
+    same(csc, ("row_indices", "column_offset", "edge_weight"), want_c)
+    same(cootocsc(ei_g, w_g, V), ("row_indices", "column_offset", "edge_weight"), want_c)     # sorts
+    same(cootocsr(ei_g, w_g, V), ("column_indices", "row_offset", "edge_weight"), want_r)
+
+    # weights written in place after the normalisation, or another node count: the order is not used
+    ei2, w2 = (gcn_norm if norm == "gcn" else sage_norm)(to_gpu(ei), None, V)
+    w2.mul_(2.0)
+    same(cootocsc(ei2, w2, V), ("row_indices", "column_offset", "edge_weight"),
+         oracle.cootocsc(ei2.cpu().numpy(), w2.cpu().numpy(), V))
+    ei3, w3 = (gcn_norm if norm == "gcn" else sage_norm)(to_gpu(ei), None, V)
+    same(cootocsc(ei3, w3, V + 7), ("row_indices", "column_offset", "edge_weight"),
+         oracle.cootocsc(ei3.cpu().numpy(), w3.cpu().numpy(), V + 7))
+
+
+@pytest.mark.parametrize("V,E,extra,hubs", [(300, 5000, 40, 1), (4000, 90000, 0, 2), (1, 3000, 0, 0), (70000, 9000, 0, 0)])
+def test_weights_scaled_in_compressed_order_equal_the_conversion_of_scaled_weights(V, E, extra, hubs):
+    """jgamd_scale_csx_weights on the arrays of one conversion = the conversion of
+    jgamd_scale_edge_weights's result, bit for bit, slots of dropped edges (keys outside [0, V))
+    included; either factor array may be missing."""
+    from jittorgeometric_amd import _lib
+    from jittorgeometric_amd.ops.cootocsr import _convert
+    lib = _lib.load()
+    rng = np.random.default_rng(32 + V)
+    ei, w = rand_graph(rng, V + extra, E, hubs)          # with extra > 0 some destinations are outside [0, V)
+    ei_g, w_g = to_gpu(ei), to_gpu(w)
+    N = V + extra
+    a = to_gpu(rng.standard_normal(N).astype(np.float32))
+    b = to_gpu(rng.standard_normal(N).astype(np.float32))
+    idx, off, ws, _ = _convert(ei_g, w_g, V, 1)
+    for fa, fb in ((a, b), (None, b), (a, None)):
+        coo = torch.empty(E, device=dev())
+        _lib.check(lib.jgamd_scale_edge_weights(_lib.ptr(ei_g), _lib.ptr(w_g), _lib.ptr(fa), _lib.ptr(fb), E, N,
+                                                _lib.ptr(coo), _lib.stream_ptr(dev())))
+        want = _convert(ei_g, coo, V, 1)[2]
+        got = torch.full((E,), 7.0, device=dev())
+        nbytes = _lib.query(lib.jgamd_scale_csx_weights_workspace, E)
+        wsp = _lib.workspace(nbytes, dev())
+        _lib.check(lib.jgamd_scale_csx_weights(_lib.ptr(off), _lib.ptr(idx), _lib.ptr(ws), _lib.ptr(fa), _lib.ptr(fb), V, E,
+                                               N, _lib.ptr(got), _lib.ptr(wsp), nbytes, _lib.stream_ptr(dev())))
+        assert np.array_equal(got.cpu().numpy().view(np.int32), want.cpu().numpy().view(np.int32))
+    # and the COO form against numpy
+    ref = a.cpu().numpy()[ei[0]] * w * b.cpu().numpy()[ei[1]]
+    coo = torch.empty(E, device=dev())
+    _lib.check(lib.jgamd_scale_edge_weights(_lib.ptr(ei_g), _lib.ptr(w_g), _lib.ptr(a), _lib.ptr(b), E, N, _lib.ptr(coo),
+                                            _lib.stream_ptr(dev())))
+    assert np.array_equal(coo.cpu().numpy(), (a.cpu().numpy()[ei[0]] * w) * b.cpu().numpy()[ei[1]]) or \
+        np.allclose(coo.cpu().numpy(), ref, rtol=1e-6)
