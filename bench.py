@@ -631,18 +631,18 @@ def config5(b):
     x = torch.randn(V, 100, device=dev)
     y = torch.randint(0, 47, (V,), device=dev)
 
-    def model_step(layers, call, loss_fn=cross_entropy_loss):
+    def model_step(layers, call, loss_fn=cross_entropy_loss, relu_inside=False):
         for layer in layers:
             layer.zero_grad(set_to_none=True)
         hcur = x
         for i, layer in enumerate(layers):
             hcur = call(layer, hcur)
-            if i < 2:
+            if i < 2 and not relu_inside:
                 hcur = torch.relu(hcur)
         loss_fn(hcur, y).backward()
 
     main_only = args.part == "main"
-    gcn_ms = sage_ms = gcn_af_ms = sage_tf_ms = gcn_torch_loss_ms = 0.0
+    gcn_ms = sage_ms = gcn_af_ms = sage_tf_ms = gcn_torch_loss_ms = gcn_act_ms = sage_act_ms = 0.0
     if not main_only:
         gcn = [GCNConv(dims[i], dims[i + 1], spmm=False).to(dev) for i in range(3)]
         gcn_ms = b.timed(lambda: model_step(gcn, lambda l, t: l(t, csc, csr)), args.steps, args.warmup)
@@ -653,6 +653,10 @@ def config5(b):
         gcn_af = [GCNConv(dims[i], dims[i + 1], spmm=False, aggregate_first=dims[i] < dims[i + 1]).to(dev) for i in range(3)]
         gcn_af_ms = b.timed(lambda: model_step(gcn_af, lambda l, t: l(t, csc, csr)), args.steps, args.warmup)
         del gcn_af
+        # the same model with the activation applied in the product's row store (an option of this build's GCNConv)
+        gcn_act = [GCNConv(dims[i], dims[i + 1], spmm=False, activation="relu" if i < 2 else None).to(dev) for i in range(3)]
+        gcn_act_ms = b.timed(lambda: model_step(gcn_act, lambda l, t: l(t, csc, csr), relu_inside=True), args.steps, args.warmup)
+        del gcn_act
         from jittorgeometric_amd.nn import sage_norm
         sei, sw = sage_norm(ei[:, :E - V].contiguous(), None, V)       # same edges, mean weights
         sei = sei.contiguous()
@@ -662,7 +666,11 @@ def config5(b):
         sage_tf = [SAGEConv(dims[i], dims[i + 1], root_weight=False, spmm=False,
                             transform_first=dims[i + 1] < dims[i]).to(dev) for i in range(3)]
         sage_tf_ms = b.timed(lambda: model_step(sage_tf, lambda l, t: l(t, None, None, scsc, scsr)), args.steps, args.warmup)
-        del sei, sw, scsc, scsr, sage, gcn, sage_tf
+        sage_act = [SAGEConv(dims[i], dims[i + 1], root_weight=False, spmm=False,
+                             activation="relu" if i < 2 else None).to(dev) for i in range(3)]
+        sage_act_ms = b.timed(lambda: model_step(sage_act, lambda l, t: l(t, None, None, scsc, scsr), relu_inside=True),
+                              args.steps, args.warmup)
+        del sei, sw, scsc, scsr, sage, gcn, sage_tf, sage_act
     widths = (256,) if main_only else (100, 256, 47)
     prod = {}
     for F in widths:
@@ -681,6 +689,8 @@ def config5(b):
                  "gcn3_with_torch_cross_entropy_ms": round(gcn_torch_loss_ms, 3),
                  "sage3_fullgraph_fwd_bwd_ms": round(sage_ms, 3),
                  "gcn3_aggregate_first_where_narrower_ms": round(gcn_af_ms, 3),
+                 "gcn3_relu_in_row_store_ms": round(gcn_act_ms, 3),
+                 "sage3_relu_in_dense_store_ms": round(sage_act_ms, 3),
                  "sage3_transform_first_where_narrower_ms": round(sage_tf_ms, 3),
                  "coo_to_csr_ms": round(conv_csr_ms, 4), "coo_to_csr_edges_per_s": round(E / (conv_csr_ms * 1e-3)),
                  "coo_to_csc_edges_per_s": round(E / (conv_csc_ms * 1e-3))})
@@ -696,7 +706,7 @@ def config5(b):
         ms = prod[256][0]
         line.update({"metric": "spmm_f256_algorithmic_bandwidth", "value": round(spmm_bytes(V, E, 256) / (ms * 1e-3) / 1e9, 1),
                      "unit": "GB/s", "ms_per_step": round(ms, 4), "higher_is_better": True})
-        for k in ("loss", "gcn3_with_torch_cross_entropy_ms", "sage3_fullgraph_fwd_bwd_ms",
+        for k in ("loss", "gcn3_with_torch_cross_entropy_ms", "sage3_fullgraph_fwd_bwd_ms", "gcn3_relu_in_row_store_ms", "sage3_relu_in_dense_store_ms",
                   "gcn3_aggregate_first_where_narrower_ms", "sage3_transform_first_where_narrower_ms"):
             line.pop(k, None)
     return line, err

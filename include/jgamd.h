@@ -40,6 +40,9 @@ extern "C" {
 #define JGAMD_ERR_UNSUPPORTED (-4) /* shape outside what the kernels handle   */
 #define JGAMD_ERR_ALIGN (-5)       /* pointer not 4-byte aligned              */
 
+/* flag of the entry points that finish output rows: clamp the row at zero (ReLU) */
+#define JGAMD_ROW_RELU 1
+
 /* Library version, major*10000 + minor*100 + patch. */
 int32_t jgamd_version(void);
 /* Thread-local text of the last error returned on this thread ("" if none). */
@@ -176,14 +179,18 @@ int32_t jgamd_csx_plan_counts(const void *plan, int32_t *n_fix, int32_t *n_grp, 
  * NULL, not both; rows of 1, 2, 4 or 8 floats use `tiles` when it is given,
  * every other width needs `plan`).  beta = 1, alpha = 0 or h = NULL is the
  * plain product of AggregateOp::jit_run (ops/cpp/aggregate_op.cc:26-71).
+ * flags: JGAMD_ROW_RELU clamps every finished row at zero in the row store,
+ * out = max(0, beta * A x + alpha * h): the activation the reference's models
+ * apply in a pass of their own after the layer (examples/gcn_example.py:84-90).
  * The workspace holds row pieces only (jgamd_spmm_csx_planned_workspace).
  */
 int32_t jgamd_spmm_csx_planned_workspace(int32_t R, int64_t E, int32_t F, size_t *bytes);
 int32_t jgamd_spmm_csx_planned(const void *plan, const void *tiles, int32_t n_fix, int32_t n_grp,
                                const int32_t *off, const int32_t *idx, const float *w,
                                const float *x, float *out, float beta, float alpha,
-                               const float *h, int32_t h_rows, int32_t R, int32_t C, int64_t E,
-                               int32_t F, void *ws, size_t ws_bytes, void *stream);
+                               const float *h, int32_t h_rows, int32_t flags, int32_t R,
+                               int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes,
+                               void *stream);
 
 /* jgamd_spmm_csx without a workspace argument.  No counterpart in the
  * reference: it is for callers that cannot allocate device memory or own a
@@ -361,12 +368,14 @@ int32_t jgamd_spmm_csx_blocked_timed(const int32_t *b_off, const int32_t *b_idx,
  * and N must be multiples of 4 with K1 + K2 <= 256 (jgamd_dense_rows_supported
  * returns 1 for such a shape, else 0; other shapes stay with the BLAS
  * library); x1, x2, out and bias 16-byte aligned.  K2 = 0 leaves out the
- * second product, bias = NULL the added row.  Needs no workspace.
+ * second product, bias = NULL the added row.  flags: JGAMD_ROW_RELU clamps
+ * the result at zero in the store (see jgamd_spmm_csx_planned).  Needs no
+ * workspace.
  */
 int32_t jgamd_dense_rows_supported(int32_t K1, int32_t K2, int32_t N);
 int32_t jgamd_dense_rows(const float *x1, const float *w1, int32_t K1, const float *x2,
                          const float *w2, int32_t K2, const float *bias, float *out, int32_t V,
-                         int32_t N, void *stream);
+                         int32_t N, int32_t flags, void *stream);
 
 /* ------------------------------------------------------------------------
  * Column sums of a row-major [R,F] matrix: out[f] = sum_r x[r,f].  The bias
@@ -377,6 +386,19 @@ int32_t jgamd_dense_rows(const float *x1, const float *w1, int32_t K1, const flo
 int32_t jgamd_column_sum_workspace(int64_t R, int32_t F, size_t *bytes);
 int32_t jgamd_column_sum(const float *x, float *out, int64_t R, int32_t F, void *ws,
                          size_t ws_bytes, void *stream);
+
+/* The gradient in front of a ReLU and its column sums in one pass:
+ *   masked[r,c] = y[r,c] > 0 ? g[r,c] : 0,   out[c] = sum_r masked[r,c]
+ * for the upstream gradient g and the ReLU's output y, both [R,F]; masked must
+ * not be g.  Together with JGAMD_ROW_RELU this is the backward of a layer whose
+ * activation was applied in the product's row store: the bias gradient reads
+ * the upstream gradient anyway (nn/conv/gcn_conv.py:109-110 adds the bias,
+ * examples/gcn_example.py:84-90 applies relu after the layer).  Same workspace
+ * as jgamd_column_sum.
+ */
+int32_t jgamd_relu_backward_column_sum(const float *g, const float *y, float *masked, float *out,
+                                       int64_t R, int32_t F, void *ws, size_t ws_bytes,
+                                       void *stream);
 
 /* ------------------------------------------------------------------------
  * Mean cross-entropy of row-major logits [V,C] against integer labels, the

@@ -38,8 +38,8 @@ SIGNATURES = {
     "jgamd_csx_plan": [_P, _I32, _I64, _I32, _P, _c.c_size_t, _P],
     "jgamd_csx_plan_counts": [_P, _c.POINTER(_I32), _c.POINTER(_I32), _P],
     "jgamd_spmm_csx_planned_workspace": [_I32, _I64, _I32, _SZP],
-    "jgamd_spmm_csx_planned": [_P, _P, _I32, _I32, _P, _P, _P, _P, _P, _F32, _F32, _P, _I32, _I32, _I32, _I64, _I32,
-                               _P, _c.c_size_t, _P],
+    "jgamd_spmm_csx_planned": [_P, _P, _I32, _I32, _P, _P, _P, _P, _P, _F32, _F32, _P, _I32, _I32, _I32, _I32, _I64,
+                               _I32, _P, _c.c_size_t, _P],
     "jgamd_spmm_block_plan": [_I32, _I32, _I64, _I32, _c.POINTER(_I32), _c.POINTER(_I32)],
     "jgamd_csx_block_columns_workspace": [_I32, _I32, _SZP],
     "jgamd_csx_block_columns": [_P, _P, _P, _I32, _I64, _I32, _I32, _P, _P, _P, _P, _c.c_size_t, _P],
@@ -57,9 +57,10 @@ SIGNATURES = {
     "jgamd_edge_softmax_bwd_planned": [_P, _P, _P, _P, _P, _I32, _I64, _I32, _P, _c.c_size_t, _P],
     "jgamd_scatter_to_edge": [_P, _P, _P, _P, _I32, _I64, _I32, _I32, _P],
     "jgamd_dense_rows_supported": [_I32, _I32, _I32],
-    "jgamd_dense_rows": [_P, _P, _I32, _P, _P, _I32, _P, _P, _I32, _I32, _P],
+    "jgamd_dense_rows": [_P, _P, _I32, _P, _P, _I32, _P, _P, _I32, _I32, _I32, _P],
     "jgamd_column_sum_workspace": [_I64, _I32, _SZP],
     "jgamd_column_sum": [_P, _P, _I64, _I32, _P, _c.c_size_t, _P],
+    "jgamd_relu_backward_column_sum": [_P, _P, _P, _P, _I64, _I32, _P, _c.c_size_t, _P],
     "jgamd_cross_entropy_workspace": [_I64, _I32, _SZP],
     "jgamd_cross_entropy_fwd": [_P, _P, _I32, _I32, _I64, _I32, _P, _P, _P, _P, _c.c_size_t, _P],
     "jgamd_cross_entropy_bwd": [_P, _P, _I32, _P, _P, _P, _I64, _I32, _P, _P],

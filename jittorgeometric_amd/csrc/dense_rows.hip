@@ -45,6 +45,7 @@ struct DenseArgs {
     const float *bias;         // [N] or NULL
     float *out;                // [V,N]
     int V, K1, K2, N;
+    int relu;                  // the result is clamped at zero (a layer's activation in the store)
 };
 
 // KQ = 16-float steps held in registers (K1 + K2 <= 16 * KQ); WAVES per workgroup
@@ -143,12 +144,17 @@ __global__ __launch_bounds__(WAVES *kWave) void dense_rows(DenseArgs a)
             const int row = tile * kDenseRows + 4 * kg + r;
             if (row < a.V) {
                 float *dst = a.out + (size_t)row * a.N;
-                if (cl < a.N)
-                    __builtin_nontemporal_store(f32x4{acc[0][r] + bl[0], acc[1][r] + bl[1], acc[2][r] + bl[2], acc[3][r] + bl[3]},
-                                                reinterpret_cast<f32x4 *>(dst + cl));
-                if (ch < a.N)
-                    __builtin_nontemporal_store(f32x4{acc[4][r] + bh[0], acc[5][r] + bh[1], acc[6][r] + bh[2], acc[7][r] + bh[3]},
-                                                reinterpret_cast<f32x4 *>(dst + ch));
+                f32x4 lo4 = {acc[0][r] + bl[0], acc[1][r] + bl[1], acc[2][r] + bl[2], acc[3][r] + bl[3]};
+                f32x4 hi4 = {acc[4][r] + bh[0], acc[5][r] + bh[1], acc[6][r] + bh[2], acc[7][r] + bh[3]};
+                if (a.relu) {
+#pragma unroll
+                    for (int c = 0; c < 4; c++) {
+                        lo4[c] = fmaxf(lo4[c], 0.f);
+                        hi4[c] = fmaxf(hi4[c], 0.f);
+                    }
+                }
+                if (cl < a.N) __builtin_nontemporal_store(lo4, reinterpret_cast<f32x4 *>(dst + cl));
+                if (ch < a.N) __builtin_nontemporal_store(hi4, reinterpret_cast<f32x4 *>(dst + ch));
             }
         }
     }
@@ -187,9 +193,10 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_dense_rows_suppo
 extern "C" __attribute__((visibility("default"))) int32_t jgamd_dense_rows(const float *x1, const float *w1, int32_t K1,
                                                                            const float *x2, const float *w2, int32_t K2,
                                                                            const float *bias, float *out, int32_t V,
-                                                                           int32_t N, void *stream)
+                                                                           int32_t N, int32_t flags, void *stream)
 {
     if (V < 0) return fail(JGAMD_ERR_SIZE, "dense_rows: negative V");
+    if (flags & ~JGAMD_ROW_RELU) return fail(JGAMD_ERR_SIZE, "dense_rows: unknown flags %d", flags);
     if (!jgamd_dense_rows_supported(K1, K2, N))
         return fail(JGAMD_ERR_UNSUPPORTED, "dense_rows: K1=%d K2=%d N=%d (multiples of 4, K1 + K2 <= %d)", K1, K2, N,
                     kDenseMaxK);
@@ -198,7 +205,8 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_dense_rows(const
     if ((((uintptr_t)x1 | (uintptr_t)x2 | (uintptr_t)out | (uintptr_t)bias) & 15) != 0 ||
         (((uintptr_t)w1 | (uintptr_t)w2) & 3) != 0)
         return fail(JGAMD_ERR_ALIGN, "dense_rows: x / out / bias must be 16-byte aligned");
-    const DenseArgs a{x1, K2 > 0 ? x2 : nullptr, w1, K2 > 0 ? w2 : nullptr, bias, out, V, K1, K2 > 0 ? K2 : 0, N};
+    const DenseArgs a{x1, K2 > 0 ? x2 : nullptr, w1, K2 > 0 ? w2 : nullptr, bias, out, V, K1, K2 > 0 ? K2 : 0, N,
+                      (flags & JGAMD_ROW_RELU) ? 1 : 0};
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int K = a.K1 + a.K2;
     if (K <= 64) launch_dense<4, 8>(a, s);

@@ -79,6 +79,7 @@ struct RowFinish {
     const float *h;
     int h_stride;   // floats between the rows of h: F, or 0 when one row serves every output row
     int x_stride;   // floats between the rows of x when they are padded apart; 0 = F
+    int relu;       // the finished row is clamped at zero (a layer's activation in the row store)
 };
 
 template <int VEC, int NT, int UNROLL, bool WIDE, bool LDS, bool EPI>
@@ -161,7 +162,10 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_merge(const int32_t *__rest
 #pragma unroll
                 for (int t = 0; t < NT; t++)
 #pragma unroll
-                    for (int v = 0; v < VEC; v++) acc[t][v] = fmaf(fin.alpha, hrow[t][v], fin.beta * acc[t][v]);
+                    for (int v = 0; v < VEC; v++) {
+                        acc[t][v] = fmaf(fin.alpha, hrow[t][v], fin.beta * acc[t][v]);
+                        if (fin.relu) acc[t][v] = fmaxf(acc[t][v], 0.f);
+                    }
             }
         }
 #pragma unroll
@@ -410,6 +414,12 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_fixup(const int32_t *__rest
                     for (int v = 0; v < VEC; v++) acc[t][v] = fmaf(fin.alpha, hv[t][v], acc[t][v]);
                 }
             }
+            if (fin.relu) {
+#pragma unroll
+                for (int t = 0; t < NT; t++)
+#pragma unroll
+                    for (int v = 0; v < VEC; v++) acc[t][v] = fmaxf(acc[t][v], 0.f);
+            }
         }
 #pragma unroll
         for (int t = 0; t < NT; t++)
@@ -420,10 +430,13 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_fixup(const int32_t *__rest
 // out = beta * out + alpha * h, element-wise (the finish as a pass of its own, for the
 // shapes the fused kernels do not cover).
 __global__ void spmm_finish_rows(float *__restrict__ out, const float *__restrict__ h, int64_t n, int F,
-                                 int h_stride, float beta, float alpha)
+                                 int h_stride, float beta, float alpha, int relu)
 {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) out[i] = fmaf(alpha, h ? h[h_stride ? i : i % F] : 0.f, beta * out[i]);
+    if (i < n) {
+        const float v = fmaf(alpha, h ? h[h_stride ? i : i % F] : 0.f, beta * out[i]);
+        out[i] = relu ? fmaxf(v, 0.f) : v;
+    }
 }
 
 // ------------------------------------------------------------------ host ---
@@ -526,7 +539,7 @@ static void launch_spmm(const SpmmShape &s, const int32_t *off, const int32_t *i
     const bool narrow = (uint64_t)C * (uint64_t)(x_stride ? x_stride : F) * 4u < ((uint64_t)1 << 32);
     // the fused row finish exists for 32-bit offsets only; wide shapes finish in a pass of their own
     const bool fused = fin && narrow;
-    const RowFinish none{1.f, 0.f, nullptr, 0, 0};
+    const RowFinish none{1.f, 0.f, nullptr, 0, 0, 0};
     RowFinish f = fused ? *fin : none;
     f.x_stride = x_stride;
 #define JG_GO(W, L, P)                                                                                              \
@@ -562,7 +575,7 @@ static void launch_spmm(const SpmmShape &s, const int32_t *off, const int32_t *i
     if (fin && !fused) {
         const int64_t n = (int64_t)R * F;
         hipLaunchKernelGGL(spmm_finish_rows, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, st, out, fin->h, n, F,
-                           fin->h_stride, fin->beta, fin->alpha);
+                           fin->h_stride, fin->beta, fin->alpha, fin->relu);
     }
 }
 
@@ -673,7 +686,7 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_axpby(
     if (h && (((uintptr_t)h & 3) != 0)) return fail(JGAMD_ERR_ALIGN, "spmm_csx_axpby: h not 4-byte aligned");
     if (h && h_rows != 1 && h_rows != R)
         return fail(JGAMD_ERR_SIZE, "spmm_csx_axpby: h has %d rows, expected %d or 1", h_rows, R);
-    const RowFinish fin{beta, alpha, alpha != 0.f ? h : nullptr, h_rows == 1 ? 0 : F, 0};
+    const RowFinish fin{beta, alpha, alpha != 0.f ? h : nullptr, h_rows == 1 ? 0 : F, 0, 0};
     return spmm_call(off, idx, w, x, out, R, C, E, F, ws, ws_bytes, stream, nullptr, nullptr, &fin);
 }
 
@@ -681,9 +694,10 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_axpby(
 // starts, and the piece kernels run over the plan's lists only.
 extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_planned(
     const void *plan, const void *tiles, int32_t n_fix, int32_t n_grp, const int32_t *off, const int32_t *idx,
-    const float *w, const float *x, float *out, float beta, float alpha, const float *h, int32_t h_rows, int32_t R,
-    int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, void *stream)
+    const float *w, const float *x, float *out, float beta, float alpha, const float *h, int32_t h_rows,
+    int32_t flags, int32_t R, int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, void *stream)
 {
+    if (flags & ~JGAMD_ROW_RELU) return fail(JGAMD_ERR_SIZE, "spmm_csx_planned: unknown flags %d", flags);
     if (!plan && !tiles) return fail(JGAMD_ERR_NULL, "spmm_csx_planned: plan and tiles are both NULL");
     if (!plan && !narrow_width(F))
         return fail(JGAMD_ERR_NULL, "spmm_csx_planned: rows of %d floats need the chunk plan, not the tile plan", F);
@@ -695,8 +709,8 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_planned
     PlanHints hints;
     hints.n_fix = n_fix < 0 ? -1 : n_fix;
     hints.n_grp = n_grp < 0 ? -1 : n_grp;
-    const bool plain = beta == 1.f && (alpha == 0.f || !h);
-    const RowFinish fin{beta, alpha, alpha != 0.f ? h : nullptr, h_rows == 1 ? 0 : F, 0};
+    const bool plain = beta == 1.f && (alpha == 0.f || !h) && flags == 0;
+    const RowFinish fin{beta, alpha, alpha != 0.f ? h : nullptr, h_rows == 1 ? 0 : F, 0, (flags & JGAMD_ROW_RELU) ? 1 : 0};
     return spmm_call(off, idx, w, x, out, R, C, E, F, ws, ws_bytes, stream, nullptr, nullptr, plain ? nullptr : &fin,
                      false, 0, plan, tiles, hints);
 }

@@ -9,7 +9,7 @@ from ...ops.propagate import aggregate_bias
 from ...utils import add_remaining_self_loops
 from ...utils.num_nodes import maybe_num_nodes
 from ...ops._common import both_orders, spmm, spmm_axpby
-from ..dense import add_bias, column_sum, rows_times, xt_g, xw
+from ..dense import add_bias, column_sum, relu_backward_column_sum, rows_times, xt_g, xw
 from ..inits import glorot, zeros
 
 
@@ -93,23 +93,36 @@ class GcnLayerFunc(torch.autograd.Function):
     the product over the graph at the narrower input width."""
 
     @staticmethod
-    def forward(ctx, x, weight, bias, fwd, bwd):
+    def forward(ctx, x, weight, bias, fwd, bwd, relu=False):
         h = rows_times(x, weight)
-        if bias is not None:
-            out = spmm_axpby(fwd[0], fwd[1], fwd[2], h, x.shape[0], 1.0, 1.0, bias)
+        if bias is not None or relu:
+            out = spmm_axpby(fwd[0], fwd[1], fwd[2], h, x.shape[0], 1.0, 1.0, bias, relu)
         else:
             out = spmm(fwd[0], fwd[1], fwd[2], h, x.shape[0])
-        ctx.fwd, ctx.bwd = fwd, bwd
-        ctx.save_for_backward(x, weight)
+        ctx.fwd, ctx.bwd, ctx.relu = fwd, bwd, relu
+        if relu:
+            ctx.save_for_backward(x, weight, out)       # the mask of the activation is the output's sign
+        else:
+            ctx.save_for_backward(x, weight)
         return out
 
     @staticmethod
     def backward(ctx, g):
-        x, weight = ctx.saved_tensors
+        x, weight = ctx.saved_tensors[:2]
         g = g.contiguous()
         need_x, need_w, need_b = ctx.needs_input_grad[:3]
         gx = gw = gb = None
-        if need_b:
+        if ctx.relu:
+            # the gradient in front of the activation and the bias gradient in one pass over g
+            out = ctx.saved_tensors[2]
+            if g.dtype == torch.float32:
+                g, gb = relu_backward_column_sum(g, out)
+            else:
+                g = g * (out > 0)
+                gb = g.sum(0)
+            if not need_b:
+                gb = None
+        elif need_b:
             gb = column_sum(g) if g.dtype == torch.float32 else g.sum(0)
         f_in, f_out = weight.shape
         if need_x or (need_w and f_out <= f_in):
@@ -122,7 +135,7 @@ class GcnLayerFunc(torch.autograd.Function):
         elif need_w:
             off, idx, w = ctx.fwd
             gw = xt_g(spmm(off, idx, w, x, x.shape[0]), g)
-        return gx, gw, gb, None, None
+        return gx, gw, gb, None, None, None
 
 
 class GCNConv(nn.Module):
@@ -134,10 +147,20 @@ class GCNConv(nn.Module):
     expression as (A_hat x) W + b: the product over the graph then runs at the input
     width, which is the cheaper order when in_channels < out_channels (100 -> 256:
     half the gathered bytes); the dense product takes the bias in its own pass.  The
-    two orders differ in rounding only."""
+    two orders differ in rounding only.
 
-    def __init__(self, in_channels, out_channels, bias=True, spmm=True, aggregate_first=False, **kwargs):
+    `activation="relu"` (not in the reference, off by default) returns relu(A_hat (x W) + b) with the
+    clamp applied in the product's row store and, in the backward pass, the activation's mask
+    applied in the pass that sums the bias gradient: what examples/gcn_example.py:84-90 writes as
+    `x = nn.relu(self.conv1(x, csc, csr))`, without the two passes over [V,F] of a separate
+    activation.  Same values as relu(layer(x))."""
+
+    def __init__(self, in_channels, out_channels, bias=True, spmm=True, aggregate_first=False, activation=None,
+                 **kwargs):
         super().__init__()
+        if activation not in (None, "relu"):
+            raise ValueError("activation must be None or 'relu', got %r" % (activation,))
+        self.activation = activation
         self.aggregate_first = bool(aggregate_first)
         self.in_channels = in_channels
         self.out_channels = out_channels
@@ -151,6 +174,18 @@ class GCNConv(nn.Module):
         zeros(self.bias)
 
     def forward(self, x, csc, csr):
+        if self.activation == "relu" and self._fused_route(x):
+            fwd, bwd = both_orders(None if self.spmm and csr is not None else csc, csr)
+            return GcnLayerFunc.apply(x.to(torch.float32).contiguous(), self.weight, self.bias, fwd, bwd, True)
+        out = self._layer(x, csc, csr)
+        return torch.relu(out) if self.activation == "relu" else out
+
+    def _fused_route(self, x):
+        """The layer runs as one autograd node (dense kernel, product with the bias in its row store)."""
+        return (not self.aggregate_first and x.dim() == 2 and x.is_floating_point()
+                and not (self.spmm and _spmmcsr.REFERENCE_GRAD))
+
+    def _layer(self, x, csc, csr):
         if x.is_floating_point() and x.dtype != torch.float32:
             x = x.to(torch.float32)      # the kernels and the parameters are float32; other widths are narrowed
         if self.aggregate_first and x.dim() == 2:
@@ -159,7 +194,7 @@ class GCNConv(nn.Module):
         if x.dim() == 2 and x.dtype == torch.float32 and not (self.spmm and _spmmcsr.REFERENCE_GRAD):
             # spmm=True only needs the CSR (:96-97); both routes give the same product
             fwd, bwd = both_orders(None if self.spmm and csr is not None else csc, csr)
-            return GcnLayerFunc.apply(x.contiguous(), self.weight, self.bias, fwd, bwd)
+            return GcnLayerFunc.apply(x.contiguous(), self.weight, self.bias, fwd, bwd, False)
         x = xw(x, self.weight)
         if self.bias is not None and x.dim() == 2 and not (self.spmm and _spmmcsr.REFERENCE_GRAD):
             # product and bias in one kernel; spmm=True only needs the CSR (:96-97)

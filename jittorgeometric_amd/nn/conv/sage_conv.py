@@ -6,7 +6,7 @@ from torch import nn
 from ...ops import SpmmCsr, aggregateWithWeight, cootocsc, cootocsr
 from ...ops import spmmcsr as _spmmcsr
 from ...ops._common import both_orders, spmm, spmm_axpby
-from ..dense import add_bias, column_sum, rows_times, xt_g, xw
+from ..dense import add_bias, column_sum, relu_backward_column_sum, rows_times, xt_g, xw
 from ..inits import glorot, zeros
 from .gcn_conv import _degree_norm, _normalised, _scale
 
@@ -24,20 +24,32 @@ class SageLayerFunc(torch.autograd.Function):
     store, so no pass over a [V,F] array only adds two arrays."""
 
     @staticmethod
-    def forward(ctx, x, w1, w_root, bias, fwd, bwd):
+    def forward(ctx, x, w1, w_root, bias, fwd, bwd, relu=False):
         agg = spmm(fwd[0], fwd[1], fwd[2], x, x.shape[0])
-        out = rows_times(agg, w1, x if w_root is not None else None, w_root, bias)
-        ctx.bwd = bwd
-        ctx.save_for_backward(x, agg, w1, w_root)
+        out = rows_times(agg, w1, x if w_root is not None else None, w_root, bias, relu)
+        ctx.bwd, ctx.relu = bwd, relu
+        if relu:
+            ctx.save_for_backward(x, agg, w1, w_root, out)      # the activation's mask is the output's sign
+        else:
+            ctx.save_for_backward(x, agg, w1, w_root)
         return out
 
     @staticmethod
     def backward(ctx, g):
-        x, agg, w1, w_root = ctx.saved_tensors
+        x, agg, w1, w_root = ctx.saved_tensors[:4]
         g = g.contiguous()
         need_x, need_w1, need_root, need_b = ctx.needs_input_grad[:4]
         gx = gw1 = groot = gb = None
-        if need_b:
+        if ctx.relu:
+            out = ctx.saved_tensors[4]
+            if g.dtype == torch.float32:
+                g, gb = relu_backward_column_sum(g, out)          # mask and bias gradient in one pass
+            else:
+                g = g * (out > 0)
+                gb = g.sum(0)
+            if not need_b:
+                gb = None
+        elif need_b:
             gb = column_sum(g) if g.dtype == torch.float32 else g.sum(0)
         if need_w1:
             gw1 = xt_g(agg, g)
@@ -60,7 +72,7 @@ class SageLayerFunc(torch.autograd.Function):
                     gx = spmm_axpby(off, idx, w, g_agg, g.shape[0], 1.0, 1.0, rows_times(g, w_root.t().contiguous()))
                 else:
                     gx = spmm(off, idx, w, g_agg, g.shape[0])
-        return gx, gw1, groot, gb, None, None
+        return gx, gw1, groot, gb, None, None, None
 
 
 class SageTransformFirstFunc(torch.autograd.Function):
@@ -114,8 +126,14 @@ class SAGEConv(nn.Module):
 
     def __init__(self, in_channels, out_channels, improved=False, cached=False, add_self_loops=True,
                  normalize=True, project=False, root_weight=True, bias=True, spmm=True, transform_first=False,
-                 **kwargs):
+                 activation=None, **kwargs):
         super().__init__()
+        if activation not in (None, "relu"):
+            raise ValueError("activation must be None or 'relu', got %r" % (activation,))
+        # not in the reference, off by default: relu(layer(x)) with the clamp in the dense kernel's store
+        # and the mask applied in the pass that sums the bias gradient (examples/sage_example.py applies
+        # the activation in a pass of its own after the layer)
+        self.activation = activation
         self.transform_first = bool(transform_first)      # not in the reference: see SageTransformFirstFunc
         self.in_channels = in_channels
         self.out_channels = out_channels
@@ -147,6 +165,11 @@ class SAGEConv(nn.Module):
         self._cached_edge_index = None
 
     def forward(self, x, edge_index=None, edge_weight=None, csc=None, csr=None):
+        out, activated = self._layer(x, edge_index, edge_weight, csc, csr)
+        return torch.relu(out) if self.activation == "relu" and not activated else out
+
+    def _layer(self, x, edge_index, edge_weight, csc, csr):
+        """(output, whether the activation has been applied already)."""
         if x.is_floating_point() and x.dtype != torch.float32:
             x = x.to(torch.float32)      # the kernels and the parameters are float32; other widths are narrowed
         if csc is None or csr is None:
@@ -166,8 +189,11 @@ class SAGEConv(nn.Module):
         if self.weight_proj is None and x.dim() == 2 and x.dtype == torch.float32 and not reference_grad:
             # spmm=True only needs the CSR arrays (:183-184); both routes give the same product
             fwd, bwd = both_orders(None if self.spmm and csr is not None else csc, csr)
-            func = SageTransformFirstFunc if self.transform_first else SageLayerFunc
-            return func.apply(x.contiguous(), self.weight1, self.root_weight, self.bias, fwd, bwd)
+            if self.transform_first:
+                return SageTransformFirstFunc.apply(x.contiguous(), self.weight1, self.root_weight, self.bias, fwd,
+                                                    bwd), False
+            fused = self.activation == "relu"
+            return SageLayerFunc.apply(x.contiguous(), self.weight1, self.root_weight, self.bias, fwd, bwd, fused), fused
         xs = (x, x)
         if self.weight_proj is not None:
             xs = (torch.relu(xs[0] @ self.weight_proj + self.bias_proj), xs[1])
@@ -180,7 +206,7 @@ class SAGEConv(nn.Module):
             out = out + xw(xs[1], self.root_weight)
         if self.bias is not None:
             out = add_bias(out, self.bias)
-        return out
+        return out, False
 
     execute = forward
 

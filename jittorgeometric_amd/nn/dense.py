@@ -17,9 +17,10 @@ def _plain(t):
     return t.dtype == torch.float32 and t.is_cuda and t.dim() == 2 and t.is_contiguous() and t.data_ptr() % 16 == 0
 
 
-def rows_times(x1, w1, x2=None, w2=None, bias=None):
-    """x1 @ w1 (+ x2 @ w2) (+ bias) in one pass over the rows: the library's matrix-core kernel
-    (csrc/dense_rows.hip) for the shapes it covers, torch's BLAS products otherwise."""
+def rows_times(x1, w1, x2=None, w2=None, bias=None, relu=False):
+    """x1 @ w1 (+ x2 @ w2) (+ bias), clamped at zero with relu, in one pass over the rows: the
+    library's matrix-core kernel (csrc/dense_rows.hip) for the shapes it covers, torch's BLAS
+    products otherwise."""
     from .. import _lib
     two = x2 is not None
     K1, N = w1.shape
@@ -34,7 +35,8 @@ def rows_times(x1, w1, x2=None, w2=None, bias=None):
         ok = bool(lib.jgamd_dense_rows_supported(K1, K2, N))
     if not ok:
         out = torch.addmm(bias, x1, w1) if bias is not None else x1 @ w1
-        return out.addmm_(x2, w2) if two else out
+        out = out.addmm_(x2, w2) if two else out
+        return out.relu_() if relu else out
     dev = _lib.require_gpu(x1, w1, x2, w2, bias)
     w1 = w1.contiguous()
     w2 = w2.contiguous() if two else None
@@ -43,7 +45,7 @@ def rows_times(x1, w1, x2=None, w2=None, bias=None):
         bias = bias.clone()
     out = torch.empty((x1.shape[0], N), dtype=torch.float32, device=dev)
     _lib.check(lib.jgamd_dense_rows(_lib.ptr(x1), _lib.ptr(w1), K1, _lib.ptr(x2), _lib.ptr(w2), K2, _lib.ptr(bias),
-                                    _lib.ptr(out), x1.shape[0], N, _lib.stream_ptr(dev)))
+                                    _lib.ptr(out), x1.shape[0], N, 1 if relu else 0, _lib.stream_ptr(dev)))
     return out
 
 
@@ -101,6 +103,22 @@ def column_sum(x):
     ws = _lib.workspace(nbytes, dev)
     _lib.check(lib.jgamd_column_sum(_lib.ptr(x), _lib.ptr(out), R, F, _lib.ptr(ws), nbytes, _lib.stream_ptr(dev)))
     return out
+
+
+def relu_backward_column_sum(g, y):
+    """(g where y > 0 else 0, its sum over rows) for the upstream gradient g and a ReLU's output y,
+    both contiguous [R,F] float32 GPU tensors, in one pass (csrc/dense_ops.hip)."""
+    from .. import _lib
+    lib = _lib.load()
+    dev = _lib.require_gpu(g, y)
+    R, F = g.shape
+    masked = torch.empty_like(g)
+    out = torch.empty(F, dtype=torch.float32, device=dev)
+    nbytes = _lib.query(lib.jgamd_column_sum_workspace, R, F)
+    ws = _lib.workspace(nbytes, dev)
+    _lib.check(lib.jgamd_relu_backward_column_sum(_lib.ptr(g), _lib.ptr(y), _lib.ptr(masked), _lib.ptr(out), R, F,
+                                                  _lib.ptr(ws), nbytes, _lib.stream_ptr(dev)))
+    return masked, out
 
 
 class _AddBias(torch.autograd.Function):

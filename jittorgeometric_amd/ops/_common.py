@@ -184,8 +184,9 @@ def _blocked_arrays(off, idx, w, R, E, nb, cols):
     return b_off, b_idx, b_w
 
 
-def _product(off, idx, w, x, R, beta, alpha, h):
-    """beta * (A x) + alpha * h through the plain or the column-blocked kernels."""
+def _product(off, idx, w, x, R, beta, alpha, h, relu=False):
+    """beta * (A x) + alpha * h through the plain or the column-blocked kernels; with relu the
+    result is clamped at zero, in the product's row store where the kernels offer it."""
     lib = _lib.load()
     dev = _lib.require_gpu(off, x, idx, w, h)
     x = as_f32(x, "x")
@@ -213,7 +214,7 @@ def _product(off, idx, w, x, R, beta, alpha, h):
         _lib.check(lib.jgamd_spmm_csx_blocked(_lib.ptr(b_off), _lib.ptr(b_idx), _lib.ptr(b_w), _lib.ptr(x), _lib.ptr(out),
                                               float(beta), float(alpha), _lib.ptr(h), h_rows, R, C, E, F, nb.value,
                                               _lib.ptr(ws), nbytes, stream))
-        return out
+        return out.relu_() if relu else out
     # the partition of the rows is kept with the offsets: the chunk plan, or the tile plan for
     # rows of 1, 2, 4 or 8 floats
     narrow = F in (1, 2, 4, 8) and E > 0
@@ -223,8 +224,8 @@ def _product(off, idx, w, x, R, beta, alpha, h):
         ws = _lib.workspace(nbytes, dev)
         _lib.check(lib.jgamd_spmm_csx_planned(None if narrow else _lib.ptr(plan), _lib.ptr(plan) if narrow else None,
                                               n_fix, n_grp, _lib.ptr(off), _lib.ptr(idx), _lib.ptr(w), _lib.ptr(x),
-                                              _lib.ptr(out), float(beta), float(alpha), _lib.ptr(h), h_rows, R, C, E,
-                                              F, _lib.ptr(ws), nbytes, stream))
+                                              _lib.ptr(out), float(beta), float(alpha), _lib.ptr(h), h_rows,
+                                              1 if relu else 0, R, C, E, F, _lib.ptr(ws), nbytes, stream))
         return out
     nbytes = _lib.query(lib.jgamd_spmm_csx_workspace, R, E, F)
     ws = _lib.workspace(nbytes, dev)
@@ -235,7 +236,7 @@ def _product(off, idx, w, x, R, beta, alpha, h):
         _lib.check(lib.jgamd_spmm_csx_axpby(_lib.ptr(off), _lib.ptr(idx), _lib.ptr(w), _lib.ptr(x), _lib.ptr(out),
                                             float(beta), float(alpha), _lib.ptr(h), h_rows, R, C, E, F, _lib.ptr(ws),
                                             nbytes, stream))
-    return out
+    return out.relu_() if relu else out
 
 
 def spmm(off, idx, w, x, R):
@@ -243,10 +244,10 @@ def spmm(off, idx, w, x, R):
     return _product(off, idx, w, x, R, 1.0, 0.0, None)
 
 
-def spmm_axpby(off, idx, w, x, R, beta, alpha, h):
+def spmm_axpby(off, idx, w, x, R, beta, alpha, h, relu=False):
     """out[r,:] = beta * sum_j w[j] * x[idx[j],:] + alpha * h[r,:]; h is [R,F], or [F] / [1,F]
-    for one row added to every output row, or None."""
-    return _product(off, idx, w, x, R, beta, alpha, h)
+    for one row added to every output row, or None.  relu clamps the result at zero."""
+    return _product(off, idx, w, x, R, beta, alpha, h, relu)
 
 
 def both_orders(csc, csr):

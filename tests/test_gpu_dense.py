@@ -57,7 +57,7 @@ def test_rows_past_the_inputs_are_not_touched_and_special_values_stay_in_their_r
     x[17, 99] = float("nan")
     w = torch.randn((K, N), device=dev(), generator=gen)
     buf = torch.full((V + 16, N), 7.0, device=dev())
-    L.check(l.jgamd_dense_rows(L.ptr(x), L.ptr(w), K, None, None, 0, None, L.ptr(buf), V, N, L.stream_ptr(dev())))
+    L.check(l.jgamd_dense_rows(L.ptr(x), L.ptr(w), K, None, None, 0, None, L.ptr(buf), V, N, 0, L.stream_ptr(dev())))
     out = buf.cpu().numpy()
     assert (out[V:] == 7.0).all()
     finite = np.isfinite(out[:V]).all(axis=1)
@@ -78,7 +78,7 @@ def test_shapes_outside_the_kernel_fall_back_and_are_refused_by_the_entry_point(
     assert_close(rows_times(x, w, bias=b).cpu().numpy(), ref, scale, what="BLAS route")
     out = torch.empty((5000, 41), device=dev())
     with pytest.raises(JgamdError):
-        L.check(l.jgamd_dense_rows(L.ptr(x), L.ptr(w), 47, None, None, 0, None, L.ptr(out), 5000, 41, L.stream_ptr(dev())))
+        L.check(l.jgamd_dense_rows(L.ptr(x), L.ptr(w), 47, None, None, 0, None, L.ptr(out), 5000, 41, 0, L.stream_ptr(dev())))
     xs = torch.randn((5000, 256), device=dev(), generator=gen)[:, ::2]          # not contiguous: BLAS route
     w2 = torch.randn((128, 64), device=dev(), generator=gen)
     ref, scale = reference(xs, w2, None, None, None)

@@ -503,3 +503,93 @@ def test_sage_training_loop_through_the_edge_list_route(root):
     for p, q in zip(params, ref_params):
         q = q.detach().numpy()
         assert_close(p.detach().cpu().numpy(), q, np.abs(q) + np.abs(q).mean(), rtol=1e-4, what="parameters after 15 steps")
+
+
+@pytest.mark.parametrize("spmm,bias", [(False, True), (True, True), (False, False)])
+@pytest.mark.parametrize("f_in,f_out", [(48, 96), (96, 47)])
+def test_gcn_layer_with_the_activation_in_its_row_store_is_relu_of_the_layer(spmm, bias, f_in, f_out):
+    """GCNConv(activation="relu") = relu(GCNConv(...)) as examples/gcn_example.py:84-90 writes it:
+    same output and same gradients bit for bit (the clamp and its mask are exact operations), and
+    both within tolerance of a dense float64 model."""
+    from jittorgeometric_amd.nn import GCNConv, gcn_norm
+    from jittorgeometric_amd.ops import cootocsc, cootocsr
+    from util import rand_graph
+    rng = np.random.default_rng(f_in + 3 * f_out)
+    V, E = 6000, 90000
+    ei, _ = rand_graph(rng, V, E, 2)
+    ei_g, w_g = gcn_norm(to_gpu(ei), None, V)
+    csc, csr = cootocsc(ei_g, w_g, V), cootocsr(ei_g, w_g, V)
+    torch.manual_seed(3)
+    plain = GCNConv(f_in, f_out, bias=bias, spmm=spmm).to(dev())
+    fused = GCNConv(f_in, f_out, bias=bias, spmm=spmm, activation="relu").to(dev())
+    fused.load_state_dict(plain.state_dict())
+    if bias:
+        with torch.no_grad():
+            plain.bias.copy_(torch.randn(f_out, device=dev()) * 0.1)
+            fused.bias.copy_(plain.bias)
+    x = rng.standard_normal((V, f_in)).astype(np.float32)
+    g = rng.standard_normal((V, f_out)).astype(np.float32)
+    xa, xb = to_gpu(x).requires_grad_(True), to_gpu(x).requires_grad_(True)
+    out_a = torch.relu(plain(xa, csc, csr))
+    out_b = fused(xb, csc, csr)
+    assert torch.equal(out_a, out_b) and (out_b >= 0).all() and (out_b == 0).any()
+    out_a.backward(to_gpu(g))
+    out_b.backward(to_gpu(g))
+    assert torch.equal(xa.grad, xb.grad) and torch.equal(plain.weight.grad, fused.weight.grad)
+    if bias:
+        assert torch.equal(plain.bias.grad, fused.bias.grad)
+    # dense float64 model of relu(A (x W) + b)
+    A = dense_adj(ei_g.cpu().numpy(), w_g.cpu().numpy(), V)
+    x64 = torch.from_numpy(x.astype(np.float64)).requires_grad_(True)
+    W64 = plain.weight.detach().cpu().double().requires_grad_(True)
+    pre = A @ (x64 @ W64) + (plain.bias.detach().cpu().double() if bias else 0)
+    torch.relu(pre).backward(torch.from_numpy(g.astype(np.float64)))
+    scale = (A.abs() @ (x64.detach().abs() @ W64.detach().abs())).numpy() + 1
+    near_zero = np.abs(pre.detach().numpy()) < 1e-4 * scale       # the mask may flip where the pre-activation is ~0
+    assert_close(np.where(near_zero, 0, out_b.detach().cpu().numpy()), np.where(near_zero, 0, torch.relu(pre).detach().numpy()),
+                 scale, what="activated output")
+    if not near_zero.any():
+        assert_close(fused.weight.grad.cpu().numpy(), W64.grad.numpy(), rtol=1e-4, atol=1e-4, what="weight gradient")
+
+
+@pytest.mark.parametrize("R,F", [(1, 1), (5000, 47), (70000, 128), (3000, 602), (2049, 256)])
+def test_relu_backward_with_column_sum_in_one_pass(R, F):
+    from jittorgeometric_amd.nn.dense import column_sum, relu_backward_column_sum
+    rng = np.random.default_rng(R + F)
+    g = to_gpu(rng.standard_normal((R, F)).astype(np.float32))
+    y = to_gpu(np.maximum(rng.standard_normal((R, F)), 0).astype(np.float32))
+    masked, gb = relu_backward_column_sum(g, y)
+    want = g * (y > 0)
+    assert torch.equal(masked, want)
+    assert torch.equal(gb, column_sum(want))                       # the same sums in the same order
+    assert_close(gb.cpu().numpy(), want.double().sum(0).cpu().numpy(), want.abs().double().sum(0).cpu().numpy(),
+                 what="bias gradient behind a relu")
+
+
+@pytest.mark.parametrize("root,f_in,f_out", [(True, 64, 96), (False, 100, 48)])
+def test_sage_layer_with_the_activation_in_its_store_is_relu_of_the_layer(root, f_in, f_out):
+    """SAGEConv(activation="relu") = relu(SAGEConv(...)), outputs and gradients bit for bit."""
+    from jittorgeometric_amd.nn import SAGEConv, sage_norm
+    from jittorgeometric_amd.ops import cootocsc, cootocsr
+    from util import rand_graph
+    rng = np.random.default_rng(f_in + f_out)
+    V, E = 6000, 80000
+    ei, _ = rand_graph(rng, V, E, 2)
+    ei_g, w_g = sage_norm(to_gpu(ei), None, V)
+    csc, csr = cootocsc(ei_g, w_g, V), cootocsr(ei_g, w_g, V)
+    torch.manual_seed(4)
+    plain = SAGEConv(f_in, f_out, root_weight=root, spmm=False).to(dev())
+    fused = SAGEConv(f_in, f_out, root_weight=root, spmm=False, activation="relu").to(dev())
+    fused.load_state_dict(plain.state_dict())
+    x = rng.standard_normal((V, f_in)).astype(np.float32)
+    g = to_gpu(rng.standard_normal((V, f_out)).astype(np.float32))
+    xa, xb = to_gpu(x).requires_grad_(True), to_gpu(x).requires_grad_(True)
+    out_a = torch.relu(plain(xa, None, None, csc, csr))
+    out_b = fused(xb, None, None, csc, csr)
+    assert torch.equal(out_a, out_b) and (out_b == 0).any()
+    out_a.backward(g)
+    out_b.backward(g)
+    assert torch.equal(xa.grad, xb.grad) and torch.equal(plain.weight1.grad, fused.weight1.grad)
+    assert torch.equal(plain.bias.grad, fused.bias.grad)
+    if root:
+        assert torch.equal(plain.root_weight.grad, fused.root_weight.grad)

@@ -120,7 +120,7 @@ def test_plan_arrays_follow_the_partition_rule(V, E, hubs, share, kind, seed):
         assert n_fix == 0 and n_grp == 0
 
 
-def planned(plan, tiles, hints, off, idx, w, x, R, beta=1.0, alpha=0.0, h=None):
+def planned(plan, tiles, hints, off, idx, w, x, R, beta=1.0, alpha=0.0, h=None, flags=0):
     L, l = lib()
     C, F = x.shape
     E = idx.shape[0] if idx is not None else C
@@ -129,8 +129,8 @@ def planned(plan, tiles, hints, off, idx, w, x, R, beta=1.0, alpha=0.0, h=None):
     ws = L.workspace(nbytes, dev())
     h_rows = R if h is None or h.dim() == 2 else 1
     L.check(l.jgamd_spmm_csx_planned(L.ptr(plan), L.ptr(tiles), hints[0], hints[1], L.ptr(off), L.ptr(idx), L.ptr(w),
-                                     L.ptr(x), L.ptr(out), beta, alpha, L.ptr(h), h_rows, R, C, E, F, L.ptr(ws), nbytes,
-                                     L.stream_ptr(dev())))
+                                     L.ptr(x), L.ptr(out), beta, alpha, L.ptr(h), h_rows, flags, R, C, E, F, L.ptr(ws),
+                                     nbytes, L.stream_ptr(dev())))
     return out
 
 
@@ -186,6 +186,11 @@ def test_planned_product_with_row_finish_and_without_indices():
     for hh in (to_gpu(h), to_gpu(b)):
         got = planned(plan, None, (n_fix, n_grp), off_g, idx_g, w_g, x_g, V, 0.9, 0.1, hh)
         assert torch.equal(got, unplanned(off_g, idx_g, w_g, x_g, V, 0.9, 0.1, hh))
+    # the row clamped at zero in the row store (a layer's relu): exactly max(0, .) of the unclamped call
+    for hh in (to_gpu(h), to_gpu(b), None):
+        got = planned(plan, None, (n_fix, n_grp), off_g, idx_g, w_g, x_g, V, 1.0, 1.0 if hh is not None else 0.0, hh, flags=1)
+        ref = planned(plan, None, (n_fix, n_grp), off_g, idx_g, w_g, x_g, V, 1.0, 1.0 if hh is not None else 0.0, hh)
+        assert torch.equal(got, torch.relu(ref)) and (got == 0).any()
     # per-entry rows summed per column (ScatterToVertex): idx = NULL, w = NULL
     xe = to_gpu(rng.standard_normal((E, F)).astype(np.float32))
     got = planned(plan, None, (n_fix, n_grp), off_g, None, None, xe, V)
@@ -305,6 +310,8 @@ def test_plan_entry_points_reject_bad_arguments():
     assert l.jgamd_csx_plan(None, 10, 20, 0, bad, 1 << 20, None) == -1
     assert l.jgamd_csx_plan(bad, 10, 20, 0, bad, 8, None) == -3             # plan too small
     assert l.jgamd_csx_plan(bad, 10, 20, 0, ctypes.c_void_p(260), 1 << 20, None) == -5
-    assert l.jgamd_spmm_csx_planned(None, None, -1, -1, bad, bad, bad, bad, bad, 1.0, 0.0, None, 1, 4, 4, 5, 16, bad,
+    assert l.jgamd_spmm_csx_planned(None, None, -1, -1, bad, bad, bad, bad, bad, 1.0, 0.0, None, 1, 0, 4, 4, 5, 16, bad,
                                     1 << 20, None) == -1
+    assert l.jgamd_spmm_csx_planned(bad, None, -1, -1, bad, bad, bad, bad, bad, 1.0, 0.0, None, 1, 2, 4, 4, 5, 16, bad,
+                                    1 << 20, None) == -2                        # unknown flag
     assert l.jgamd_edge_softmax_fwd_planned(None, bad, bad, bad, 4, 5, 1, bad, 1 << 20, None) == -1
