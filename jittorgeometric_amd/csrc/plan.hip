@@ -102,20 +102,31 @@ __global__ __launch_bounds__(kListThreads) void plan_chunk_lists(const int32_t *
 }
 
 // Tiles.  tile_first[i] / tile_last[i] = column of the first / last covered entry of tile i
-// (tiles of T entries); one thread per column marks the tiles whose first or last entry falls
-// among its entries.  Tiles without a covered entry keep what the arrays held.
+// (tiles of T entries).  One thread per tile finds both by bisection of the offsets: the column
+// of entry p is the largest c with off[c] <= p (of several columns that share an offset, empty
+// ones followed by the one that holds p, that is the last).  A column with millions of entries
+// costs what any other costs.  Tiles without a covered entry keep what the arrays held.
+__device__ __forceinline__ int column_of_entry(const int32_t *__restrict__ off, int V, int p)
+{
+    int lo = 0, hi = V;                      // largest c in [0,V) with off[c] <= p
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (off[mid] <= p) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
 __global__ void plan_tile_columns(const int32_t *__restrict__ off, int V, int E, int T, int32_t *__restrict__ tile_first,
                                   int32_t *__restrict__ tile_last)
 {
-    const int c = blockIdx.x * blockDim.x + threadIdx.x;
-    if (c >= V) return;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
     const int covered = min(max(off[V], 0), E);
-    const int s = off[c], e = min(off[c + 1], covered);
-    if (e <= s) return;
     const int ntiles = (covered + T - 1) / T;
-    for (int i = (s + T - 1) / T; i < ntiles && (int64_t)i * T < e; i++) tile_first[i] = c;
-    for (int i = s / T + 1; i <= ntiles && (int64_t)i * T <= e; i++) tile_last[i - 1] = c;   // last entry i*T - 1
-    if (e == covered) tile_last[ntiles - 1] = c;
+    if (i >= ntiles) return;
+    const int64_t first = (int64_t)i * T;
+    const int last = (int)min(first + T, (int64_t)covered) - 1;
+    tile_first[i] = column_of_entry(off, V, (int)first);
+    tile_last[i] = column_of_entry(off, V, last);
 }
 
 int plan_chunk_for(int kind, int64_t M)
@@ -197,8 +208,8 @@ TilePlan tile_plan_view(int64_t E, int T, const void *plan)
 void tile_columns_enqueue(const int32_t *off, int32_t V, int64_t E, int T, int32_t *tile_first, int32_t *tile_last,
                           hipStream_t s)
 {
-    hipLaunchKernelGGL(plan_tile_columns, dim3((unsigned)ceil_div(V > 0 ? V : 1, 256)), dim3(256), 0, s, off, V, (int)E,
-                       T, tile_first, tile_last);
+    hipLaunchKernelGGL(plan_tile_columns, dim3((unsigned)ceil_div(ceil_div(E > 0 ? E : 1, T), 256)), dim3(256), 0, s, off,
+                       V, (int)E, T, tile_first, tile_last);
 }
 
 }  // namespace jg
