@@ -10,11 +10,15 @@
 //                     column of its first and of its last entry (plan.hip;
 //                     once per graph when the caller keeps a tile plan).
 //   1. tile kernel  : a lane holds K consecutive entries (all H heads, loaded
-//                     as vectors).  Each entry's column is found from the
-//                     offsets staged in LDS; per-column totals (max, then sum
-//                     of exp; or sum of y*g) come from a lane-local reduction
-//                     over runs of equal columns plus one segmented scan over
-//                     the block's lanes, in a fixed order (no float atomics).
+//                     as vectors).  The tile's columns mark their first entry
+//                     in a bitmap in LDS; a lane reads the K bits of its
+//                     entries and never learns a column id.  Per-column totals
+//                     (max, then sum of exp; or sum of y*g): runs of one column
+//                     inside a lane are folded in registers, the run that
+//                     reaches a lane from the lanes before it and the run that
+//                     leaves it go through one segmented scan over the block's
+//                     lanes and a table in LDS indexed by the position of the
+//                     column's first entry, in a fixed order (no float atomics).
 //                     Columns that lie inside the tile are finished from
 //                     registers: x is read once, y written once.  A column
 //                     that crosses a tile edge leaves a piece per tile.
@@ -57,16 +61,25 @@ struct FlatMeta {
 __host__ __device__ constexpr int flat_pad(int f) { return f + (f >> 5) * 4; }
 
 template <int H, int T> struct FlatLds {
-    int off[T + 2];
+    unsigned bits[T / 32 + 1];      // bit p: a column begins at entry p of the tile; the last word stays zero
+    int edge[4];                    // off[c_lo], off[c_lo + 1], off[c_hi], off[c_hi + 1]
     __attribute__((aligned(16))) float tot[flat_pad(T * H)];
     float carry[kFlatWaves * H];
     int wflag[kFlatWaves];
-    int wlast[kFlatWaves];
-    int wfirst[kFlatWaves];
+    int wmax[kFlatWaves];
 };
 
 struct OpMax {
-    __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); }
+    // The bare instruction: fmaxf() first passes each operand through a max with itself (it must
+    // quiet signalling NaNs), which doubles the instructions of a pass that is nothing but
+    // maxima.  Volatile so that it stays where it is written, ahead of the select that follows,
+    // instead of moving into a branch of its own.  A NaN operand gives a NaN column either way.
+    __device__ __forceinline__ float operator()(float a, float b) const
+    {
+        float r;
+        asm volatile("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+        return r;
+    }
 };
 struct OpAdd {
     __device__ __forceinline__ float operator()(float a, float b) const { return a + b; }
@@ -100,62 +113,90 @@ __device__ __forceinline__ bool skip_uncovered_tile(int t0, int covered, int E, 
     return true;
 }
 
-// What a tile knows about its entries' columns.
+// What a lane knows about the columns of its K entries.
 template <int K> struct LaneColumns {
-    int slot[K];
-    unsigned closed;   // bit k: entry k is valid and its column lies inside the tile
-    int tail_slot;     // slot of the tile's last column
+    unsigned starts;            // bit k: a column begins at the lane's entry k
+    int first_slot, last_slot;  // slots of the columns of the lane's first and last entry
+    bool ends_here;             // the column of the lane's last entry ends with that entry (or the tile does)
+    unsigned closed;            // bit k: entry k is valid and its column lies inside the tile
+    int tail_slot;              // slot of the tile's last column
     int closed_lo, closed_hi;   // the valid entries of columns inside the tile, relative to t0
-    bool staged;                // the tile's offsets are in L.off (else read from memory)
 };
 
-// Stages the offsets of the tile's columns [c_lo, c_hi] and resolves the column
-// of each of this lane's K entries (entries past the tile's end take the
-// column of the tile's last entry).  Thread 0 records the tile's metadata.
+// One step of an inclusive maximum scan over the wavefront (values >= 0; lanes
+// without a source keep their own).
+template <int CTRL, int ROWS> __device__ __forceinline__ int max_scan_step(int v)
+{
+    return max(v, __builtin_amdgcn_update_dpp(0, v, CTRL, ROWS, 0xf, false));
+}
+
+// The value of the lane before (wave_shr:1); lane 0 receives `first`.
+__device__ __forceinline__ int from_lane_before(int v, int first)
+{
+    return __builtin_amdgcn_update_dpp(first, v, 0x138, 0xf, 0xf, false);
+}
+__device__ __forceinline__ float from_lane_before(float v, float first)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(first), __float_as_int(v), 0x138, 0xf, 0xf, false));
+}
+
+// Marks the first entries of the tile's columns [c_lo, c_hi] in L.bits and gives every lane the
+// bits of its K entries and the slots of its first and last column (entries past the tile's end
+// belong to the column of the tile's last entry).  Thread 0 records the tile's metadata.
+// Contains barriers; L.bits and L.edge stay valid afterwards.
 template <int H, int K, int T>
 __device__ __forceinline__ void resolve_columns(const int32_t *__restrict__ off, int c_lo, int c_hi, int t0, int n,
                                                 FlatLds<H, T> &L, LaneColumns<K> &cols, FlatMeta *meta_out)
 {
-    const int ncol = c_hi - c_lo + 1;
-    const bool staged = ncol + 1 <= T + 2;
-    if (staged)
-        for (int i = threadIdx.x; i <= ncol; i += kFlatThreads) L.off[i] = off[c_lo + i];
+    static_assert(32 % K == 0 && T / 32 + 1 <= kFlatThreads, "a lane's bits lie in one word");
+    const int tid = threadIdx.x;
+    if (tid <= T / 32) L.bits[tid] = 0;
+    if (tid < 4) L.edge[tid] = off[tid < 2 ? c_lo + tid : c_hi + tid - 2];
     __syncthreads();
-    auto offv = [&](int c) { return staged ? L.off[c - c_lo] : off[c]; };
-    const int last = t0 + n - 1;
-    const int j0 = t0 + threadIdx.x * K;
-    const int jc = min(j0, last);
-    int lo = c_lo, hi = c_hi;
-    while (lo < hi) {
-        const int mid = (lo + hi + 1) >> 1;
-        if (offv(mid) <= jc) lo = mid;
-        else hi = mid - 1;
+    // empty columns repeat the position of the column after them; positions outside the tile
+    // (offsets that are not monotone) are left out
+    for (int c = c_lo + tid; c <= c_hi; c += kFlatThreads) {
+        const int pos = off[c] - t0;
+        if (pos >= 0 && pos < n) atomicOr(&L.bits[pos >> 5], 1u << (pos & 31));
     }
-    int c = lo, cs = offv(c), ce = offv(c + 1);
-    cols.closed = 0;
+    __syncthreads();
+    const int p0 = tid * K;
+    cols.starts = (L.bits[p0 >> 5] >> (p0 & 31)) & ((1u << K) - 1u);
+    cols.ends_here = tid == kFlatThreads - 1 || ((L.bits[(p0 + K) >> 5] >> ((p0 + K) & 31)) & 1u);
+    // slot of a lane's last column: the latest first entry at or before the lane's end
+    const int own = cols.starts ? p0 + 31 - __clz((int)cols.starts) : 0;
+    int incl = own;
+    incl = max_scan_step<0x111, 0xf>(incl);
+    incl = max_scan_step<0x112, 0xf>(incl);
+    incl = max_scan_step<0x114, 0xf>(incl);
+    incl = max_scan_step<0x118, 0xf>(incl);
+    incl = max_scan_step<0x142, 0xa>(incl);
+    incl = max_scan_step<0x143, 0xc>(incl);
+    const int w = uniform(tid >> 6);
+    if (lane_id() == kWave - 1) L.wmax[w] = incl;
+    __syncthreads();
+    int before = 0;
 #pragma unroll
-    for (int k = 0; k < K; k++) {
-        const int j = min(j0 + k, last);
-        while (ce <= j && c < c_hi) {      // c < c_hi only matters if off[V] != E
-            c++;
-            cs = ce;
-            ce = offv(c + 1);
-        }
-        cols.slot[k] = min(max(cs - t0, 0), T - 1);     // the upper clamp only matters for inconsistent offsets
-        if (j0 + k <= last && cs >= t0 && ce <= t0 + n) cols.closed |= 1u << k;
-    }
-    cols.staged = staged;
-    cols.tail_slot = min(max(offv(c_hi) - t0, 0), T - 1);
-    cols.closed_lo = offv(c_lo) < t0 ? min(offv(c_lo + 1) - t0, n) : 0;
-    cols.closed_hi = offv(c_hi + 1) > t0 + n ? max(offv(c_hi) - t0, cols.closed_lo) : n;
-    if (threadIdx.x == 0) {
+    for (int u = 0; u < kFlatWaves - 1; u++)
+        if (u < w) before = max(before, L.wmax[u]);
+    const int prev = max(before, from_lane_before(incl, 0));
+    cols.first_slot = (cols.starts & 1u) ? p0 : prev;
+    cols.last_slot = max(prev, own);
+    const int e0 = L.edge[0], e1 = L.edge[1], e2 = L.edge[2], e3 = L.edge[3];
+    const bool head_open = e0 < t0, tail_open = e3 > t0 + n;
+    cols.tail_slot = min(max(e2 - t0, 0), T - 1);     // the upper clamp only matters for inconsistent offsets
+    cols.closed_lo = head_open ? min(max(e1 - t0, 0), n) : 0;
+    cols.closed_hi = tail_open ? min(max(e2 - t0, cols.closed_lo), n) : n;
+    const int lo_k = min(max(cols.closed_lo - p0, 0), K), hi_k = min(max(cols.closed_hi - p0, 0), K);
+    cols.closed = ((1u << hi_k) - 1u) & ~((1u << lo_k) - 1u);
+    if (tid == 0) {
         FlatMeta m;
-        m.head_cs = offv(c_lo);
-        m.head_ce = offv(c_lo + 1);
-        m.head_open = m.head_cs < t0;
-        m.tail_cs = offv(c_hi);
-        m.tail_ce = offv(c_hi + 1);
-        m.tail_open = m.tail_ce > t0 + n;
+        m.head_cs = e0;
+        m.head_ce = e1;
+        m.head_open = head_open;
+        m.tail_cs = e2;
+        m.tail_ce = e3;
+        m.tail_open = tail_open;
         m.tail_col = c_hi;
         m.pad1 = 0;
         *meta_out = m;
@@ -174,7 +215,8 @@ __device__ __forceinline__ void seg_scan_step(float (&v)[H], int &fl, Op op, flo
     for (int h = 0; h < H; h++) {
         const float up = __int_as_float(
             __builtin_amdgcn_update_dpp(__float_as_int(ident), __float_as_int(v[h]), CTRL, ROWS, 0xf, false));
-        v[h] = fl ? v[h] : op(up, v[h]);
+        const float folded = op(up, v[h]);
+        v[h] = fl ? v[h] : folded;
     }
     fl |= fu;
 }
@@ -200,60 +242,42 @@ template <int H> __device__ __forceinline__ void read_totals(const float *tot, i
     }
 }
 
-// Per-column totals of val over the tile -> L.tot[slot*H + h].  Entries that
-// do not count must hold the identity.  Starts and ends with a barrier.
-template <int H, int K, int T, typename Op>
-__device__ __forceinline__ void segment_totals(const float (&val)[K][H], const int (&slot)[K], FlatLds<H, T> &L, Op op,
-                                               float ident)
+// tot[k] = the fold of val over the whole column of the lane's entry k, as far as the column
+// lies in the tile.  Entries that do not count must hold the identity.  A run that begins and
+// ends inside the lane never leaves its registers; the lane's first run (it may reach back
+// into earlier lanes) and its last (it may go on in later ones) are completed by the segmented
+// scan, and the lane in which a column ends publishes its total in L.tot[slot].  Afterwards
+// L.tot holds the totals of every column that crosses a lane edge, the tile's first column
+// (slot 0) and its last (tail_slot) among them; TABLE adds the columns inside one lane, and
+// a barrier, so that L.tot can be read for any column that begins in the tile.
+template <int H, int K, int T, bool TABLE = false, typename Op>
+__device__ __forceinline__ void segment_totals(const float (&val)[K][H], const LaneColumns<K> &cols, FlatLds<H, T> &L,
+                                               Op op, float ident, float (&tot)[K][H])
 {
     const int lane = lane_id();
-    const int w = threadIdx.x >> 6;
-    __syncthreads();
-    // runs of equal columns inside the lane: the first and the last may go on
-    // in the neighbouring lanes, the ones between are complete
-    float acc[H], headv[H];
-    bool multi = false;
+    const int w = uniform(threadIdx.x >> 6);
+    bool st[K];
 #pragma unroll
-    for (int h = 0; h < H; h++) acc[h] = val[0][h];
+    for (int k = 0; k < K; k++) st[k] = (cols.starts >> k) & 1u;
+    // a[k]: fold of the entries of k's run up to k, inside the lane
+    float a[K][H];
 #pragma unroll
-    for (int k = 1; k < K; k++) {
-        if (slot[k] != slot[k - 1]) {
-            if (!multi) {
+    for (int h = 0; h < H; h++) a[0][h] = val[0][h];
 #pragma unroll
-                for (int h = 0; h < H; h++) headv[h] = acc[h];
-                multi = true;
-            } else {
+    for (int k = 1; k < K; k++)
 #pragma unroll
-                for (int h = 0; h < H; h++) L.tot[slot[k - 1] * H + h] = acc[h];
-            }
-#pragma unroll
-            for (int h = 0; h < H; h++) acc[h] = val[k][h];
-        } else {
-#pragma unroll
-            for (int h = 0; h < H; h++) acc[h] = op(acc[h], val[k][h]);
+        for (int h = 0; h < H; h++) {
+            const float folded = op(a[k - 1][h], val[k][h]);     // computed either way: a select, not a branch
+            a[k][h] = st[k] ? val[k][h] : folded;
         }
-    }
-    if (!multi) {
-#pragma unroll
-        for (int h = 0; h < H; h++) headv[h] = acc[h];
-    }
-    const int firstslot = slot[0], lastslot = slot[K - 1];
-    if (lane == kWave - 1) L.wlast[w] = lastslot;
-    if (lane == 0) L.wfirst[w] = firstslot;
-    __syncthreads();
-    int prevlast = __shfl_up(lastslot, 1, kWave);
-    if (lane == 0) prevlast = w > 0 ? L.wlast[w - 1] : -1;
-    int nextfirst = __shfl_down(firstslot, 1, kWave);
-    if (lane == kWave - 1) nextfirst = w < kFlatWaves - 1 ? L.wfirst[w + 1] : -2;
-    // inclusive segmented scan of the last runs: a lane starts a new segment
-    // if a column begins inside it or at its first entry
-    int fl = (multi || firstslot != prevlast) ? 1 : 0;
+    // inclusive segmented scan of the last runs: a lane in which a column begins starts a segment.
+    // Rows of 16 lanes with row shifts, then lane 15 -> next row (rows 1, 3) and lane 31 -> rows
+    // 2, 3: all data-parallel moves on the vector ALU (a step changes nothing once every lane
+    // has seen a segment start)
+    int fl = cols.starts != 0;
     float v[H];
 #pragma unroll
-    for (int h = 0; h < H; h++) v[h] = acc[h];
-    // rows of 16 lanes with row shifts, then lane 15 -> next row (rows 1, 3)
-    // and lane 31 -> rows 2, 3: all data-parallel moves on the vector ALU
-    // (a step changes nothing once every lane has seen a segment start)
+    for (int h = 0; h < H; h++) v[h] = a[K - 1][h];
     seg_scan_step<0x111, 0xf>(v, fl, op, ident);
     seg_scan_step<0x112, 0xf>(v, fl, op, ident);
     if (__ballot(fl == 0)) {
@@ -273,21 +297,55 @@ __device__ __forceinline__ void segment_totals(const float (&val)[K][H], const i
     float carry[H];
 #pragma unroll
     for (int h = 0; h < H; h++) carry[h] = ident;
-    for (int u = 0; u < w; u++) {
-        const bool cut = L.wflag[u] != 0;
 #pragma unroll
-        for (int h = 0; h < H; h++) carry[h] = cut ? L.carry[u * H + h] : op(carry[h], L.carry[u * H + h]);
-    }
+    for (int u = 0; u < kFlatWaves - 1; u++)
+        if (u < w) {
+            const bool cut = L.wflag[u] != 0;
+#pragma unroll
+            for (int h = 0; h < H; h++) {
+                const float folded = op(carry[h], L.carry[u * H + h]);
+                carry[h] = cut ? L.carry[u * H + h] : folded;
+            }
+        }
+    // the column that ends inside this lane after reaching it from the lanes before: its total is
+    // what those lanes hold plus this lane's entries below its first column start
+    const bool head_ends = cols.starts != 0 && !(cols.starts & 1u);
+    float head_total[H];
 #pragma unroll
     for (int h = 0; h < H; h++) {
-        if (!fl) v[h] = op(carry[h], v[h]);
-        // total of the previous lane's last column up to that lane
-        float prev = __shfl_up(v[h], 1, kWave);
-        if (lane == 0) prev = carry[h];
-        if (multi) L.tot[firstslot * H + h] = firstslot == prevlast ? op(prev, headv[h]) : headv[h];
-        if (nextfirst != lastslot) L.tot[lastslot * H + h] = v[h];
+        const float with_carry = op(carry[h], v[h]);
+        v[h] = fl ? v[h] : with_carry;
+        const float prev = from_lane_before(v[h], carry[h]);
+        float hd = a[K - 1][h];
+#pragma unroll
+        for (int k = K - 1; k >= 1; k--) hd = st[k] ? a[k - 1][h] : hd;
+        head_total[h] = op(prev, hd);
+        if (head_ends) L.tot[cols.first_slot * H + h] = head_total[h];
+        if (cols.ends_here) L.tot[cols.last_slot * H + h] = v[h];
     }
     __syncthreads();
+    float run[H];
+    read_totals<H>(L.tot, cols.last_slot, run);
+    const int k0 = cols.starts ? __builtin_ctz(cols.starts) : 0;     // entries below k0: the column that ends here
+#pragma unroll
+    for (int k = K - 1; k >= 0; k--) {
+#pragma unroll
+        for (int h = 0; h < H; h++) {
+            tot[k][h] = k < k0 ? head_total[h] : run[h];
+            if (k >= 1) run[h] = st[k] ? a[k - 1][h] : run[h];
+        }
+    }
+    if constexpr (TABLE) {
+        // columns inside the lane (the last run is published by the lane it ends in)
+        const int top = cols.starts ? 31 - __clz((int)cols.starts) : 0;
+#pragma unroll
+        for (int k = 0; k < K; k++)
+            if (st[k] && k != top) {
+#pragma unroll
+                for (int h = 0; h < H; h++) L.tot[((int)threadIdx.x * K + k) * H + h] = tot[k][h];
+            }
+        __syncthreads();
+    }
 }
 
 template <int N> struct __attribute__((aligned(N >= 4 ? 16 : 4 * N))) FloatVec {
@@ -448,37 +506,43 @@ __global__ __launch_bounds__(kFlatThreads) void esm_fwd_tile(const int32_t *__re
     else load_lane<H, K>(x, aligned, j0, E, v);
     LaneColumns<K> cols;
     resolve_columns<H, K, T>(off, c_lo, c_hi, t0, n, L, cols, meta + tile);
+    const bool partial = n < T;      // only the last covered tile holds entries that do not count
+    if (partial) {
 #pragma unroll
-    for (int k = 0; k < K; k++)
-        if (j0 + k >= t0 + n) {
+        for (int k = 0; k < K; k++)
+            if (j0 + k >= t0 + n) {
 #pragma unroll
-            for (int h = 0; h < H; h++) v[k][h] = -INFINITY;
-        }
-    segment_totals<H, K, T>(v, cols.slot, L, OpMax(), -INFINITY);
+                for (int h = 0; h < H; h++) v[k][h] = -INFINITY;
+            }
+    }
+    float t[K][H];
+    segment_totals<H, K, T>(v, cols, L, OpMax(), -INFINITY, t);
     const int tail_slot = cols.tail_slot;
     if (threadIdx.x < H) {
         piece<H>(pieces, tile, 0)[threadIdx.x] = L.tot[threadIdx.x];
         piece<H>(pieces, tile, 1)[threadIdx.x] = L.tot[tail_slot * H + threadIdx.x];
     }
 #pragma unroll
-    for (int k = 0; k < K; k++) {
-        float m[H];
-        read_totals<H>(L.tot, cols.slot[k], m);
+    for (int k = 0; k < K; k++)
 #pragma unroll
-        for (int h = 0; h < H; h++) v[k][h] = j0 + k < t0 + n ? __expf(v[k][h] - m[h]) : 0.f;
+        for (int h = 0; h < H; h++) v[k][h] = __expf(v[k][h] - t[k][h]);
+    if (partial) {
+#pragma unroll
+        for (int k = 0; k < K; k++)
+            if (j0 + k >= t0 + n) {
+#pragma unroll
+                for (int h = 0; h < H; h++) v[k][h] = 0.f;
+            }
     }
-    segment_totals<H, K, T>(v, cols.slot, L, OpAdd(), 0.f);
+    segment_totals<H, K, T>(v, cols, L, OpAdd(), 0.f, t);
     if (threadIdx.x < H) {
         piece<H>(pieces, tile, 0)[H + threadIdx.x] = L.tot[threadIdx.x];
         piece<H>(pieces, tile, 1)[H + threadIdx.x] = L.tot[tail_slot * H + threadIdx.x];
     }
 #pragma unroll
-    for (int k = 0; k < K; k++) {
-        float t[H];
-        read_totals<H>(L.tot, cols.slot[k], t);
+    for (int k = 0; k < K; k++)
 #pragma unroll
-        for (int h = 0; h < H; h++) v[k][h] = v[k][h] * __frcp_rn(t[h]);
-    }
+        for (int h = 0; h < H; h++) v[k][h] = v[k][h] * __builtin_amdgcn_rcpf(t[k][h]);
     if (through_lds) store_tile<H, K>(y, t0, cols.closed_lo, cols.closed_hi, L.tot, v);
     else store_lane<H, K>(y, aligned, j0, cols.closed, v);
 }
@@ -519,20 +583,26 @@ __global__ __launch_bounds__(kFlatThreads) void esm_bwd_tile(const int32_t *__re
 #pragma unroll
     for (int k = 0; k < K; k++)
 #pragma unroll
-        for (int h = 0; h < H; h++) yg[k][h] = j0 + k < t0 + n ? yv[k][h] * yg[k][h] : 0.f;
-    segment_totals<H, K, T>(yg, cols.slot, L, OpAdd(), 0.f);
+        for (int h = 0; h < H; h++) yg[k][h] = yv[k][h] * yg[k][h];
+    if (n < T) {
+#pragma unroll
+        for (int k = 0; k < K; k++)
+            if (j0 + k >= t0 + n) {
+#pragma unroll
+                for (int h = 0; h < H; h++) yg[k][h] = 0.f;
+            }
+    }
+    float t[K][H];
+    segment_totals<H, K, T>(yg, cols, L, OpAdd(), 0.f, t);
     const int tail_slot = cols.tail_slot;
     if (threadIdx.x < H) {
         piece<H>(pieces, tile, 0)[threadIdx.x] = L.tot[threadIdx.x];
         piece<H>(pieces, tile, 1)[threadIdx.x] = L.tot[tail_slot * H + threadIdx.x];
     }
 #pragma unroll
-    for (int k = 0; k < K; k++) {
-        float t[H];
-        read_totals<H>(L.tot, cols.slot[k], t);
+    for (int k = 0; k < K; k++)
 #pragma unroll
-        for (int h = 0; h < H; h++) yg[k][h] = yg[k][h] - yv[k][h] * t[h];
-    }
+        for (int h = 0; h < H; h++) yg[k][h] = yg[k][h] - yv[k][h] * t[k][h];
     if (through_lds) store_tile<H, K>(dx, t0, cols.closed_lo, cols.closed_hi, L.tot, yg);
     else store_lane<H, K>(dx, aligned, j0, cols.closed, yg);
 }
@@ -596,7 +666,8 @@ __global__ __launch_bounds__(kFlatThreads) void esm_colsum_tile(const int32_t *_
     for (int k = 0; k < K; k++)
 #pragma unroll
         for (int h = 0; h < H; h++) v[k][h] *= wk[k];
-    segment_totals<H, K, T>(v, cols.slot, L, OpAdd(), 0.f);
+    float t[K][H];
+    segment_totals<H, K, T, true>(v, cols, L, OpAdd(), 0.f, t);
     if (threadIdx.x < H) {
         piece<H>(pieces, tile, 0)[threadIdx.x] = L.tot[threadIdx.x];
         piece<H>(pieces, tile, 1)[threadIdx.x] = L.tot[cols.tail_slot * H + threadIdx.x];
@@ -606,14 +677,14 @@ __global__ __launch_bounds__(kFlatThreads) void esm_colsum_tile(const int32_t *_
     const int c_to = t0 + T >= covered ? V - 1 : c_hi;
     for (int c = c_from + (int)threadIdx.x; c <= c_to; c += kFlatThreads) {
         const bool inside = c >= c_lo && c <= c_hi;
-        const int cs = !inside ? 0 : cols.staged ? L.off[c - c_lo] : off[c];
-        const int ce = !inside ? 0 : cols.staged ? L.off[c - c_lo + 1] : off[c + 1];
+        const int cs = inside ? off[c] : 0;
+        const int ce = inside ? off[c + 1] : 0;
         if (ce > cs) {
             if (cs >= t0 && ce <= t0 + n) {
-                float t[H];
-                read_totals<H>(L.tot, cs - t0, t);
+                float r[H];
+                read_totals<H>(L.tot, cs - t0, r);
 #pragma unroll
-                for (int h = 0; h < H; h++) out[(int64_t)c * H + h] = t[h];
+                for (int h = 0; h < H; h++) out[(int64_t)c * H + h] = r[h];
             }
         } else {
 #pragma unroll
@@ -622,12 +693,60 @@ __global__ __launch_bounds__(kFlatThreads) void esm_colsum_tile(const int32_t *_
     }
 }
 
-// One wavefront per tile in which a crossing column begins: folds the tail
-// piece of that tile and the head pieces of the tiles the column runs
-// through into stat[tile] (forward: H maxima, H sums; backward: H sums).
+// Folding the pieces of a column that crosses tile edges: (max, sum relative to that max) for
+// the softmax, plain sums otherwise.
+template <int H, bool SOFT> struct PieceFold {
+    float mx[H], sum[H];
+    __device__ __forceinline__ PieceFold()
+    {
+#pragma unroll
+        for (int h = 0; h < H; h++) {
+            mx[h] = -INFINITY;
+            sum[h] = 0.f;
+        }
+    }
+    __device__ __forceinline__ void fold(int h, float m2, float s2)
+    {
+        if (SOFT) {
+            const float mm = fmaxf(mx[h], m2);
+            sum[h] = (mx[h] == -INFINITY ? 0.f : sum[h] * __expf(mx[h] - mm)) + (m2 == -INFINITY ? 0.f : s2 * __expf(m2 - mm));
+            mx[h] = mm;
+        } else {
+            sum[h] += s2;
+        }
+    }
+    // pieces of the tiles first..last of one column (its tail piece in the tile it begins in,
+    // head pieces after that).  Most crossing columns end in the next tile: a short chain is
+    // folded in order by every lane alike; a long one is dealt round-robin over the wavefront's
+    // lanes, each lane keeping tile order, then folded across the lanes (fold is symmetric in
+    // its operands, so every lane ends with the same bits).  The same order whoever computes it.
+    __device__ __forceinline__ void chain(const float *pieces, int first, int last)
+    {
+        const bool chain_short = last - first < 4;
+        for (int j = first + (chain_short ? 0 : lane_id()); j <= last; j += chain_short ? 1 : kWave) {
+            const float *p = pieces + ((int64_t)j * 2 + (j == first ? 1 : 0)) * 2 * H;
+#pragma unroll
+            for (int h = 0; h < H; h++) fold(h, SOFT ? p[h] : 0.f, SOFT ? p[H + h] : p[h]);
+        }
+        if (chain_short) return;
+#pragma unroll
+        for (int o = 1; o < kWave; o <<= 1) {
+#pragma unroll
+            for (int h = 0; h < H; h++) {
+                const float m2 = SOFT ? __shfl_xor(mx[h], o, kWave) : 0.f;
+                const float s2 = __shfl_xor(sum[h], o, kWave);
+                fold(h, m2, s2);
+            }
+        }
+    }
+};
+
+// One wavefront per tile in which a crossing column begins folds the column's pieces into
+// stat[tile] (forward: H maxima, H reciprocals of the sums; backward: H sums), or, for column
+// sums, into the column's slot of the result.
 template <int H, int T, bool FWD>
 __global__ __launch_bounds__(kFlatThreads) void esm_merge(const FlatMeta *__restrict__ meta,
-                                                          float *__restrict__ pieces, float *__restrict__ stat,
+                                                          const float *__restrict__ pieces, float *__restrict__ stat,
                                                           int ntiles, float *__restrict__ column_out = nullptr)
 {
     const int tile = blockIdx.x * kFlatWaves + (threadIdx.x >> 6);
@@ -635,66 +754,25 @@ __global__ __launch_bounds__(kFlatThreads) void esm_merge(const FlatMeta *__rest
     const FlatMeta m = meta[tile];
     if (!m.tail_open || m.tail_cs < tile * T) return;
     const int last_tile = min((m.tail_ce - 1) / T, ntiles - 1);   // the clamp only matters for offsets past E
-    const int lane = lane_id();
-    float mx[H], sum[H];
-#pragma unroll
-    for (int h = 0; h < H; h++) {
-        mx[h] = -INFINITY;
-        sum[h] = 0.f;
-    }
-    auto fold = [&](int h, float m2, float s2) {
-        if (FWD) {
-            const float mm = fmaxf(mx[h], m2);
-            sum[h] = (mx[h] == -INFINITY ? 0.f : sum[h] * expf(mx[h] - mm)) + (m2 == -INFINITY ? 0.f : s2 * expf(m2 - mm));
-            mx[h] = mm;
-        } else {
-            sum[h] += s2;
-        }
-    };
-    // lane 0 starts from the tail piece of this tile; head pieces of the
-    // following tiles are dealt round-robin, each lane keeping tile order.
-    // Most crossing columns end in the next tile: short chains are folded by
-    // lane 0 alone and skip the exchange between lanes.
-    const bool chain_short = last_tile - tile < 4;
-    if (chain_short) {
-        if (lane == 0)
-            for (int j = tile; j <= last_tile; j++) {
-                const float *p = piece<H>(pieces, j, j == tile ? 1 : 0);
-#pragma unroll
-                for (int h = 0; h < H; h++) fold(h, FWD ? p[h] : 0.f, FWD ? p[H + h] : p[h]);
-            }
-    } else {
-        for (int j = tile + lane; j <= last_tile; j += kWave) {
-            const float *p = piece<H>(pieces, j, j == tile ? 1 : 0);
-#pragma unroll
-            for (int h = 0; h < H; h++) fold(h, FWD ? p[h] : 0.f, FWD ? p[H + h] : p[h]);
-        }
-#pragma unroll
-        for (int o = 1; o < kWave; o <<= 1) {
-#pragma unroll
-            for (int h = 0; h < H; h++) {
-                const float m2 = FWD ? __shfl_xor(mx[h], o, kWave) : 0.f;
-                const float s2 = __shfl_xor(sum[h], o, kWave);
-                fold(h, m2, s2);
-            }
-        }
-    }
-    if (lane == 0) {
+    PieceFold<H, FWD> f;
+    f.chain(pieces, tile, last_tile);
+    if (lane_id() == 0) {
 #pragma unroll
         for (int h = 0; h < H; h++) {
             if (FWD) {
-                stat[(int64_t)tile * 2 * H + h] = mx[h];
-                stat[(int64_t)tile * 2 * H + H + h] = sum[h];
+                stat[(int64_t)tile * 2 * H + h] = f.mx[h];
+                stat[(int64_t)tile * 2 * H + H + h] = 1.f / f.sum[h];
             } else if (column_out) {
-                column_out[(int64_t)m.tail_col * H + h] = sum[h];     // column sums: the total is the result
+                column_out[(int64_t)m.tail_col * H + h] = f.sum[h];     // column sums: the total is the result
             } else {
-                stat[(int64_t)tile * 2 * H + h] = sum[h];
+                stat[(int64_t)tile * 2 * H + h] = f.sum[h];
             }
         }
     }
 }
 
-// Entries of crossing columns.  a = x (forward) or y (backward); b = g.
+// Entries of crossing columns.  a = x (forward) or y (backward); b = g.  Four floats per lane and
+// access where the arrays are aligned; the two ends of a range float by float.
 template <int H, int T, bool FWD>
 __global__ __launch_bounds__(kFlatThreads) void esm_finish(const FlatMeta *__restrict__ meta,
                                                            const float *__restrict__ stat, const float *__restrict__ a,
@@ -704,38 +782,68 @@ __global__ __launch_bounds__(kFlatThreads) void esm_finish(const FlatMeta *__res
     const int t0 = tile * T;
     const int n = min(T, E - t0);
     const FlatMeta m = meta[tile];
+    const bool vec = both_aligned(a, out) && (FWD || ((uintptr_t)b & 15) == 0);
 #pragma unroll
     for (int part = 0; part < 2; part++) {
-        int src, s, e;
+        int src;
+        int64_t lo, hi;
         if (part == 0) {
             if (!m.head_open) continue;
             src = min(max(m.head_cs, 0) / T, tile);
-            s = t0;
-            e = min(m.head_ce, t0 + n);
+            lo = (int64_t)t0 * H;
+            hi = (int64_t)min(m.head_ce, t0 + n) * H;
         } else {
             if (!m.tail_open || m.tail_cs < t0) continue;
             src = tile;
-            s = m.tail_cs;
-            e = t0 + n;
+            lo = (int64_t)m.tail_cs * H;
+            hi = (int64_t)(t0 + n) * H;
         }
         const float *st = stat + (int64_t)src * 2 * H;
-        // kFlatThreads % H == 0: a thread stays on one head
-        const int h = (int)(((int64_t)s * H + threadIdx.x) % H);
-        const float s0 = st[h], s1 = FWD ? st[H + h] : 0.f;
-        const int64_t end = (int64_t)e * H;
-        constexpr int kBatch = 4;
-        for (int64_t p0 = (int64_t)s * H + threadIdx.x; p0 < end; p0 += (int64_t)kBatch * kFlatThreads) {
-            float va[kBatch], vb[kBatch];
+        if (vec) {
+            // the heads of a lane's four floats are the same at every step (the stride is a multiple of H)
+            const int64_t q0 = (lo >> 2) + threadIdx.x;
+            const int hb = (int)((q0 * 4) % H);
+            float s0[4], s1[4];
 #pragma unroll
-            for (int i = 0; i < kBatch; i++) {
-                const int64_t p = min(p0 + (int64_t)i * kFlatThreads, end - 1);
-                va[i] = a[p];
-                vb[i] = FWD ? 0.f : b[p];
+            for (int i = 0; i < 4; i++) {
+                s0[i] = st[(hb + i) % H];
+                s1[i] = FWD ? st[H + (hb + i) % H] : 0.f;
             }
+            auto value = [&](int i, float va, float vb) { return FWD ? __expf(va - s0[i]) * s1[i] : va * vb - va * s0[i]; };
+            constexpr int kBatch = 2;
+            for (int64_t qb = q0; qb * 4 < hi; qb += (int64_t)kBatch * kFlatThreads) {
+                float4 va[kBatch], vb[kBatch];
+                bool whole[kBatch];
 #pragma unroll
-            for (int i = 0; i < kBatch; i++) {
-                const int64_t p = p0 + (int64_t)i * kFlatThreads;
-                if (p < end) out[p] = FWD ? expf(va[i] - s0) / s1 : va[i] * vb[i] - va[i] * s0;
+                for (int u = 0; u < kBatch; u++) {
+                    const int64_t p = (qb + (int64_t)u * kFlatThreads) * 4;
+                    whole[u] = p >= lo && p + 4 <= hi;
+                    if (whole[u]) {
+                        va[u] = *reinterpret_cast<const float4 *>(a + p);
+                        if (!FWD) vb[u] = *reinterpret_cast<const float4 *>(b + p);
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < kBatch; u++) {
+                    const int64_t p = (qb + (int64_t)u * kFlatThreads) * 4;
+                    if (whole[u]) {
+                        float4 r;
+                        r.x = value(0, va[u].x, FWD ? 0.f : vb[u].x);
+                        r.y = value(1, va[u].y, FWD ? 0.f : vb[u].y);
+                        r.z = value(2, va[u].z, FWD ? 0.f : vb[u].z);
+                        r.w = value(3, va[u].w, FWD ? 0.f : vb[u].w);
+                        *reinterpret_cast<float4 *>(out + p) = r;
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 4; i++)
+                            if (p + i >= lo && p + i < hi) out[p + i] = value(i, a[p + i], FWD ? 0.f : b[p + i]);
+                    }
+                }
+            }
+        } else {
+            for (int64_t p = lo + threadIdx.x; p < hi; p += kFlatThreads) {
+                const int h = (int)(p % H);
+                out[p] = FWD ? __expf(a[p] - st[h]) * st[H + h] : a[p] * b[p] - a[p] * st[h];
             }
         }
     }
@@ -811,13 +919,13 @@ static void colsum_launch(const int32_t *off, const int32_t *idx, const float *w
     const size_t cap = (size_t)ceil_div(E, (int64_t)FlatShape<8>::T);
     FlatMeta *meta = carve.take<FlatMeta>(cap);
     float *pieces = carve.take<float>(cap * 4 * 8);
-    float *stat = carve.take<float>(cap * 2 * 8);
+    carve.take<float>(cap * 2 * 8);      // the softmax kernels' merged totals: not used here
     const TilePlan tp = tile_columns(tiles, off, R, E, T, carve.take<int32_t>(cap), carve.take<int32_t>(cap), s);
     const int32_t *tile_first = tp.tile_first, *tile_last = tp.tile_last;
     hipLaunchKernelGGL(esm_colsum_tile<H>, dim3(ntiles), dim3(kFlatThreads), 0, s, off, idx, w, x, out, tile_first,
                        tile_last, R, C, (int)E, meta, pieces);
     hipLaunchKernelGGL((esm_merge<H, T, false>), dim3((unsigned)ceil_div(ntiles, kFlatWaves)), dim3(kFlatThreads), 0, s,
-                       meta, pieces, stat, ntiles, out);
+                       meta, pieces, (float *)nullptr, ntiles, out);
 }
 
 // out[r,:] = sum_j w[j] * x[idx[j],:] for rows of F = 1, 2, 4 or 8 floats.  Needs R > 0,

@@ -81,6 +81,67 @@ def test_edgesoftmax_forward_backward(V, E, H, hubs, seed):
     assert_close(xt.grad.cpu().numpy(), wantg, scale=np.abs(wantg) + want * scale[seg], what="softmax backward")
 
 
+def _column_layouts():
+    """Column lengths whose first entries fall on the places the tile kernels treat differently:
+    lane edges (a lane holds 8 or 4 consecutive entries), tile edges (2048 / 1024 entries),
+    every entry a column of its own, columns inside one lane, columns over many lanes, runs of
+    empty columns (more than a block has threads, more than a tile has entries)."""
+    rng = np.random.default_rng(77)
+    lay = {
+        "lane_edges": [8] * 300 + [4] * 100 + [16] * 50 + [3, 5] * 80 + [1] * 64 + [7, 9] * 60,
+        "tile_edges": [2048, 1024, 1024, 2047, 1, 2049, 1023, 1, 1024, 4096, 5, 3, 2040],
+        "singles": [1] * 5000,
+        "empties": [0] * 700 + [3] + [0] * 3000 + [2, 0, 0, 5] * 300 + [0] * 2500 + [2048] + [0] * 10,
+        "long_inside": [1, 700, 2, 1300, 45, 2048 - 45, 6, 2000, 42],
+        "mixed": list(rng.integers(0, 40, 800)) + [5000] + list(rng.integers(0, 6, 3000)) + [1, 9000, 1],
+    }
+    return lay
+
+
+@pytest.mark.parametrize("layout", sorted(_column_layouts()))
+@pytest.mark.parametrize("H", [1, 2, 4, 8])
+def test_edgesoftmax_and_narrow_sums_on_built_columns(layout, H):
+    from jittorgeometric_amd import CSC
+    from jittorgeometric_amd.ops import EdgeSoftmax
+    from jittorgeometric_amd.ops._common import spmm
+    lens = np.asarray(_column_layouts()[layout], dtype=np.int64)
+    V, E = len(lens), int(lens.sum())
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    rng = np.random.default_rng(len(lens) + H)
+    row = rng.integers(0, V, E).astype(np.int32)
+    w = rng.standard_normal(E).astype(np.float32)
+    csc = CSC(to_gpu(row), to_gpu(off), to_gpu(w))
+    x = (4 * rng.standard_normal((E, H))).astype(np.float32)
+    g = rng.standard_normal((E, H)).astype(np.float32)
+    xt = to_gpu(x).requires_grad_(True)
+    y = EdgeSoftmax(xt, csc)
+    y.backward(to_gpu(g))
+    seg = np.repeat(np.arange(V), lens)
+    x64 = x.astype(np.float64)
+    mx = np.full((V, H), -np.inf)
+    np.maximum.at(mx, seg, x64)
+    p64 = np.exp(x64 - mx[seg])
+    den = np.zeros((V, H))
+    np.add.at(den, seg, p64)
+    y64 = p64 / den[seg]
+    assert_close(y.detach().cpu().numpy(), y64, rtol=1e-5, atol=1e-7, what="softmax vs fp64")
+    dot = np.zeros((V, H))
+    np.add.at(dot, seg, y64 * g)
+    absdot = np.zeros((V, H))
+    np.add.at(absdot, seg, np.abs(y64 * g))
+    assert_close(xt.grad.cpu().numpy(), y64 * (g - dot[seg]), scale=np.abs(y64 * g) + y64 * absdot[seg],
+                 what="softmax backward vs fp64")
+    # the gather-sum over the same columns at the same widths (rows of H floats)
+    feat = rng.standard_normal((V, H)).astype(np.float32)
+    out = spmm(csc.column_offset, csc.row_indices, csc.edge_weight, to_gpu(feat), V).cpu().numpy()
+    terms = w.astype(np.float64)[:, None] * feat.astype(np.float64)[row]
+    want = np.zeros((V, H))
+    np.add.at(want, seg, terms)
+    mag = np.zeros((V, H))
+    np.add.at(mag, seg, np.abs(terms))
+    assert_close(out, want, scale=mag, what="narrow gather-sum vs fp64")
+
+
 def test_edgesoftmax_reference_shapes_E_and_E1():
     from jittorgeometric_amd.ops import EdgeSoftmax
     rng = np.random.default_rng(30)
