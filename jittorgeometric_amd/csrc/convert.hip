@@ -160,14 +160,16 @@ __device__ __forceinline__ int tile_of_workgroup(int nblocks)
 // lanes, which the shift does not cross), so unsorted keys pay a few ALU instructions, no LDS trip.
 __device__ __forceinline__ void count_runs(uint32_t *bins, int b, uint32_t unit)
 {
-    const int lane = lane_id();
+    const int l15 = lane_id() & 15;
     const int prev = __builtin_amdgcn_update_dpp(b, b, 0x111 /* row_shr:1 */, 0xf, 0xf, false);
-    const bool start = (lane & 15) == 0 || b != prev;
+    const bool start = l15 == 0 || b != prev;
     const uint64_t starts = __ballot(start);
     if (start && b >= 0) {
-        const uint64_t later = lane == kWave - 1 ? 0ull : (starts >> (lane + 1));
-        const int len = later ? __ffsll((unsigned long long)later) : kWave - lane;
-        atomicAdd(&bins[b], (uint32_t)len * unit);
+        // the starts of this row of 16 lanes after this lane; none: the run goes to the row's end
+        const uint32_t row = (uint32_t)(starts >> (lane_id() & 48)) & 0xffffu;
+        const uint32_t later = row >> (l15 + 1);
+        const uint32_t len = min(later ? (uint32_t)__builtin_ctz(later) : 31u, (uint32_t)(15 - l15)) + 1u;
+        atomicAdd(&bins[b], len * unit);
     }
 }
 
@@ -238,8 +240,16 @@ inline size_t tile_lds_bytes(int nbins, size_t rec_bytes)
 {
     return tile_bins_bytes(nbins) + (size_t)tile_stage_records(nbins, rec_bytes) * rec_bytes;
 }
+// the stage area also holds a byte per (wavefront, bin) while the items are ranked
+constexpr bool tile_stage_holds_tags(size_t rec_bytes)
+{
+    return ((kTileLdsBytes - ((size_t)(kPartWaves / 2 + 2) * kMaxBins + kTileMisc) * 4) / rec_bytes / kPartThreads *
+            kPartThreads) * rec_bytes >= (size_t)kPartWaves * kMaxBins;
+}
+static_assert(tile_stage_holds_tags(8) && tile_stage_holds_tags(12) && tile_stage_holds_tags(16),
+              "stage area too small for the tag table at the largest number of bins");
 template <typename Rec, typename Base>
-__device__ __forceinline__ int tile_sort(uint32_t *raw, int stage_n, TileLds &L, int nbins, int nbits,
+__device__ __forceinline__ int tile_sort(uint32_t *raw, int stage_n, TileLds &L, int nbins,
                                          const int (&bin)[kItems], int (&lp)[kItems], Base gbase)
 {
     L.stage = raw;
@@ -307,25 +317,38 @@ __device__ __forceinline__ int tile_sort(uint32_t *raw, int stage_n, TileLds &L,
         }
     if (threadIdx.x == kPartThreads - 1) L.misc[kPartWaves] = base;
     __syncthreads();
-    const uint64_t below = lane == 0 ? 0ull : (~0ull >> (kWave - lane));
+    // Lanes of one round with the same bin.  Comparing the bins themselves takes one vote per bit
+    // of the bin (9 to 11); instead every lane leaves its number in a table indexed by bin (the
+    // stage area is idle until the records move) and reads the slot back: lanes of one bin read the
+    // same number, whichever of them wrote last, and telling those numbers apart takes 6 votes.
+    // The LDS executes a wavefront's accesses in order, so the read sees every lane's write.
+    uint8_t *tags = reinterpret_cast<uint8_t *>(L.stage) + w * nbins;
 #pragma unroll
     for (int r = 0; r < kItems; r++) {
         const int b = bin[r];
         const bool valid = b >= 0;
-        uint64_t peers = __ballot(valid);
-        for (int t = 0; t < nbits; t++) {
-            const bool bit = (b >> t) & 1;
-            const uint64_t vote = __ballot(bit);
-            peers &= bit ? vote : ~vote;
+        if (valid) tags[b] = (uint8_t)lane;
+        asm volatile("" ::: "memory");      // the slot is read back from LDS, not from the value just stored
+        const int tag = valid ? tags[b] : 0;
+        // peers: valid lanes of this round with the same bin as this lane, kept as two halves;
+        // m is all ones where the tag's bit is set, so ~(vote ^ m) keeps the lanes that voted alike
+        const uint64_t voters = __ballot(valid);
+        uint32_t plo = (uint32_t)voters, phi = (uint32_t)(voters >> 32);
+#pragma unroll
+        for (int t = 0; t < 6; t++) {
+            const int m = (tag << (31 - t)) >> 31;
+            const uint64_t vote = __ballot(m != 0);
+            plo &= ~((uint32_t)vote ^ (uint32_t)m);
+            phi &= ~((uint32_t)(vote >> 32) ^ (uint32_t)m);
         }
-        // peers: valid lanes of this round with the same bin as this lane
-        const int leader = __ffsll((unsigned long long)peers) - 1;
-        const int rank = __popcll(peers & below);
+        const int rank = (int)__builtin_amdgcn_mbcnt_hi(phi, __builtin_amdgcn_mbcnt_lo(plo, 0u));    // peers in lower lanes
+        // the lane whose number the group read adds the group's size to the bin's counter
         uint32_t old = 0;
-        if (valid && lane == leader) old = atomicAdd(&mine[b], (uint32_t)__popcll(peers) << half);
-        old = __shfl(old, leader < 0 ? 0 : leader, kWave);
+        if (valid && lane == tag) old = atomicAdd(&mine[b], (uint32_t)(__popc(plo) + __popc(phi)) << half);
+        old = __shfl(old, tag, kWave);
         lp[r] = (int)((old >> half) & 0xffff) + rank;
     }
+    __syncthreads();      // the stage area is the records' from here on
     return L.misc[kPartWaves];
 }
 
@@ -360,10 +383,11 @@ template <typename Rec> struct CooLoader {
     int64_t n;
     int32_t V;
     uint32_t omask;     // endpoints from this value up do not pack (0: nothing is packed, LSD passes)
-    // Branch-free: the index is clamped, validity is judged afterwards.
-    __device__ __forceinline__ void load(int64_t e, Rec &r) const
+    // Branch-free: the index is clamped, validity is judged afterwards.  INSIDE: the caller knows
+    // e < n (a tile that ends before the list does), so the addresses are the lane's base plus a constant.
+    template <bool INSIDE = false> __device__ __forceinline__ void load(int64_t e, Rec &r) const
     {
-        const int64_t c = e < n ? e : n - 1;
+        const int64_t c = (INSIDE || e < n) ? e : n - 1;
         r.key = keys[c];
         r.other = others[c];
         r.w = w ? w[c] : 0u;
@@ -377,9 +401,9 @@ template <typename Rec> struct CooLoader {
             }
         }
     }
-    __device__ __forceinline__ bool valid(int64_t e, const Rec &r) const
+    template <bool INSIDE = false> __device__ __forceinline__ bool valid(int64_t e, const Rec &r) const
     {
-        return e < n && (uint32_t)r.key < (uint32_t)V;
+        return (INSIDE || e < n) && (uint32_t)r.key < (uint32_t)V;
     }
 };
 // Loader for the later LSD passes: items are records; only the first *count
@@ -443,7 +467,7 @@ __global__ void csx_unpack_sorted(const Rec *__restrict__ recs, const int32_t *_
 
 template <typename Rec, typename Loader>
 __global__ __launch_bounds__(kPartThreads) void csx_partition(Loader in, int shift, int mask, int nbins,
-                                                              int nbits, const int32_t *__restrict__ table,
+                                                              const int32_t *__restrict__ table,
                                                               int nblocks, Rec *__restrict__ out, int stage_n)
 {
     extern __shared__ uint32_t lds_raw[];
@@ -460,7 +484,7 @@ __global__ __launch_bounds__(kPartThreads) void csx_partition(Loader in, int shi
         bin[r] = in.valid(base + (int64_t)r * kWave, rec[r]) ? ((rec[r].key >> shift) & mask) : -1;
 
     TileLds L;
-    const int total = tile_sort<Rec>(lds_raw, stage_n, L, nbins, nbits, bin, lp,
+    const int total = tile_sort<Rec>(lds_raw, stage_n, L, nbins, bin, lp,
                                      [&](int b) { return table[(int64_t)b * nblocks + blk]; });
     tile_emit(L, total, [&](const Rec &q) { return (q.key >> shift) & mask; }, rec, bin, lp,
               [&](int pos, const Rec &q) { out[pos] = q; });
@@ -468,7 +492,7 @@ __global__ __launch_bounds__(kPartThreads) void csx_partition(Loader in, int shi
 
 // The first partition of the two-level path: same tile sort, the records leave packed.
 template <typename Rec, typename Out>
-__global__ __launch_bounds__(kPartThreads) void csx_partition_pack(CooLoader<Rec> in, PackRule rule, int nbins, int nbits,
+__global__ __launch_bounds__(kPartThreads) void csx_partition_pack(CooLoader<Rec> in, PackRule rule, int nbins,
                                                                    const int32_t *__restrict__ table, int nblocks,
                                                                    Out *__restrict__ out, int stage_n)
 {
@@ -479,13 +503,22 @@ __global__ __launch_bounds__(kPartThreads) void csx_partition_pack(CooLoader<Rec
     const int64_t base = (int64_t)blk * kTile + (int64_t)w * kWaveSpan + lane_id();
     Rec rec[kItems];
     int bin[kItems], lp[kItems];
+    if ((int64_t)(blk + 1) * kTile <= in.n) {
 #pragma unroll
-    for (int r = 0; r < kItems; r++) in.load(base + (int64_t)r * kWave, rec[r]);
+        for (int r = 0; r < kItems; r++) in.template load<true>(base + r * kWave, rec[r]);
 #pragma unroll
-    for (int r = 0; r < kItems; r++) bin[r] = in.valid(base + (int64_t)r * kWave, rec[r]) ? (rec[r].key >> rule.shift) : -1;
+        for (int r = 0; r < kItems; r++)
+            bin[r] = in.template valid<true>(base + r * kWave, rec[r]) ? (rec[r].key >> rule.shift) : -1;
+    } else {
+#pragma unroll
+        for (int r = 0; r < kItems; r++) in.load(base + (int64_t)r * kWave, rec[r]);
+#pragma unroll
+        for (int r = 0; r < kItems; r++)
+            bin[r] = in.valid(base + (int64_t)r * kWave, rec[r]) ? (rec[r].key >> rule.shift) : -1;
+    }
 
     TileLds L;
-    const int total = tile_sort<Rec>(lds_raw, stage_n, L, nbins, nbits, bin, lp,
+    const int total = tile_sort<Rec>(lds_raw, stage_n, L, nbins, bin, lp,
                                      [&](int b) { return table[(int64_t)b * nblocks + blk]; });
     tile_emit(L, total, [&](const Rec &q) { return q.key >> rule.shift; }, rec, bin, lp,
               [&](int pos, const Rec &q) { out[pos] = pack(q, rule); });
@@ -713,7 +746,7 @@ __global__ __launch_bounds__(kPartThreads) void csx_sub_scatter(const Rec *__res
 #pragma unroll
     for (int r = 0; r < kItems; r++) bin[r] = base + r * kWave < sr.end ? view.key_low(rec[r]) : -1;
     TileLds L;
-    const int total = tile_sort<Rec>(lds_raw, stage_n, L, nkeys, shift, bin, lp,
+    const int total = tile_sort<Rec>(lds_raw, stage_n, L, nkeys, bin, lp,
                                      [&](int k) { return cnt2[(int64_t)sub * nkeys + k]; });
     tile_emit(L, total, [&](const Rec &q) { return view.key_low(q); }, rec, bin, lp, [&](int pos, const Rec &q) {
         int32_t other, id;
@@ -872,7 +905,7 @@ static int32_t convert(const int32_t *keys, const int32_t *others, const float *
                 auto part = csx_partition<Rec, CooLoader<Rec>>;
                 allow_lds(part, lds);
                 hipLaunchKernelGGL(part, dim3((nb + 7) / 8 * 8), dim3(kPartThreads), lds, s, in, shift, kMaxBins - 1, kMaxBins,
-                                   kMaxBinBits, table, nblk, dst, stage_n);
+                                   table, nblk, dst, stage_n);
             } else {
                 RecLoader<Rec> in{bufs[(d - 1) & 1], count, E};
                 hipLaunchKernelGGL((csx_digit_histogram<Rec, RecLoader<Rec>>), dim3((nb + 7) / 8 * 8), dim3(kPartThreads), 0, s, in,
@@ -881,7 +914,7 @@ static int32_t convert(const int32_t *keys, const int32_t *others, const float *
                 auto part = csx_partition<Rec, RecLoader<Rec>>;
                 allow_lds(part, lds);
                 hipLaunchKernelGGL(part, dim3((nb + 7) / 8 * 8), dim3(kPartThreads), lds, s, in, shift, kMaxBins - 1, kMaxBins,
-                                   kMaxBinBits, table, nblk, dst, stage_n);
+                                   table, nblk, dst, stage_n);
             }
         }
         hipLaunchKernelGGL((csx_unpack_sorted<Rec, PERM>), dim3((unsigned)ceil_div(E + 1, 256)), dim3(256), 0, s,
@@ -891,8 +924,6 @@ static int32_t convert(const int32_t *keys, const int32_t *others, const float *
         return launch_status("coo_to_csx(lsd)");
     }
 
-    int bbits = 0;
-    while ((1 << bbits) < p.nbuckets) bbits++;
     hipLaunchKernelGGL(csx_bucket_histogram, dim3((nb + 7) / 8 * 8), dim3(kPartThreads), 0, s, keys, E, V, p.shift, p.nbuckets,
                        table, nblk);
     if ((rc = exclusive_scan_i32(table, table, (int64_t)table_n, sums, s))) return rc;
@@ -933,14 +964,14 @@ static int32_t convert(const int32_t *keys, const int32_t *others, const float *
         CooLoader<Rec> in{keys, others, wbits, E, V, rule.omask};
         auto part = csx_partition_pack<Rec, Packed>;
         allow_lds(part, part_lds);
-        hipLaunchKernelGGL(part, dim3((nb + 7) / 8 * 8), dim3(kPartThreads), part_lds, s, in, rule, p.nbuckets, bbits, table, nblk, packed,
+        hipLaunchKernelGGL(part, dim3((nb + 7) / 8 * 8), dim3(kPartThreads), part_lds, s, in, rule, p.nbuckets, table, nblk, packed,
                            tile_stage_records(p.nbuckets, sizeof(Rec)));
         level2(packed, PackedView{rule});
     } else {
         CooLoader<Rec> in{keys, others, wbits, E, V, 0u};
         auto part = csx_partition<Rec, CooLoader<Rec>>;
         allow_lds(part, part_lds);
-        hipLaunchKernelGGL(part, dim3((nb + 7) / 8 * 8), dim3(kPartThreads), part_lds, s, in, p.shift, 0x7fffffff, p.nbuckets, bbits,
+        hipLaunchKernelGGL(part, dim3((nb + 7) / 8 * 8), dim3(kPartThreads), part_lds, s, in, p.shift, 0x7fffffff, p.nbuckets,
                            table, nblk, recs, tile_stage_records(p.nbuckets, sizeof(Rec)));
         level2(recs, PlainView{nkeys - 1});
     }
