@@ -59,8 +59,9 @@ def spmm_compulsory_bytes(R, C, E, feat):
 
 
 def read_profile(name, expect):
-    """Key figures of a rocprofv3 summary under profiles/ ('@key value' lines).  The summary
-    must have been taken on the workload of this run."""
+    """Key figures of a rocprofv3 summary under profiles/ ('@key value' lines), or None when there
+    is no summary or it was taken on another workload than this run's (then the line carries no
+    counted traffic, and says why)."""
     path = os.path.join(ROOT, "profiles", name)
     if not os.path.exists(path):
         return None
@@ -70,9 +71,18 @@ def read_profile(name, expect):
         if m:
             vals[m.group(1)] = m.group(2)
     for key, want in expect.items():
-        if key not in vals or int(float(vals[key])) != int(want):
-            sys.exit("bench.py: %s describes %s=%s, this run has %s=%s; take the counters again "
-                     "(the command is in the file's header)" % (path, key, vals.get(key), key, want))
+        have = int(float(vals[key])) if key in vals else None
+        # The generators call the host's math library; a last-bit difference between two hosts can
+        # move an edge or two.  Up to 0.1 % of the edge count the counted bytes are scaled with it.
+        if key == "E" and have and have != int(want) and abs(have - int(want)) <= 1e-3 * have:
+            if "traffic_bytes" in vals:
+                vals["traffic_bytes"] = str(float(vals["traffic_bytes"]) * int(want) / have)
+            continue
+        if have != int(want):
+            print("bench.py: %s describes %s=%s, this run has %s=%s: its counters are not used; take them "
+                  "again (the command is in the file's header)" % (path, key, vals.get(key), key, want),
+                  file=sys.stderr)
+            return None
     return vals
 
 

@@ -13,6 +13,7 @@ constexpr int kColThreads = 256;
 constexpr int kColStripe = 512;    // rows per block: about 2000 blocks at V = 10^6, eight per CU, to keep enough loads in flight
 constexpr int kColMinStripe = 16;
 constexpr int kColMaxBlocks = 2048;     // more rows per block beyond that: the second stage reads one partial row per block
+constexpr int kColOneStage = 8192;      // up to this many rows the second stage's kernel sums the matrix itself: one launch
 
 // W = floats per lane (1, or 4 when F % 4 == 0 and x is 16-byte aligned): a row is then F / W
 // lanes wide and every load moves 16 bytes.
@@ -83,9 +84,12 @@ __global__ __launch_bounds__(kColThreads) void column_partial_sums(const float *
 // sums are then added in group order.  COLS = 16 keeps a narrow matrix (a few dozen to a few
 // hundred columns, two thousand partial rows) from being two or three blocks' serial work:
 // 128 columns are 8 blocks of 64 groups instead of 2 blocks of 16 (32 -> 9 us at 1954 rows).
-template <int COLS>
+// MASK: the rows are an upstream gradient itself (a matrix of few rows needs no first stage),
+// masked by the ReLU output y as in column_partial_sums.
+template <int COLS, bool MASK = false>
 __global__ __launch_bounds__(1024) void column_final_sums(const float *__restrict__ partial, int nblocks, int F,
-                                                          float *__restrict__ out)
+                                                          float *__restrict__ out, const float *__restrict__ y = nullptr,
+                                                          float *__restrict__ masked = nullptr)
 {
     constexpr int GROUPS = 1024 / COLS;
     __shared__ float part[GROUPS][COLS];
@@ -95,12 +99,22 @@ __global__ __launch_bounds__(1024) void column_final_sums(const float *__restric
     if (col < F) {
         constexpr int kB = 4;               // rows fetched together, added in the same order as one by one
         for (int b0 = grp; b0 < nblocks; b0 += GROUPS * kB) {
-            float v[kB];
+            float v[kB], yv[MASK ? kB : 1];
 #pragma unroll
-            for (int i = 0; i < kB; i++) v[i] = partial[(size_t)min(b0 + GROUPS * i, nblocks - 1) * F + col];
+            for (int i = 0; i < kB; i++) {
+                const size_t at = (size_t)min(b0 + GROUPS * i, nblocks - 1) * F + col;
+                v[i] = partial[at];
+                if constexpr (MASK) yv[i] = y[at];
+            }
 #pragma unroll
             for (int i = 0; i < kB; i++)
-                if (b0 + GROUPS * i < nblocks) s += v[i];
+                if (b0 + GROUPS * i < nblocks) {
+                    if constexpr (MASK) {
+                        v[i] = yv[i] > 0.f ? v[i] : 0.f;
+                        masked[(size_t)(b0 + GROUPS * i) * F + col] = v[i];
+                    }
+                    s += v[i];
+                }
         }
     }
     part[grp][c] = s;
@@ -152,6 +166,13 @@ static int32_t column_sum(const float *x, const float *y, float *masked, float *
     if (!ws || ws_bytes < need) return fail(JGAMD_ERR_WORKSPACE, "column_sum: workspace %zu < %zu bytes", ws ? ws_bytes : (size_t)0, need);
     if (((uintptr_t)ws & 255) != 0) return fail(JGAMD_ERR_ALIGN, "column_sum: workspace not 256-byte aligned");
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (R > 0 && R <= kColOneStage && F <= 2048) {
+        // a few thousand rows (a citation graph's logits): the rows are the "partial rows"
+        const dim3 grid((unsigned)ceil_div(F, 16)), block(1024);
+        if (y) hipLaunchKernelGGL((column_final_sums<16, true>), grid, block, 0, st, x, (int)R, F, out, y, masked);
+        else hipLaunchKernelGGL((column_final_sums<16, false>), grid, block, 0, st, x, (int)R, F, out);
+        return launch_status("column_sum");
+    }
     float *partial = static_cast<float *>(ws);
     const int nblocks = col_blocks(R);
     const int stripe = col_stripe(R);

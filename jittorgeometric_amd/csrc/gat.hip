@@ -283,21 +283,29 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_merge(
 #pragma unroll
                         for (int t = 0; t < NT; t++)
                             if (act[t]) {
+                                // One of the two factors of the running softmax is always 1: the old sums
+                                // shrink by e when the entry raises the maximum, else the entry weighs e
+                                // (e = 0 on a row's first entry, m = -inf).  One exp per entry, and the
+                                // accumulators are scaled in place before the entry is added, which keeps
+                                // each of them in its register.
                                 const float z = sv[u][t] + er_r[t];
-                                const float s = lrelu(z, slope);
-                                const float mn = fmaxf(m[t], s);
-                                const float sc = fast_exp(m[t] - mn);   // 0 on the first entry (m = -inf)
-                                const float p = fast_exp(s - mn);
+                                const bool above = z > 0.f;
+                                const float s = above ? z : slope * z;
+                                const float d = s - m[t];
+                                const float e = fast_exp(-fabsf(d));
+                                const bool up = d > 0.f;
+                                const float sc = up ? e : 1.f, p = up ? 1.f : e;
+                                m[t] = up ? s : m[t];
                                 l[t] = fmaf(l[t], sc, p);
 #pragma unroll
-                                for (int v = 0; v < VEC; v++) acc[t][v] = fmaf(acc[t][v], sc, p * xv[u][t][v]);
+                                for (int v = 0; v < VEC; v++) acc[t][v] = fmaf(p, xv[u][t][v], __fmul_rn(acc[t][v], sc));
                                 if constexpr (POS) {
-                                    const float pp = z > 0.f ? p : 0.f;
+                                    const float pp = above ? p : 0.f;
                                     lp[t] = fmaf(lp[t], sc, pp);
 #pragma unroll
-                                    for (int v = 0; v < VEC; v++) pacc[t][v] = fmaf(pacc[t][v], sc, pp * xv[u][t][v]);
+                                    for (int v = 0; v < VEC; v++)
+                                        pacc[t][v] = fmaf(pp, xv[u][t][v], __fmul_rn(pacc[t][v], sc));
                                 }
-                                m[t] = mn;
                             }
                     }
                 }

@@ -97,7 +97,13 @@ def lognormal_degree(num_nodes, mean_degree, sigma=1.0, seed=0):
     self-loops dropped."""
     rng = np.random.default_rng(seed)
     mu = np.log(mean_degree) - 0.5 * sigma * sigma
-    deg = np.maximum(np.rint(rng.lognormal(mu, sigma, num_nodes)), 0).astype(np.int64)
+    # Normal variates from two uniforms each (Box-Muller), not from the generator's own normal
+    # sampler: that one rejects and redraws on a comparison of library logarithms, so a last-bit
+    # difference between two hosts' math libraries shifts every later draw and the graph comes
+    # out with another edge count.  Here such a difference can only move one degree by one.
+    u1, u2 = rng.random(num_nodes), rng.random(num_nodes)
+    z = np.sqrt(-2.0 * np.log1p(-u1)) * np.cos(2.0 * np.pi * u2)
+    deg = np.maximum(np.rint(np.exp(mu + sigma * z)), 0).astype(np.int64)
     src = np.repeat(np.arange(num_nodes, dtype=np.int32), deg)
     dst = rng.integers(0, num_nodes, src.shape[0], dtype=np.int32)
     keep = src != dst
