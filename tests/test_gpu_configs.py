@@ -4,9 +4,10 @@ the CPU oracle.
 What the oracle can finish in seconds is compared directly: the conversions (bit
 for bit) and, for the products, a sample of output rows that always holds the
 rows with the most entries (the hubs) next to random ones, summed by the oracle's
-own sequential loop over exactly those rows.  Every row is covered by the
-transpose identity <A x, g> = <x, A^T g>, which ties the forward product over the
-CSC arrays to the backward product over the CSR arrays.  Layers are checked by
+own sequential loop over exactly those rows.  Every row of every product is also held to
+float64 sums computed on the GPU with torch operators over the oracle's compressed arrays, and
+the transpose identity <A x, g> = <x, A^T g> ties the forward product over the CSC arrays to
+the backward product over the CSR arrays.  Layers are checked by
 what the reference's call order fixes: a sample of rows of each layer's output
 recomputed by the oracle from that layer's input, equal losses and gradients
 through the two routes a layer offers (SpmmCsr / aggregateWithWeight), finiteness.
@@ -76,6 +77,46 @@ def dot64(a, b, rows=1 << 18):
     return s, t
 
 
+def all_rows_f64(x, idx, off, wt, entries=1 << 20):
+    """Every row of the product in float64 on the GPU, and the sums of the absolute terms: an
+    arbiter that shares nothing with the kernels under test.  The compressed arrays are the
+    oracle's; a slice of entries is multiplied out in float64, summed by a running sum along the
+    entries, and a row's share of the slice is the difference of that running sum between the
+    row's two ends (no atomics, so a row of millions of entries costs what any other does; the
+    running sum's rounding, 1e-16 of at most a slice's total, is far below the 1e-6 allowed)."""
+    V, F = off.shape[0] - 1, x.shape[1]
+    d = dev()
+    off_g = torch.from_numpy(off.astype(np.int64)).to(d)
+    idx_g, w_g = torch.from_numpy(idx.astype(np.int64)).to(d), torch.from_numpy(wt).to(d).double()
+    exact = torch.zeros((V, F), dtype=torch.float64, device=d)
+    terms = torch.zeros((V, F), dtype=torch.float64, device=d)
+    step = max(1, entries * 64 // max(F, 1))
+    zero = torch.zeros((F, 1), dtype=torch.float64, device=d)
+    for s in range(0, idx_g.shape[0], step):
+        n = min(step, idx_g.shape[0] - s)
+        r_lo = int(np.searchsorted(off, s, side="right")) - 1
+        r_hi = int(np.searchsorted(off, s + n - 1, side="right")) - 1
+        pos = (off_g[r_lo:r_hi + 2] - s).clamp_(0, n)
+        # entries along the contiguous dimension: torch's running sum is two orders of magnitude
+        # faster that way round
+        t = (w_g[s:s + n, None] * x[idx_g[s:s + n]].double()).t().contiguous()
+        for acc, val in ((exact, t), (terms, t.abs())):
+            run = torch.cat([zero, val.cumsum(1)], dim=1)
+            acc[r_lo:r_hi + 1] += (run[:, pos[1:]] - run[:, pos[:-1]]).t()
+    return exact, terms
+
+
+def check_all_rows(got, x, idx, off, wt, what):
+    exact, terms = all_rows_f64(x, idx, off, wt)
+    err = (got.double() - exact).abs_()
+    bad = err > 1e-6 + 1e-5 * terms
+    if bad.any():
+        r, c = (int(v) for v in torch.nonzero(bad)[0])
+        raise AssertionError("%s: %d of %d elements out of tolerance, first at row %d col %d: got %r want %r (terms %r)"
+                             % (what, int(bad.sum()), bad.numel(), r, c, float(got[r, c]), float(exact[r, c]),
+                                float(terms[r, c])))
+
+
 def product_checks(name, F, seed):
     """Forward and backward product of one configuration at width F."""
     from jittorgeometric_amd.ops import aggregateWithWeight
@@ -91,6 +132,9 @@ def product_checks(name, F, seed):
     lhs, lscale = dot64(out, g)
     rhs, _ = dot64(gx, x.detach())
     assert abs(lhs - rhs) <= 1e-6 * lscale, "transpose identity %s F=%d: %r vs %r" % (name, F, lhs, rhs)
+    # every row against float64 sums, then a sample of rows against the oracle's own loop
+    check_all_rows(out, x.detach(), *ocsc, what="%s forward F=%d, all rows" % (name, F))
+    check_all_rows(gx, g, *ocsr, what="%s backward F=%d, all rows" % (name, F))
     x_h, g_h = x.detach().cpu().numpy(), g.cpu().numpy()
     for label, got, src, (idx, off, wt) in (("forward", out, x_h, ocsc), ("backward", gx, g_h, ocsr)):
         rows = sample_rows(off, seed)
