@@ -323,6 +323,8 @@ def config2(b):
     if args.calibrate_copy:
         b.calibrate_copy()
 
+    if args.part == "softmax":
+        return config2_softmax(b, csc, V, E), 0.0
     step = lambda: spmm(csc.column_offset, csc.row_indices, csc.edge_weight, x, V)
     bytes_step = spmm_bytes(V, E, F)
     setup_ms = None
@@ -443,6 +445,46 @@ def config2(b):
                                        "the same SpMM workload (V=%d, E=%d, F=%d)" % (V, E, F))
     line["cpu_baseline"] = cpu
     return line, err
+
+
+def config2_softmax(b, csc, V, E):
+    """Only the standalone edge softmax on config 2's graph, forward and backward at 1 and 8 heads
+    (what profiles/edge_softmax_powerlaw_1m.txt is taken from).  Times are of the operator's
+    C entry points through the wrappers, without autograd's dispatch."""
+    from jittorgeometric_amd.ops import EdgeSoftmax
+    from jittorgeometric_amd.ops.edgesoftmax import EdgeSoftmaxFunc
+    torch, args, dev = b.torch, b.args, b.dev
+    iters, warm = max(args.steps, 5), args.warmup
+    out = {}
+
+    class Ctx:      # what EdgeSoftmaxFunc.backward reads from its context
+        pass
+    for H in (1, 8):
+        x = torch.randn(E, H, device=dev)
+        g = torch.randn(E, H, device=dev)
+        y = EdgeSoftmax(x, csc)
+        fwd = b.timed(lambda: EdgeSoftmax(x, csc), iters, warm)
+        ctx = Ctx()
+        ctx.saved_tensors, ctx.csc = (y,), csc
+        bwd = b.timed(lambda: EdgeSoftmaxFunc.backward(ctx, g), iters, warm)
+        fb, bb = 8 * E * H + 4 * (V + 1), 12 * E * H + 4 * (V + 1)
+        out["edge_softmax_h%d_fwd_ms" % H] = round(fwd, 4)
+        out["edge_softmax_h%d_fwd_frac_hbm_peak" % H] = round(fb / (fwd * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)
+        out["edge_softmax_h%d_bwd_ms" % H] = round(bwd, 4)
+        out["edge_softmax_h%d_bwd_frac_hbm_peak" % H] = round(bb / (bwd * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)
+        del x, g, y
+    ms = out["edge_softmax_h1_fwd_ms"]
+    line = base_line(args, "edge_softmax_fwd_ms", ms, "ms", ms, False,
+                     "config 2 graph, standalone edge softmax over the CSC columns, [E,1] and [E,8] logits",
+                     {"V": V, "E": E})
+    line.update(out)
+    line["roofline"] = {"bound": "hbm", "peak": HBM_PEAK_GBPS, "unit": "GB/s", "kernel": "esm_fwd_tile + esm_merge + esm_finish",
+                        "algorithmic_bytes": 8 * E + 4 * (V + 1),
+                        "achieved": round((8 * E + 4 * (V + 1)) / (ms * 1e-3) / 1e9, 1),
+                        "frac": out["edge_softmax_h1_fwd_frac_hbm_peak"], "traffic": None,
+                        "achieved_basis": "algorithmic bytes / operator time"}
+    line["cpu_baseline"] = None
+    return line
 
 
 # --------------------------------------------------------------------------------- config 1
@@ -730,14 +772,14 @@ def main():
     ap.add_argument("--config", type=int, default=2, choices=[1, 2, 3, 4, 5],
                     help="benchmark configuration; 2 (the headline SpMM workload) is the default")
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the single-thread CPU timing")
-    ap.add_argument("--part", default="all", choices=["all", "main", "layers"],
+    ap.add_argument("--part", default="all", choices=["all", "main", "layers", "softmax"],
                     help="main: only the timed workload of the metric (what the counter profiles under profiles/ "
                          "are taken from); layers: only the GCN and GraphSAGE layer steps of config 2")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (known traffic, for scaling rocprof counters)")
     args = ap.parse_args()
-    if args.part == "layers" and args.config != 2:
-        sys.exit("bench.py: --part layers belongs to --config 2")
+    if args.part in ("layers", "softmax") and args.config != 2:
+        sys.exit("bench.py: --part %s belongs to --config 2" % args.part)
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only; --gpus %d is not supported "
                  "(no collectives or sharding are part of it)" % args.gpus)
