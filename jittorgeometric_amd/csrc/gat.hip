@@ -125,6 +125,12 @@ __global__ __launch_bounds__(256) void gat_node_scores_vec(const float4 *__restr
     }
 }
 
+// The value lane CTRL (0x00, 0x55, 0xAA, 0xFF = 0, 1, 2, 3) of every quad holds, in all four lanes.
+template <int CTRL> __device__ __forceinline__ float quad_lane(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+
 // Sum of v over aligned groups of `lanes` consecutive lanes (a power of two), left in every
 // lane of the group.  Up to 16 lanes the exchanges are DPP modifiers on the adds (quad
 // permutes, then the half-row and row mirrors); only 32 and 64 go through the LDS crossbar.
@@ -607,7 +613,7 @@ __global__ __launch_bounds__(256) void gat_bwd_node_stats_vec(const float *__res
 // ends the row is stored as it is in g_h / g_el_row, and gat_bwd_fixup adds everything up.
 // lph = lanes per head (power of two) when H > 1; for H == 1 the whole
 // wavefront (all tiles) reduces into the single head.
-template <int VEC, int NT>
+template <int VEC, int NT, bool QUADS>
 __global__ __launch_bounds__(kGatThreads) void gat_bwd_merge(
     const int32_t *__restrict__ t_off, const int32_t *__restrict__ t_idx,
     const float *__restrict__ h, const float *__restrict__ el, const float4 *__restrict__ stat,
@@ -640,6 +646,7 @@ __global__ __launch_bounds__(kGatThreads) void gat_bwd_merge(
         lead[t] = act[t] && (f % D == 0);
         fo[t] = act[t] ? f : 0;
     }
+    constexpr bool quads = QUADS;      // the lanes of a head are whole quads (D a multiple of 4 VEC)
     // this wavefront's share of the gradients of a_src and a_dst
     float pas[NT][VEC], pad[NT][VEC];
 #pragma unroll
@@ -741,7 +748,13 @@ __global__ __launch_bounds__(kGatThreads) void gat_bwd_merge(
             }
             for (int i0 = 0; i0 < n; i0 += kGatUnroll) {
                 float gv[kGatUnroll][NT][VEC];
-                float3 st[kGatUnroll][NT];          // (er, smax + log ssum, g.out) of the destination
+                // (er, smax + log ssum, g.out) of the destination and head: one float per lane, the
+                // lane's number inside its quad choosing which (a head's lanes are whole quads when
+                // quads holds; the three values are spread over the quad when they are used).  Twelve
+                // bytes per lane instead cost the address unit three times as long per entry, more
+                // than the 512-byte row gathered beside them.
+                float sq[QUADS ? kGatUnroll : 1][QUADS ? NT : 1];
+                float3 st[QUADS ? 1 : kGatUnroll][QUADS ? 1 : NT];
 #pragma unroll
                 for (int u = 0; u < kGatUnroll; u++) {
                     const int c = max(bcast_i(my_c, (i0 + u) & (kWave - 1)), 0);
@@ -750,7 +763,8 @@ __global__ __launch_bounds__(kGatThreads) void gat_bwd_merge(
 #pragma unroll
                     for (int t = 0; t < NT; t++) {
                         gload<VEC>(gv[u][t], src + fo[t]);
-                        st[u][t] = *reinterpret_cast<const float3 *>(ss + head[t]);
+                        if constexpr (quads) sq[u][t] = reinterpret_cast<const float *>(ss + head[t])[lane & 3];
+                        else st[u][t] = *reinterpret_cast<const float3 *>(ss + head[t]);
                     }
                 }
 #pragma unroll
@@ -781,15 +795,24 @@ __global__ __launch_bounds__(kGatThreads) void gat_bwd_merge(
                                 for (int t = 0; t < NT; t++) dot[t] = lane_group_sum(dot[t], lph);
                             }
 #pragma unroll
-                            for (int t = 0; t < NT; t++)
+                            for (int t = 0; t < NT; t++) {
+                                float3 sv;
+                                if constexpr (quads) {
+                                    sv.x = quad_lane<0x00>(sq[u][t]);
+                                    sv.y = quad_lane<0x55>(sq[u][t]);
+                                    sv.z = quad_lane<0xAA>(sq[u][t]);
+                                } else {
+                                    sv = st[u][t];
+                                }
                                 if (act[t]) {
-                                    const float z = el_r[t] + st[u][t].x;
-                                    const float alpha = fast_exp(lrelu(z, slope) - st[u][t].y);
-                                    const float gz = alpha * (dot[t] - st[u][t].z) * (z > 0.f ? 1.f : slope);
+                                    const float z = el_r[t] + sv.x;
+                                    const float alpha = fast_exp(lrelu(z, slope) - sv.y);
+                                    const float gz = alpha * (dot[t] - sv.z) * (z > 0.f ? 1.f : slope);
                                     gel[t] += gz;
 #pragma unroll
                                     for (int v = 0; v < VEC; v++) acc[t][v] = fmaf(alpha, gv[u][t][v], acc[t][v]);
                                 }
+                            }
                         }
                     }
                 }
@@ -1269,9 +1292,14 @@ JG_EXPORT int32_t jgamd_gat_bwd(const void *t_plan, int32_t n_fix, int32_t n_grp
     const dim3 fgrid(listed ? gat_list_grid(n_fix, s.nchunks) : grid.x);
 #define JG_BWD(VV, NN)                                                                                             \
     case VV * 16 + NN:                                                                                             \
-        hipLaunchKernelGGL((gat_bwd_merge<VV, NN>), grid, block, 0, st, t_off, t_idx, h, el, stat, g_er, g_out,    \
-                           a_src, a_dst, slope, g_h, g_el_row, partial, pel, red, pv.start, V, (int)E, H, D,       \
-                           s.lph, s.nchunks);                                                                      \
+        if (D % (4 * VV) == 0)                                                                                     \
+            hipLaunchKernelGGL((gat_bwd_merge<VV, NN, true>), grid, block, 0, st, t_off, t_idx, h, el, stat, g_er, \
+                               g_out, a_src, a_dst, slope, g_h, g_el_row, partial, pel, red, pv.start, V, (int)E,  \
+                               H, D, s.lph, s.nchunks);                                                            \
+        else                                                                                                       \
+            hipLaunchKernelGGL((gat_bwd_merge<VV, NN, false>), grid, block, 0, st, t_off, t_idx, h, el, stat,      \
+                               g_er, g_out, a_src, a_dst, slope, g_h, g_el_row, partial, pel, red, pv.start, V,    \
+                               (int)E, H, D, s.lph, s.nchunks);                                                    \
         if (ngroups > 1 && n_grp != 0 && n_fix != 0)                                                               \
             hipLaunchKernelGGL((gat_bwd_group<VV, NN>), ggrid, block, 0, st, t_off, partial, pel, gvec, ggel,      \
                                pv.start, pv.grp, pv.counts + 1, V, H, D, s.chunk, s.nchunks);                      \
