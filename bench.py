@@ -325,6 +325,28 @@ def config2(b):
 
     if args.part == "softmax":
         return config2_softmax(b, csc, V, E), 0.0
+    if args.part == "convert":
+        # only the two conversions of the normalised edge list (what profiles/coo_to_csx_powerlaw_1m.txt
+        # is taken from)
+        from jittorgeometric_amd.ops import cootocsr
+        iters, warm = max(args.steps, 10), args.warmup
+        csr_ms = b.timed(lambda: cootocsr(ei, w, V), iters, warm)
+        csc_ms = b.timed(lambda: cootocsc(ei, w, V), iters, warm)
+        conv_bytes = 24 * E + 8 * (V + 1)
+        line = base_line(args, "coo_to_csr_edges_per_s", round(E / (csr_ms * 1e-3)), "edges/s", csr_ms, True,
+                         "config 2: cootocsr / cootocsc of the gcn_norm edge list, V=1,000,000, E=%d" % E,
+                         {"V": V, "E": E})
+        line.update({"coo_to_csr_ms": round(csr_ms, 4), "coo_to_csc_ms": round(csc_ms, 4),
+                     "coo_to_csr_ms_event_median": round(csr_ms.median, 4),
+                     "coo_to_csc_edges_per_s": round(E / (csc_ms * 1e-3)),
+                     "roofline": {"bound": "hbm", "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                                  "kernel": "csx_partition_pack + csx_sub_scatter (+ 7 short kernels)",
+                                  "algorithmic_bytes": conv_bytes,
+                                  "achieved": round(conv_bytes / (csr_ms * 1e-3) / 1e9, 1),
+                                  "frac": round(conv_bytes / (csr_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                                  "traffic": None, "achieved_basis": "algorithmic bytes / operator time"},
+                     "cpu_baseline": None})
+        return line, 0.0
     step = lambda: spmm(csc.column_offset, csc.row_indices, csc.edge_weight, x, V)
     bytes_step = spmm_bytes(V, E, F)
     setup_ms = None
@@ -772,13 +794,13 @@ def main():
     ap.add_argument("--config", type=int, default=2, choices=[1, 2, 3, 4, 5],
                     help="benchmark configuration; 2 (the headline SpMM workload) is the default")
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the single-thread CPU timing")
-    ap.add_argument("--part", default="all", choices=["all", "main", "layers", "softmax"],
+    ap.add_argument("--part", default="all", choices=["all", "main", "layers", "softmax", "convert"],
                     help="main: only the timed workload of the metric (what the counter profiles under profiles/ "
                          "are taken from); layers: only the GCN and GraphSAGE layer steps of config 2")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (known traffic, for scaling rocprof counters)")
     args = ap.parse_args()
-    if args.part in ("layers", "softmax") and args.config != 2:
+    if args.part in ("layers", "softmax", "convert") and args.config != 2:
         sys.exit("bench.py: --part %s belongs to --config 2" % args.part)
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only; --gpus %d is not supported "
