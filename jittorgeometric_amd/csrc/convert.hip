@@ -133,6 +133,28 @@ struct PlainView {
     }
 };
 
+// A record out of an array, field by field for the 16-byte kind: copied as one aligned block, a
+// lane's sixteen of them stayed in scratch memory (272 bytes per lane) instead of registers.  The
+// kernels take the same time either way (more registers, fewer wavefronts); without scratch
+// memory no launch of this library makes the runtime set any aside.
+template <typename Rec> __device__ __forceinline__ Rec read_rec(const Rec *p) { return *p; }
+template <> __device__ __forceinline__ Rec4 read_rec<Rec4>(const Rec4 *p)
+{
+    const uint4 q = *reinterpret_cast<const uint4 *>(p);
+    Rec4 r;
+    r.key = (int32_t)q.x;
+    r.other = (int32_t)q.y;
+    r.w = q.z;
+    r.id = (int32_t)q.w;
+    return r;
+}
+
+template <typename Rec> __device__ __forceinline__ void write_rec(Rec *p, const Rec &r) { *p = r; }
+template <> __device__ __forceinline__ void write_rec<Rec4>(Rec4 *p, const Rec4 &r)
+{
+    *reinterpret_cast<uint4 *>(p) = make_uint4((uint32_t)r.key, (uint32_t)r.other, r.w, (uint32_t)r.id);
+}
+
 template <bool PERM> struct RecOf { using type = Rec3; };
 template <> struct RecOf<true> { using type = Rec4; };
 
@@ -360,12 +382,12 @@ __device__ __forceinline__ void tile_emit(const TileLds &L, int total, BinOfRec 
     for (int h0 = 0; h0 < total; h0 += L.stage_n) {
 #pragma unroll
         for (int r = 0; r < kItems; r++)
-            if (bin[r] >= 0 && (unsigned)(lp[r] - h0) < (unsigned)L.stage_n) stage[lp[r] - h0] = rec[r];
+            if (bin[r] >= 0 && (unsigned)(lp[r] - h0) < (unsigned)L.stage_n) write_rec(stage + (lp[r] - h0), rec[r]);
         __syncthreads();
         const int n = min(total - h0, L.stage_n);
 #pragma unroll 4
         for (int j = threadIdx.x; j < n; j += kPartThreads) {
-            const Rec q = stage[j];
+            const Rec q = read_rec(stage + j);
             emit(L.delta[bin_of_rec(q)] + h0 + j, q);
         }
         __syncthreads();
@@ -412,7 +434,7 @@ template <typename Rec> struct RecLoader {
     const Rec *recs;
     const int32_t *count;
     int64_t cap;      // upper bound of *count (> 0)
-    __device__ __forceinline__ void load(int64_t e, Rec &r) const { r = recs[e < cap ? e : cap - 1]; }
+    __device__ __forceinline__ void load(int64_t e, Rec &r) const { r = read_rec(recs + (e < cap ? e : cap - 1)); }
     __device__ __forceinline__ bool valid(int64_t e, const Rec &) const { return e < (int64_t)*count; }
 };
 
@@ -487,7 +509,7 @@ __global__ __launch_bounds__(kPartThreads) void csx_partition(Loader in, int shi
     const int total = tile_sort<Rec>(lds_raw, stage_n, L, nbins, bin, lp,
                                      [&](int b) { return table[(int64_t)b * nblocks + blk]; });
     tile_emit(L, total, [&](const Rec &q) { return (q.key >> shift) & mask; }, rec, bin, lp,
-              [&](int pos, const Rec &q) { out[pos] = q; });
+              [&](int pos, const Rec &q) { write_rec(out + pos, q); });
 }
 
 // The first partition of the two-level path: same tile sort, the records leave packed.
@@ -742,7 +764,7 @@ __global__ __launch_bounds__(kPartThreads) void csx_sub_scatter(const Rec *__res
     Rec rec[kItems];
     int bin[kItems], lp[kItems];
 #pragma unroll
-    for (int r = 0; r < kItems; r++) rec[r] = recs[min(base + r * kWave, sr.end - 1)];
+    for (int r = 0; r < kItems; r++) rec[r] = read_rec(recs + min(base + r * kWave, sr.end - 1));
 #pragma unroll
     for (int r = 0; r < kItems; r++) bin[r] = base + r * kWave < sr.end ? view.key_low(rec[r]) : -1;
     TileLds L;
@@ -758,15 +780,64 @@ __global__ __launch_bounds__(kPartThreads) void csx_sub_scatter(const Rec *__res
     });
 }
 
-// Expands compressed offsets into one row id per entry (for the transpose).
-__global__ void csx_expand_rows(const int32_t *__restrict__ off, int32_t R, int32_t *__restrict__ rows)
+// Expands compressed offsets into one row id per entry (for the transpose).  A block takes a tile
+// of kTileEntriesNarrow entries; the rows of its first and last entry come from the tile -> row
+// map (plan.hip), their offsets are staged in LDS, a thread finds the row of its first entry by
+// bisection there and walks on from it, and stores its four row ids as 16 bytes.  (One wavefront
+// per row, the first form of this kernel, wrote 0.3 TB/s on rows of a few dozen entries.)
+// Entries past off[R] belong to no row and get row 0.
+constexpr int kExpandSlots = 4;
+__global__ __launch_bounds__(256) void csx_expand_rows(const int32_t *__restrict__ off,
+                                                       const int32_t *__restrict__ tile_first,
+                                                       const int32_t *__restrict__ tile_last, int32_t R, int64_t E,
+                                                       int32_t *__restrict__ rows)
 {
-    // one wave per row keeps long rows coalesced; short rows cost one store
-    const int wave = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-    const int nwaves = gridDim.x * (blockDim.x >> 6);
-    for (int r = wave; r < R; r += nwaves) {
-        const int s = off[r], e = off[r + 1];
-        for (int j = s + lane_id(); j < e; j += kWave) rows[j] = r;
+    typedef int i32x4 __attribute__((ext_vector_type(4)));
+    constexpr int T = kTileEntriesNarrow;
+    static_assert(T == 256 * kExpandSlots, "one tile per block");
+    __shared__ int s_off[T + 2];
+    const int tile = blockIdx.x;
+    const int64_t t0 = (int64_t)tile * T;
+    const int covered = min(max(off[R], 0), (int)E);
+    const int64_t j0 = t0 + (int64_t)threadIdx.x * kExpandSlots;
+    if (t0 >= covered) {
+        for (int k = 0; k < kExpandSlots; k++)
+            if (j0 + k < E) rows[j0 + k] = 0;
+        return;
+    }
+    const int c_lo = min(max(tile_first[tile], 0), R - 1);
+    const int c_hi = min(max(tile_last[tile], c_lo), R - 1);
+    const int ncol = c_hi - c_lo + 1;
+    const bool staged = ncol + 1 <= T + 2;
+    if (staged)
+        for (int i = threadIdx.x; i <= ncol; i += 256) s_off[i] = off[c_lo + i];
+    __syncthreads();
+    auto offv = [&](int c) { return staged ? s_off[c - c_lo] : off[c]; };
+    const int last = covered - 1;
+    const int jc = (int)min(j0, (int64_t)last);
+    int lo = c_lo, hi = c_hi;
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (offv(mid) <= jc) lo = mid;
+        else hi = mid - 1;
+    }
+    int c = lo, ce = offv(c + 1);
+    i32x4 r;
+#pragma unroll
+    for (int k = 0; k < kExpandSlots; k++) {
+        const int64_t j = j0 + k;
+        while (ce <= j && c < c_hi) {
+            c++;
+            ce = offv(c + 1);
+        }
+        r[k] = j > last ? 0 : c;
+    }
+    if (j0 + kExpandSlots <= E) {
+        *reinterpret_cast<i32x4 *>(rows + j0) = r;      // rows is carved 256-byte aligned, j0 a multiple of 4
+    } else {
+#pragma unroll
+        for (int k = 0; k < kExpandSlots; k++)
+            if (j0 + k < E) rows[j0 + k] = r[k];
     }
 }
 
@@ -1027,7 +1098,9 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_coo_to_csx(const
 
 static size_t transpose_ws_bytes(int64_t E, int32_t C)
 {
-    return carve_bytes((size_t)E, 4) + conv_ws_bytes(E, C, true);
+    // row of every entry, the tile -> row map it is made from, the conversion's own scratch
+    return carve_bytes((size_t)E, 4) + 2 * carve_bytes((size_t)ceil_div(E > 0 ? E : 1, kTileEntriesNarrow), 4) +
+           conv_ws_bytes(E, C, true);
 }
 
 extern "C" __attribute__((visibility("default"))) int32_t jgamd_csx_transpose_workspace(int64_t E, int32_t R, int32_t C, size_t *bytes)
@@ -1052,10 +1125,13 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_csx_transpose(co
     hipStream_t s = static_cast<hipStream_t>(stream);
     Carver carve(ws);
     int32_t *rows = carve.take<int32_t>((size_t)E);
+    const size_t ntiles = (size_t)ceil_div(E > 0 ? E : 1, kTileEntriesNarrow);
+    int32_t *tile_first = carve.take<int32_t>(ntiles), *tile_last = carve.take<int32_t>(ntiles);
     void *inner = carve.base + carve.used;
     if (E > 0 && R > 0) {
-        int blocks = (int)(ceil_div(R, 4) < 65536 ? ceil_div(R, 4) : 65536);
-        hipLaunchKernelGGL(csx_expand_rows, dim3(blocks), dim3(256), 0, s, off, R, rows);
+        tile_columns_enqueue(off, R, E, kTileEntriesNarrow, tile_first, tile_last, s);
+        hipLaunchKernelGGL(csx_expand_rows, dim3((unsigned)ntiles), dim3(256), 0, s, off, tile_first, tile_last, R, E,
+                           rows);
     }
     return out_perm ? convert<true>(idx, rows, w, E, C, out_idx, out_off, out_w, out_perm, inner, s)
                     : convert<false>(idx, rows, w, E, C, out_idx, out_off, out_w, out_perm, inner, s);
