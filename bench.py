@@ -197,7 +197,7 @@ class Bench:
                                                         ctypes.byref(c_ms)))
             return k_ms.value, c_ms.value
         from jittorgeometric_amd.ops._common import PLAN_SPMM, csx_plan
-        plan, n_fix, n_grp = csx_plan(off, R, E, PLAN_SPMM)       # the partition the operators keep with the offsets
+        plan, n_fix, n_grp = csx_plan(off, R, E, PLAN_SPMM, now=True)       # the partition the operators keep with the offsets
         nbytes = _lib.query(lib.jgamd_spmm_csx_planned_workspace, R, E, F)
         ws = _lib.workspace(nbytes, self.dev)
         torch.cuda.synchronize()

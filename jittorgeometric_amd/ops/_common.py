@@ -117,14 +117,20 @@ def transposed_inverse(holder, perm):
 PLAN_SPMM, PLAN_GAT, PLAN_TILES = 0, 1, 2
 
 
-def csx_plan(off, R, E, kind):
+def csx_plan(off, R, E, kind, now=False):
     """(plan, n_fix, n_grp) for the offsets `off` of R rows and E entries: the partition the
-    merge-path kernels (PLAN_SPMM, PLAN_GAT) or the tile kernels (PLAN_TILES) work from, built
-    on first use and kept on the offsets tensor until it is written in place (a rebound
-    attribute is another tensor and gets its own).  The two counts are the lengths of the
-    plan's lists of cut rows, read back once when the plan is built; 0 lets a call skip the
-    kernels that add up row pieces.  Returns (None, -1, -1) while a HIP graph is being captured
-    and no plan exists yet: building one would allocate from the graph's pool and read back."""
+    merge-path kernels (PLAN_SPMM, PLAN_GAT) or the tile kernels (PLAN_TILES) work from, kept on
+    the offsets tensor until it is written in place (a rebound attribute is another tensor and
+    gets its own).  The two counts are the lengths of the plan's lists of cut rows, read back
+    once when the plan is built; 0 lets a call skip the kernels that add up row pieces.
+
+    A chunk plan costs two launches and that read-back, a synchronisation with the device, so it
+    is built on the second use of the same offsets (or at once with now=True): the graph of a
+    training run is used thousands of times, the sampled subgraph of a mini-batch once, and its
+    one call takes the entry point that partitions on the fly.  A tile plan costs the one launch
+    an unplanned call makes anyway and is built on first use.  Returns (None, -1, -1) when there
+    is no plan (yet), also while a HIP graph is being captured: building one would allocate from
+    the graph's pool and read back.  Planned and unplanned calls give the same bits."""
     cache = getattr(off, "_jgamd_plans", None)
     if cache is None:
         cache = {}
@@ -134,6 +140,9 @@ def csx_plan(off, R, E, kind):
     if hit is not None and hit[0] == stamp:
         return hit[1], hit[2], hit[3]
     if torch.cuda.is_current_stream_capturing():
+        return None, -1, -1
+    if kind != PLAN_TILES and not now and cache.get(("seen", kind)) != stamp:
+        cache[("seen", kind)] = stamp
         return None, -1, -1
     lib = _lib.load()
     dev = off.device

@@ -283,16 +283,21 @@ def test_wrappers_keep_one_plan_per_offsets_and_rebuild_it_when_they_change():
     x = to_gpu(rng.standard_normal((V, F)).astype(np.float32))
     out1 = aggregateWithWeight(x, csc, None)
     off_g = csc_arrays(csc)[0]
+    # the first call partitions on the fly; the plan is built when the same offsets come again
+    assert "_jgamd_plans" in off_g.__dict__ and PLAN_SPMM not in off_g._jgamd_plans
+    assert torch.equal(aggregateWithWeight(x, csc, None), out1)
+    assert PLAN_SPMM in off_g._jgamd_plans
     p1 = csx_plan(off_g, V, E, PLAN_SPMM)
-    assert csx_plan(off_g, V, E, PLAN_SPMM)[0] is p1[0]                 # kept
+    assert p1[0] is not None and csx_plan(off_g, V, E, PLAN_SPMM)[0] is p1[0]      # kept
     assert torch.equal(aggregateWithWeight(x, csc, None), out1)
     # the same arrays regrouped: column 0 gives its entries to column 1 (offsets written in place)
     new_off = off.copy()
     new_off[1] = 0
     csc.column_offset.copy_(to_gpu(new_off))
     out2 = aggregateWithWeight(x, csc, None)
-    p2 = csx_plan(csc_arrays(csc)[0], V, E, PLAN_SPMM)
-    assert p2[0] is not p1[0]                                           # rebuilt
+    assert torch.equal(aggregateWithWeight(x, csc, None), out2)         # without a plan, then with the new one
+    p2 = csx_plan(csc_arrays(csc)[0], V, E, PLAN_SPMM, now=True)
+    assert p2[0] is not None and p2[0] is not p1[0]                     # rebuilt
     want, terms = oracle.aggregate_f64(x.cpu().numpy(), idx, new_off, wt)
     assert_close(out2.cpu().numpy(), want, terms, what="after the offsets changed in place")
     # a rebound attribute is another tensor with its own plan
