@@ -230,7 +230,9 @@ __global__ __launch_bounds__(kLongThreads) void edge_softmax_bwd_long(const int3
     long_walk2(y, g, s, e, [&](int64_t p, float yv, float gv) { dx[p] = yv * gv - yv * dot; });
 }
 
-// Any H (not a power of two, or above 64): one thread per (column, head).
+// Any H (not a power of two, or above 64): one thread per (column, head).  The thread adds a
+// column's terms one after the other, as the reference's loop does, but in double: a column of
+// 10^4 entries would otherwise be 10^4 roundings away from the sum the tile kernels compute.
 __global__ void edge_softmax_fwd_any(const int32_t *__restrict__ off, const float *__restrict__ x,
                                      float *__restrict__ y, int V, int H)
 {
@@ -240,8 +242,9 @@ __global__ void edge_softmax_fwd_any(const int32_t *__restrict__ off, const floa
     const int s = off[c], e = off[c + 1];
     float m = -INFINITY;
     for (int j = s; j < e; j++) m = fmaxf(m, x[(int64_t)j * H + h]);
-    float t = 0.f;
-    for (int j = s; j < e; j++) t += expf(x[(int64_t)j * H + h] - m);
+    double sum = 0.0;
+    for (int j = s; j < e; j++) sum += (double)expf(x[(int64_t)j * H + h] - m);
+    const float t = (float)sum;
     for (int j = s; j < e; j++) y[(int64_t)j * H + h] = expf(x[(int64_t)j * H + h] - m) / t;
 }
 
@@ -252,8 +255,9 @@ __global__ void edge_softmax_bwd_any(const int32_t *__restrict__ off, const floa
     if (i >= (int64_t)V * H) return;
     const int c = (int)(i / H), h = (int)(i % H);
     const int s = off[c], e = off[c + 1];
-    float dot = 0.f;
-    for (int j = s; j < e; j++) dot += y[(int64_t)j * H + h] * g[(int64_t)j * H + h];
+    double sum = 0.0;
+    for (int j = s; j < e; j++) sum += (double)y[(int64_t)j * H + h] * (double)g[(int64_t)j * H + h];
+    const float dot = (float)sum;
     for (int j = s; j < e; j++) {
         const int64_t p = (int64_t)j * H + h;
         dx[p] = y[p] * g[p] - y[p] * dot;
