@@ -605,7 +605,7 @@ static int32_t spmm_call(const int32_t *off, const int32_t *idx, const float *w,
                          int32_t R, int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, void *stream,
                          hipEvent_t k0, hipEvent_t k1, const RowFinish *fin = nullptr, bool narrow_slabs = false,
                          int x_stride = 0, const void *plan = nullptr, const void *tiles = nullptr,
-                         PlanHints hints = PlanHints())
+                         PlanHints hints = PlanHints(), bool planned_call = false)
 {
     if (int32_t rc = check_spmm_sizes(R, E, F)) return rc;
     if (C < 0) return fail(JGAMD_ERR_SIZE, "spmm_csx: negative C");
@@ -622,6 +622,10 @@ static int32_t spmm_call(const int32_t *off, const int32_t *idx, const float *w,
     }();
     const bool narrow_route = !fin && !k0 && !narrow_off && x_stride == 0 && E > 0 && narrow_width(F) &&
                               narrow_spmm_supported(F, x) && (tiles || !plan);
+    // a planned call that brought the tile plan only: the tile kernels must be able to take it
+    if (planned_call && !plan && !narrow_route)
+        return fail(JGAMD_ERR_NULL, "spmm_csx_planned: this product (F=%d%s) takes the chunk kernels: pass the chunk plan, "
+                    "not only the tile plan", F, fin ? ", with a row finish" : "");
     const size_t need = narrow_route ? entry_tiles_ws_bytes(E) : spmm_scratch_bytes(R, E, F, plan == nullptr);
     if (!ws || ws_bytes < need)
         return fail(JGAMD_ERR_WORKSPACE, "spmm_csx: workspace %zu < %zu bytes", ws ? ws_bytes : (size_t)0, need);
@@ -712,7 +716,7 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_planned
     const bool plain = beta == 1.f && (alpha == 0.f || !h) && flags == 0;
     const RowFinish fin{beta, alpha, alpha != 0.f ? h : nullptr, h_rows == 1 ? 0 : F, 0, (flags & JGAMD_ROW_RELU) ? 1 : 0};
     return spmm_call(off, idx, w, x, out, R, C, E, F, ws, ws_bytes, stream, nullptr, nullptr, plain ? nullptr : &fin,
-                     false, 0, plan, tiles, hints);
+                     false, 0, plan, tiles, hints, true);
 }
 
 extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_planned_workspace(int32_t R, int64_t E,

@@ -1,5 +1,6 @@
 """Helpers shared by the operator wrappers."""
 import ctypes as _c
+import os
 
 import torch
 
@@ -225,8 +226,11 @@ def _product(off, idx, w, x, R, beta, alpha, h, relu=False):
                                               _lib.ptr(ws), nbytes, stream))
         return out.relu_() if relu else out
     # the partition of the rows is kept with the offsets: the chunk plan, or the tile plan for
-    # rows of 1, 2, 4 or 8 floats
-    narrow = F in (1, 2, 4, 8) and E > 0
+    # plain products with rows of 1, 2, 4 or 8 floats (the tile kernels have no row finish and
+    # read whole aligned rows)
+    plain = h is None and beta == 1.0 and not relu
+    narrow = (F in (1, 2, 4, 8) and E > 0 and plain and x.data_ptr() % min(16, 4 * F) == 0
+              and not os.environ.get("JGAMD_SPMM_NARROW", "").startswith("m"))
     plan, n_fix, n_grp = csx_plan(off, R, E, PLAN_TILES if narrow else PLAN_SPMM) if R > 0 else (None, -1, -1)
     if plan is not None:
         nbytes = _lib.query(lib.jgamd_spmm_csx_planned_workspace, R, E, F)

@@ -240,6 +240,37 @@ def test_narrow_rows_with_a_tile_plan(case, F):
     assert (got.cpu().numpy()[np.diff(off) == 0] == 0).all()
 
 
+@pytest.mark.parametrize("F", [1, 2, 4, 8])
+def test_narrow_rows_with_a_row_finish_take_the_chunk_kernels(F):
+    """The tile kernels have no row finish: beta * A x + alpha * h (a layer's bias, an APPNP hop, a
+    fused relu) at 1, 2, 4 or 8 floats per row goes through the chunk kernels, through the
+    wrappers on the first use of the offsets (no plan yet) and on the second (planned); a planned
+    call that brings only the tile plan for such a product is refused with a message, before
+    anything is enqueued."""
+    from jittorgeometric_amd.ops._common import spmm, spmm_axpby
+    L, l = lib()
+    rng = np.random.default_rng(20 + F)
+    V, E = 3000, 90000
+    idx, off, wt = csc_of(rng, V, E, 2, 0.4)
+    x = rng.standard_normal((V, F)).astype(np.float32)
+    h = rng.standard_normal((V, F)).astype(np.float32)
+    off_g, idx_g, w_g, x_g, h_g = to_gpu(off), to_gpu(idx), to_gpu(wt), to_gpu(x), to_gpu(h)
+    want, terms = oracle.aggregate_f64(x, idx, off, wt)
+    for use in range(3):
+        got = spmm_axpby(off_g, idx_g, w_g, x_g, V, 0.9, 0.1, h_g).cpu().numpy()
+        assert_close(got, 0.9 * want + 0.1 * h, 0.9 * terms + 0.1 * np.abs(h), what="axpby F=%d, use %d" % (F, use))
+        got = spmm_axpby(off_g, idx_g, w_g, x_g, V, 1.0, 1.0, h_g[0], relu=True).cpu().numpy()
+        assert_close(got, np.maximum(want + h[0], 0), terms + np.abs(h[0]), what="relu F=%d, use %d" % (F, use))
+        assert_close(spmm(off_g, idx_g, w_g, x_g, V).cpu().numpy(), want, terms, what="plain F=%d, use %d" % (F, use))
+    tiles, _, _ = build_plan(off_g, V, E, TILES)
+    out = torch.empty((V, F), device=dev())
+    nbytes = L.query(l.jgamd_spmm_csx_planned_workspace, V, E, F)
+    ws = L.workspace(nbytes, dev())
+    rc = l.jgamd_spmm_csx_planned(None, L.ptr(tiles), -1, -1, L.ptr(off_g), L.ptr(idx_g), L.ptr(w_g), L.ptr(x_g), L.ptr(out),
+                                  0.9, 0.1, L.ptr(h_g), V, 0, V, V, E, F, L.ptr(ws), nbytes, L.stream_ptr(dev()))
+    assert rc == -1 and b"chunk plan" in l.jgamd_last_error()
+
+
 @pytest.mark.parametrize("H", [1, 2, 4, 8])
 def test_planned_edge_softmax_equals_unplanned(H):
     L, l = lib()
