@@ -176,9 +176,11 @@ int32_t jgamd_csx_plan_counts(const void *plan, int32_t *n_fix, int32_t *n_grp, 
 
 /* jgamd_spmm_csx_axpby with the partition taken from a plan of `off`:
  * plan = a JGAMD_PLAN_SPMM plan, tiles = a JGAMD_PLAN_TILES plan (either may be
- * NULL, not both; rows of 1, 2, 4 or 8 floats use `tiles` when it is given,
- * every other width needs `plan`).  beta = 1, alpha = 0 or h = NULL is the
- * plain product of AggregateOp::jit_run (ops/cpp/aggregate_op.cc:26-71).
+ * NULL, not both).  The plain product (beta = 1, alpha = 0 or h = NULL, no
+ * flags: AggregateOp::jit_run, ops/cpp/aggregate_op.cc:26-71) at rows of 1, 2,
+ * 4 or 8 floats, x aligned to min(16, 4 F) bytes, uses `tiles` when it is
+ * given; every other width, and any product with a row finish, needs `plan`
+ * and is refused with JGAMD_ERR_NULL when only `tiles` came.
  * flags: JGAMD_ROW_RELU clamps every finished row at zero in the row store,
  * out = max(0, beta * A x + alpha * h): the activation the reference's models
  * apply in a pass of their own after the layer (examples/gcn_example.py:84-90).
