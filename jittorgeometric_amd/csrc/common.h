@@ -42,6 +42,10 @@ int32_t exclusive_scan_i32(const int32_t *in, int32_t *out, int64_t n, int32_t *
 
 // ---- per-graph partition for the merge-path and tile kernels (plan.hip) ------
 constexpr int kPlanGroup = 32;             // chunks per group of pre-summed row pieces
+// A row of the product that crosses at most this many group boundaries has its group sums formed
+// by the wavefront that finishes the row; only longer rows use (and a plan only lists) pre-summed
+// groups.  At most (kSpmmInlineGroups + 1) * kPlanGroup pieces are then added by one wavefront.
+constexpr int kSpmmInlineGroups = 2;
 constexpr int kTileEntriesWide = 2048;     // entries per tile at 1 or 2 floats per entry
 constexpr int kTileEntriesNarrow = 1024;   // and at 4 or 8
 

@@ -18,7 +18,10 @@
 // Lists.  fix[] = the chunks whose first row began in an earlier chunk and ends
 // in this one (its pieces have to be added up); grp[] = the groups of kPlanGroup
 // chunks past whose end a row continues (their pieces are pre-summed).  Both
-// ascending; their lengths sit at the start of the plan.
+// ascending; their lengths sit at the start of the plan.  A plan for the product
+// leaves out the groups of rows that cross at most kSpmmInlineGroups group
+// boundaries: the kernel that finishes such a row sums its groups itself, and on
+// a graph without longer rows no group kernel is launched at all.
 #include <stdlib.h>
 
 #include "common.h"
@@ -78,7 +81,8 @@ __device__ __forceinline__ int compact_ascending(int n, int32_t *__restrict__ li
 }
 
 __global__ __launch_bounds__(kListThreads) void plan_chunk_lists(const int32_t *__restrict__ off,
-                                                                 const int2 *__restrict__ start, int R, int nchunks,
+                                                                 const int2 *__restrict__ start, int R, int chunk,
+                                                                 int nchunks, int inline_groups,
                                                                  int32_t *__restrict__ fix, int32_t *__restrict__ grp,
                                                                  int32_t *__restrict__ header)
 {
@@ -91,7 +95,11 @@ __global__ __launch_bounds__(kListThreads) void plan_chunk_lists(const int32_t *
         const int kend = (g + 1) * kPlanGroup;
         if (kend >= nchunks) return false;
         const int2 a = start[kend];
-        return a.x < R && a.y > off[a.x];
+        if (a.x < 0 || a.x >= R || a.y <= off[a.x]) return false;
+        // a cut row begins in the chunk of its first item and ends in that of its end marker
+        const int64_t r = a.x;
+        const int first = (int)((max(off[r], 0) + r) / chunk), last = (int)((max(off[r + 1], 0) + r) / chunk);
+        return last / kPlanGroup - first / kPlanGroup > inline_groups;
     });
     if (threadIdx.x == 0) {
         header[0] = n_fix;
@@ -257,8 +265,8 @@ JG_EXPORT int32_t jgamd_csx_plan(const int32_t *off, int32_t R, int64_t E, int32
     if (R == 0) return 0;
     const ChunkPlan v = chunk_plan_view(kind, R, E, plan);
     chunk_starts_enqueue(off, R, E, v.chunk, v.nchunks, const_cast<int2 *>(v.start), s);
-    hipLaunchKernelGGL(plan_chunk_lists, dim3(1), dim3(kListThreads), 0, s, off, v.start, R, v.nchunks,
-                       const_cast<int32_t *>(v.fix), const_cast<int32_t *>(v.grp), const_cast<int32_t *>(v.counts));
+    hipLaunchKernelGGL(plan_chunk_lists, dim3(1), dim3(kListThreads), 0, s, off, v.start, R, v.chunk, v.nchunks,
+                       kind == JGAMD_PLAN_SPMM ? kSpmmInlineGroups : 0, const_cast<int32_t *>(v.fix), const_cast<int32_t *>(v.grp), const_cast<int32_t *>(v.counts));
     return launch_status("csx_plan");
 }
 

@@ -289,7 +289,7 @@ template <int VEC, int NT>
 __device__ __forceinline__ void add_pieces(float (&acc)[NT][VEC], const float *__restrict__ src, int first, int last,
                                            int F, int f0)
 {
-    constexpr int kBatch = VEC * NT >= 16 ? 2 : (VEC * NT >= 8 ? 4 : 8);
+    constexpr int kBatch = VEC * NT >= 16 ? 2 : (VEC * NT >= 8 ? 4 : (VEC * NT >= 4 ? 8 : 16));
     for (int kb = first; kb < last; kb += kBatch) {
         // issue phase without branches: slots past `last` re-read the last piece, lanes past F
         // read offset 0; both are ignored below
@@ -391,6 +391,22 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_fixup(const int32_t *__rest
         const int ga = a / kGroup, gb = k / kGroup;
         if (ga == gb) {
             add_pieces<VEC, NT>(acc, partial, a, k, F, f0);
+        } else if (gb - ga <= kSpmmInlineGroups) {
+            // few groups: their sums are formed here, piece by piece from zero and then added in
+            // order, exactly as spmm_group_sums and the branch below would
+            for (int g = ga; g < gb; g++) {
+                float gs[NT][VEC];
+#pragma unroll
+                for (int t = 0; t < NT; t++)
+#pragma unroll
+                    for (int v = 0; v < VEC; v++) gs[t][v] = 0.f;
+                add_pieces<VEC, NT>(gs, partial, max(a, g * kGroup), (g + 1) * kGroup, F, f0);
+#pragma unroll
+                for (int t = 0; t < NT; t++)
+#pragma unroll
+                    for (int v = 0; v < VEC; v++) acc[t][v] += gs[t][v];
+            }
+            add_pieces<VEC, NT>(acc, partial, gb * kGroup, k, F, f0);
         } else {
             // group ga's sum starts at piece a (the row continues past that group),
             // groups ga+1 .. gb-1 belong to the row entirely, the rest of gb is added piecewise

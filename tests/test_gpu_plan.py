@@ -52,7 +52,10 @@ def gat_chunk(M):
     return c
 
 
-def model_partition(off, R, E, chunk):
+INLINE_GROUPS = 2      # the product's finishing kernel sums the groups of a row that crosses at most this many
+
+
+def model_partition(off, R, E, chunk, inline_groups=0):
     """start[k] = (row, entry), the fix list and the group list, as the kernels define them."""
     M = R + E
     nchunks = max(-(-M // chunk), 1)
@@ -73,6 +76,11 @@ def model_partition(off, R, E, chunk):
     grp = [g for g in range(ngroups)
            if (g + 1) * GROUP < nchunks and start[(g + 1) * GROUP, 0] < R
            and start[(g + 1) * GROUP, 1] > off[start[(g + 1) * GROUP, 0]]]
+
+    def crossings(g):     # group boundaries crossed by the row that continues past group g
+        r = int(start[(g + 1) * GROUP, 0])
+        return (int(off[r + 1]) + r) // chunk // GROUP - (int(off[r]) + r) // chunk // GROUP
+    grp = [g for g in grp if crossings(g) > inline_groups]
     return nchunks, start, fix, grp
 
 
@@ -100,6 +108,7 @@ def csc_of(rng, V, E, hubs, hub_share=0.3):
     (3000, 60000, 2, 0.4, SPMM, 1),          # two hubs of thousands of entries
     (500, 400000, 1, 0.7, SPMM, 2),          # one row across hundreds of chunks (several groups)
     (40000, 3000, 0, 0.0, SPMM, 3),          # mostly empty rows
+    (3000, 60000, 2, 0.05, SPMM, 6),         # rows across a few dozen chunks: cut, but no group is listed
     (3000, 60000, 2, 0.4, GAT, 4),
     (200, 2000000, 1, 0.9, GAT, 5),          # chunk 128, a row across thousands of chunks
 ])
@@ -107,7 +116,7 @@ def test_plan_arrays_follow_the_partition_rule(V, E, hubs, share, kind, seed):
     rng = np.random.default_rng(seed)
     idx, off, wt = csc_of(rng, V, E, hubs, share)
     chunk = (spmm_chunk if kind == SPMM else gat_chunk)(V + E)
-    nchunks, start, fix, grp = model_partition(off, V, E, chunk)
+    nchunks, start, fix, grp = model_partition(off, V, E, chunk, INLINE_GROUPS if kind == SPMM else 0)
     plan, n_fix, n_grp = build_plan(to_gpu(off), V, E, kind)
     counts, g_start, g_fix, g_grp = read_plan(plan, nchunks)
     assert np.array_equal(g_start, start.astype(np.int32))
@@ -118,6 +127,10 @@ def test_plan_arrays_follow_the_partition_rule(V, E, hubs, share, kind, seed):
     assert (np.diff(pos) > 0).all() and (np.abs(np.diff(pos)[:-1] - chunk) <= chunk // 2).all()
     if hubs == 0 and np.diff(off).max() <= chunk // 2:
         assert n_fix == 0 and n_grp == 0
+    if seed == 6:
+        assert n_grp == 0 and len(model_partition(off, V, E, chunk)[3]) > 0 and np.diff(off).max() > GROUP * chunk
+    if seed in (1, 2):
+        assert n_grp > 0
 
 
 def planned(plan, tiles, hints, off, idx, w, x, R, beta=1.0, alpha=0.0, h=None, flags=0):
@@ -152,7 +165,8 @@ def unplanned(off, idx, w, x, R, beta=1.0, alpha=0.0, h=None):
 
 
 @pytest.mark.parametrize("F", [3, 16, 47, 64, 100, 128, 256, 300])
-@pytest.mark.parametrize("V,E,hubs,share", [(3000, 20000, 0, 0.0), (3000, 90000, 2, 0.4), (400, 600000, 1, 0.8)])
+@pytest.mark.parametrize("V,E,hubs,share", [(3000, 20000, 0, 0.0), (3000, 90000, 2, 0.4), (400, 600000, 1, 0.8),
+                                            (3000, 60000, 2, 0.05)])
 def test_planned_product_equals_unplanned_and_oracle(V, E, hubs, share, F):
     rng = np.random.default_rng(F * 7 + V)
     idx, off, wt = csc_of(rng, V, E, hubs, share)
