@@ -97,7 +97,7 @@ __global__ __launch_bounds__(1024) void column_final_sums(const float *__restric
     const int col = blockIdx.x * COLS + c;
     float s = 0.f;
     if (col < F) {
-        constexpr int kB = 4;               // rows fetched together, added in the same order as one by one
+        constexpr int kB = 8;               // rows fetched together, added in the same order as one by one
         for (int b0 = grp; b0 < nblocks; b0 += GROUPS * kB) {
             float v[kB], yv[MASK ? kB : 1];
 #pragma unroll

@@ -153,7 +153,8 @@ __global__ __launch_bounds__(kCeThreads) void ce_final(const double *__restrict_
     if (threadIdx.x == 0) {
         double tt = 0.0;
         long long nn = 0;
-        for (int i = 0; i < kCeThreads; i++) {
+        const int used = nblocks < kCeThreads ? nblocks : kCeThreads;     // the other threads hold zeros
+        for (int i = 0; i < used; i++) {
             tt += s_sum[i];
             nn += s_cnt[i];
         }

@@ -131,7 +131,7 @@ class GcnLayerFunc(torch.autograd.Function):
             if need_w:
                 gw = xt_g(x, gh)
             if need_x:
-                gx = rows_times(gh, weight.t().contiguous())
+                gx = rows_times(gh, weight.t())
         elif need_w:
             off, idx, w = ctx.fwd
             gw = xt_g(spmm(off, idx, w, x, x.shape[0]), g)

@@ -63,13 +63,13 @@ class SageLayerFunc(torch.autograd.Function):
                 # one pass.  Same gradient, summed in another order; the forward pass is untouched.
                 t = spmm(off, idx, w, g, g.shape[0])
                 if w_root is not None:
-                    gx = rows_times(t, w1.t().contiguous(), g, w_root.t().contiguous())
+                    gx = rows_times(t, w1.t(), g, w_root.t())
                 else:
-                    gx = rows_times(t, w1.t().contiguous())
+                    gx = rows_times(t, w1.t())
             else:
-                g_agg = rows_times(g, w1.t().contiguous())
+                g_agg = rows_times(g, w1.t())
                 if w_root is not None:
-                    gx = spmm_axpby(off, idx, w, g_agg, g.shape[0], 1.0, 1.0, rows_times(g, w_root.t().contiguous()))
+                    gx = spmm_axpby(off, idx, w, g_agg, g.shape[0], 1.0, 1.0, rows_times(g, w_root.t()))
                 else:
                     gx = spmm(off, idx, w, g_agg, g.shape[0])
         return gx, gw1, groot, gb, None, None, None
@@ -114,9 +114,9 @@ class SageTransformFirstFunc(torch.autograd.Function):
                 gw1 = xt_g(x, g_h1)
             if need_x:
                 if w_root is not None:
-                    gx = rows_times(g_h1, w1.t().contiguous(), g, w_root.t().contiguous())
+                    gx = rows_times(g_h1, w1.t(), g, w_root.t())
                 else:
-                    gx = rows_times(g_h1, w1.t().contiguous())
+                    gx = rows_times(g_h1, w1.t())
         return gx, gw1, groot, gb, None, None
 
 

@@ -76,7 +76,7 @@ class _XW(torch.autograd.Function):
         gx = gw = gb = None
         g = g.contiguous()
         if ctx.needs_input_grad[0]:
-            gx = rows_times(g, weight.t().contiguous())
+            gx = rows_times(g, weight.t())      # copied row-major only where the library's kernel runs
         if ctx.needs_input_grad[1]:
             gw = xt_g(x, g)
         if ctx.needs_input_grad[2]:
