@@ -325,6 +325,8 @@ def config2(b):
 
     if args.part == "softmax":
         return config2_softmax(b, csc, V, E), 0.0
+    if args.part == "propagate":
+        return config2_propagate(b, csc, csr, V, E), 0.0
     if args.part == "convert":
         # only the two conversions of the normalised edge list (what profiles/coo_to_csx_powerlaw_1m.txt
         # is taken from)
@@ -505,6 +507,43 @@ def config2_softmax(b, csc, V, E):
                         "achieved": round((8 * E + 4 * (V + 1)) / (ms * 1e-3) / 1e9, 1),
                         "frac": out["edge_softmax_h1_fwd_frac_hbm_peak"], "traffic": None,
                         "achieved_basis": "algorithmic bytes / operator time"}
+    line["cpu_baseline"] = None
+    return line
+
+
+def config2_propagate(b, csc, csr, V, E):
+    """Forward passes of the propagation layers on config 2's graph at 64 features: each layer
+    as this build runs it (the element-wise tail of every hop in the product's row store; BernNet
+    by Horner's rule) and as the reference's chain of operators (fused=False)."""
+    from jittorgeometric_amd.nn import APPNP, BernNet, ChebNetII, EvenNet, GCN2Conv
+    torch, args, dev = b.torch, b.args, b.dev
+    F, K = 64, 10
+    iters, warm = max(args.steps // 5, 5), 2
+    x = torch.randn(V, F, device=dev)
+    x0 = torch.randn(V, F, device=dev)
+    out = {}
+    with torch.no_grad():
+        for name, make, call in (
+                ("appnp_k10", lambda f: APPNP(K, 0.1, spmm=False, fused=f), lambda l: l(x, csc, csr)),
+                ("chebnet2_k10", lambda f: ChebNetII(K, spmm=False, fused=f).to(dev), lambda l: l(x, csc, csr)),
+                ("evennet_k10", lambda f: EvenNet(K, 0.1, spmm=False, fused=f), lambda l: l(x, csc, csr)),
+                ("gcn2conv", lambda f: GCN2Conv(F, F, spmm=False, fused=f).to(dev), lambda l: l(x, x0, csc, csr, 0.1, 0.4)),
+                ("bernnet_k10", lambda f: BernNet(K, spmm=False, fused=f).to(dev), lambda l: l(x, csc, csr, csc, csr))):
+            for fused in (True, False):
+                layer = make(fused)
+                out["%s_f64_fwd_%s_ms" % (name, "fused" if fused else "chain")] = round(
+                    b.timed(lambda: call(layer), iters if fused or name != "bernnet_k10" else 3, warm), 4)
+    ms = out["chebnet2_k10_f64_fwd_fused_ms"]
+    line = base_line(args, "chebnet2_k10_f64_fwd_ms", ms, "ms", ms, False,
+                     "config 2 graph, forward of the propagation layers at 64 features (K = 10 hops where the layer has K)",
+                     {"V": V, "E": E, "F": F, "K": K})
+    line.update(out)
+    hop_bytes = 4 * (V + 1) + 8 * E + 4 * E * F + 4 * V * F
+    line["roofline"] = {"bound": "hbm", "peak": HBM_PEAK_GBPS, "unit": "GB/s", "kernel": "spmm_merge (one per hop)",
+                        "algorithmic_bytes": hop_bytes + 4 * V * F, "traffic": None,
+                        "achieved": round(K * (hop_bytes + 4 * V * F) / (ms * 1e-3) / 1e9, 1),
+                        "frac": round(K * (hop_bytes + 4 * V * F) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                        "achieved_basis": "K hops x (product bytes + the added row) / layer time"}
     line["cpu_baseline"] = None
     return line
 
@@ -794,13 +833,13 @@ def main():
     ap.add_argument("--config", type=int, default=2, choices=[1, 2, 3, 4, 5],
                     help="benchmark configuration; 2 (the headline SpMM workload) is the default")
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the single-thread CPU timing")
-    ap.add_argument("--part", default="all", choices=["all", "main", "layers", "softmax", "convert"],
+    ap.add_argument("--part", default="all", choices=["all", "main", "layers", "softmax", "convert", "propagate"],
                     help="main: only the timed workload of the metric (what the counter profiles under profiles/ "
                          "are taken from); layers: only the GCN and GraphSAGE layer steps of config 2")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (known traffic, for scaling rocprof counters)")
     args = ap.parse_args()
-    if args.part in ("layers", "softmax", "convert") and args.config != 2:
+    if args.part in ("layers", "softmax", "convert", "propagate") and args.config != 2:
         sys.exit("bench.py: --part %s belongs to --config 2" % args.part)
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only; --gpus %d is not supported "

@@ -20,6 +20,13 @@ jittor==1.3.9.14).  Pins of the numpy restatements at the end of this file:
                 PageRank limit alpha * (I - (1 - alpha) A)^-1 h on a small graph
   sgconv        dense fp64 A^K x W
   gprgnn        dense fp64 sum_k temp[k] A^k x
+  lightgcn      dense fp64 A x
+  gcn2conv      dense fp64 A ((1-b)(1-a) x + b x W1) + (1-b) a x0 + b x0 W2
+  evennet       dense fp64 t0 x + t3 A^3 x + t4 A^4 x (the hops the loop adds as written)
+  chebnet2      T_i(A) from the eigenvalues of a symmetric A (cos(i arccos lambda)); a
+                polynomial sampled at the Chebyshev nodes comes back as that polynomial of A
+  bernnet       dense fp64 sum_i C(K,i)/2^K t_i A1^i A2^(K-i) x; the binomial theorem
+                (A1 = L, A2 = 2I - L, t = 1 gives x back)
   gpuinitco / getweight / csctocsr  brute-force Python loops on small graphs,
                 the README's CSC -> CSR known answer
   sampleprocessing  "parity unpinned": the reference draws with rand() /
@@ -440,6 +447,96 @@ def gprgnn(x, csc, temp):
     for k in range(temp.shape[0] - 1):
         x = aggregate_with_weight(x, csc)
         out = (out + temp[k + 1] * x).astype(np.float32)
+    return out
+
+
+def lightgcn(x, csc):
+    """nn/conv/lightgcn_conv.py:28-44: one product, no weights."""
+    return aggregate_with_weight(_f32(x), csc)
+
+
+def gcn2conv(x, x_0, csc, weight1, weight2, alpha, beta):
+    """nn/conv/gcn2_conv.py:66-73: support = (1-beta)(1-alpha) x + beta x W1,
+    initial = (1-beta) alpha x_0 + beta x_0 W2, out = propagate(support) + initial."""
+    x, x_0 = _f32(x), _f32(x_0)
+    mm = lambda a, w: (a.astype(np.float64) @ np.asarray(w, np.float64)).astype(np.float32)
+    support = (np.float32((1 - beta) * (1 - alpha)) * x + np.float32(beta) * mm(x, weight1)).astype(np.float32)
+    initial = (np.float32((1 - beta) * alpha) * x_0 + np.float32(beta) * mm(x_0, weight2)).astype(np.float32)
+    return (aggregate_with_weight(support, csc) + initial).astype(np.float32)
+
+
+def evennet_temp(K, alpha):
+    """nn/conv/even_conv.py:48-50: alpha (1-alpha)^k, the last one (1-alpha)^K."""
+    t = alpha * (1 - alpha) ** np.arange(K + 1)
+    t[-1] = (1 - alpha) ** K
+    return t
+
+
+def evennet(x, csc, K, alpha):
+    """nn/conv/even_conv.py:53-61: out = x * temp[0]; K hops; hop k (from 0) is added with
+    temp[k+1] when k // 2 == 1, i.e. the third and the fourth hop, as the loop is written."""
+    temp = evennet_temp(K, alpha)
+    x = _f32(x)
+    out = (x * np.float32(temp[0])).astype(np.float32)
+    for k in range(K):
+        x = aggregate_with_weight(x, csc)
+        if k // 2 == 1:
+            out = (out + np.float32(temp[k + 1]) * x).astype(np.float32)
+    return out
+
+
+def chebnet2_coefficients(temp):
+    """nn/conv/chebnet2_conv.py:22-33,68-75: coe[i] = 2/(K+1) sum_j relu(temp)[j] T_i(x_j) with
+    x_j = cos((K - j + 0.5) pi / (K + 1)), T_i by the three-term recurrence."""
+    t = np.maximum(np.asarray(temp, np.float64), 0.0)
+    K = t.shape[0] - 1
+
+    def cheb(i, v):
+        if i == 0:
+            return 1.0
+        t0, t1 = 1.0, v
+        for _ in range(2, i + 1):
+            t0, t1 = t1, 2 * v * t1 - t0
+        return t1
+    coe = np.zeros(K + 1)
+    for i in range(K + 1):
+        acc = 0.0
+        for j in range(K + 1):
+            acc += t[j] * cheb(i, np.cos((K - j + 0.5) * np.pi / (K + 1)))
+        coe[i] = 2 * acc / (K + 1)
+    return coe
+
+
+def chebnet2(x, csc, temp):
+    """nn/conv/chebnet2_conv.py:77-93: out = coe[0]/2 Tx_0 + coe[1] Tx_1, then
+    Tx_2 = 2 propagate(Tx_1) - Tx_0 and out += coe[i] Tx_2 for i = 2..K."""
+    coe = chebnet2_coefficients(temp).astype(np.float32)
+    K = coe.shape[0] - 1
+    t0 = _f32(x)
+    t1 = aggregate_with_weight(t0, csc)
+    out = (coe[0] / np.float32(2) * t0 + coe[1] * t1).astype(np.float32)
+    for i in range(2, K + 1):
+        t2 = (np.float32(2) * aggregate_with_weight(t1, csc) - t0).astype(np.float32)
+        out = (out + coe[i] * t2).astype(np.float32)
+        t0, t1 = t1, t2
+    return out
+
+
+def bernnet(x, csc1, csc2, temp):
+    """nn/conv/bernnet_conv.py:56-80: tmp[k] = A2^k x; out = C(K,0)/2^K t[0] tmp[K], then for
+    i = 0..K-1: out += C(K,i+1)/2^K t[i+1] A1^(i+1) tmp[K-i-1], with t = relu(temp)."""
+    from math import comb
+    t = np.maximum(_f32(temp), 0)
+    K = t.shape[0] - 1
+    tmp = [_f32(x)]
+    for _ in range(K):
+        tmp.append(aggregate_with_weight(tmp[-1], csc2))
+    out = (np.float32(comb(K, 0) / 2 ** K) * t[0] * tmp[K]).astype(np.float32)
+    for i in range(K):
+        v = tmp[K - i - 1]
+        for _ in range(i + 1):
+            v = aggregate_with_weight(v, csc1)
+        out = (out + np.float32(comb(K, i + 1) / 2 ** K) * t[i + 1] * v).astype(np.float32)
     return out
 
 

@@ -1,6 +1,8 @@
 """Callers either side of the SpMM path on the GPU against the CPU oracle: the
-product with a fused row finish, APPNP / SGConv built on it, SpmmCoo and
-toUndirected.  fp32, 1e-5 relative to the sum of absolute terms."""
+product with a fused row finish, the propagation layers built on it (APPNP, SGConv,
+GPRGNN, LightGCNConv, GCN2Conv, EvenNet, ChebNetII, BernNet), SpmmCoo and
+toUndirected.  fp32, 1e-5 relative to the sum of absolute terms for one product,
+1e-4 for the layers of several hops."""
 import json
 import os
 
@@ -276,3 +278,174 @@ def test_gprgnn_forward_backward(init):
     gx = sum(float(temp[k]) * gs[k].astype(np.float64) for k in range(K + 1))
     gxs = sum(abs(float(temp[k])) * np.abs(gs[k]).astype(np.float64) for k in range(K + 1))
     assert_close(xt.grad.cpu().numpy(), gx, scale=gxs + 1e-3, rtol=1e-4)
+
+
+# ------------------------------------------- polynomial layers built on the fused hop ---
+def _dense64(ei, w, V):
+    A = torch.zeros((V, V), dtype=torch.float64)
+    A.index_put_((torch.from_numpy(ei[1].astype(np.int64)), torch.from_numpy(ei[0].astype(np.int64))),
+                 torch.from_numpy(w.astype(np.float64)), accumulate=True)
+    return A
+
+
+def _check_layer(run_gpu, model, A_list, x_list, params, what, rtol=1e-4):
+    """Forward and every gradient of a layer on the GPU against a float64 dense model of it.
+    model(As, xs, ps, sub) is written with sub(a, b) for every subtraction, so that the same
+    expression on absolute values (sub = add) bounds the size of the terms that were added."""
+    rng = np.random.default_rng(5)
+    xs_g = [to_gpu(x).requires_grad_(True) for x in x_list]
+    out = run_gpu(xs_g)
+    g = rng.standard_normal(tuple(out.shape)).astype(np.float32)
+    out.backward(to_gpu(g))
+    xs64 = [torch.from_numpy(x).double().requires_grad_(True) for x in x_list]
+    ps64 = [p.detach().cpu().double().requires_grad_(True) for p in params]
+    want = model(A_list, xs64, ps64, lambda a, b: a - b)
+    want.backward(torch.from_numpy(g).double())
+    mag = model([A.abs() for A in A_list], [x.detach().abs() for x in xs64], [p.detach().abs() for p in ps64],
+                lambda a, b: a + b).detach().numpy()
+    assert_close(out.detach().cpu().numpy(), want.detach().numpy(), scale=mag + 1e-30, rtol=rtol, what=what + " forward")
+    # gradients: the size of their terms comes from the same model run on |g| through the transposes
+    for got, ref64, name in [(t.grad, r.grad, "x%d" % i) for i, (t, r) in enumerate(zip(xs_g, xs64))] + \
+                            [(p.grad, r.grad, "param%d" % i) for i, (p, r) in enumerate(zip(params, ps64))]:
+        if ref64 is None:
+            assert got is None or float(got.abs().max()) == 0.0
+            continue
+        ref = ref64.numpy()
+        bound = np.abs(ref).max() + 1e-30
+        assert got is not None, name
+        err = np.abs(got.cpu().numpy().astype(np.float64) - ref).max()
+        # a coefficient's gradient is one sum over all V * F products, whose terms cancel: looser
+        tol = 1e-4 if name.startswith("x") else 2e-3
+        assert err <= tol * bound, "%s gradient of %s: err %g against max %g" % (what, name, err, bound)
+    return out.detach().cpu().numpy()
+
+
+def _poly_graph(V=1500, E=25000, seed=90):
+    rng, ei, w, csc_o, csr_o, csc, csr = graphs(V, E, 1, seed)
+    return rng, ei, w, csc_o, csc, csr, _dense64(ei, w, V)
+
+
+@pytest.mark.parametrize("spmm", [True, False])
+def test_lightgcn_and_gcn2conv(spmm):
+    from jittorgeometric_amd.nn import GCN2Conv, LightGCNConv
+    V, F = 1500, 24
+    rng, ei, w, csc_o, csc, csr, A = _poly_graph()
+    x = rng.standard_normal((V, F)).astype(np.float32)
+    x0 = rng.standard_normal((V, F)).astype(np.float32)
+    layer = LightGCNConv(spmm=spmm)
+    got = _check_layer(lambda xs: layer(xs[0], csc, csr), lambda As, xs, ps, sub: As[0] @ xs[0], [A], [x], [], "LightGCNConv")
+    assert_close(got, oracle.lightgcn(x, csc_o), scale=abs_prod(x, csc_o) + 1e-30)
+    a, b = 0.1, 0.35
+    for fused in (True, False):
+        conv = GCN2Conv(F, F, spmm=spmm, fused=fused).to(dev())
+
+        def model(As, xs, ps, sub):
+            support = (1 - b) * (1 - a) * xs[0] + b * xs[0] @ ps[0]
+            return As[0] @ support + (1 - b) * a * xs[1] + b * xs[1] @ ps[1]
+        got = _check_layer(lambda xs: conv(xs[0], xs[1], csc, csr, a, b), model, [A], [x, x0], [conv.weight1, conv.weight2],
+                           "GCN2Conv fused=%s" % fused)
+        want = oracle.gcn2conv(x, x0, csc_o, conv.weight1.detach().cpu().numpy(), conv.weight2.detach().cpu().numpy(), a, b)
+        assert np.abs(got - want).max() <= 1e-4 * np.abs(want).max()
+
+
+@pytest.mark.parametrize("K", [1, 2, 3, 4, 7])
+def test_evennet(K):
+    from jittorgeometric_amd.nn import EvenNet
+    V, F, alpha = 1500, 20, 0.2
+    rng, ei, w, csc_o, csc, csr, A = _poly_graph(seed=91)
+    x = rng.standard_normal((V, F)).astype(np.float32)
+    t = oracle.evennet_temp(K, alpha)
+
+    def model(As, xs, ps, sub):
+        out, v = t[0] * xs[0], xs[0]
+        for k in range(K):
+            v = As[0] @ v
+            if k // 2 == 1:
+                out = out + t[k + 1] * v
+        return out
+    want = oracle.evennet(x, csc_o, K, alpha)
+    for fused, spmm in ((True, True), (True, False), (False, False)):
+        layer = EvenNet(K, alpha, spmm=spmm, fused=fused)
+        assert np.allclose(layer.temp, t)
+        got = _check_layer(lambda xs: layer(xs[0], csc, csr), model, [A], [x], [], "EvenNet K=%d fused=%s" % (K, fused))
+        assert np.abs(got - want).max() <= 1e-4 * np.abs(want).max()
+
+
+@pytest.mark.parametrize("K", [1, 2, 5])
+def test_chebnet2(K):
+    from jittorgeometric_amd.nn import ChebNetII
+    from jittorgeometric_amd.nn.conv.chebnet2_conv import node_table
+    V, F = 1500, 20
+    rng, ei, w, csc_o, csc, csr, A = _poly_graph(seed=92)
+    x = rng.standard_normal((V, F)).astype(np.float32)
+    temp0 = (rng.random(K + 1) * 2 - 0.4).astype(np.float32)       # some below zero: clamped
+    table = torch.from_numpy(node_table(K) * (2.0 / (K + 1)))
+
+    def model(As, xs, ps, sub):
+        # the run on absolute values (sub adds) takes the table's absolute values too
+        coe = (table.abs() if sub(1.0, 1.0) == 2.0 else table) @ torch.relu(ps[0])
+        t0 = xs[0]
+        t1 = As[0] @ t0
+        out = coe[0] / 2 * t0 + coe[1] * t1
+        for i in range(2, K + 1):
+            t2 = sub(2 * (As[0] @ t1), t0)
+            out = out + coe[i] * t2
+            t0, t1 = t1, t2
+        return out
+    with pytest.raises(ValueError):
+        ChebNetII(0)
+    for fused, spmm in ((True, True), (True, False), (False, False)):
+        layer = ChebNetII(K, spmm=spmm, fused=fused).to(dev())
+        assert torch.equal(layer.temp.detach().cpu(), torch.ones(K + 1))
+        with torch.no_grad():
+            layer.temp.copy_(to_gpu(temp0))
+        np.testing.assert_allclose(layer.coefficients().detach().cpu().numpy(), oracle.chebnet2_coefficients(temp0),
+                                   rtol=1e-5, atol=1e-6)
+        got = _check_layer(lambda xs: layer(xs[0], csc, csr), model, [A], [x], [layer.temp], "ChebNetII K=%d fused=%s" % (K, fused))
+        want = oracle.chebnet2(x, csc_o, temp0)
+        assert np.abs(got - want).max() <= 1e-4 * np.abs(want).max()
+
+
+@pytest.mark.parametrize("K", [1, 2, 4])
+def test_bernnet(K):
+    from math import comb
+    from jittorgeometric_amd.nn import BernNet
+    from jittorgeometric_amd.ops import cootocsc, cootocsr
+    V, F = 1200, 16
+    rng, ei, w, csc_o, csc, csr, A = _poly_graph(V=V, E=20000, seed=93)
+    loops = np.stack([np.arange(V), np.arange(V)]).astype(np.int32)
+    ei2 = np.concatenate([ei, loops], axis=1)
+    w1 = np.concatenate([-w, np.ones(V, np.float32)])              # L = I - A
+    w2 = np.concatenate([w, np.ones(V, np.float32)])               # 2I - L = I + A
+    csc1, csr1 = cootocsc(to_gpu(ei2), to_gpu(w1), V), cootocsr(to_gpu(ei2), to_gpu(w1), V)
+    csc2, csr2 = cootocsc(to_gpu(ei2), to_gpu(w2), V), cootocsr(to_gpu(ei2), to_gpu(w2), V)
+    A1, A2 = _dense64(ei2, w1, V), _dense64(ei2, w2, V)
+    x = rng.standard_normal((V, F)).astype(np.float32)
+    temp0 = (rng.random(K + 1) * 2 - 0.3).astype(np.float32)
+
+    def model(As, xs, ps, sub):
+        t = torch.relu(ps[0])
+        tmp = [xs[0]]
+        for _ in range(K):
+            tmp.append(As[1] @ tmp[-1])
+        out = 0
+        for i in range(K + 1):
+            v = tmp[K - i]
+            for _ in range(i):
+                v = As[0] @ v
+            out = out + comb(K, i) / 2 ** K * t[i] * v
+        return out
+    want = oracle.bernnet(x, oracle.cootocsc(ei2, w1, V), oracle.cootocsc(ei2, w2, V), temp0)
+    for fused, spmm in ((True, True), (True, False), (False, False)):
+        layer = BernNet(K, spmm=spmm, fused=fused).to(dev())
+        with torch.no_grad():
+            layer.temp.copy_(to_gpu(temp0))
+        got = _check_layer(lambda xs: layer(xs[0], csc1, csr1, csc2, csr2), model, [A1, A2], [x], [layer.temp],
+                           "BernNet K=%d fused=%s" % (K, fused))
+        scale = np.abs(model([A1.abs(), A2.abs()], [torch.from_numpy(np.abs(x)).double()], [torch.from_numpy(np.abs(temp0)).double()],
+                             None).numpy())
+        assert_close(got, want, scale=scale + 1e-30, rtol=1e-4, what="BernNet against the oracle's order of products")
+    # all weights one on (L, 2I - L): the binomial theorem gives x back
+    layer = BernNet(3).to(dev())
+    out = layer(to_gpu(x), csc1, csr1, csc2, csr2).cpu().detach().numpy()
+    assert np.abs(out - x).max() < 1e-4

@@ -449,6 +449,104 @@ def test_gprgnn_dense_closed_form():
     np.testing.assert_allclose(oracle.gprgnn(x, csc, temp), want, rtol=1e-5, atol=1e-5)
 
 
+def _small_symmetric(seed, V=30, E=200):
+    """A gcn-normalised undirected graph (symmetric, eigenvalues in [-1, 1]), its CSC and dense form."""
+    rng = np.random.default_rng(seed)
+    ei, _ = rand_graph(rng, V, E, loops=False)
+    ei = np.concatenate([ei, ei[::-1]], axis=1)
+    ei = np.unique(ei, axis=1).astype(np.int32)
+    ei, w = oracle.gcn_norm(ei, None, V)
+    A = sp.coo_matrix((w.astype(np.float64), (ei[1], ei[0])), shape=(V, V)).toarray()
+    assert np.allclose(A, A.T)
+    return rng, ei, w, oracle.cootocsc(ei, w, V), A
+
+
+def test_lightgcn_and_gcn2conv_dense_closed_forms():
+    rng, ei, w, csc, A = _small_symmetric(75)
+    V = A.shape[0]
+    x, x0 = rng.standard_normal((V, 6)).astype(np.float32), rng.standard_normal((V, 6)).astype(np.float32)
+    np.testing.assert_allclose(oracle.lightgcn(x, csc), A @ x.astype(np.float64), rtol=1e-5, atol=1e-6)
+    W1, W2 = rng.standard_normal((6, 6)).astype(np.float32), rng.standard_normal((6, 6)).astype(np.float32)
+    a, b = 0.1, 0.4
+    x64, x064 = x.astype(np.float64), x0.astype(np.float64)
+    want = A @ ((1 - b) * (1 - a) * x64 + b * x64 @ W1) + (1 - b) * a * x064 + b * x064 @ W2
+    np.testing.assert_allclose(oracle.gcn2conv(x, x0, csc, W1, W2, a, b), want, rtol=1e-5, atol=1e-5)
+    # beta = 0, alpha = 0: the plain product; alpha = 1: the input of the first layer comes back
+    np.testing.assert_allclose(oracle.gcn2conv(x, x0, csc, W1, W2, 0.0, 0.0), A @ x64, rtol=1e-5, atol=1e-6)
+    assert np.array_equal(oracle.gcn2conv(x, x0, csc, W1, W2, 1.0, 0.0), x0)
+
+
+def test_evennet_adds_the_hops_the_loop_names():
+    rng, ei, w, csc, A = _small_symmetric(76)
+    V = A.shape[0]
+    x = rng.standard_normal((V, 5)).astype(np.float32)
+    x64 = x.astype(np.float64)
+    alpha = 0.2
+    for K in (1, 2, 3, 4, 6):
+        t = alpha * (1 - alpha) ** np.arange(K + 1)
+        t[-1] = (1 - alpha) ** K
+        assert np.allclose(oracle.evennet_temp(K, alpha), t)
+        want = t[0] * x64
+        if K >= 3:
+            want = want + t[3] * np.linalg.matrix_power(A, 3) @ x64
+        if K >= 4:
+            want = want + t[4] * np.linalg.matrix_power(A, 4) @ x64
+        np.testing.assert_allclose(oracle.evennet(x, csc, K, alpha), want, rtol=1e-5, atol=1e-6)
+
+
+def test_chebnet2_is_the_interpolating_polynomial_of_the_node_values():
+    rng, ei, w, csc, A = _small_symmetric(77)
+    V = A.shape[0]
+    x = rng.standard_normal((V, 4)).astype(np.float32)
+    x64 = x.astype(np.float64)
+    lam, Q = np.linalg.eigh(A)
+    assert lam.min() > -1 - 1e-9 and lam.max() < 1 + 1e-9
+    K = 5
+    nodes = np.cos((K - np.arange(K + 1) + 0.5) * np.pi / (K + 1))
+    # a polynomial of degree <= K, positive at the nodes, sampled there: the filter is that polynomial of A
+    f = lambda v: 0.7 + 0.3 * v - 0.5 * v ** 2 + 0.2 * v ** 3 + v ** 4
+    assert (f(nodes) > 0).all()
+    want = (Q * f(lam)) @ Q.T @ x64
+    np.testing.assert_allclose(oracle.chebnet2(x, csc, f(nodes)), want, rtol=1e-5, atol=1e-5)
+    # any non-negative values: sum' coe_i T_i(A) with T_i(A) = Q cos(i arccos lambda) Q^T
+    temp = rng.random(K + 1) + 0.1
+    coe = oracle.chebnet2_coefficients(temp)
+    ref = np.polynomial.chebyshev.chebinterpolate(lambda v: np.interp(v, nodes, temp), K)   # same nodes, library routine
+    assert np.allclose(coe[0] / 2, ref[0]) and np.allclose(coe[1:], ref[1:])
+    Ti = lambda i: (Q * np.cos(i * np.arccos(np.clip(lam, -1, 1)))) @ Q.T
+    want = (coe[0] / 2 * Ti(0) + sum(coe[i] * Ti(i) for i in range(1, K + 1))) @ x64
+    np.testing.assert_allclose(oracle.chebnet2(x, csc, temp), want, rtol=1e-5, atol=1e-5)
+    # negative parameters are clamped at zero first
+    assert np.array_equal(oracle.chebnet2(x, csc, [-1.0, 2.0, -3.0]), oracle.chebnet2(x, csc, [0.0, 2.0, 0.0]))
+
+
+def test_bernnet_dense_closed_form_and_binomial_theorem():
+    from math import comb
+    rng, ei, w, csc, A = _small_symmetric(78)
+    V = A.shape[0]
+    x = rng.standard_normal((V, 4)).astype(np.float32)
+    x64 = x.astype(np.float64)
+    # L = I - A and 2I - L = I + A as weighted graphs of their own
+    def as_csc(M):
+        r, c = np.nonzero(M)
+        e = np.stack([c, r]).astype(np.int32)             # edge j -> i carries M[i, j]
+        return oracle.cootocsc(e, M[r, c].astype(np.float32), V)
+    L, L2 = np.eye(V) - A, np.eye(V) + A
+    csc1, csc2 = as_csc(L), as_csc(L2)
+    K = 4
+    temp = rng.random(K + 1).astype(np.float32)
+    want = sum(comb(K, i) / 2 ** K * float(temp[i]) * np.linalg.matrix_power(L, i) @ np.linalg.matrix_power(L2, K - i) @ x64
+               for i in range(K + 1))
+    np.testing.assert_allclose(oracle.bernnet(x, csc1, csc2, temp), want, rtol=1e-5, atol=1e-5)
+    # all weights one: ((L + (2I - L)) / 2)^K = I
+    np.testing.assert_allclose(oracle.bernnet(x, csc1, csc2, np.ones(K + 1)), x64, rtol=1e-5, atol=1e-5)
+    # two unrelated matrices (they do not commute): the order A1^i A2^(K-i) matters
+    B = rng.standard_normal((V, V)) * (rng.random((V, V)) < 0.2)
+    want = sum(comb(3, i) / 8 * np.linalg.matrix_power(L, i) @ np.linalg.matrix_power(B, 3 - i) @ x64 for i in range(4))
+    np.testing.assert_allclose(oracle.bernnet(x, csc1, as_csc(B), np.ones(4)), want, rtol=1e-4, atol=1e-4)
+    assert np.array_equal(oracle.bernnet(x, csc1, csc2, [-1.0, 1.0, -2.0]), oracle.bernnet(x, csc1, csc2, [0.0, 1.0, 0.0]))
+
+
 # -------------------------------------------------- sampled-subgraph operators ---
 
 def _global_csc(rng, V, E):
