@@ -1,6 +1,7 @@
 from .appnp_conv import APPNP  # noqa: F401
 from .bernnet_conv import BernNet  # noqa: F401
 from .chebnet2_conv import ChebNetII  # noqa: F401
+from .clustergcn_conv import ClusterGCNConv, clustergcn_norm  # noqa: F401
 from .even_conv import EvenNet  # noqa: F401
 from .gat_conv import GATConv  # noqa: F401
 from .gcn2_conv import GCN2Conv  # noqa: F401

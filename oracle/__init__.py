@@ -20,6 +20,11 @@ jittor==1.3.9.14).  Pins of the numpy restatements at the end of this file:
                 PageRank limit alpha * (I - (1 - alpha) A)^-1 h on a small graph
   sgconv        dense fp64 A^K x W
   gprgnn        dense fp64 sum_k temp[k] A^k x
+  clustergcn_norm  integer degrees: 1 / deg[row] exactly; on a symmetric graph every row's
+                outgoing weights sum to 1 (mass is kept: sum_v (A x)[v] = sum_v x[v]), which
+                scaling by the other endpoint's degree does not give; the trace grows by
+                diag_lambda * sum 1 / deg
+  clustergcn_conv  dense fp64 (A x) W_out + x W_root + b
   lightgcn      dense fp64 A x
   gcn2conv      dense fp64 A ((1-b)(1-a) x + b x W1) + (1-b) a x0 + b x0 W2
   evennet       dense fp64 t0 x + t3 A^3 x + t4 A^4 x (the hops the loop adds as written)
@@ -299,6 +304,28 @@ def sage_norm(edge_index, edge_weight=None, num_nodes=None, improved=False, add_
     return edge_index, (edge_weight * di[col]).astype(np.float32)
 
 
+def clustergcn_norm(edge_index, edge_weight=None, num_nodes=None, improved=False, add_self_loops=True,
+                    diag_lambda=0.0):
+    """nn/conv/clustergcn_conv.py:14-39: deg summed by col, w = w * deg^-1[row], and every
+    self-loop gets diag_lambda * deg^-1[row] on top."""
+    edge_index = np.asarray(edge_index)
+    N = int(edge_index.max()) + 1 if num_nodes is None else int(num_nodes)
+    fill = 2.0 if improved else 1.0
+    if edge_weight is None:
+        edge_weight = np.ones(edge_index.shape[1], np.float32)
+    if add_self_loops:
+        edge_index, edge_weight = add_remaining_self_loops(edge_index, edge_weight, fill, N)
+    row, col = edge_index[0], edge_index[1]
+    deg = _degree_by_col(col, edge_weight, N)
+    with np.errstate(divide="ignore"):
+        di = np.power(deg, np.float32(-1.0)).astype(np.float32)
+    di[np.isinf(di)] = 0
+    w = (edge_weight * di[row]).astype(np.float32)
+    loop = row == col
+    w[loop] = (w[loop] + np.float32(diag_lambda) * di[row[loop]]).astype(np.float32)
+    return edge_index, w
+
+
 # ------------------------------------------------------ numpy: op wrappers ---
 
 def aggregate_with_weight(x, csc, csr=None):
@@ -538,6 +565,14 @@ def bernnet(x, csc1, csc2, temp):
             v = aggregate_with_weight(v, csc1)
         out = (out + np.float32(comb(K, i + 1) / 2 ** K) * t[i + 1] * v).astype(np.float32)
     return out
+
+
+def clustergcn_conv(x, csc, weight_out, weight_root, bias=None):
+    """nn/conv/clustergcn_conv.py:136-143: propagate(x) @ weight_out + x @ weight_root (+ bias)."""
+    x = _f32(x)
+    mm = lambda a, w: (a.astype(np.float64) @ np.asarray(w, np.float64)).astype(np.float32)
+    out = (mm(aggregate_with_weight(x, csc), weight_out) + mm(x, weight_root)).astype(np.float32)
+    return out if bias is None else (out + _f32(bias)).astype(np.float32)
 
 
 def gpuinitco(dst_size, fanout_i, csc_layer_dst, csc_global_column_offset):

@@ -593,3 +593,44 @@ def test_sage_layer_with_the_activation_in_its_store_is_relu_of_the_layer(root, 
     assert torch.equal(plain.bias.grad, fused.bias.grad)
     if root:
         assert torch.equal(plain.root_weight.grad, fused.root_weight.grad)
+
+
+@pytest.mark.parametrize("spmm,lam,weighted", [(True, 0.0, False), (False, 0.3, False), (True, 0.3, True)])
+def test_clustergcn_layer(spmm, lam, weighted):
+    """clustergcn_norm's weights are asymmetric on an irregular graph (scaled by the source's
+    degree only), so the backward must be the true transpose, as for SAGEConv."""
+    from jittorgeometric_amd.nn import ClusterGCNConv, clustergcn_norm
+    from jittorgeometric_amd import synthetic
+    V = 3000
+    ei = synthetic.chung_lu(V, 40000, 2.1, max_degree=800, seed=19)
+    rng = np.random.default_rng(3)
+    w = (rng.random(ei.shape[1]) + 0.5).astype(np.float32) if weighted else None
+    x = rng.standard_normal((V, 64)).astype(np.float32)
+    g = rng.standard_normal((V, 24)).astype(np.float32)
+    eit, wt = clustergcn_norm(to_gpu(ei), None if w is None else to_gpu(w), V, diag_lambda=lam)
+    oei, ow = oracle.clustergcn_norm(ei, w, V, diag_lambda=lam)
+    assert np.array_equal(eit.cpu().numpy(), oei)
+    assert_close(wt.cpu().numpy(), ow, rtol=2e-6, atol=0)
+    torch.manual_seed(1)
+    layer = ClusterGCNConv(64, 24, diag_lambda=lam, spmm=spmm, cached=True).to(dev())
+    with torch.no_grad():
+        layer.bias.copy_(to_gpu(rng.standard_normal(24).astype(np.float32)))
+    xt = to_gpu(x).requires_grad_(True)
+    out = layer(xt, to_gpu(ei), None if w is None else to_gpu(w))
+    out.backward(to_gpu(g))
+    again = layer(to_gpu(x), None, None)                      # from the cached arrays
+    assert torch.equal(again, out.detach())
+    params = [p.detach().cpu().numpy() for p in (layer.weight_out, layer.weight_root, layer.bias)]
+    want = oracle.clustergcn_conv(x, oracle.cootocsc(oei, ow, V), *params)
+    assert_close(out.detach().cpu().numpy(), want, rtol=1e-4, atol=1e-5, what="against the oracle")
+
+    A = dense_adj(oei, ow, V)
+    x64 = torch.from_numpy(x.astype(np.float64)).requires_grad_(True)
+    Wo, Wr, b = [torch.from_numpy(p.astype(np.float64)).requires_grad_(True) for p in params]
+    ref = (A @ x64) @ Wo + x64 @ Wr + b
+    ref.backward(torch.from_numpy(g.astype(np.float64)))
+    assert_close(out.detach().cpu().numpy(), ref.detach().numpy(), rtol=1e-4, atol=1e-5, what="out")
+    for got, want, name in ((xt.grad, x64.grad, "x"), (layer.weight_out.grad, Wo.grad, "W_out"),
+                            (layer.weight_root.grad, Wr.grad, "W_root"), (layer.bias.grad, b.grad, "bias")):
+        want = want.numpy()
+        assert_close(got.cpu().numpy(), want, np.abs(want) + np.abs(want).max() * 1e-2, rtol=1e-4, what="grad " + name)

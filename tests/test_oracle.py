@@ -271,6 +271,44 @@ def test_gcn_and_sage_norm_closed_forms():
     np.testing.assert_allclose(colsum, 1, rtol=1e-5)
 
 
+def test_clustergcn_norm_and_conv_closed_forms():
+    rng = np.random.default_rng(81)
+    V = 40
+    ei, _ = rand_graph(rng, V, 260, loops=False)
+    ei = np.unique(np.concatenate([ei, ei[::-1]], axis=1), axis=1).astype(np.int32)      # symmetric, no repeats
+    oi, ow = oracle.clustergcn_norm(ei, None, V)
+    assert oi.shape[1] == ei.shape[1] + V
+    deg = np.bincount(oi[1], minlength=V).astype(np.float64)
+    assert deg.min() >= 1 and len(set(deg.tolist())) > 3                                  # irregular
+    np.testing.assert_allclose(ow, 1 / deg[oi[0]], rtol=1e-6)
+    A = sp.coo_matrix((ow.astype(np.float64), (oi[1], oi[0])), shape=(V, V)).toarray()   # A[dst, src]
+    np.testing.assert_allclose(A.sum(0), 1, rtol=1e-5)             # what leaves a node sums to 1 ...
+    assert np.abs(A.sum(1) - 1).max() > 0.05                       # ... what arrives does not
+    x = rng.standard_normal((V, 5)).astype(np.float32)
+    csc = oracle.cootocsc(oi, ow, V)
+    np.testing.assert_allclose(oracle.aggregate_with_weight(x, csc).astype(np.float64).sum(0), x.astype(np.float64).sum(0),
+                               rtol=1e-4, atol=1e-4)
+    # diagonal enhancement: only the self-loops change, by lambda / deg
+    li, lw = oracle.clustergcn_norm(ei, None, V, diag_lambda=0.7)
+    assert np.array_equal(li, oi)
+    loop = li[0] == li[1]
+    np.testing.assert_allclose(lw[~loop], ow[~loop], rtol=0)
+    np.testing.assert_allclose(lw[loop], (1 + 0.7) / deg[li[0][loop]], rtol=1e-6)
+    # weighted, improved self-loops
+    w = (rng.random(ei.shape[1]) + 0.5).astype(np.float32)
+    wi, ww = oracle.clustergcn_norm(ei, w, V, improved=True, diag_lambda=0.25)
+    full_w = np.concatenate([w, np.full(V, 2.0, np.float32)]).astype(np.float64)
+    degw = np.zeros(V)
+    np.add.at(degw, wi[1], full_w)
+    want = full_w / degw[wi[0]] + 0.25 * (wi[0] == wi[1]) / degw[wi[0]]
+    np.testing.assert_allclose(ww, want, rtol=1e-5)
+    # the layer
+    Wo, Wr, b = rng.standard_normal((5, 3)), rng.standard_normal((5, 3)), rng.standard_normal(3)
+    want = A @ x.astype(np.float64) @ Wo + x.astype(np.float64) @ Wr + b
+    np.testing.assert_allclose(oracle.clustergcn_conv(x, csc, Wo, Wr, b), want, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(oracle.clustergcn_conv(x, csc, Wo, Wr), want - b, rtol=1e-5, atol=1e-5)
+
+
 # ------------------------------------------------------------ GAT pieces ----
 
 def test_gat_forward_matches_dense_fp64():
