@@ -273,7 +273,10 @@ int32_t jgamd_scatter_to_edge(const int32_t *off, const int32_t *idx, const floa
  * [E,2C]x[2C,1] product, leaky_relu, EdgeSoftmax, multiply, ScatterToVertex.
  *   h      [V,H,D]   node features after vertex_forward
  *   a_src  [H,D], a_dst [H,D]  the two halves of GATConv.edge_weight
- *   el,er  [V,H]  outputs: a_src.h and a_dst.h per node and head
+ *   el,er  [V,H]  outputs: a_src.h and a_dst.h per node and head; both NULL
+ *          when no backward pass follows (pos, spos and alpha then NULL as
+ *          well): the scores are then taken inside the aggregation kernel and
+ *          the pass over h that computes the two arrays is not run
  *   smax, ssum [V,H] outputs: per destination and head, the max logit and
  *          the sum of exp(logit - max) (what backward needs to rebuild alpha)
  *   pos [V,H,D], spos [V,H]  optional outputs (both or neither): the share of

@@ -160,13 +160,21 @@ struct GatPieces {
     float *pvec, *psum;        // the positive-logit share, POS only
 };
 
-template <int VEC, int NT, bool POS>
+// SCORES (one tile per lane, lph = D / VEC lanes per head, a power of two): the caller wants no
+// el / er arrays (no backward pass follows), and the two dot products are taken where the rows
+// pass through registers anyway -- a_src.h[src] from every gathered row, a_dst.h[r] from the
+// destination's own row, fetched one row ahead as er is otherwise -- folded over the head's
+// lanes with DPP adds.  The pass over h that computes the two arrays (a sixth of the forward
+// time at 169k nodes of 8 x 16 features) and one 4-byte gather per entry then fall away.
+template <int VEC, int NT, bool POS, bool SCORES = false>
 __global__ __launch_bounds__(kGatThreads) void gat_fwd_merge(
     const int32_t *__restrict__ off, const int32_t *__restrict__ idx, const float *__restrict__ h,
     const float *__restrict__ el, const float *__restrict__ er, float slope, float *__restrict__ out,
     float *__restrict__ smax, float *__restrict__ ssum, float *__restrict__ pos, float *__restrict__ spos,
-    GatPieces piece, const int2 *__restrict__ start, int R, int E, int H, int D, int nchunks)
+    GatPieces piece, const int2 *__restrict__ start, int R, int E, int H, int D, int nchunks,
+    const float *__restrict__ a_src = nullptr, const float *__restrict__ a_dst = nullptr, int lph = 0)
 {
+    static_assert(!SCORES || (NT == 1 && !POS), "scores in the kernel: one tile, inference only");
     constexpr int kGatUnroll = gat_unroll(VEC * NT * (POS ? 2 : 1));
     const int k = blockIdx.x * kGatWaves + wave_in_block();
     if (k >= nchunks) return;
@@ -200,10 +208,25 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_merge(
     // wait for a fresh load (rows are a handful of entries long)
     float m[NT], l[NT], acc[NT][VEC], er_r[NT], er_next[NT];
     float lp[POS ? NT : 1], pacc[POS ? NT : 1][POS ? VEC : 1];
+    // SCORES: this lane's slices of a_src / a_dst, and the next destination's own slice of h
+    float as_[SCORES ? NT : 1][SCORES ? VEC : 1], ad_[SCORES ? NT : 1][SCORES ? VEC : 1];
+    float hr_next[SCORES ? NT : 1][SCORES ? VEC : 1];
+    if constexpr (SCORES) {
+#pragma unroll
+        for (int t = 0; t < NT; t++)
+#pragma unroll
+            for (int v = 0; v < VEC; v++) {
+                as_[t][v] = a_src[fo[t] + v];
+                ad_[t][v] = a_dst[fo[t] + v];
+            }
+    }
     auto fetch_row = [&](int row) {
         const size_t rn = (size_t)min(row, R - 1);
 #pragma unroll
-        for (int t = 0; t < NT; t++) er_next[t] = er[rn * H + head[t]];
+        for (int t = 0; t < NT; t++) {
+            if constexpr (SCORES) gload<VEC>(hr_next[t], h + rn * F + fo[t]);
+            else er_next[t] = er[rn * H + head[t]];
+        }
     };
     auto fetch_next = [&]() { fetch_row(r + 1); };
     auto reset = [&]() {
@@ -218,7 +241,14 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_merge(
 #pragma unroll
                 for (int v = 0; v < VEC; v++) pacc[t][v] = 0.f;
             }
-            er_r[t] = er_next[t];
+            if constexpr (SCORES) {
+                float d = 0.f;
+#pragma unroll
+                for (int v = 0; v < VEC; v++) d = fmaf(hr_next[t][v], ad_[t][v], d);
+                er_r[t] = lane_group_sum(d, lph);      // every lane runs this: row ends are wave-uniform
+            } else {
+                er_r[t] = er_next[t];
+            }
         }
         fetch_next();
     };
@@ -276,7 +306,7 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_merge(
 #pragma unroll
                 for (int t = 0; t < NT; t++) {
                     gload<VEC>(xv[u][t], src + fo[t]);
-                    sv[u][t] = sl[head[t]];
+                    if constexpr (!SCORES) sv[u][t] = sl[head[t]];
                 }
             }
 #pragma unroll
@@ -286,6 +316,16 @@ __global__ __launch_bounds__(kGatThreads) void gat_fwd_merge(
                     while (jj == row_end && r < r1) flush_row();
                     const int c = bcast_i(my_c, i0 + u);
                     if (c >= 0) {
+                        if constexpr (SCORES) {
+                            // all lanes take part (c is wave-uniform): the adds read neighbouring lanes
+#pragma unroll
+                            for (int t = 0; t < NT; t++) {
+                                float d = 0.f;
+#pragma unroll
+                                for (int v = 0; v < VEC; v++) d = fmaf(xv[u][t][v], as_[t][v], d);
+                                sv[u][t] = lane_group_sum(d, lph);
+                            }
+                        }
 #pragma unroll
                         for (int t = 0; t < NT; t++)
                             if (act[t]) {
@@ -1100,8 +1140,9 @@ static size_t gat_fwd_ws(int32_t V, int64_t E, int32_t H, int32_t D)
 {
     GatShape s = gat_shape(V, E, H, D);
     const size_t ng = (size_t)ceil_div(s.nchunks, kGatGroup);
+    // + el / er of a call that brings none and whose shape the in-kernel scores do not cover
     return carve_bytes((size_t)s.nchunks + 1, sizeof(int2)) + pieces_bytes((size_t)s.nchunks, H, D) +
-           pieces_bytes(ng, H, D);
+           pieces_bytes(ng, H, D) + 2 * carve_bytes((size_t)V * H, 4);
 }
 
 static size_t gat_bwd_ws(int32_t V, int64_t E, int32_t H, int32_t D)
@@ -1144,8 +1185,10 @@ JG_EXPORT int32_t jgamd_gat_fwd(const void *plan, int32_t n_fix, int32_t n_grp, 
 {
     if (int32_t rc = check_gat("gat_fwd", V, E, H, D)) return rc;
     if (V == 0) return 0;
-    if (!off || !h || !a_src || !a_dst || !el || !er || !smax || !ssum || !out)
+    if (!off || !h || !a_src || !a_dst || !smax || !ssum || !out)
         return fail(JGAMD_ERR_NULL, "gat_fwd: NULL array");
+    if ((el == nullptr) != (er == nullptr)) return fail(JGAMD_ERR_NULL, "gat_fwd: el and er go together");
+    if (!el && (pos || alpha)) return fail(JGAMD_ERR_NULL, "gat_fwd: pos / alpha need el and er");
     if ((pos == nullptr) != (spos == nullptr)) return fail(JGAMD_ERR_NULL, "gat_fwd: pos and spos go together");
     if (E > 0 && !idx) return fail(JGAMD_ERR_NULL, "gat_fwd: idx is NULL with E > 0");
     if ((((uintptr_t)h | (uintptr_t)out | (uintptr_t)pos) & 15) != 0)
@@ -1171,7 +1214,17 @@ JG_EXPORT int32_t jgamd_gat_fwd(const void *plan, int32_t n_fix, int32_t n_grp, 
     const GatPieces group = carve_pieces(carve, (size_t)ngroups, H, D);
     const int64_t VH = (int64_t)V * H;
     if (pos && !s.bwd_ok) return fail(JGAMD_ERR_UNSUPPORTED, "gat_fwd: pos / spos need a shape jgamd_gat_bwd takes");
-    if (vec_nodes_ok(D) && (((uintptr_t)a_src | (uintptr_t)a_dst) & 15) == 0)
+    float *own_el = carve.take<float>((size_t)V * H), *own_er = carve.take<float>((size_t)V * H);
+    // no el / er wanted: the scores are taken inside the merge kernel where its lane layout allows
+    static const bool no_fuse = [] { const char *e = getenv("JGAMD_GAT_SCORES"); return e && e[0] == 'n'; }();
+    const bool fuse = !el && !no_fuse && s.nt == 1 && D % s.vec == 0 && s.lph >= 1 && s.lph <= kWave &&
+                      (s.lph & (s.lph - 1)) == 0;
+    if (!el) {
+        el = own_el;
+        er = own_er;
+    }
+    if (fuse) {
+    } else if (vec_nodes_ok(D) && (((uintptr_t)a_src | (uintptr_t)a_dst) & 15) == 0)
         hipLaunchKernelGGL(gat_node_scores_vec, dim3((unsigned)ceil_div(VH * (D / 4), 256)), dim3(256), 0, st,
                            reinterpret_cast<const float4 *>(h), reinterpret_cast<const float4 *>(a_src),
                            reinterpret_cast<const float4 *>(a_dst), el, er, VH * (D / 4), H, D / 4);
@@ -1186,8 +1239,13 @@ JG_EXPORT int32_t jgamd_gat_fwd(const void *plan, int32_t n_fix, int32_t n_grp, 
     const bool with_group = ngroups > 1 && n_grp != 0 && n_fix != 0;
 #define JG_FWD_P(VV, NN, PP)                                                                                     \
     {                                                                                                            \
-        hipLaunchKernelGGL((gat_fwd_merge<VV, NN, PP>), grid, block, 0, st, off, idx, h, el, er, slope, out,     \
-                           smax, ssum, pos, spos, piece, pv.start, V, (int)E, H, D, s.nchunks);                  \
+        if (!PP && fuse)                                                                                         \
+            hipLaunchKernelGGL((gat_fwd_merge<VV, 1, false, true>), grid, block, 0, st, off, idx, h, el, er,     \
+                               slope, out, smax, ssum, pos, spos, piece, pv.start, V, (int)E, H, D, s.nchunks,   \
+                               a_src, a_dst, s.lph);                                                             \
+        else                                                                                                     \
+            hipLaunchKernelGGL((gat_fwd_merge<VV, NN, PP>), grid, block, 0, st, off, idx, h, el, er, slope, out, \
+                               smax, ssum, pos, spos, piece, pv.start, V, (int)E, H, D, s.nchunks);              \
         if (with_group)                                                                                          \
             hipLaunchKernelGGL((gat_fwd_group<VV, NN, PP>), ggrid, block, 0, st, off, piece, group, pv.start,    \
                                pv.grp, pv.counts + 1, V, H, D, s.chunk, s.nchunks);                              \

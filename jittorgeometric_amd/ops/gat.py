@@ -23,10 +23,11 @@ def fused_supported(H, D, backward=True):
     return True
 
 
-def gat_forward_raw(h, csc, a_src, a_dst, slope=0.2, want_alpha=False, for_backward=False):
+def gat_forward_raw(h, csc, a_src, a_dst, slope=0.2, want_alpha=False, for_backward=False, want_scores=None):
     """h [V,H,D], a_src/a_dst [H,D] -> dict(out, el, er, smax, ssum, alpha, pos, spos); pos / spos
     (the positive-logit share of out and of the attention, which the backward kernels read) are
-    only computed with for_backward."""
+    only computed with for_backward, and el / er only when something reads them (want_scores;
+    by default with want_alpha or for_backward): without them the kernel takes the scores itself."""
     lib = _lib.load()
     dev = _lib.require_gpu(h, csc.row_indices, csc.column_offset, a_src, a_dst)
     h, a_src, a_dst = as_f32(h, "h"), as_f32(a_src, "a_src"), as_f32(a_dst, "a_dst")
@@ -39,7 +40,12 @@ def gat_forward_raw(h, csc, a_src, a_dst, slope=0.2, want_alpha=False, for_backw
         raise _lib.JgamdError("gat: %d column offsets for %d nodes" % (off.shape[0], V))
     E = idx.shape[0]
     mk = lambda *s: torch.empty(s, dtype=torch.float32, device=dev)
-    out, el, er, smax, ssum = mk(V, H, D), mk(V, H), mk(V, H), mk(V, H), mk(V, H)
+    if want_scores is None:
+        want_scores = want_alpha or for_backward
+    if (want_alpha or for_backward) and not want_scores:
+        raise _lib.JgamdError("gat: alpha and the backward arrays need el / er")
+    out, smax, ssum = mk(V, H, D), mk(V, H), mk(V, H)
+    el, er = (mk(V, H), mk(V, H)) if want_scores else (None, None)
     alpha = mk(E, H) if want_alpha else None
     pos, spos = (mk(V, H, D), mk(V, H)) if for_backward else (None, None)
     nbytes = _lib.query(lib.jgamd_gat_fwd_workspace, V, E, H, D)

@@ -101,6 +101,17 @@ def run_case(V, E, H, D, hubs, seed, check_oracle=True):
     hs = torch.zeros((V, H, D), dtype=torch.float64).index_add(
         0, torch.from_numpy(dst.astype(np.int64)), ref_alpha.detach().unsqueeze(-1) * h64.detach().abs()[row]).numpy()
     check_against_fp64(raw["alpha"], out, ht.grad, ast.grad, adt.grad, ref, ref_alpha, h64, as64, ad64, g, row, dst, V)
+    # the forward alone, as a caller without a backward pass runs it: no el / er arrays, the scores
+    # are taken inside the aggregation kernel where its lane layout allows (else in a workspace)
+    inf = gat_forward_raw(to_gpu(h), csc, to_gpu(a_src), to_gpu(a_dst), 0.2)
+    assert inf["el"] is None and inf["er"] is None and raw["el"] is not None
+    assert_close(inf["out"].cpu().numpy(), ref.detach().numpy(), hs, what="out of the forward without el / er")
+    finite = lambda t: np.nan_to_num(t.cpu().numpy(), neginf=-1e30)       # destinations without entries hold -inf
+    assert_close(finite(inf["smax"]), finite(raw["smax"]), rtol=1e-5, atol=1e-6, what="smax")
+    assert_close(inf["ssum"].cpu().numpy(), raw["ssum"].cpu().numpy(), rtol=1e-4, atol=1e-6, what="ssum")
+    with torch.no_grad():
+        out_ng = gat_aggregate(to_gpu(h), csc, to_gpu(a_src), to_gpu(a_dst), 0.2)
+    assert torch.equal(out_ng, inf["out"])
     if check_oracle:
         # the reference's loops add a destination's terms one by one in fp32, so the
         # oracle itself is only good to about deg * 2^-24 relative on long columns
