@@ -383,11 +383,17 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_fixup(const int32_t *__rest
         const int a = min((int)(((int64_t)max(s, 0) + r0) / chunk), k);
         const int lane = lane_id();
         const int f0 = blockIdx.y * (kWave * VEC * NT) + lane * VEC;
-        float acc[NT][VEC];
+        float acc[NT][VEC], last[NT][VEC];
+        float *dst = out + (size_t)r0 * F;
+        // the row's last piece, as the chunk's wavefront stored it: fetched with the first pieces
+        // rather than after them (one memory round trip less), added last as before
 #pragma unroll
-        for (int t = 0; t < NT; t++)
+        for (int t = 0; t < NT; t++) {
+            const int f = f0 + t * kWave * VEC;
+            vload<VEC>(last[t], dst + (f < F ? f : 0));
 #pragma unroll
             for (int v = 0; v < VEC; v++) acc[t][v] = 0.f;
+        }
         const int ga = a / kGroup, gb = k / kGroup;
         if (ga == gb) {
             add_pieces<VEC, NT>(acc, partial, a, k, F, f0);
@@ -413,8 +419,10 @@ __global__ __launch_bounds__(kSpmmThreads) void spmm_fixup(const int32_t *__rest
             add_pieces<VEC, NT>(acc, group_sum, ga, gb, F, f0);
             add_pieces<VEC, NT>(acc, partial, gb * kGroup, k, F, f0);
         }
-        float *dst = out + (size_t)r0 * F;
-        add_pieces<VEC, NT>(acc, dst, 0, 1, F, f0);
+#pragma unroll
+        for (int t = 0; t < NT; t++)
+#pragma unroll
+            for (int v = 0; v < VEC; v++) acc[t][v] += last[t][v];
         if constexpr (EPI) {
 #pragma unroll
             for (int t = 0; t < NT; t++)
