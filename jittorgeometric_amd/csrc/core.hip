@@ -138,5 +138,5 @@ int32_t exclusive_scan_i32(const int32_t *in, int32_t *out, int64_t n, int32_t *
 
 }  // namespace jg
 
-extern "C" __attribute__((visibility("default"))) int32_t jgamd_version(void) { return 100; }
+extern "C" __attribute__((visibility("default"))) int32_t jgamd_version(void) { return 300; }
 extern "C" __attribute__((visibility("default"))) const char *jgamd_last_error(void) { return jg::g_err; }
