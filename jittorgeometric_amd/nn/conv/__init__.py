@@ -1,5 +1,6 @@
 from .appnp_conv import APPNP  # noqa: F401
 from .bernnet_conv import BernNet  # noqa: F401
+from .cheb_conv import ChebConv  # noqa: F401
 from .chebnet2_conv import ChebNetII  # noqa: F401
 from .clustergcn_conv import ClusterGCNConv, clustergcn_norm  # noqa: F401
 from .even_conv import EvenNet  # noqa: F401

@@ -34,3 +34,23 @@ def add_remaining_self_loops(edge_index, edge_weight=None, fill_value=1.0, num_n
     if edge_index.dtype != torch.int32:
         out_index = out_index.to(edge_index.dtype)
     return out_index, (out_w[:n_out] if edge_weight is not None else None)
+
+
+def remove_self_loops(edge_index, edge_attr=None):
+    """The edges with two different endpoints, in their order (utils/loop.py:22-38)."""
+    mask = edge_index[0] != edge_index[1]
+    edge_index = edge_index[:, mask]
+    return edge_index, (None if edge_attr is None else edge_attr[mask])
+
+
+def add_self_loops(edge_index, edge_weight=None, fill_value=1.0, num_nodes=None):
+    """One loop (i, i) per node appended after the edges, with weight fill_value when the
+    edges carry weights (utils/loop.py:64-95); existing loops stay."""
+    N = int(maybe_num_nodes(edge_index, num_nodes))
+    loop_index = torch.arange(N, dtype=edge_index.dtype, device=edge_index.device).unsqueeze(0).repeat(2, 1)
+    if edge_weight is not None:
+        if edge_weight.numel() != edge_index.size(1):
+            raise ValueError("add_self_loops: %d weights for %d edges" % (edge_weight.numel(), edge_index.size(1)))
+        loop_weight = torch.full((N,), fill_value, dtype=edge_weight.dtype, device=edge_weight.device)
+        edge_weight = torch.cat([edge_weight, loop_weight], dim=0)
+    return torch.cat([edge_index, loop_index], dim=1), edge_weight

@@ -25,6 +25,10 @@ jittor==1.3.9.14).  Pins of the numpy restatements at the end of this file:
                 scaling by the other endpoint's degree does not give; the trace grows by
                 diag_lambda * sum 1 / deg
   clustergcn_conv  dense fp64 (A x) W_out + x W_root + b
+  get_laplacian scipy.sparse.csgraph.laplacian on a symmetric weighted graph (all three
+                normalisations; 'rw' against I - D^-1 A); rows of D - A sum to zero
+  cheb_norm / cheb_conv  dense fp64: L^ = 2 L / lambda - I and T_k(L^) from the eigenvalues
+                of the symmetric L^ (cos(k arccos .) inside [-1, 1], cosh outside)
   lightgcn      dense fp64 A x
   gcn2conv      dense fp64 A ((1-b)(1-a) x + b x W1) + (1-b) a x0 + b x0 W2
   evennet       dense fp64 t0 x + t3 A^3 x + t4 A^4 x (the hops the loop adds as written)
@@ -324,6 +328,68 @@ def clustergcn_norm(edge_index, edge_weight=None, num_nodes=None, improved=False
     loop = row == col
     w[loop] = (w[loop] + np.float32(diag_lambda) * di[row[loop]]).astype(np.float32)
     return edge_index, w
+
+
+def get_laplacian(edge_index, edge_weight=None, normalization=None, num_nodes=None):
+    """utils/get_laplacian.py:9-81: self-loops removed, degree summed by row (the source),
+    None: L = D - A; 'sym': I - D^-1/2 A D^-1/2; 'rw': I - D^-1 A; the N diagonal entries are
+    appended after the other edges."""
+    ei = np.asarray(edge_index)
+    keep = ei[0] != ei[1]
+    w = np.ones(ei.shape[1], np.float32) if edge_weight is None else _f32(edge_weight)
+    ei, w = ei[:, keep], w[keep]
+    N = int(ei.max()) + 1 if num_nodes is None else int(num_nodes)
+    row, col = ei[0], ei[1]
+    deg = np.zeros(N, np.float32)
+    np.add.at(deg, row, w)
+    loops = np.stack([np.arange(N)] * 2).astype(ei.dtype)
+    if normalization is None:
+        return np.concatenate([ei, loops], axis=1), np.concatenate([-w, deg]).astype(np.float32)
+    with np.errstate(divide="ignore"):
+        if normalization == "sym":
+            d = np.power(deg, np.float32(-0.5)).astype(np.float32)
+            d[np.isinf(d)] = 0
+            a = (d[row] * w * d[col]).astype(np.float32)
+        else:
+            d = (np.float32(1.0) / deg).astype(np.float32)
+            d[np.isinf(d)] = 0
+            a = (d[row] * w).astype(np.float32)
+    return np.concatenate([ei, loops], axis=1), np.concatenate([-a, np.ones(N, np.float32)]).astype(np.float32)
+
+
+def cheb_norm(edge_index, num_nodes, edge_weight=None, normalization="sym", lambda_max=None, batch=None):
+    """nn/conv/cheb_conv.py:97-122: the Laplacian scaled to 2 L / lambda_max - I (lambda_max
+    defaults to twice the largest entry; infinite weights become 0; 1 is taken off the loops)."""
+    ei, w = get_laplacian(edge_index, edge_weight, normalization, num_nodes)
+    lam = np.float32(2.0) * w.max() if lambda_max is None else np.asarray(lambda_max, np.float32).reshape(-1)
+    if batch is not None and np.size(lam) > 1:
+        lam = lam[np.asarray(batch)[ei[0]]]
+    with np.errstate(divide="ignore", invalid="ignore"):
+        w = ((np.float32(2.0) * w) / lam).astype(np.float32)
+    w[np.isinf(w)] = 0
+    loop = ei[0] == ei[1]
+    w[loop] = w[loop] - np.float32(1)
+    return ei, w
+
+
+def cheb_conv(x, edge_index, weights, bias=None, edge_weight=None, normalization="sym", lambda_max=None, batch=None):
+    """nn/conv/cheb_conv.py:124-155: out = Tx_0 W_0 + Tx_1 W_1 + ..., Tx_1 = L^ x,
+    Tx_k = 2 L^ Tx_{k-1} - Tx_{k-2}, messages norm_e * x[src] summed at dst; weights[k] is [in, out]."""
+    x = _f32(x)
+    V = x.shape[0]
+    ei, norm = cheb_norm(edge_index, V, edge_weight, normalization, lambda_max, batch)
+    csc = cootocsc(ei.astype(np.int32), norm, V)
+    mm = lambda a, w: (a.astype(np.float64) @ np.asarray(w, np.float64)).astype(np.float32)
+    t0 = t1 = x
+    out = mm(t0, weights[0])
+    if len(weights) > 1:
+        t1 = aggregate_with_weight(x, csc)
+        out = (out + mm(t1, weights[1])).astype(np.float32)
+    for wk in weights[2:]:
+        t2 = (np.float32(2) * aggregate_with_weight(t1, csc) - t0).astype(np.float32)
+        out = (out + mm(t2, wk)).astype(np.float32)
+        t0, t1 = t1, t2
+    return out if bias is None else (out + _f32(bias)).astype(np.float32)
 
 
 # ------------------------------------------------------ numpy: op wrappers ---

@@ -634,3 +634,82 @@ def test_clustergcn_layer(spmm, lam, weighted):
                             (layer.weight_root.grad, Wr.grad, "W_root"), (layer.bias.grad, b.grad, "bias")):
         want = want.numpy()
         assert_close(got.cpu().numpy(), want, np.abs(want) + np.abs(want).max() * 1e-2, rtol=1e-4, what="grad " + name)
+
+
+@pytest.mark.parametrize("normalization", [None, "sym", "rw"])
+def test_get_laplacian(normalization):
+    from jittorgeometric_amd.utils import get_laplacian
+    from jittorgeometric_amd import synthetic
+    V = 4000
+    ei = synthetic.chung_lu(V, 50000, 2.1, max_degree=900, seed=29)
+    rng = np.random.default_rng(4)
+    loops = np.stack([rng.integers(0, V, 50)] * 2).astype(ei.dtype)          # a few self-loops: dropped
+    ei = np.concatenate([ei[:, :20000], loops, ei[:, 20000:]], axis=1)
+    ei[:, 100:110] = V - 1 - np.arange(10)[None, :]                          # more loops, in the middle
+    for w in (None, (rng.random(ei.shape[1]) + 0.5).astype(np.float32)):
+        gi, gw = get_laplacian(to_gpu(ei), None if w is None else to_gpu(w), normalization, num_nodes=V)
+        oi, ow = oracle.get_laplacian(ei, w, normalization, V)
+        assert np.array_equal(gi.cpu().numpy(), oi)
+        # the degree is a sum of up to 900 weights: fixed order here, numpy's own order in the oracle
+        assert_close(gw.cpu().numpy(), ow, rtol=1e-5 if w is not None else 2e-6, atol=0)
+    # nodes without an outgoing edge: D^-1/2 = inf becomes 0
+    few = np.array([[0, 1, 2], [1, 2, 0]], np.int32)
+    gi, gw = get_laplacian(to_gpu(few), None, normalization, num_nodes=6)
+    oi, ow = oracle.get_laplacian(few, None, normalization, 6)
+    assert np.array_equal(gi.cpu().numpy(), oi) and np.array_equal(gw.cpu().numpy(), ow)
+
+
+@pytest.mark.parametrize("K,normalization,lam", [(1, "sym", None), (2, "sym", None), (4, "sym", 2.5), (3, "rw", None),
+                                                 (3, None, 40.0)])
+def test_cheb_conv(K, normalization, lam):
+    """The reference sends norm_e * x[src] messages; here the scaled Laplacian is a compressed
+    matrix and every recurrence step one product with `2 * ... - T_{k-2}` in its row store."""
+    from jittorgeometric_amd.nn import ChebConv
+    from jittorgeometric_amd import synthetic
+    V, Fin, Fout = 2500, 32, 12
+    ei = synthetic.chung_lu(V, 30000, 2.1, max_degree=600, seed=39)
+    rng = np.random.default_rng(6)
+    w = (rng.random(ei.shape[1]) + 0.5).astype(np.float32)
+    x = rng.standard_normal((V, Fin)).astype(np.float32)
+    g = rng.standard_normal((V, Fout)).astype(np.float32)
+    torch.manual_seed(2)
+    layer = ChebConv(Fin, Fout, K, normalization=normalization).to(dev())
+    with torch.no_grad():
+        layer.bias.copy_(to_gpu(rng.standard_normal(Fout).astype(np.float32)))
+    ei_g, w_g = to_gpu(ei), to_gpu(w)
+    xt = to_gpu(x).requires_grad_(True)
+    out = layer(xt, ei_g, w_g, None, lam)
+    out.backward(to_gpu(g))
+    assert torch.equal(layer(to_gpu(x), ei_g, w_g, None, lam), out.detach())           # from the kept conversion
+    Ws = [lin.weight.detach().cpu().numpy().T for lin in layer.lins]                     # [in, out]
+    b = layer.bias.detach().cpu().numpy()
+    want = oracle.cheb_conv(x, ei, Ws, b, w, normalization, lam)
+    assert np.abs(out.detach().cpu().numpy() - want).max() <= 1e-4 * np.abs(want).max()
+
+    ni, nw = oracle.cheb_norm(ei, V, w, normalization, lam)
+    L = dense_adj(ni, nw, V)
+    x64 = torch.from_numpy(x.astype(np.float64)).requires_grad_(True)
+    W64 = [torch.from_numpy(W.astype(np.float64)).requires_grad_(True) for W in Ws]
+    b64 = torch.from_numpy(b.astype(np.float64)).requires_grad_(True)
+    t0 = t1 = x64
+    ref = t0 @ W64[0]
+    if K > 1:
+        t1 = L @ x64
+        ref = ref + t1 @ W64[1]
+    for k in range(2, K):
+        t0, t1 = t1, 2 * (L @ t1) - t0
+        ref = ref + t1 @ W64[k]
+    ref = ref + b64
+    ref.backward(torch.from_numpy(g.astype(np.float64)))
+    scale = np.abs(ref.detach().numpy()).max()
+    assert np.abs(out.detach().cpu().numpy() - ref.detach().numpy()).max() <= 1e-4 * scale
+    pairs = [(xt.grad, x64.grad, "x"), (layer.bias.grad, b64.grad, "bias")] + \
+            [(lin.weight.grad.t(), W.grad, "W%d" % k) for k, (lin, W) in enumerate(zip(layer.lins, W64))]
+    for got, ref_g, name in pairs:
+        ref_g = ref_g.numpy()
+        assert np.abs(got.cpu().numpy() - ref_g).max() <= 2e-4 * np.abs(ref_g).max(), name
+    # other edge tensors: the conversion is redone
+    ei2 = to_gpu(ei[:, :20000].copy())
+    out2 = layer(to_gpu(x), ei2, to_gpu(w[:20000].copy()), None, lam)
+    want2 = oracle.cheb_conv(x, ei[:, :20000], Ws, b, w[:20000], normalization, lam)
+    assert np.abs(out2.detach().cpu().numpy() - want2).max() <= 1e-4 * np.abs(want2).max()

@@ -309,6 +309,62 @@ def test_clustergcn_norm_and_conv_closed_forms():
     np.testing.assert_allclose(oracle.clustergcn_conv(x, csc, Wo, Wr), want - b, rtol=1e-5, atol=1e-5)
 
 
+def test_get_laplacian_against_scipy_and_cheb_conv_dense():
+    from scipy.sparse.csgraph import laplacian
+    rng = np.random.default_rng(83)
+    V = 35
+    ei, _ = rand_graph(rng, V, 220, loops=True)                      # some self-loops: they must be dropped
+    und = np.unique(np.sort(ei[:, ei[0] != ei[1]], axis=0), axis=1)
+    wu = (rng.random(und.shape[1]) + 0.5).astype(np.float32)
+    loops = np.stack([np.arange(0, V, 5)] * 2)
+    ei = np.concatenate([und, und[::-1], loops], axis=1).astype(np.int32)
+    w = np.concatenate([wu, wu, np.full(loops.shape[1], 9.0, np.float32)])
+    A = sp.coo_matrix((np.concatenate([wu, wu]).astype(np.float64), (np.concatenate([und[0], und[1]]), np.concatenate([und[1], und[0]]))),
+                      shape=(V, V)).toarray()
+    dense = lambda e, v: sp.coo_matrix((v.astype(np.float64), (e[1], e[0])), shape=(V, V)).toarray()   # [dst, src]
+    li, lw = oracle.get_laplacian(ei, w, None, V)
+    assert li.shape[1] == 2 * und.shape[1] + V and np.array_equal(li[:, -V:], np.stack([np.arange(V)] * 2))
+    np.testing.assert_allclose(dense(li, lw), laplacian(A), rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(dense(li, lw).sum(1), 0, atol=1e-4)
+    si, sw = oracle.get_laplacian(ei, w, "sym", V)
+    np.testing.assert_allclose(dense(si, sw), laplacian(A, normed=True), rtol=1e-5, atol=1e-6)
+    ri, rw = oracle.get_laplacian(ei, w, "rw", V)
+    deg = A.sum(1)
+    # entry (src -> dst) carries -w / deg[src]: as a [dst, src] matrix that is I - A D^-1
+    np.testing.assert_allclose(dense(ri, rw), np.eye(V) - A / deg[None, :], rtol=1e-5, atol=1e-6)
+    # unweighted
+    ui, uw = oracle.get_laplacian(ei, None, None, V)
+    np.testing.assert_allclose(dense(ui, uw), laplacian((A > 0).astype(np.float64)), atol=1e-6)
+
+    # scaled Laplacian and the layer, symmetric case: T_k from the eigenvalues
+    for lam in (None, 2.0, 3.5):
+        ni, nw = oracle.cheb_norm(ei, V, w, "sym", lam)
+        L = laplacian(A, normed=True)
+        lam_used = 2.0 * max(1.0, np.abs(L).max()) if lam is None else lam      # largest entry of L is its unit diagonal
+        Lh = 2.0 * L / lam_used - np.eye(V)
+        np.testing.assert_allclose(dense(ni, nw), Lh, rtol=1e-5, atol=1e-6)
+        x = rng.standard_normal((V, 4)).astype(np.float32)
+        Ws = [rng.standard_normal((4, 3)).astype(np.float32) for _ in range(4)]
+        b = rng.standard_normal(3).astype(np.float32)
+        ev, Q = np.linalg.eigh(Lh)
+
+        def T(k):
+            inside = np.abs(ev) <= 1
+            t = np.where(inside, np.cos(k * np.arccos(np.clip(ev, -1, 1))),
+                         np.sign(ev) ** k * np.cosh(k * np.arccosh(np.maximum(np.abs(ev), 1))))
+            return (Q * t) @ Q.T
+        for K in (1, 2, 4):
+            want = sum(T(k) @ x.astype(np.float64) @ Ws[k].astype(np.float64) for k in range(K)) + b
+            np.testing.assert_allclose(oracle.cheb_conv(x, ei, Ws[:K], b, w, "sym", lam), want, rtol=1e-4, atol=1e-4)
+    # per-graph lambda_max through the batch vector: two halves scaled apart
+    batch = (np.arange(V) >= V // 2).astype(np.int64)
+    lam2 = np.array([2.0, 4.0], np.float32)
+    bi, bw = oracle.cheb_norm(ei, V, w, "sym", lam2, batch)
+    si, sw = oracle.get_laplacian(ei, w, "sym", V)
+    want = 2 * sw / lam2[batch[si[0]]] - (si[0] == si[1])
+    np.testing.assert_allclose(bw, want, rtol=1e-6)
+
+
 # ------------------------------------------------------------ GAT pieces ----
 
 def test_gat_forward_matches_dense_fp64():
