@@ -37,7 +37,10 @@ jittor==1.3.9.14).  Pins of the numpy restatements at the end of this file:
   bernnet       dense fp64 sum_i C(K,i)/2^K t_i A1^i A2^(K-i) x; the binomial theorem
                 (A1 = L, A2 = 2I - L, t = 1 gives x back)
   gpuinitco / getweight / csctocsr  brute-force Python loops on small graphs,
-                the README's CSC -> CSR known answer
+                the README's CSC -> CSR known answer, the inputs of the reference's
+                test_getweight.py with the expected list that test carries, those of
+                test_gpuinitco.py / test_fromtonodes.py / test_edgetovertex.py /
+                test_scatter_to_edge.py with hand-derived answers
   sampleprocessing  "parity unpinned": the reference draws with rand() /
                 clock-seeded curand, so no output of it can be reproduced.  Pinned
                 here: the copy branch exactly, and for the sampled branch the

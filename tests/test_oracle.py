@@ -747,3 +747,26 @@ def test_cross_entropy_closed_forms():
     # very large logits stay finite
     big = np.array([[1e4, -1e4, 0.0]])
     assert abs(oracle.cross_entropy_loss(big, [1])[0] - 2e4) < 1e-6
+
+
+# ------------------------------------- literal inputs of the reference's remaining tests ---
+def test_reference_test_inputs_getweight_gpuinitco_fromtonodes_scatter():
+    g = GOLD["getweight_v4"]
+    w = oracle.getweight(g["vtx_size"], np.array(g["dst"]), np.array(g["src"]), np.array(g["column_offset"]),
+                         np.array(g["row_indices"]))
+    np.testing.assert_allclose(w, g["edge_weight"], rtol=2e-7)
+    g = GOLD["gpuinitco_v4"]
+    out = oracle.gpuinitco(g["dst_size"], g["fanout"], np.array(g["csc_layer_dst"]), np.array(g["csc_global_column_offset"]))
+    assert out.tolist() == g["out"]
+    g = GOLD["fromtonodes_v5"]
+    a = oracle.from_nodes(g["column_offset"], g["row_indices"], g["nodes"])
+    b = oracle.from_nodes(g["row_offset"], g["column_indices"], g["nodes"])
+    assert a.tolist() == g["from_nodes"] and b.tolist() == g["to_nodes"]
+    assert sorted(set(a.tolist())) == g["from_nodes_as_set"] and sorted(set(b.tolist())) == g["to_nodes_as_set"]
+    g = GOLD["edgetovertex_v3"]
+    out = oracle.edgetovertex(np.array(g["x"], np.float32), g["row_indices"], g["column_offset"], 1)
+    assert out.tolist() == g["out"]
+    g = GOLD["scatter_to_edge_v3"]
+    x = np.array(g["x"], np.float32)
+    assert oracle.scattertoedge(x, g["row_indices"], g["column_offset"], 1).tolist() == g["out_dst"]
+    assert oracle.scattertoedge(x, g["row_indices"], g["column_offset"], 0).tolist() == g["out_src"]
