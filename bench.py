@@ -790,6 +790,12 @@ def config5(b):
         xf = torch.randn(V, F, device=dev)
         prod[F] = (b.timed(lambda xf=xf: spmm(csc.column_offset, csc.row_indices, csc.edge_weight, xf, V), 10, 2),
                    b.spmm_kernel_ms(csc.column_offset, csc.row_indices, csc.edge_weight, xf, V, 10)[0], xf)
+    f47_padded_ms = None
+    if not main_only:
+        # the same product with the rows of x 64 floats apart, as the 256 -> 47 layer's x @ W is written
+        x47 = torch.randn(V, 64, device=dev)[:, :47]
+        f47_padded_ms = b.timed(lambda: spmm(csc.column_offset, csc.row_indices, csc.edge_weight, x47, V), 10, 2)
+        del x47
     cpu, err = (None, 0.0)
     if not args.no_cpu_baseline and not main_only:
         xf = prod[256][2]
@@ -810,6 +816,9 @@ def config5(b):
     for F in widths:
         line["spmm_f%d_ms" % F] = round(prod[F][0], 4)
         line["spmm_f%d_algorithmic_gbps" % F] = round(spmm_bytes(V, E, F) / (prod[F][0] * 1e-3) / 1e9, 1)
+    if f47_padded_ms is not None:
+        line["spmm_f47_rows_64_apart_ms"] = round(f47_padded_ms, 4)
+        line["spmm_f47_rows_64_apart_algorithmic_gbps"] = round(spmm_bytes(V, E, 47) / (f47_padded_ms * 1e-3) / 1e9, 1)
     line["roofline"] = roofline("spmm_merge_powerlaw_2m4_f256.txt", {"V": V, "E": E, "F": 256}, "spmm_merge", prod[256][1],
                                 spmm_bytes(V, E, 256), spmm_compulsory_bytes(V, V, E, 256), "hipEvents in this run",
                                 b.copy_rate_gbps())

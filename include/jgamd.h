@@ -42,6 +42,10 @@ extern "C" {
 
 /* flag of the entry points that finish output rows: clamp the row at zero (ReLU) */
 #define JGAMD_ROW_RELU 1
+/* jgamd_spmm_csx_planned, or-ed into `flags`: the rows of x lie n floats apart (n >= F, a
+ * multiple of 4; a producer that pads its rows to whole 128-byte lines, e.g. a BLAS product
+ * written with that leading dimension, spares the gathers the lines an odd width straddles) */
+#define JGAMD_ROW_X_STRIDE(n) ((int32_t)(n) << 8)
 
 /* Library version, major*10000 + minor*100 + patch. */
 int32_t jgamd_version(void);

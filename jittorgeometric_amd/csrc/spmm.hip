@@ -725,7 +725,15 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_planned
     const float *w, const float *x, float *out, float beta, float alpha, const float *h, int32_t h_rows,
     int32_t flags, int32_t R, int32_t C, int64_t E, int32_t F, void *ws, size_t ws_bytes, void *stream)
 {
+    // bits 8 and up: floats between the rows of x when they are padded apart (0 = F)
+    const int32_t x_stride = flags >> 8;
+    flags &= 0xff;
     if (flags & ~JGAMD_ROW_RELU) return fail(JGAMD_ERR_SIZE, "spmm_csx_planned: unknown flags %d", flags);
+    if (x_stride != 0 && (x_stride < F || (x_stride & 3) != 0))
+        return fail(JGAMD_ERR_SIZE, "spmm_csx_planned: x row stride %d must be a multiple of 4 floats and at least F=%d",
+                    x_stride, F);
+    if (x_stride != 0 && !plan)
+        return fail(JGAMD_ERR_NULL, "spmm_csx_planned: rows of x padded apart take the chunk kernels: pass the chunk plan");
     if (!plan && !tiles) return fail(JGAMD_ERR_NULL, "spmm_csx_planned: plan and tiles are both NULL");
     if (!plan && !narrow_width(F))
         return fail(JGAMD_ERR_NULL, "spmm_csx_planned: rows of %d floats need the chunk plan, not the tile plan", F);
@@ -740,7 +748,7 @@ extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_planned
     const bool plain = beta == 1.f && (alpha == 0.f || !h) && flags == 0;
     const RowFinish fin{beta, alpha, alpha != 0.f ? h : nullptr, h_rows == 1 ? 0 : F, 0, (flags & JGAMD_ROW_RELU) ? 1 : 0};
     return spmm_call(off, idx, w, x, out, R, C, E, F, ws, ws_bytes, stream, nullptr, nullptr, plain ? nullptr : &fin,
-                     false, 0, plan, tiles, hints, true);
+                     false, x_stride == F ? 0 : x_stride, plan, tiles, hints, true);
 }
 
 extern "C" __attribute__((visibility("default"))) int32_t jgamd_spmm_csx_planned_workspace(int32_t R, int64_t E,

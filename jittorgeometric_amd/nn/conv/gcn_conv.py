@@ -94,7 +94,7 @@ class GcnLayerFunc(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, weight, bias, fwd, bwd, relu=False):
-        h = rows_times(x, weight)
+        h = rows_times(x, weight, pad_rows=True)      # gathered next: rows of an odd width start on a line
         if bias is not None or relu:
             out = spmm_axpby(fwd[0], fwd[1], fwd[2], h, x.shape[0], 1.0, 1.0, bias, relu)
         else:

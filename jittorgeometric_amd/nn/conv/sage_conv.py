@@ -83,7 +83,7 @@ class SageTransformFirstFunc(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, w1, w_root, bias, fwd, bwd):
-        h1 = rows_times(x, w1)
+        h1 = rows_times(x, w1, pad_rows=True)     # gathered next
         rest = None
         if w_root is not None:
             rest = rows_times(x, w_root, bias=bias)

@@ -199,7 +199,14 @@ def _product(off, idx, w, x, R, beta, alpha, h, relu=False):
     result is clamped at zero, in the product's row store where the kernels offer it."""
     lib = _lib.load()
     dev = _lib.require_gpu(off, x, idx, w, h)
-    x = as_f32(x, "x")
+    # rows padded apart (a [V,F] view of a wider buffer, as rows_times(..., pad_rows=True) returns):
+    # gathered in place by the planned chunk kernels
+    x_stride = 0
+    if (x.dim() == 2 and x.dtype == torch.float32 and x.stride(1) == 1 and x.stride(0) > x.shape[1]
+            and x.stride(0) % 4 == 0 and x.stride(0) < 1 << 22 and x.data_ptr() % 16 == 0):
+        x_stride = x.stride(0)
+    else:
+        x = as_f32(x, "x")
     off, idx, w = _raw_arrays(off, idx, w, R)
     if x.dim() != 2:
         raise _lib.JgamdError("x must be [rows, F], got %s" % (tuple(x.shape),))
@@ -218,6 +225,8 @@ def _product(off, idx, w, x, R, beta, alpha, h, relu=False):
     if idx is not None:
         _lib.check(lib.jgamd_spmm_block_plan(R, C, E, F, _c.byref(nb), _c.byref(cols)))
     if nb.value > 0:
+        x = x.contiguous()
+        x_stride = 0
         b_off, b_idx, b_w = _blocked_arrays(off, idx, w, R, E, nb.value, cols.value)
         nbytes = _lib.query(lib.jgamd_spmm_csx_blocked_workspace, R, C, E, F, nb.value)
         ws = _lib.workspace(nbytes, dev)
@@ -229,16 +238,20 @@ def _product(off, idx, w, x, R, beta, alpha, h, relu=False):
     # plain products with rows of 1, 2, 4 or 8 floats (the tile kernels have no row finish and
     # read whole aligned rows)
     plain = h is None and beta == 1.0 and not relu
-    narrow = (F in (1, 2, 4, 8) and E > 0 and plain and x.data_ptr() % min(16, 4 * F) == 0
+    narrow = (F in (1, 2, 4, 8) and E > 0 and plain and x.data_ptr() % min(16, 4 * F) == 0 and not x_stride
               and not os.environ.get("JGAMD_SPMM_NARROW", "").startswith("m"))
     plan, n_fix, n_grp = csx_plan(off, R, E, PLAN_TILES if narrow else PLAN_SPMM) if R > 0 else (None, -1, -1)
+    if plan is None and x_stride:
+        x = x.contiguous()          # only the planned entry point takes padded rows
+        x_stride = 0
     if plan is not None:
         nbytes = _lib.query(lib.jgamd_spmm_csx_planned_workspace, R, E, F)
         ws = _lib.workspace(nbytes, dev)
         _lib.check(lib.jgamd_spmm_csx_planned(None if narrow else _lib.ptr(plan), _lib.ptr(plan) if narrow else None,
                                               n_fix, n_grp, _lib.ptr(off), _lib.ptr(idx), _lib.ptr(w), _lib.ptr(x),
                                               _lib.ptr(out), float(beta), float(alpha), _lib.ptr(h), h_rows,
-                                              1 if relu else 0, R, C, E, F, _lib.ptr(ws), nbytes, stream))
+                                              (1 if relu else 0) | (x_stride << 8), R, C, E, F, _lib.ptr(ws), nbytes,
+                                              stream))
         return out
     nbytes = _lib.query(lib.jgamd_spmm_csx_workspace, R, E, F)
     ws = _lib.workspace(nbytes, dev)

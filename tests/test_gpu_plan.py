@@ -365,3 +365,55 @@ def test_plan_entry_points_reject_bad_arguments():
     assert l.jgamd_spmm_csx_planned(bad, None, -1, -1, bad, bad, bad, bad, bad, 1.0, 0.0, None, 1, 2, 4, 4, 5, 16, bad,
                                     1 << 20, None) == -2                        # unknown flag
     assert l.jgamd_edge_softmax_fwd_planned(None, bad, bad, bad, 4, 5, 1, bad, 1 << 20, None) == -1
+
+
+@pytest.mark.parametrize("F,wide", [(47, 64), (33, 64), (100, 128), (130, 160), (64, 96)])
+def test_rows_of_x_padded_apart(F, wide):
+    """x as a [C,F] view of rows `wide` floats apart: gathered in place, the same bits as from a
+    dense copy, with and without a row finish."""
+    from jittorgeometric_amd.ops._common import csx_plan, spmm, spmm_axpby
+    rng = np.random.default_rng(F)
+    V, E = 3000, 90000
+    idx, off, wt = csc_of(rng, V, E, 2, 0.4)
+    off_g, idx_g, w_g = to_gpu(off), to_gpu(idx), to_gpu(wt)
+    buf = torch.full((V, wide), float("nan"), dtype=torch.float32, device=dev())
+    x = buf[:, :F]
+    x.copy_(to_gpu(rng.standard_normal((V, F)).astype(np.float32)))
+    assert x.stride(0) == wide and not x.is_contiguous()
+    dense = x.contiguous()
+    h = to_gpu(rng.standard_normal((V, F)).astype(np.float32))
+    csx_plan(off_g, V, E, SPMM, now=True)                 # the planned entry point is the one that takes a stride
+    assert torch.equal(spmm(off_g, idx_g, w_g, x, V), spmm(off_g, idx_g, w_g, dense, V))
+    assert torch.equal(spmm_axpby(off_g, idx_g, w_g, x, V, 0.7, 0.3, h, relu=True),
+                       spmm_axpby(off_g, idx_g, w_g, dense, V, 0.7, 0.3, h, relu=True))
+    want, terms = oracle.aggregate_f64(dense.cpu().numpy(), idx, off, wt)
+    assert_close(spmm(off_g, idx_g, w_g, x, V).cpu().numpy(), want, terms, what="padded rows F=%d" % F)
+    # offsets without a plan yet (first use): the wrapper falls back to a dense copy, same result
+    off2 = off_g.clone()
+    assert torch.equal(spmm(off2, idx_g, w_g, x, V), spmm(off_g, idx_g, w_g, dense, V))
+    # through the C ABI: a stride below F, or not a multiple of 4 floats, is refused
+    L, l = lib()
+    plan, n_fix, n_grp = build_plan(off_g, V, E, SPMM)
+    out = torch.empty((V, F), dtype=torch.float32, device=dev())
+    nbytes = L.query(l.jgamd_spmm_csx_planned_workspace, V, E, F)
+    ws = L.workspace(nbytes, dev())
+    for bad in (F - 1 if (F - 1) % 4 == 0 else F - (F % 4) - 4, wide + 2):
+        rc = l.jgamd_spmm_csx_planned(L.ptr(plan), None, n_fix, n_grp, L.ptr(off_g), L.ptr(idx_g), L.ptr(w_g), L.ptr(x),
+                                      L.ptr(out), 1.0, 0.0, None, V, bad << 8, V, V, E, F, L.ptr(ws), nbytes,
+                                      L.stream_ptr(dev()))
+        assert rc == -2 and b"stride" in l.jgamd_last_error(), bad
+
+
+def test_blas_route_writes_padded_rows():
+    from jittorgeometric_amd.nn.dense import padded_width, rows_times
+    assert [padded_width(n) for n in (7, 32, 33, 40, 41, 47, 64, 80, 100, 128, 130)] == [7, 32, 33, 40, 64, 64, 64, 80, 100, 128, 130]
+    rng = np.random.default_rng(3)
+    x = to_gpu(rng.standard_normal((5000, 256)).astype(np.float32))
+    w = to_gpu(rng.standard_normal((256, 47)).astype(np.float32))
+    b = to_gpu(rng.standard_normal(47).astype(np.float32))
+    for bias in (None, b):
+        got = rows_times(x, w, bias=bias, pad_rows=True)
+        assert got.shape == (5000, 47) and got.stride() == (64, 1)
+        ref = rows_times(x, w, bias=bias)
+        assert ref.is_contiguous() and torch.allclose(got, ref, rtol=1e-5, atol=1e-5)
+    assert rows_times(x, to_gpu(rng.standard_normal((256, 128)).astype(np.float32)), pad_rows=True).is_contiguous()
